@@ -1,0 +1,328 @@
+#!/usr/bin/env python3
+"""Benchmark of the KV-cache / attention hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-cpu-baseline]
+
+A step is one pass of the hot path over one batch of synthetic input:
+
+  decode workloads   one decode step = for every layer (append one token if the workload says so,
+                     then split-K decode attention + merge).  Metric: KV bytes read per second.
+  prefill workload   for every layer: append the 512-token chunk, then causal batched attention.
+                     Metric: TFLOP/s.
+
+The default workload is the one the headline metric is quoted on: 32 layers, FP8 KV, 32768 keys,
+32/8/128 heads.  Inputs are resident in HBM before the timed region.  After the timed region the
+same launches are replayed with HIP events around each launch of the dominant kernel (on the
+stream it runs on) to obtain its average duration for the roofline entry, and the CPU oracle is
+timed on a bounded sample of the same workload on the host cores of this machine.
+Prints one JSON line.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0       # MI355X HBM3E, published
+MFMA_F16_PEAK_TFLOPS = 2500.0
+
+
+def parse_args():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--workload", default="decode_fp8_32k_32layers")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--cpu-seconds", type=float, default=12.0, help="target CPU time of the baseline sample")
+    ap.add_argument("--seed", type=int, default=1234)
+    ap.add_argument("--no-graph", action="store_true",
+                    help="launch every kernel from Python instead of replaying one captured HIP graph per step")
+    return ap.parse_args()
+
+
+def fill_cache(torch, vf, fwd, wl, n_tokens, seed, outliers):
+    """Seeded synthetic K/V: N(0,1) rounded to fp16 (or N(0,1)*0.5 with a 1 % tail at +-40), written
+    through the append kernels so the cache holds exactly what the product would have written."""
+    g = torch.Generator(device="cuda").manual_seed(seed)
+    cache = fwd.kv_cache
+    chunk = 4096
+    for layer in range(wl.n_layers):
+        row = cache.kv_heads_for(layer) * cache.head_dim_for(layer)
+        for base in range(0, n_tokens, chunk):
+            n = min(chunk, n_tokens - base)
+            ks = torch.randn((n, row), device="cuda", generator=g)
+            vs = torch.randn((n, row), device="cuda", generator=g)
+            if outliers:
+                for x in (ks, vs):
+                    x.mul_(0.5)
+                    hit = torch.rand(x.shape, device="cuda", generator=g) < 0.01
+                    sign = torch.where(torch.rand(x.shape, device="cuda", generator=g) < 0.5, -40.0, 40.0)
+                    x.copy_(torch.where(hit, sign, x))
+            else:
+                ks, vs = ks.half().float(), vs.half().float()
+            fwd.b_step_kv_write(layer, base, n, ks, vs)
+    torch.cuda.synchronize()
+
+
+def time_steps(torch, step, args):
+    """W untimed steps, then exactly K timed steps between two device synchronisations.  One step's
+    launches are captured once into a HIP graph and replayed, so the host's per-launch cost (Python
+    and ctypes here) does not gate a step that is only a few hundred microseconds of GPU work."""
+    run = step
+    if not args.no_graph:
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            step()                       # first-use initialisation must not happen under capture
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            step()
+        run = graph.replay
+    for _ in range(args.warmup):
+        run()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        run()
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) / args.steps
+
+
+def bench_decode(args, wl):
+    import torch
+
+    import vulkanforge_amd as vf
+    from vulkanforge_amd import _ffi
+
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    L, H, Hkv, D = wl.n_layers, wl.n_heads, wl.n_kv_heads, wl.head_dim
+    max_seq = wl.context
+    es = wl.dtype.element_size()
+    nbytes = L * max_seq * Hkv * D * es
+    kbuf = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+    vbuf = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+    cache = vf.KvCache(vf.KvCacheConfig(L, Hkv, D, max_seq, dtype=wl.dtype), k_buffer=kbuf.data_ptr(),
+                       v_buffer=vbuf.data_ptr())
+    fwd = vf.Forward(cache, H)
+    outliers = wl.name == "decode_fp8_8k_32layers"
+    fill_cache(torch, vf, fwd, wl, max_seq, args.seed, outliers)
+
+    g = torch.Generator(device="cuda").manual_seed(args.seed + 1)
+    q = torch.randn((L, H, D), device=dev, generator=g).half().float()
+    o = torch.zeros((L, H, D), device=dev)
+    k_new = torch.randn((L, Hkv * D), device=dev, generator=g).half().float()
+    v_new = torch.randn((L, Hkv * D), device=dev, generator=g).half().float()
+    pos = wl.context - 1
+    scale = 1.0 / (D ** 0.5)
+    starts = [_ffi.lib().vfkv_kv_start_decode(pos, wl.layer_window(i)) if wl.layer_window(i) else 0 for i in range(L)]
+
+    def step():
+        for layer in range(L):
+            if wl.append:
+                fwd.step_kv_write(layer, pos, k_new[layer], v_new[layer])
+            fwd.run_scalar_attn(layer, pos, q[layer], o[layer], kv_start=starts[layer], scale=scale,
+                                softcap=wl.softcap)
+
+    sec_per_step = time_steps(torch, step, args)
+    bytes_step = wl.kv_bytes_step()
+
+    # ---- replay with HIP events around every launch of the split worker (the dominant kernel) ----
+    stream = torch.cuda.current_stream()
+    lib = _ffi.lib()
+    max_tiles = (max_seq + 63) // 64
+    so = torch.empty((H * max_tiles * D,), device=dev)
+    sm = torch.empty((H * max_tiles,), device=dev)
+    ss = torch.empty((H * max_tiles,), device=dev)
+    n_ev = min(args.steps, 20)
+    pairs = []
+    for _ in range(n_ev):
+        for layer in range(L):
+            span = wl.context - starts[layer]
+            tile = lib.vfkv_decode_tile_for(span, H, Hkv)
+            klay = cache.k_ptr + cache.layer_offset_bytes(layer)
+            vlay = cache.v_ptr + cache.layer_offset_bytes(layer)
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record(stream)
+            nt = fwd.run_flash_attn_split(q[layer], klay, vlay, wl.dtype, so, sm, ss, H, Hkv, D, wl.context, scale,
+                                          kv_start=starts[layer], tile=tile, softcap=wl.softcap)
+            e1.record(stream)
+            fwd.run_flash_attn_reduce(so, sm, ss, o[layer], H, D, nt)
+            pairs.append((layer, e0, e1))
+    torch.cuda.synchronize()
+    # byte-weighted: total algorithmic bytes / total kernel time == bytes per launch / mean duration
+    split_ms = sum(e0.elapsed_time(e1) for _l, e0, e1 in pairs)
+    launches = len(pairs)
+    bytes_launch = bytes_step / L
+    avg_ms = split_ms / launches
+    achieved = bytes_launch / (avg_ms * 1e-3) / 1e9
+
+    result = {
+        "metric": "kv_read_GBps_decode_step",
+        "value": bytes_step / sec_per_step / 1e9,
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": sec_per_step * 1e3,
+        "us_per_decode_step": sec_per_step * 1e6,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "kv_dtype": wl.dtype.label(),
+        "launch": "eager" if args.no_graph else "hip_graph",
+        "data": "synthetic (seeded N(0,1) rounded to fp16; cache written by the append kernels)",
+        "config": {"workload": wl.name, "n_layers": L, "n_heads": H, "n_kv_heads": Hkv, "head_dim": D,
+                   "context": wl.context, "append_per_step": wl.append, "kv_bytes_per_step": bytes_step,
+                   "pct_of_hbm_peak": 100.0 * bytes_step / sec_per_step / 1e9 / HBM_PEAK_GBPS},
+        "roofline": {"bound": "hbm", "kernel": "split_kernel", "achieved": achieved, "peak": HBM_PEAK_GBPS,
+                     "unit": "GB/s", "frac": achieved / HBM_PEAK_GBPS, "traffic": None,
+                     "avg_launch_us": avg_ms * 1e3, "launches_timed": launches,
+                     "algorithmic_bytes_per_launch": bytes_launch},
+    }
+
+    if not args.no_cpu_baseline:
+        import numpy as np
+
+        import oracle
+        threads = len(os.sched_getaffinity(0))
+        per_layer = L * max_seq * Hkv * D * es // L
+        done_bytes, spent, layers_done = 0, 0.0, 0
+        for layer in range(L):
+            lo = layer * per_layer
+            kh = kbuf[lo:lo + per_layer].cpu().numpy().view(oracle.NP_DTYPE[int(wl.dtype)]).reshape(max_seq, Hkv, D)
+            vh = vbuf[lo:lo + per_layer].cpu().numpy().view(oracle.NP_DTYPE[int(wl.dtype)]).reshape(max_seq, Hkv, D)
+            qh = q[layer].cpu().numpy()
+            c0 = time.perf_counter()
+            ref = oracle.attn_decode_ref(qh, kh, vh, int(wl.dtype), H, Hkv, D, wl.context, scale,
+                                         kv_start=starts[layer], softcap=wl.softcap, threads=threads)
+            spent += time.perf_counter() - c0
+            done_bytes += wl.kv_bytes_layer(layer)
+            layers_done += 1
+            if layer == 0:   # the timed GPU output of this layer also has to agree with the oracle
+                err = float(np.abs(o[layer].cpu().numpy() - ref).max())
+                result["config"]["max_abs_err_vs_oracle_layer0"] = err
+            if spent >= args.cpu_seconds:
+                break
+        result["cpu_baseline"] = {"value": done_bytes / spent / 1e9, "unit": "GB/s", "cores": threads, "kind": "port",
+                                  "sample": f"{layers_done} of {L} layers of the same step, CPU oracle "
+                                            f"(attn_decode_ref, f64 accumulation), {spent:.1f} s"}
+    cache.destroy()
+    return result
+
+
+def bench_prefill(args, wl):
+    import torch
+
+    import vulkanforge_amd as vf
+
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    L, H, Hkv, D = wl.n_layers, wl.n_heads, wl.n_kv_heads, wl.head_dim
+    max_seq = wl.base_pos + wl.m
+    es = wl.dtype.element_size()
+    per_layer = max_seq * Hkv * D * es
+    kbuf = torch.empty(L * per_layer, dtype=torch.uint8, device=dev)
+    vbuf = torch.empty(L * per_layer, dtype=torch.uint8, device=dev)
+    cache = vf.KvCache(vf.KvCacheConfig(L, Hkv, D, max_seq, dtype=wl.dtype), k_buffer=kbuf.data_ptr(),
+                       v_buffer=vbuf.data_ptr())
+    fwd = vf.Forward(cache, H)
+
+    class _W:  # fill_cache only needs n_layers
+        n_layers = L
+    fill_cache(torch, vf, fwd, _W, wl.base_pos, args.seed, False)
+    g = torch.Generator(device="cuda").manual_seed(args.seed + 1)
+    q = torch.randn((wl.m, H, D), device=dev, generator=g).half().float()
+    kn = torch.randn((wl.m, Hkv * D), device=dev, generator=g).half().float()
+    vn = torch.randn((wl.m, Hkv * D), device=dev, generator=g).half().float()
+    o = torch.zeros((wl.m, H, D), device=dev)
+
+    def step():
+        for layer in range(L):
+            fwd.b_step_kv_write(layer, wl.base_pos, wl.m, kn, vn)
+            fwd.b_step_attention(layer, wl.base_pos, wl.m, q, o)
+
+    sec_per_step = time_steps(torch, step, args)
+    flops_step = wl.flops_layer() * L
+
+    stream = torch.cuda.current_stream()
+    pairs = []
+    for _ in range(min(args.steps, 5)):
+        for layer in range(L):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record(stream)
+            fwd.b_step_attention(layer, wl.base_pos, wl.m, q, o)
+            e1.record(stream)
+            pairs.append((e0, e1))
+    torch.cuda.synchronize()
+    avg_ms = sum(a.elapsed_time(b) for a, b in pairs) / len(pairs)
+    achieved = wl.flops_layer() / (avg_ms * 1e-3) / 1e12
+    result = {
+        "metric": "prefill_attention_TFLOPs",
+        "value": flops_step / sec_per_step / 1e12,
+        "unit": "TFLOP/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": sec_per_step * 1e3,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f16", "kv_dtype": wl.dtype.label(),
+        "data": "synthetic (seeded N(0,1) rounded to fp16)",
+        "config": {"workload": wl.name, "n_layers": L, "n_heads": H, "n_kv_heads": Hkv, "head_dim": D,
+                   "m": wl.m, "q_start": wl.base_pos, "n_kv": max_seq, "flop_per_step": flops_step},
+        "roofline": {"bound": "mfma", "kernel": "flash_attn_batch", "achieved": achieved, "peak": MFMA_F16_PEAK_TFLOPS,
+                     "unit": "TFLOP/s", "frac": achieved / MFMA_F16_PEAK_TFLOPS, "traffic": None,
+                     "avg_launch_us": avg_ms * 1e3},
+    }
+    if not args.no_cpu_baseline:
+        import numpy as np
+
+        import oracle
+        threads = len(os.sched_getaffinity(0))
+        kh = kbuf[:per_layer].cpu().numpy().view(oracle.NP_DTYPE[int(wl.dtype)]).reshape(max_seq, Hkv, D)
+        vh = vbuf[:per_layer].cpu().numpy().view(oracle.NP_DTYPE[int(wl.dtype)]).reshape(max_seq, Hkv, D)
+        ms = 8                       # the last `ms` query rows of layer 0, repeated until the time target
+        qs = wl.base_pos + wl.m - ms
+        qh = q[wl.m - ms:].cpu().numpy()
+        flops_sample = sum(qs + i + 1 for i in range(ms)) * H * 4 * D
+        spent, reps, ref = 0.0, 0, None
+        while spent < args.cpu_seconds and reps < 64:
+            c0 = time.perf_counter()
+            ref = oracle.attn_batch_ref(qh, kh, vh, int(wl.dtype), ms, max_seq, H, Hkv, D, qs, 1.0 / D ** 0.5,
+                                        threads=threads)
+            spent += time.perf_counter() - c0
+            reps += 1
+        err = float(np.abs(o[wl.m - ms:].cpu().numpy() - ref).max())
+        result["config"]["max_abs_err_vs_oracle_last_rows"] = err
+        result["cpu_baseline"] = {"value": flops_sample * reps / spent / 1e12, "unit": "TFLOP/s", "cores": threads,
+                                  "kind": "port",
+                                  "sample": f"last {ms} of {wl.m} query rows of layer 0, {reps} repetitions, CPU "
+                                            f"oracle (attn_batch_ref, f64), {spent:.1f} s"}
+    cache.destroy()
+    return result
+
+
+def main():
+    args = parse_args()
+    if args.gpus != 1:
+        print(f"bench.py measures one GPU only (got --gpus {args.gpus}): this build has no multi-GPU path.",
+              file=sys.stderr)
+        sys.exit(2)
+    from vulkanforge_amd import workloads
+    if args.workload in workloads.DECODE:
+        res = bench_decode(args, workloads.DECODE[args.workload])
+    elif args.workload in workloads.PREFILL:
+        res = bench_prefill(args, workloads.PREFILL[args.workload])
+    else:
+        print("unknown workload; choose from: " + ", ".join(list(workloads.DECODE) + list(workloads.PREFILL)),
+              file=sys.stderr)
+        sys.exit(2)
+    print(json.dumps(res))
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,226 @@
+/*
+ * vfkv.h -- C ABI of the MI355X (gfx950) KV-cache / attention hot path.
+ *
+ * Every entry point replaces one piece of the reference's Vulkan dispatch layer; the reference
+ * location is cited next to it (paths relative to the reference tree).  Conventions:
+ *
+ *   - All data pointers are HIP device pointers owned by the caller, except the two cache
+ *     buffers owned by a `vfkv_cache` created with vfkv_cache_create().
+ *   - `stream` is a hipStream_t passed as void* (NULL = the default stream).  Functions only
+ *     enqueue work on it (the analogue of "record into the open command buffer") and never
+ *     synchronise; ordering between calls is stream order, which replaces the reference's
+ *     in-command-buffer barriers (executor/attention.rs:583-595, runs.rs:1539-1541).
+ *   - Return value: VFKV_OK (0) or a negative vfkv_status.  Nothing panics or aborts across the
+ *     ABI; vfkv_last_error() returns a thread-local description of the last failure.
+ *   - Thread-compatible: distinct caches / workspaces / streams may be used from distinct
+ *     threads; one workspace must not be used by two in-flight calls at once.
+ *   - There is no CPU fallback: without a HIP device every compute entry point fails with
+ *     VFKV_ERR_HIP / VFKV_ERR_NO_DEVICE.  Layout arithmetic works without a device.
+ */
+#ifndef VFKV_H
+#define VFKV_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define VFKV_ABI_VERSION 1u
+
+typedef void* vfkv_stream; /* hipStream_t */
+
+typedef enum vfkv_status {
+    VFKV_OK = 0,
+    VFKV_ERR_INVALID_ARG = -1, /* NULL pointer, zero dimension, n_heads % n_kv_heads != 0, ... */
+    VFKV_ERR_OVERFLOW = -2,    /* size arithmetic does not fit (kv_cache.rs:270-291) */
+    VFKV_ERR_ALIGNMENT = -3,   /* dst_byte_offset % 4 != 0 (runs.rs:2400-2404, 2448-2453) */
+    VFKV_ERR_UNSUPPORTED = -4, /* shape outside what the kernels cover (e.g. head_dim > 512) */
+    VFKV_ERR_HIP = -5,         /* a HIP runtime call failed; see vfkv_last_error() */
+    VFKV_ERR_NO_DEVICE = -6,
+    VFKV_ERR_WORKSPACE = -7    /* workspace too small for the requested launch */
+} vfkv_status;
+
+/* KvDtype, kv_cache.rs:42-74 (element_size 4 / 2 / 1). */
+typedef enum vfkv_dtype { VFKV_F32 = 0, VFKV_F16 = 1, VFKV_F8E4M3 = 2 } vfkv_dtype;
+
+const char* vfkv_status_string(int status);
+const char* vfkv_last_error(void);
+uint32_t vfkv_abi_version(void);
+/* Number of visible HIP devices (0 when there is none or the runtime cannot initialise). */
+int vfkv_device_count(void);
+
+/* ------------------------------------------------------------------------------------------ */
+/* KV cache object -- replaces `KvCache` (kv_cache.rs:204-500).                                */
+/* Pos-major layout K[layer][pos][kv_head][d] (kv_cache.rs:3-12), two buffers K and V.         */
+/* ------------------------------------------------------------------------------------------ */
+
+/* KvCacheConfig, kv_cache.rs:153-174.  The per-layer tables may be NULL (uniform layout); when
+ * given they hold n_layers entries and select the cumulative-offset layout (kv_cache.rs:256-283). */
+typedef struct vfkv_cache_config {
+    uint32_t n_layers;
+    uint32_t n_kv_heads;
+    uint32_t head_dim;
+    uint32_t max_seq_len;
+    const uint32_t* per_layer_head_dim;
+    const uint32_t* per_layer_n_kv_heads;
+    uint32_t dtype; /* vfkv_dtype; the reference reads it from the environment (kv_cache.rs:85-101) */
+} vfkv_cache_config;
+
+typedef struct vfkv_cache vfkv_cache;
+
+/* KvCache::new (kv_cache.rs:224-339): checked size arithmetic, then two device allocations. */
+int vfkv_cache_create(const vfkv_cache_config* cfg, vfkv_cache** out);
+/* Same layout object over caller-owned buffers (either may be NULL for layout-only use, e.g. on a
+ * host without a GPU).  No allocation happens and destroy() leaves the buffers alone. */
+int vfkv_cache_create_external(const vfkv_cache_config* cfg, void* k_buffer, void* v_buffer,
+                               vfkv_cache** out);
+/* KvCache::destroy (kv_cache.rs:496-499). */
+void vfkv_cache_destroy(vfkv_cache* c);
+/* KvCache::zero_fill (kv_cache.rs:357-380) / zero_layer (kv_cache.rs:389-407). */
+int vfkv_cache_zero_fill(vfkv_cache* c, vfkv_stream stream);
+int vfkv_cache_zero_layer(vfkv_cache* c, uint32_t layer, vfkv_stream stream);
+/* current_seq_len field and KvCache::reset (kv_cache.rs:492-494). */
+uint32_t vfkv_cache_current_seq_len(const vfkv_cache* c);
+void vfkv_cache_set_current_seq_len(vfkv_cache* c, uint32_t n);
+void vfkv_cache_reset(vfkv_cache* c);
+
+void* vfkv_cache_k_ptr(const vfkv_cache* c);
+void* vfkv_cache_v_ptr(const vfkv_cache* c);
+uint32_t vfkv_cache_dtype(const vfkv_cache* c);
+uint64_t vfkv_cache_bytes_per_buffer(const vfkv_cache* c);                       /* kv_cache.rs:383 */
+uint32_t vfkv_cache_head_dim_for(const vfkv_cache* c, uint32_t layer);           /* kv_cache.rs:412 */
+uint32_t vfkv_cache_kv_heads_for(const vfkv_cache* c, uint32_t layer);           /* kv_cache.rs:422 */
+uint64_t vfkv_cache_layer_offset_elems(const vfkv_cache* c, uint32_t layer);     /* kv_cache.rs:431 */
+uint64_t vfkv_cache_pos_offset_bytes(const vfkv_cache* c, uint32_t layer, uint32_t pos); /* :446 */
+uint64_t vfkv_cache_row_bytes(const vfkv_cache* c, uint32_t layer);              /* kv_cache.rs:456 */
+uint64_t vfkv_cache_layer_offset_bytes(const vfkv_cache* c, uint32_t layer);     /* kv_cache.rs:466 */
+uint64_t vfkv_cache_layer_size_bytes(const vfkv_cache* c, uint32_t layer);       /* kv_cache.rs:485 */
+/* kv_bytes_per_token (kv_cache.rs:186-202), saturating. */
+uint64_t vfkv_kv_bytes_per_token(uint32_t n_layers, uint32_t n_kv_heads, uint32_t head_dim,
+                                 const uint32_t* per_layer_head_dim,
+                                 const uint32_t* per_layer_n_kv_heads, uint64_t elem_size);
+/* guard_kv_precision_inner (kv_cache.rs:127-151): 0 when the combination is allowed. */
+int vfkv_guard_kv_precision(int is_gemma4_moe, uint32_t dtype, int force);
+/* gemma4_kv_start (forward/arch/gemma4.rs:59-73): max(0, position + 1 - sliding_window). */
+uint32_t vfkv_kv_start_decode(uint32_t position, uint32_t sliding_window);
+/* b_step_attention (executor/attention.rs:2215-2219): window of the LAST query of the batch. */
+uint32_t vfkv_kv_start_batch(uint32_t base_pos, uint32_t seq_len, uint32_t window);
+
+/* ------------------------------------------------------------------------------------------ */
+/* KV append and expansion kernels.                                                           */
+/* ------------------------------------------------------------------------------------------ */
+
+/* Forward::run_kv_store_fp8 (forward/runs.rs:2437-2478) + kv_store_fp8.comp:42-67.
+ * dst[dst_byte_offset + i] = e4m3(src[i]) for i < n_elements, saturating round-to-nearest-even
+ * E4M3FN (fp8_ext.rs:126-186); the tail of the last 32-bit word is zero-filled. */
+int vfkv_store_fp8(const float* src, void* dst, uint32_t n_elements, uint64_t dst_byte_offset,
+                   vfkv_stream stream);
+/* Forward::run_kv_copy_fp16 (forward/runs.rs:2389-2430) + kv_copy_fp16.comp:39-51. */
+int vfkv_copy_fp16(const float* src, void* dst, uint32_t n_elements, uint64_t dst_byte_offset,
+                   vfkv_stream stream);
+/* The kv_fp8_to_f16 pass of run_flash_attn_cm_gemma_rs (forward/runs.rs:1105-1137) +
+ * kv_fp8_to_f16.comp:28-33: dst_f16[i] = f16(e4m3_decode(src[i])), i < n_elems. */
+int vfkv_fp8_to_f16(const void* src, void* dst_f16, uint64_t n_elems, vfkv_stream stream);
+
+/* step_kv_write (executor/attention.rs:546-597) and b_step_kv_write (:2134-2190): append
+ * `n_tokens` rows of K and of V (f32, [n_tokens, kv_heads_for(layer) * head_dim_for(layer)]) at
+ * position `pos` of `layer`, in the cache's dtype.  K and V go out in one launch.  For an F32
+ * cache this is the reference's plain buffer copy. */
+int vfkv_kv_write(vfkv_cache* c, uint32_t layer, uint32_t pos, uint32_t n_tokens,
+                  const float* k_src, const float* v_src, vfkv_stream stream);
+
+/* ------------------------------------------------------------------------------------------ */
+/* Decode attention: split-K worker + log-sum-exp merge.                                      */
+/* ------------------------------------------------------------------------------------------ */
+
+/* FlashAttnSplitPushConstants, pipeline.rs:553-569 (32 bytes, same field order). */
+typedef struct vfkv_split_params {
+    uint32_t n_heads;
+    uint32_t n_kv_heads;
+    uint32_t head_dim;
+    uint32_t seq_len;
+    uint32_t max_seq; /* unused by the kernels, kept for layout compatibility */
+    float scale;
+    uint32_t n_tiles; /* ceil(seq_len / tile) */
+    uint32_t kv_start;
+} vfkv_split_params;
+
+/* Forward::run_flash_attn_split_reduce, worker half (forward/runs.rs:1463-1537) +
+ * flash_attn_split.comp:82-162.  `k_layer` / `v_layer` point at the start of the layer's slab
+ * (buffer + layer_offset_bytes(kv_layer), runs.rs:1507-1508).  Tile j covers keys
+ * [j*tile, (j+1)*tile); partials go to scratch_out[(h*n_tiles + j)*head_dim + d] and
+ * scratch_max / scratch_sum[h*n_tiles + j].  The reference fixes tile = 64
+ * (flash_attn_split.comp:23-24); here it is a parameter (multiple of 16, <= 65536).
+ * `softcap` > 0 applies s <- softcap * tanh(s / softcap) after scaling (an extension: the
+ * reference has no attention soft-cap); 0 disables it. */
+int vfkv_flash_attn_split(const float* q, const void* k_layer, const void* v_layer, uint32_t kv_dtype,
+                          float* scratch_out, float* scratch_max, float* scratch_sum,
+                          const vfkv_split_params* p, uint32_t tile, float softcap,
+                          vfkv_stream stream);
+
+/* Forward::run_flash_attn_split_reduce, reducer half (forward/runs.rs:1543-1571) +
+ * flash_attn_reduce.comp:35-81 (FlashAttnReducePushConstants, pipeline.rs:573-580). */
+int vfkv_flash_attn_reduce(const float* scratch_out, const float* scratch_max,
+                           const float* scratch_sum, float* o, uint32_t n_heads, uint32_t head_dim,
+                           uint32_t n_tiles, vfkv_stream stream);
+
+/* Scratch for vfkv_decode_attention -- replaces fa_scratch_out/max/sum (forward/setup.rs:203-230),
+ * sized for ceil(max_seq_len / 64) tiles of n_heads * head_dim floats. */
+typedef struct vfkv_workspace vfkv_workspace;
+int vfkv_workspace_create(uint32_t n_heads, uint32_t head_dim, uint32_t max_seq_len,
+                          vfkv_workspace** out);
+void vfkv_workspace_destroy(vfkv_workspace* w);
+
+/* Tile length (keys per workgroup) vfkv_decode_attention uses for `span` visible keys.  No
+ * counterpart in the reference, which hard-codes 64 (runs.rs:766); exposed so that callers who
+ * drive vfkv_flash_attn_split / _reduce themselves can reproduce the same launch.  The
+ * environment variable VFKV_DECODE_TILE (a multiple of 64) overrides the choice. */
+uint32_t vfkv_decode_tile_for(uint32_t span, uint32_t n_heads, uint32_t n_kv_heads);
+
+/* Forward::run_scalar_attn (forward/runs.rs:722-822) == step_attention's body
+ * (executor/attention.rs:599-625): one decode query per head over keys [kv_start, position].
+ * `kv_layer` is the layer whose slab is read (Gemma-4 KV share, gemma4.rs:27-49; equals `layer`
+ * otherwise), `layer` selects head_dim_for / kv_heads_for.  `scale` and `kv_start` are supplied
+ * by the caller (runs.rs:734-760).  Chooses the tile length itself so that the launch fills the
+ * GPU, skips tiles below kv_start, and merges the partials on the same stream.  Short contexts
+ * go through the same kernels (the reference routes seq_len <= 64 to a single-workgroup shader,
+ * runs.rs:766-821; the result is the same attention). */
+int vfkv_decode_attention(vfkv_cache* c, uint32_t layer, uint32_t kv_layer, uint32_t n_heads,
+                          const float* q, float* o, uint32_t position, uint32_t kv_start, float scale,
+                          float softcap, vfkv_workspace* ws, vfkv_stream stream);
+
+/* ------------------------------------------------------------------------------------------ */
+/* Chunked-prefill causal attention over the cache.                                           */
+/* ------------------------------------------------------------------------------------------ */
+
+/* FlashAttnBatchPushConstants, pipeline.rs:592-611 (32 bytes, same field order). */
+typedef struct vfkv_batch_params {
+    uint32_t n_heads;
+    uint32_t n_kv_heads;
+    uint32_t head_dim;
+    uint32_t m;       /* queries in this batch */
+    uint32_t n_kv;    /* populated KV positions (= q_start + m) */
+    uint32_t q_start; /* KV position of the first query */
+    float scale;
+    uint32_t kv_start; /* one lower bound for the whole batch */
+} vfkv_batch_params;
+
+/* Forward::run_flash_attn_batch (forward/runs.rs:933-1010) + flash_attn_batch.comp:105-208.
+ * q and o are [m, n_heads, head_dim] row-major f32; query i sees keys
+ * [kv_start, min(q_start + i + 1, n_kv)). */
+int vfkv_flash_attn_batch(const float* q, const void* k_layer, const void* v_layer, uint32_t kv_dtype,
+                          float* o, const vfkv_batch_params* p, float softcap, vfkv_stream stream);
+
+/* b_step_attention's fallback route (executor/attention.rs:2192-2219, 2383-2390): batch attention
+ * of `m` queries starting at `base_pos` over the cache, kv_start derived from `window`
+ * (0 = full history) exactly as the reference does. */
+int vfkv_prefill_attention(vfkv_cache* c, uint32_t layer, uint32_t kv_layer, uint32_t n_heads,
+                           const float* q, float* o, uint32_t m, uint32_t base_pos, uint32_t window,
+                           float scale, float softcap, vfkv_stream stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* VFKV_H */

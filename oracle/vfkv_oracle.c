@@ -271,10 +271,17 @@ uint32_t vfo_kv_start_batch(uint32_t base_pos, uint32_t seq_len, uint32_t window
 /* ------------------------------------------------------------------------------------------
  * Element fetch by cache dtype  (flash_attn_split.comp:29-58 load_k/load_v)
  * ---------------------------------------------------------------------------------------- */
+static float g_e4m3_lut[256];
+static int g_e4m3_lut_ready = 0;
+__attribute__((constructor)) static void init_e4m3_lut(void) {
+    for (int i = 0; i < 256; ++i) g_e4m3_lut[i] = vfo_e4m3_to_f32((uint8_t)i);
+    g_e4m3_lut_ready = 1;
+}
+
 static inline float load_kv(const void* base, uint32_t dtype, uint64_t idx) {
     if (dtype == VFO_DTYPE_F32) return ((const float*)base)[idx];
     if (dtype == VFO_DTYPE_F16) return vfo_f16_to_f32(((const uint16_t*)base)[idx]);
-    return vfo_e4m3_to_f32(((const uint8_t*)base)[idx]);
+    return g_e4m3_lut[((const uint8_t*)base)[idx]]; /* table of vfo_e4m3_to_f32 over all 256 codes */
 }
 
 static inline float softcap_f32(float s, float cap) { return cap > 0.0f ? cap * tanhf(s / cap) : s; }

@@ -1,0 +1,169 @@
+"""CPU-only checks of the C-ABI library: it loads, exports every symbol the header declares, does
+the layout arithmetic of the reference (kv_cache.rs), and rejects bad arguments before touching a
+device.  No compute entry point is exercised here."""
+import ctypes as C
+import os
+import re
+
+import numpy as np
+import pytest
+
+import oracle
+import vulkanforge_amd as vf
+from vulkanforge_amd import _ffi
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared_symbols():
+    text = open(os.path.join(ROOT, "include", "vfkv.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(vfkv_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    L = _ffi.lib()
+    names = _declared_symbols()
+    assert len(names) >= 35
+    for n in names:
+        assert hasattr(L, n), n
+    assert sorted(_ffi.SIGNATURES) == names          # the ctypes table and the header agree
+    assert L.vfkv_abi_version() == 1
+    assert L.vfkv_status_string(0) == b"ok" and L.vfkv_status_string(-3) == b"misaligned offset"
+
+
+def test_param_structs_are_32_bytes():
+    # pipeline.rs:569 and :611
+    assert C.sizeof(_ffi.SplitParams) == 32 and C.sizeof(_ffi.BatchParams) == 32
+    assert _ffi.SplitParams.scale.offset == 20 and _ffi.SplitParams.kv_start.offset == 28
+    assert _ffi.BatchParams.scale.offset == 24 and _ffi.BatchParams.kv_start.offset == 28
+
+
+@pytest.mark.parametrize("dtype", list(vf.KvDtype))
+def test_uniform_layout_matches_reference_figures(dtype):
+    # kv_cache.rs:553-587: 36 x 8 x 128 x 2048 -> 576 / 288 MiB (and 144 for FP8)
+    c = vf.KvCache(vf.KvCacheConfig(36, 8, 128, 2048, dtype=dtype), layout_only=True)
+    es = dtype.element_size()
+    assert 2 * c.bytes_per_buffer() == {4: 576, 2: 288, 1: 144}[es] * 1024 * 1024
+    assert c.row_bytes(0) == 8 * 128 * es
+    assert c.layer_size_bytes(5) == 2048 * 8 * 128 * es
+    assert c.layer_offset_bytes(5) == 5 * 2048 * 8 * 128 * es
+    assert c.layer_offset_elems(5) == 5 * 2048 * 8 * 128
+    assert c.pos_offset_bytes(5, 77) == c.layer_offset_bytes(5) + 77 * c.row_bytes(5)
+    assert c.head_dim_for(3) == 128 and c.kv_heads_for(3) == 8
+    off = oracle.layout_offsets(36, 8, 128, 2048, int(dtype))
+    assert [c.layer_offset_bytes(i) for i in range(36)] == list(map(int, off[:-1]))
+    assert c.current_seq_len == 0
+    c.current_seq_len = 17
+    assert c.current_seq_len == 17
+    c.reset()
+    assert c.current_seq_len == 0
+    assert c.k_ptr == 0 and c.v_ptr == 0
+    c.destroy()
+
+
+def test_heterogeneous_layout_matches_oracle():
+    hd, kvh = [256, 256, 512, 256, 512], [8, 8, 2, 8, 2]
+    c = vf.KvCache(vf.KvCacheConfig(5, 999, 999, 1000, hd, kvh, vf.KvDtype.F8), layout_only=True)
+    off = oracle.layout_offsets(5, 999, 999, 1000, oracle.F8, hd, kvh)
+    for i in range(5):
+        assert c.layer_offset_bytes(i) == int(off[i])
+        assert c.layer_size_bytes(i) == int(off[i + 1] - off[i])
+        assert c.row_bytes(i) == hd[i] * kvh[i]
+        assert c.head_dim_for(i) == hd[i] and c.kv_heads_for(i) == kvh[i]
+        assert c.pos_offset_bytes(i, 999) == int(off[i]) + 999 * hd[i] * kvh[i]
+    assert c.bytes_per_buffer() == int(off[-1])
+    with pytest.raises(ValueError):
+        vf.KvCache(vf.KvCacheConfig(5, 8, 128, 10, per_layer_head_dim=[1, 2]), layout_only=True)
+
+
+def test_kv_bytes_per_token_reference_cases():
+    # kv_cache.rs:518-551
+    assert vf.kv_bytes_per_token(40, 8, 128, None, None, 2) == 2 * 2 * 40 * 8 * 128
+    assert vf.kv_bytes_per_token(4, 999, 999, [256, 256, 512, 512], [2, 2, 4, 4], 1) == 10_240
+    assert vf.kv_bytes_per_token(3, 0xFFFFFFFF, 0xFFFFFFFF, None, None, 1 << 40) == (1 << 64) - 1  # saturates
+
+
+def test_size_overflow_is_an_error_not_a_wrap():
+    with pytest.raises(vf.VfkvError) as e:
+        vf.KvCache(vf.KvCacheConfig(0xFFFFFFFF, 0xFFFFFFFF, 0xFFFFFFFF, 0xFFFFFFFF, dtype=vf.KvDtype.F32),
+                   layout_only=True)
+    assert e.value.status == -2
+    with pytest.raises(vf.VfkvError) as e:
+        vf.KvCache(vf.KvCacheConfig(2, 8, 128, 0xFFFFFFFF, [0xFFFFFFFF, 1], [0xFFFFFFFF, 1], vf.KvDtype.F32),
+                   layout_only=True)
+    assert e.value.status == -2
+
+
+def test_guard_kv_precision():
+    # kv_cache.rs:596-630
+    for kv in (vf.KvDtype.F32, vf.KvDtype.F16):
+        with pytest.raises(vf.VfkvError) as e:
+            vf.guard_kv_precision(True, kv)
+        assert "FP8" in str(e.value)
+        vf.guard_kv_precision(True, kv, force=True)
+        vf.guard_kv_precision(False, kv)
+    vf.guard_kv_precision(True, vf.KvDtype.F8)
+
+
+def test_kv_start_helpers_match_oracle():
+    L = _ffi.lib()
+    for pos, win in ((16383, 4096), (100, 4096), (4095, 4096), (4096, 4096), (0, 1), (0xFFFFFFFE, 5)):
+        assert L.vfkv_kv_start_decode(pos, win) == oracle.kv_start_decode(pos, win)
+    for base, n, win in ((4096, 512, 0), (4096, 512, 1024), (10, 20, 1024), (0, 1, 1)):
+        assert L.vfkv_kv_start_batch(base, n, win) == oracle.kv_start_batch(base, n, win)
+
+
+def test_bad_arguments_are_rejected_before_any_device_work():
+    L = _ffi.lib()
+    fake = 0x1000  # never dereferenced: every call below must fail in validation
+    assert L.vfkv_store_fp8(fake, fake, 8, 2, None) == -3       # runs.rs:2448-2453
+    assert L.vfkv_copy_fp16(fake, fake, 8, 6, None) == -3       # runs.rs:2400-2404
+    assert b"uint-aligned" in L.vfkv_last_error()
+    assert L.vfkv_store_fp8(None, fake, 8, 0, None) == -1
+    assert L.vfkv_store_fp8(None, None, 0, 0, None) == 0        # nothing to do
+    assert L.vfkv_fp8_to_f16(None, fake, 4, None) == -1
+    p = _ffi.SplitParams(30, 8, 128, 100, 0, 0.1, 2, 0)
+    assert L.vfkv_flash_attn_split(fake, fake, fake, 2, fake, fake, fake, C.byref(p), 64, 0.0, None) == -1
+    assert b"multiple" in L.vfkv_last_error()
+    p = _ffi.SplitParams(32, 8, 128, 0, 0, 0.1, 0, 0)
+    assert L.vfkv_flash_attn_split(fake, fake, fake, 2, fake, fake, fake, C.byref(p), 64, 0.0, None) == -1
+    p = _ffi.SplitParams(32, 8, 128, 100, 0, 0.1, 3, 0)          # n_tiles must be ceil(100/64) = 2
+    assert L.vfkv_flash_attn_split(fake, fake, fake, 2, fake, fake, fake, C.byref(p), 64, 0.0, None) == -1
+    p = _ffi.SplitParams(32, 8, 1024, 100, 0, 0.1, 2, 0)
+    assert L.vfkv_flash_attn_split(fake, fake, fake, 2, fake, fake, fake, C.byref(p), 64, 0.0, None) == -4
+    p = _ffi.SplitParams(32, 8, 128, 100, 0, 0.1, 2, 0)
+    assert L.vfkv_flash_attn_split(fake, fake, fake, 7, fake, fake, fake, C.byref(p), 64, 0.0, None) == -1
+    assert L.vfkv_flash_attn_split(fake, fake, fake, 2, fake, fake, fake, C.byref(p), 60, 0.0, None) == -1
+    assert L.vfkv_flash_attn_reduce(fake, fake, fake, fake, 32, 128, 0, None) == -1
+    b = _ffi.BatchParams(32, 8, 128, 4, 64, 60, 0.1, 61)        # kv_start hides every key of query 0
+    assert L.vfkv_flash_attn_batch(fake, fake, fake, 0, fake, C.byref(b), 0.0, None) == -1
+    b = _ffi.BatchParams(32, 5, 128, 4, 64, 60, 0.1, 0)
+    assert L.vfkv_flash_attn_batch(fake, fake, fake, 0, fake, C.byref(b), 0.0, None) == -1
+    h = C.c_void_p()
+    assert L.vfkv_workspace_create(0, 128, 100, C.byref(h)) == -1
+    # a layout-only cache has no buffers: compute entry points refuse it
+    c = vf.KvCache(vf.KvCacheConfig(2, 8, 128, 64, dtype=vf.KvDtype.F8), layout_only=True)
+    assert L.vfkv_kv_write(c.handle, 0, 0, 1, fake, fake, None) == -1
+    assert L.vfkv_cache_zero_fill(c.handle, None) == -1
+    assert L.vfkv_decode_attention(c.handle, 0, 0, 32, fake, fake, 3, 0, 0.1, 0.0, None, None) == -1
+
+
+def test_product_package_does_not_reach_into_the_oracle():
+    pkg = os.path.join(ROOT, "vulkanforge_amd")
+    for dirpath, _dirs, files in os.walk(pkg):
+        for f in files:
+            if f.endswith((".py", ".hip", ".h", ".cpp", ".hpp")) or f == "Makefile":
+                text = open(os.path.join(dirpath, f)).read()
+                assert not re.search(r"import\s+oracle|from\s+oracle|oracle/|vfkv_oracle|vfo_", text), \
+                    os.path.join(dirpath, f)
+
+
+def test_no_device_means_loud_failure():
+    if _ffi.lib().vfkv_device_count() > 0:
+        pytest.skip("a GPU is present")
+    with pytest.raises(vf.VfkvError):
+        vf.KvCache(vf.KvCacheConfig(1, 1, 64, 16, dtype=vf.KvDtype.F8))
+    with pytest.raises(ValueError):
+        import torch
+        vf.Forward.run_kv_store_fp8(torch.zeros(8), torch.zeros(8, dtype=torch.uint8), 8, 0, stream=0)

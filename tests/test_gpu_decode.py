@@ -1,0 +1,275 @@
+"""GPU parity of split-K decode attention (worker + log-sum-exp merge) through the C ABI.
+
+Bars (max-abs against the CPU oracle on the same decoded inputs): F16 KV 2e-3, FP8 KV 5e-3, F32 KV
+1e-3 (the reference's own bar, tests/correctness.rs:2875-2894).  TIGHT is what f32 arithmetic is
+expected to reach and guards against regressions hiding inside the wide bars."""
+import os
+
+import numpy as np
+import pytest
+import torch
+
+import oracle
+import vulkanforge_amd as vf
+from gpu_util import (DEV, TIGHT, TOL, encode_np, fp16_normal, gpu_split_reduce, outlier_normal, rng, to_dev,
+                      to_np)
+from refgen import D, H, HKV, decode_inputs
+
+pytestmark = pytest.mark.gpu
+SCALE = float(np.float32(1.0) / np.sqrt(np.float32(D)))
+
+
+def test_single_hip_runtime_in_process():
+    torch.cuda.synchronize()
+    vf.lib()
+    libs = {line.split()[-1] for line in open("/proc/self/maps") if "libamdhip64" in line}
+    assert len(libs) == 1, libs
+
+
+@pytest.mark.parametrize("seq", (64, 200, 2048))
+def test_reference_split_fixture_f32_tile64(golden_dir, seq):
+    # tests/correctness.rs:2791-2894: FlashAttnSplit + FlashAttnReduce, F32 KV, TILE 64, tol 1e-3
+    golden = np.load(os.path.join(golden_dir, "attn_cases.npz"))[f"decode_seq{seq}_out"]
+    q, k, v = decode_inputs(seq)
+    o, so, sm, ss = gpu_split_reduce(q, k, v, vf.KvDtype.F32, H, HKV, D, seq, SCALE, tile=64)
+    assert np.isfinite(o).all()
+    assert np.abs(o - golden).max() < 1e-3
+    assert np.abs(o - golden).max() < 2e-5
+    # the per-tile partials have the reference's meaning and layout (flash_attn_split.comp:147-161)
+    eo, em, es = oracle.attn_split(q, k, v, oracle.F32, H, HKV, D, seq, SCALE, tile=64)
+    assert np.abs(sm - em).max() < 1e-5
+    assert np.abs(ss - es).max() < 1e-4 * max(1.0, np.abs(es).max())
+    assert np.abs(so - eo).max() < 1e-4 * max(1.0, np.abs(eo).max())
+
+
+def test_seq1_returns_v0_exactly():
+    q, k, v = decode_inputs(1)
+    o, *_ = gpu_split_reduce(q, k, v, vf.KvDtype.F32, H, HKV, D, 1, SCALE, tile=64)
+    assert (o == np.repeat(v[0], H // HKV, axis=0)).all()
+
+
+CASES = [
+    # dtype, H, Hkv, D, seq, tile, kv_start, softcap
+    (vf.KvDtype.F8, 32, 8, 128, 2049, 512, 0, 0.0),
+    (vf.KvDtype.F8, 32, 8, 128, 777, 64, 0, 0.0),
+    (vf.KvDtype.F8, 32, 8, 128, 1000, 256, 300, 0.0),
+    (vf.KvDtype.F8, 32, 8, 128, 1000, 128, 999, 0.0),
+    (vf.KvDtype.F8, 8, 8, 128, 500, 64, 0, 0.0),      # G = 1
+    (vf.KvDtype.F8, 16, 8, 128, 500, 192, 17, 30.0),  # G = 2
+    (vf.KvDtype.F8, 24, 8, 64, 500, 64, 0, 0.0),      # G = 3
+    (vf.KvDtype.F8, 64, 8, 128, 300, 64, 0, 0.0),     # G = 8 (two head groups)
+    (vf.KvDtype.F8, 16, 2, 256, 600, 128, 0, 0.0),
+    (vf.KvDtype.F8, 8, 2, 512, 300, 64, 100, 0.0),
+    (vf.KvDtype.F8, 16, 4, 64, 900, 320, 0, 0.0),
+    (vf.KvDtype.F16, 32, 8, 128, 2049, 512, 0, 0.0),
+    (vf.KvDtype.F16, 16, 8, 256, 1500, 256, 0, 50.0),
+    (vf.KvDtype.F16, 16, 8, 256, 1500, 64, 1100, 50.0),
+    (vf.KvDtype.F16, 8, 4, 512, 200, 64, 0, 0.0),
+    (vf.KvDtype.F16, 12, 4, 64, 1000, 512, 0, 0.0),
+    (vf.KvDtype.F32, 32, 8, 128, 700, 128, 0, 0.0),
+    (vf.KvDtype.F32, 8, 2, 256, 300, 64, 50, 0.0),
+    (vf.KvDtype.F32, 4, 2, 64, 300, 64, 0, 10.0),
+    # shapes only the generic worker covers
+    (vf.KvDtype.F32, 4, 2, 512, 200, 64, 0, 0.0),
+    (vf.KvDtype.F16, 6, 2, 80, 333, 64, 10, 0.0),
+    (vf.KvDtype.F8, 4, 4, 96, 333, 128, 0, 0.0),
+    (vf.KvDtype.F32, 3, 1, 50, 100, 64, 0, 0.0),
+]
+
+
+@pytest.mark.parametrize("dtype,heads,hkv,d,seq,tile,kv_start,cap", CASES)
+def test_split_reduce_matches_oracle(dtype, heads, hkv, d, seq, tile, kv_start, cap):
+    r = rng(hash((int(dtype), heads, hkv, d, seq, tile)) % (1 << 31))
+    q = fp16_normal(r, (heads, d))
+    kf = outlier_normal(r, (seq, hkv, d)) if dtype == vf.KvDtype.F8 else fp16_normal(r, (seq, hkv, d))
+    vfl = outlier_normal(r, (seq, hkv, d)) if dtype == vf.KvDtype.F8 else fp16_normal(r, (seq, hkv, d))
+    k, v = encode_np(kf, dtype), encode_np(vfl, dtype)
+    scale = float(1.0 / np.sqrt(d))
+    print(f"case dtype={dtype.label()} H={heads} Hkv={hkv} D={d} seq={seq} tile={tile} kv_start={kv_start} cap={cap}",
+          flush=True)
+    o, so, sm, ss = gpu_split_reduce(q, k, v, dtype, heads, hkv, d, seq, scale, tile=tile, kv_start=kv_start,
+                                     softcap=cap)
+    ref = oracle.attn_decode_ref(q, k, v, int(dtype), heads, hkv, d, seq, scale, kv_start=kv_start, softcap=cap)
+    assert np.isfinite(o).all() and np.isfinite(so).all()       # NaN-poisoned scratch fully overwritten
+    err = np.abs(o - ref).max()
+    assert err < TOL[dtype], err
+    assert err < TIGHT * max(1.0, np.abs(ref).max()), err
+    # tiles wholly below the window are empty partials (flash_attn_split.comp:64-69)
+    dead = kv_start // tile
+    if dead:
+        assert (sm[:, :dead] == np.float32(-1e30)).all() and (ss[:, :dead] == 0).all() and (so[:, :dead] == 0).all()
+
+
+def test_tile_invariance_and_linearity_full_size_fp8():
+    # size-independent properties at the benchmark's largest single-layer shape (32768 keys, FP8)
+    seq, heads, hkv, d = 32768, 32, 8, 128
+    g = torch.Generator(device=DEV).manual_seed(5)
+    kf = torch.randn((seq, hkv * d), device=DEV, generator=g)
+    v1 = torch.randn((seq, hkv * d), device=DEV, generator=g)
+    v2 = torch.randn((seq, hkv * d), device=DEV, generator=g)
+    q = torch.randn((heads, d), device=DEV, generator=g).half().float()
+    scale = float(1.0 / np.sqrt(d))
+
+    def enc(x):
+        out = torch.empty(x.numel(), dtype=torch.uint8, device=DEV)
+        vf.Forward.run_kv_store_fp8(x, out, x.numel(), 0)
+        return out
+
+    def dec(b):
+        out = torch.empty(b.numel(), dtype=torch.float16, device=DEV)
+        vf.Forward.run_kv_fp8_to_f16(b, out, b.numel())
+        return out.float()
+
+    k8, va, vb = enc(kf), enc(v1), enc(v2)
+    vsum = dec(va) + dec(vb)            # exact in f32; encode it as an F32-KV value tensor
+    ones = enc(torch.ones_like(v1))
+
+    def attn(k, v, dt, tile):
+        n_tiles = (seq + tile - 1) // tile
+        so = torch.empty((heads, n_tiles, d), device=DEV)
+        sm = torch.empty((heads, n_tiles), device=DEV)
+        ss = torch.empty((heads, n_tiles), device=DEV)
+        o = torch.empty((heads, d), device=DEV)
+        vf.Forward.run_flash_attn_split(q, k, v, dt, so, sm, ss, heads, hkv, d, seq, scale, tile=tile)
+        vf.Forward.run_flash_attn_reduce(so, sm, ss, o, heads, d, n_tiles)
+        return o
+
+    o512 = attn(k8, va, vf.KvDtype.F8, 512)
+    for tile in (64, 1024, 4096):
+        assert (attn(k8, va, vf.KvDtype.F8, tile) - o512).abs().max().item() < 2e-5
+    assert (attn(k8, ones, vf.KvDtype.F8, 512) - 1.0).abs().max().item() < 1e-5      # weights sum to one
+    ob = attn(k8, vb, vf.KvDtype.F8, 512)
+    # linearity in V needs one K for all three runs: decode K to f32 and use the F32-KV kernels
+    kf32 = dec(k8)
+    oa32 = attn(kf32, dec(va), vf.KvDtype.F32, 512)
+    ob32 = attn(kf32, dec(vb), vf.KvDtype.F32, 512)
+    os32 = attn(kf32, vsum, vf.KvDtype.F32, 512)
+    assert (oa32 + ob32 - os32).abs().max().item() < 2e-5
+    # the FP8-KV and F32-KV kernels see the same decoded values
+    assert (oa32 - o512).abs().max().item() < 2e-5 and (ob32 - ob).abs().max().item() < 2e-5
+    # and one full-size comparison with the oracle
+    ref = oracle.attn_decode_ref(to_np(q), to_np(k8).reshape(seq, hkv, d), to_np(va).reshape(seq, hkv, d),
+                                 oracle.F8, heads, hkv, d, seq, scale)
+    assert np.abs(to_np(o512) - ref).max() < 5e-3
+    assert np.abs(to_np(o512) - ref).max() < TIGHT
+
+
+def _cache_with_history(dtype, n_layers, hkv, d, max_seq, fill, seed, hd=None, kvh=None):
+    cfg = vf.KvCacheConfig(n_layers, hkv, d, max_seq, hd, kvh, dtype)
+    cache = vf.KvCache(cfg)
+    cache.zero_fill()
+    r = rng(seed)
+    hist = []
+    fwd = vf.Forward(cache, 1)
+    for layer in range(n_layers):
+        row = cache.kv_heads_for(layer) * cache.head_dim_for(layer)
+        k, v = fill(r, (max_seq, row)), fill(r, (max_seq, row))
+        fwd.b_step_kv_write(layer, 0, max_seq, to_dev(k), to_dev(v))
+        hist.append((k, v))
+    torch.cuda.synchronize()
+    return cache, hist
+
+
+def test_config1_append_then_decode_f16():
+    # BASELINE config 1: one layer, F16 KV, 32/8/128, context 2048, append one token, attend
+    heads, hkv, d, ctx = 32, 8, 128, 2048
+    cache, hist = _cache_with_history(vf.KvDtype.F16, 1, hkv, d, ctx + 1, fp16_normal, 11)
+    fwd = vf.Forward(cache, heads)
+    r = rng(12)
+    k_new, v_new, q = fp16_normal(r, (1, hkv * d)), fp16_normal(r, (1, hkv * d)), fp16_normal(r, (heads, d))
+    fwd.step_kv_write(0, ctx, to_dev(k_new), to_dev(v_new))
+    o = torch.full((heads, d), float("nan"), device=DEV)
+    fwd.run_scalar_attn(0, ctx, to_dev(q), o)
+    torch.cuda.synchronize()
+    k_all, v_all = hist[0][0].copy(), hist[0][1].copy()
+    k_all[ctx], v_all[ctx] = k_new[0], v_new[0]
+    ke, ve = encode_np(k_all, vf.KvDtype.F16), encode_np(v_all, vf.KvDtype.F16)
+    ref = oracle.attn_decode_ref(q, ke.reshape(-1, hkv, d), ve.reshape(-1, hkv, d), oracle.F16, heads, hkv, d,
+                                 ctx + 1, fwd.attn_scale)
+    err = np.abs(to_np(o) - ref).max()
+    assert err < 2e-3 and err < TIGHT, err
+
+
+def test_config2_fp8_outliers_append_then_decode_two_layers():
+    # BASELINE config 2 geometry (FP8 KV, context 8192, +-40 outlier tail), two layers of the 32
+    heads, hkv, d, ctx = 32, 8, 128, 8192
+    cache, hist = _cache_with_history(vf.KvDtype.F8, 2, hkv, d, ctx + 1, outlier_normal, 21)
+    fwd = vf.Forward(cache, heads)
+    r = rng(22)
+    for layer in range(2):
+        k_new, v_new = outlier_normal(r, (1, hkv * d)), outlier_normal(r, (1, hkv * d))
+        q = fp16_normal(r, (heads, d))
+        fwd.step_kv_write(layer, ctx, to_dev(k_new), to_dev(v_new))
+        o = torch.full((heads, d), float("nan"), device=DEV)
+        fwd.step_attention(layer, ctx, to_dev(q), o)
+        torch.cuda.synchronize()
+        k_all, v_all = hist[layer][0].copy(), hist[layer][1].copy()
+        k_all[ctx], v_all[ctx] = k_new[0], v_new[0]
+        ke, ve = encode_np(k_all, vf.KvDtype.F8), encode_np(v_all, vf.KvDtype.F8)
+        # the appended FP8 bytes are bit-exact
+        from gpu_util import read_device
+        off = cache.pos_offset_bytes(layer, ctx)
+        assert (read_device(cache.k_ptr + off, hkv * d) == ke[ctx]).all()
+        assert (read_device(cache.v_ptr + off, hkv * d) == ve[ctx]).all()
+        ref = oracle.attn_decode_ref(q, ke.reshape(-1, hkv, d), ve.reshape(-1, hkv, d), oracle.F8, heads, hkv, d,
+                                     ctx + 1, fwd.attn_scale)
+        err = np.abs(to_np(o) - ref).max()
+        assert err < 5e-3 and err < TIGHT * 40, err
+
+
+def test_config4_hd256_sliding_window_softcap_f16():
+    # BASELINE config 4 geometry: 16/8/256, F16 KV, window 4096 at context 16384, soft-cap 50;
+    # layer 0 sliding, layer 1 global
+    heads, hkv, d, ctx, window, cap = 16, 8, 256, 16384, 4096, 50.0
+    cache, hist = _cache_with_history(vf.KvDtype.F16, 2, hkv, d, ctx, fp16_normal, 31)
+    fwd = vf.Forward(cache, heads)
+    q = fp16_normal(rng(32), (heads, d))
+    scale = float(1.0 / np.sqrt(d))
+    for layer, win in ((0, window), (1, 0)):
+        kv_start = oracle.kv_start_decode(ctx - 1, win) if win else 0
+        assert kv_start == (12288 if win else 0)
+        o = torch.full((heads, d), float("nan"), device=DEV)
+        fwd.run_scalar_attn(layer, ctx - 1, to_dev(q), o, kv_start=kv_start, scale=scale, softcap=cap)
+        torch.cuda.synchronize()
+        ke, ve = encode_np(hist[layer][0], vf.KvDtype.F16), encode_np(hist[layer][1], vf.KvDtype.F16)
+        ref = oracle.attn_decode_ref(q, ke.reshape(-1, hkv, d), ve.reshape(-1, hkv, d), oracle.F16, heads, hkv, d,
+                                     ctx, scale, kv_start=kv_start, softcap=cap)
+        err = np.abs(to_np(o) - ref).max()
+        assert err < 2e-3 and err < TIGHT, (layer, err)
+
+
+def test_heterogeneous_cache_and_kv_share():
+    # per-layer head_dim / kv heads (kv_cache.rs:256-283) and reading another layer's slab
+    # (gemma4_kv_read_layer, gemma4.rs:27-49)
+    hd, kvh, heads, seq = [256, 512, 256], [4, 2, 4], 8, 300
+    cache, hist = _cache_with_history(vf.KvDtype.F8, 3, 999, 512, seq, fp16_normal, 41, hd=hd, kvh=kvh)
+    fwd = vf.Forward(cache, heads)
+    r = rng(42)
+    for layer, kv_layer in ((0, 0), (1, 1), (2, 0)):
+        d, g = hd[layer], kvh[layer]
+        q = fp16_normal(r, (heads, d))
+        o = torch.full((heads, d), float("nan"), device=DEV)
+        fwd.run_scalar_attn(layer, seq - 1, to_dev(q), o, kv_layer=kv_layer, scale=1.0 / np.sqrt(d))
+        torch.cuda.synchronize()
+        ke, ve = (encode_np(x, vf.KvDtype.F8).reshape(seq, g, d) for x in hist[kv_layer])
+        ref = oracle.attn_decode_ref(q, ke, ve, oracle.F8, heads, g, d, seq, 1.0 / np.sqrt(d))
+        assert np.abs(to_np(o) - ref).max() < TIGHT
+
+
+def test_short_context_goes_through_the_same_path():
+    # seq <= 64: the reference uses its single-workgroup shader (runs.rs:776-821); same attention
+    heads, hkv, d = 32, 8, 128
+    cache, hist = _cache_with_history(vf.KvDtype.F16, 1, hkv, d, 64, fp16_normal, 51)
+    fwd = vf.Forward(cache, heads)
+    q = fp16_normal(rng(52), (heads, d))
+    ke, ve = (encode_np(x, vf.KvDtype.F16).reshape(64, hkv, d) for x in hist[0])
+    for pos in (0, 1, 17, 63):
+        o = torch.full((heads, d), float("nan"), device=DEV)
+        fwd.run_scalar_attn(0, pos, to_dev(q), o)
+        torch.cuda.synchronize()
+        ref = oracle.attn_decode_ref(q, ke, ve, oracle.F16, heads, hkv, d, pos + 1, fwd.attn_scale)
+        assert np.abs(to_np(o) - ref).max() < TIGHT
+    with pytest.raises(vf.VfkvError):
+        fwd.run_scalar_attn(0, 64, to_dev(q), torch.empty((heads, d), device=DEV))      # beyond max_seq
+    with pytest.raises(vf.VfkvError):
+        fwd.run_scalar_attn(0, 10, to_dev(q), torch.empty((heads, d), device=DEV), kv_start=11)

@@ -1,0 +1,122 @@
+"""GPU parity of chunked-prefill causal attention (flash_attn_batch) through the C ABI."""
+import os
+
+import numpy as np
+import pytest
+import torch
+
+import oracle
+import vulkanforge_amd as vf
+from gpu_util import DEV, TIGHT, TOL, encode_np, fp16_normal, gpu_batch, outlier_normal, rng, to_dev, to_np
+from refgen import BATCH_CASES, D, H, HKV, batch_inputs, golden_rows
+
+pytestmark = pytest.mark.gpu
+SCALE = float(np.float32(1.0) / np.sqrt(np.float32(D)))
+REF_TOL = {(1, 0): 1e-4, (4, 0): 1e-3, (16, 0): 1e-3, (64, 0): 1e-3, (200, 0): 5e-3, (4, 60): 1e-3}
+
+
+@pytest.mark.parametrize("m,q_start", BATCH_CASES)
+def test_reference_batch_fixtures_f32(golden_dir, m, q_start):
+    # tests/correctness.rs:3073-3201
+    golden = np.load(os.path.join(golden_dir, "attn_cases.npz"))[f"batch_m{m}_qs{q_start}_out"]
+    q, k, v = batch_inputs(m, q_start)
+    o = gpu_batch(q, k, v, vf.KvDtype.F32, H, HKV, D, m, q_start, q_start + m, SCALE)
+    assert np.isfinite(o).all()
+    err = np.abs(o[golden_rows(m)] - golden).max()
+    assert err < REF_TOL[(m, q_start)] and err < 2e-5, err
+    ref = oracle.attn_batch_ref(q, k, v, oracle.F32, m, q_start + m, H, HKV, D, q_start, SCALE)
+    assert np.abs(o - ref).max() < 2e-5
+
+
+def test_m1_equals_decode_and_causal_isolation():
+    # tests/correctness.rs:3203-3279 (M=1 == single-query attention) and :3281-3386
+    q, k, v = batch_inputs(4, 0)
+    full = gpu_batch(q, k, v, vf.KvDtype.F32, H, HKV, D, 4, 0, 4, SCALE)
+    one = gpu_batch(q[:1].copy(), k[:1].copy(), v[:1].copy(), vf.KvDtype.F32, H, HKV, D, 1, 0, 1, SCALE)
+    assert np.abs(full[0] - one[0]).max() < 1e-5
+    assert (np.abs(full[3] - one[0]) > 1e-3).sum() > H * D // 8
+    from gpu_util import gpu_split_reduce
+    dec, *_ = gpu_split_reduce(q[3], k, v, vf.KvDtype.F32, H, HKV, D, 4, SCALE, tile=64)
+    assert np.abs(dec - full[3]).max() < 1e-5
+
+
+CASES = [
+    # dtype, H, Hkv, D, m, q_start, kv_start, softcap
+    (vf.KvDtype.F8, 32, 8, 128, 64, 200, 0, 0.0),
+    (vf.KvDtype.F8, 32, 8, 128, 37, 0, 0, 0.0),
+    (vf.KvDtype.F8, 32, 8, 128, 50, 300, 111, 0.0),
+    (vf.KvDtype.F8, 16, 8, 128, 33, 100, 0, 25.0),
+    (vf.KvDtype.F8, 8, 2, 256, 20, 150, 64, 0.0),
+    (vf.KvDtype.F16, 32, 8, 128, 64, 200, 0, 0.0),
+    (vf.KvDtype.F16, 16, 8, 256, 48, 500, 300, 50.0),
+    (vf.KvDtype.F16, 4, 1, 512, 10, 70, 0, 0.0),
+    (vf.KvDtype.F32, 12, 4, 64, 30, 90, 5, 0.0),
+    (vf.KvDtype.F8, 6, 2, 80, 19, 45, 0, 0.0),
+]
+
+
+@pytest.mark.parametrize("dtype,heads,hkv,d,m,q_start,kv_start,cap", CASES)
+def test_batch_matches_oracle(dtype, heads, hkv, d, m, q_start, kv_start, cap):
+    r = rng(hash((int(dtype), heads, hkv, d, m, q_start)) % (1 << 31))
+    n_kv = q_start + m
+    q = fp16_normal(r, (m, heads, d))
+    fill = outlier_normal if dtype == vf.KvDtype.F8 else fp16_normal
+    k, v = encode_np(fill(r, (n_kv, hkv, d)), dtype), encode_np(fill(r, (n_kv, hkv, d)), dtype)
+    scale = float(1.0 / np.sqrt(d))
+    print(f"case dtype={dtype.label()} H={heads} Hkv={hkv} D={d} m={m} q_start={q_start} kv_start={kv_start} cap={cap}",
+          flush=True)
+    o = gpu_batch(q, k, v, dtype, heads, hkv, d, m, q_start, n_kv, scale, kv_start=kv_start, softcap=cap)
+    ref = oracle.attn_batch_ref(q, k, v, int(dtype), m, n_kv, heads, hkv, d, q_start, scale, kv_start=kv_start,
+                                softcap=cap)
+    assert np.isfinite(o).all()
+    err = np.abs(o - ref).max()
+    assert err < TOL[dtype], err
+
+
+def test_config5_chunk_append_then_prefill_fp8_one_layer():
+    # BASELINE config 5, one of its 32 layers: FP8 cache filled to 4096, append 512 tokens, then
+    # 512 causal queries over 4608 keys (32/8/128).  The oracle is run on a sample of query rows.
+    heads, hkv, d, base, m = 32, 8, 128, 4096, 512
+    cache = vf.KvCache(vf.KvCacheConfig(1, hkv, d, base + m, dtype=vf.KvDtype.F8))
+    fwd = vf.Forward(cache, heads)
+    r = rng(61)
+    hist_k, hist_v = fp16_normal(r, (base, hkv * d)), fp16_normal(r, (base, hkv * d))
+    new_k, new_v = fp16_normal(r, (m, hkv * d)), fp16_normal(r, (m, hkv * d))
+    q = fp16_normal(r, (m, heads, d))
+    fwd.b_step_kv_write(0, 0, base, to_dev(hist_k), to_dev(hist_v))
+    fwd.b_step_kv_write(0, base, m, to_dev(new_k), to_dev(new_v))
+    o = torch.full((m, heads, d), float("nan"), device=DEV)
+    fwd.b_step_attention(0, base, m, to_dev(q), o)
+    torch.cuda.synchronize()
+    o = to_np(o)
+    assert np.isfinite(o).all()
+    ke = encode_np(np.concatenate([hist_k, new_k]), vf.KvDtype.F8).reshape(-1, hkv, d)
+    ve = encode_np(np.concatenate([hist_v, new_v]), vf.KvDtype.F8).reshape(-1, hkv, d)
+    from gpu_util import read_device
+    assert (read_device(cache.k_ptr, ke.size) == ke.ravel()).all()          # appended bytes bit-exact
+    for i in (0, 1, 63, 64, 255, 400, 511):
+        ref = oracle.attn_decode_ref(q[i], ke, ve, oracle.F8, heads, hkv, d, base + i + 1, fwd.attn_scale)
+        err = np.abs(o[i] - ref).max()
+        assert err < 5e-3, (i, err)
+    cache.destroy()
+
+
+def test_window_uses_the_last_querys_lower_bound():
+    # executor/attention.rs:2215-2219: kv_start = base + m - window for every row of the batch
+    heads, hkv, d, base, m, window = 8, 2, 128, 300, 40, 128
+    cache = vf.KvCache(vf.KvCacheConfig(1, hkv, d, base + m, dtype=vf.KvDtype.F16))
+    fwd = vf.Forward(cache, heads)
+    r = rng(71)
+    k, v = fp16_normal(r, (base + m, hkv * d)), fp16_normal(r, (base + m, hkv * d))
+    q = fp16_normal(r, (m, heads, d))
+    fwd.b_step_kv_write(0, 0, base + m, to_dev(k), to_dev(v))
+    o = torch.full((m, heads, d), float("nan"), device=DEV)
+    fwd.b_step_attention(0, base, m, to_dev(q), o, kv_start_window=window)
+    torch.cuda.synchronize()
+    kv_start = oracle.kv_start_batch(base, m, window)
+    assert kv_start == base + m - window
+    ke, ve = (encode_np(x, vf.KvDtype.F16).reshape(-1, hkv, d) for x in (k, v))
+    ref = oracle.attn_batch_ref(q, ke, ve, oracle.F16, m, base + m, heads, hkv, d, base, fwd.attn_scale,
+                                kv_start=kv_start)
+    assert np.abs(to_np(o) - ref).max() < TIGHT
+    cache.destroy()

@@ -1,0 +1,498 @@
+// extern "C" boundary of libvfkv: the cache object (KvCache, kv_cache.rs:204-500), the scratch
+// workspace (forward/setup.rs:203-230) and one entry point per reference dispatch helper
+// (forward/runs.rs).  Host code only; the kernels live in the other translation units.
+#include <hip/hip_runtime.h>
+
+#include <cstdarg>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <new>
+#include <vector>
+
+#include "../../include/vfkv.h"
+#include "device_utils.h"
+#include "kernels.h"
+
+namespace {
+
+thread_local char g_err[512] = "";
+
+int fail(int status, const char* fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof(g_err), fmt, ap);
+    va_end(ap);
+    return status;
+}
+
+int hip_fail(hipError_t e, const char* what) {
+    return fail(e == hipErrorNoDevice ? VFKV_ERR_NO_DEVICE : VFKV_ERR_HIP, "%s: %s", what, hipGetErrorString(e));
+}
+
+#define VFKV_HIP(call)                                  \
+    do {                                                \
+        hipError_t e_ = (call);                         \
+        if (e_ != hipSuccess) return hip_fail(e_, #call); \
+    } while (0)
+
+inline bool mul_ovf(uint64_t a, uint64_t b, uint64_t* r) { return __builtin_mul_overflow(a, b, r); }
+inline bool add_ovf(uint64_t a, uint64_t b, uint64_t* r) { return __builtin_add_overflow(a, b, r); }
+inline uint64_t esize(uint32_t dtype) { return vfkv::elem_size(dtype); }
+inline hipStream_t S(vfkv_stream s) { return reinterpret_cast<hipStream_t>(s); }
+
+}  // namespace
+
+struct vfkv_cache {
+    uint32_t n_layers, n_kv_heads, head_dim, max_seq_len, dtype;
+    std::vector<uint32_t> per_layer_head_dim;     // empty = uniform
+    std::vector<uint32_t> per_layer_n_kv_heads;   // empty = uniform
+    std::vector<uint64_t> layer_byte_offsets;     // n_layers + 1 entries when heterogeneous, else empty
+    uint64_t bytes;                               // per buffer
+    void* k;
+    void* v;
+    bool owns;
+    uint32_t current_seq_len;
+};
+
+struct vfkv_workspace {
+    uint32_t n_heads, head_dim, max_tiles;
+    float* scratch_out;
+    float* scratch_max;
+    float* scratch_sum;
+};
+
+namespace {
+
+// KvCache::new size arithmetic (kv_cache.rs:224-291).
+int build_layout(const vfkv_cache_config* cfg, vfkv_cache* c) {
+    if (!cfg) return fail(VFKV_ERR_INVALID_ARG, "cache config is NULL");
+    if (cfg->dtype > VFKV_F8E4M3) return fail(VFKV_ERR_INVALID_ARG, "unknown kv dtype %u", cfg->dtype);
+    if (cfg->n_layers == 0) return fail(VFKV_ERR_INVALID_ARG, "n_layers must be > 0");
+    c->n_layers = cfg->n_layers;
+    c->n_kv_heads = cfg->n_kv_heads;
+    c->head_dim = cfg->head_dim;
+    c->max_seq_len = cfg->max_seq_len;
+    c->dtype = cfg->dtype;
+    c->current_seq_len = 0;
+    const uint64_t es = esize(cfg->dtype);
+    const bool hetero = cfg->per_layer_head_dim || cfg->per_layer_n_kv_heads;
+    if (hetero) {
+        if (cfg->per_layer_head_dim) c->per_layer_head_dim.assign(cfg->per_layer_head_dim, cfg->per_layer_head_dim + cfg->n_layers);
+        if (cfg->per_layer_n_kv_heads) c->per_layer_n_kv_heads.assign(cfg->per_layer_n_kv_heads, cfg->per_layer_n_kv_heads + cfg->n_layers);
+        c->layer_byte_offsets.reserve((size_t)cfg->n_layers + 1);
+        uint64_t acc = 0;
+        c->layer_byte_offsets.push_back(0);
+        for (uint32_t i = 0; i < cfg->n_layers; ++i) {
+            const uint64_t hd = cfg->per_layer_head_dim ? cfg->per_layer_head_dim[i] : cfg->head_dim;
+            const uint64_t kvh = cfg->per_layer_n_kv_heads ? cfg->per_layer_n_kv_heads[i] : cfg->n_kv_heads;
+            uint64_t b;
+            if (mul_ovf(cfg->max_seq_len, kvh, &b) || mul_ovf(b, hd, &b) || mul_ovf(b, es, &b))
+                return fail(VFKV_ERR_OVERFLOW, "kv-cache per-layer size overflow");
+            if (add_ovf(acc, b, &acc)) return fail(VFKV_ERR_OVERFLOW, "kv-cache total size overflow");
+            c->layer_byte_offsets.push_back(acc);
+        }
+        c->bytes = acc;
+    } else {
+        uint64_t t;
+        if (mul_ovf(cfg->n_layers, cfg->n_kv_heads, &t) || mul_ovf(t, cfg->max_seq_len, &t) ||
+            mul_ovf(t, cfg->head_dim, &t) || mul_ovf(t, es, &t))
+            return fail(VFKV_ERR_OVERFLOW, "kv-cache size overflow");
+        c->bytes = t;
+    }
+    return VFKV_OK;
+}
+
+inline uint32_t hd_for(const vfkv_cache* c, uint32_t layer) {
+    return c->per_layer_head_dim.empty() ? c->head_dim : c->per_layer_head_dim[layer];
+}
+inline uint32_t kvh_for(const vfkv_cache* c, uint32_t layer) {
+    return c->per_layer_n_kv_heads.empty() ? c->n_kv_heads : c->per_layer_n_kv_heads[layer];
+}
+inline uint64_t layer_off(const vfkv_cache* c, uint32_t layer) {
+    if (!c->layer_byte_offsets.empty()) return c->layer_byte_offsets[layer];
+    return (uint64_t)layer * c->n_kv_heads * c->max_seq_len * c->head_dim * esize(c->dtype);
+}
+inline uint64_t row_b(const vfkv_cache* c, uint32_t layer) {
+    return (uint64_t)kvh_for(c, layer) * hd_for(c, layer) * esize(c->dtype);
+}
+
+int check_attn_dims(uint32_t n_heads, uint32_t n_kv_heads, uint32_t head_dim) {
+    if (n_heads == 0 || n_kv_heads == 0 || head_dim == 0)
+        return fail(VFKV_ERR_INVALID_ARG, "n_heads, n_kv_heads and head_dim must be > 0");
+    if (n_heads % n_kv_heads != 0)
+        return fail(VFKV_ERR_INVALID_ARG, "n_heads (%u) is not a multiple of n_kv_heads (%u)", n_heads, n_kv_heads);
+    if (head_dim > 512) return fail(VFKV_ERR_UNSUPPORTED, "head_dim %u > 512 (flash_attn_split.comp:127-132)", head_dim);
+    return VFKV_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+const char* vfkv_status_string(int status) {
+    switch (status) {
+        case VFKV_OK: return "ok";
+        case VFKV_ERR_INVALID_ARG: return "invalid argument";
+        case VFKV_ERR_OVERFLOW: return "size overflow";
+        case VFKV_ERR_ALIGNMENT: return "misaligned offset";
+        case VFKV_ERR_UNSUPPORTED: return "unsupported shape";
+        case VFKV_ERR_HIP: return "HIP runtime error";
+        case VFKV_ERR_NO_DEVICE: return "no HIP device";
+        case VFKV_ERR_WORKSPACE: return "workspace too small";
+        default: return "unknown status";
+    }
+}
+
+const char* vfkv_last_error(void) { return g_err; }
+uint32_t vfkv_abi_version(void) { return VFKV_ABI_VERSION; }
+
+int vfkv_device_count(void) {
+    int n = 0;
+    if (hipGetDeviceCount(&n) != hipSuccess) return 0;
+    return n;
+}
+
+// ---- cache ---------------------------------------------------------------------------------------
+int vfkv_cache_create_external(const vfkv_cache_config* cfg, void* k_buffer, void* v_buffer, vfkv_cache** out) {
+    if (!out) return fail(VFKV_ERR_INVALID_ARG, "out is NULL");
+    *out = nullptr;
+    vfkv_cache* c = new (std::nothrow) vfkv_cache();
+    if (!c) return fail(VFKV_ERR_HIP, "host allocation failed");
+    const int rc = build_layout(cfg, c);
+    if (rc != VFKV_OK) { delete c; return rc; }
+    c->k = k_buffer;
+    c->v = v_buffer;
+    c->owns = false;
+    *out = c;
+    return VFKV_OK;
+}
+
+int vfkv_cache_create(const vfkv_cache_config* cfg, vfkv_cache** out) {
+    vfkv_cache* c = nullptr;
+    const int rc = vfkv_cache_create_external(cfg, nullptr, nullptr, &c);
+    if (rc != VFKV_OK) return rc;
+    *out = nullptr;
+    if (c->bytes == 0) { delete c; return fail(VFKV_ERR_INVALID_ARG, "kv-cache size is zero"); }
+    hipError_t e = hipMalloc(&c->k, c->bytes);
+    if (e == hipSuccess) {
+        e = hipMalloc(&c->v, c->bytes);
+        if (e != hipSuccess) { (void)hipFree(c->k); c->k = nullptr; }
+    }
+    if (e != hipSuccess) { delete c; return hip_fail(e, "hipMalloc(kv cache)"); }
+    c->owns = true;
+    *out = c;
+    return VFKV_OK;
+}
+
+void vfkv_cache_destroy(vfkv_cache* c) {
+    if (!c) return;
+    if (c->owns) {
+        if (c->k) (void)hipFree(c->k);
+        if (c->v) (void)hipFree(c->v);
+    }
+    delete c;
+}
+
+int vfkv_cache_zero_fill(vfkv_cache* c, vfkv_stream stream) {
+    if (!c || !c->k || !c->v) return fail(VFKV_ERR_INVALID_ARG, "cache has no buffers");
+    VFKV_HIP(hipMemsetAsync(c->k, 0, c->bytes, S(stream)));
+    VFKV_HIP(hipMemsetAsync(c->v, 0, c->bytes, S(stream)));
+    return VFKV_OK;
+}
+
+int vfkv_cache_zero_layer(vfkv_cache* c, uint32_t layer, vfkv_stream stream) {
+    if (!c || !c->k || !c->v) return fail(VFKV_ERR_INVALID_ARG, "cache has no buffers");
+    if (layer >= c->n_layers) return fail(VFKV_ERR_INVALID_ARG, "layer %u out of range", layer);
+    const uint64_t off = layer_off(c, layer);
+    const uint64_t size = (uint64_t)c->max_seq_len * row_b(c, layer);
+    if (size == 0) return VFKV_OK;
+    VFKV_HIP(hipMemsetAsync((char*)c->k + off, 0, size, S(stream)));
+    VFKV_HIP(hipMemsetAsync((char*)c->v + off, 0, size, S(stream)));
+    return VFKV_OK;
+}
+
+uint32_t vfkv_cache_current_seq_len(const vfkv_cache* c) { return c ? c->current_seq_len : 0u; }
+void vfkv_cache_set_current_seq_len(vfkv_cache* c, uint32_t n) { if (c) c->current_seq_len = n; }
+void vfkv_cache_reset(vfkv_cache* c) { if (c) c->current_seq_len = 0; }
+void* vfkv_cache_k_ptr(const vfkv_cache* c) { return c ? c->k : nullptr; }
+void* vfkv_cache_v_ptr(const vfkv_cache* c) { return c ? c->v : nullptr; }
+uint32_t vfkv_cache_dtype(const vfkv_cache* c) { return c ? c->dtype : 0u; }
+uint64_t vfkv_cache_bytes_per_buffer(const vfkv_cache* c) { return c ? c->bytes : 0u; }
+uint32_t vfkv_cache_head_dim_for(const vfkv_cache* c, uint32_t layer) { return (c && layer < c->n_layers) ? hd_for(c, layer) : 0u; }
+uint32_t vfkv_cache_kv_heads_for(const vfkv_cache* c, uint32_t layer) { return (c && layer < c->n_layers) ? kvh_for(c, layer) : 0u; }
+uint64_t vfkv_cache_layer_offset_bytes(const vfkv_cache* c, uint32_t layer) { return (c && layer < c->n_layers) ? layer_off(c, layer) : 0u; }
+uint64_t vfkv_cache_layer_offset_elems(const vfkv_cache* c, uint32_t layer) {
+    return (c && layer < c->n_layers) ? layer_off(c, layer) / esize(c->dtype) : 0u;
+}
+uint64_t vfkv_cache_row_bytes(const vfkv_cache* c, uint32_t layer) { return (c && layer < c->n_layers) ? row_b(c, layer) : 0u; }
+uint64_t vfkv_cache_pos_offset_bytes(const vfkv_cache* c, uint32_t layer, uint32_t pos) {
+    return (c && layer < c->n_layers) ? layer_off(c, layer) + (uint64_t)pos * row_b(c, layer) : 0u;
+}
+uint64_t vfkv_cache_layer_size_bytes(const vfkv_cache* c, uint32_t layer) {
+    return (c && layer < c->n_layers) ? (uint64_t)c->max_seq_len * row_b(c, layer) : 0u;
+}
+
+uint64_t vfkv_kv_bytes_per_token(uint32_t n_layers, uint32_t n_kv_heads, uint32_t head_dim,
+                                 const uint32_t* per_layer_head_dim, const uint32_t* per_layer_n_kv_heads,
+                                 uint64_t elem_size) {
+    uint64_t elems = 0;
+    for (uint32_t i = 0; i < n_layers; ++i) {
+        const uint64_t hd = per_layer_head_dim ? per_layer_head_dim[i] : head_dim;
+        const uint64_t kvh = per_layer_n_kv_heads ? per_layer_n_kv_heads[i] : n_kv_heads;
+        uint64_t p;
+        if (mul_ovf(kvh, hd, &p)) p = UINT64_MAX;
+        if (add_ovf(elems, p, &elems)) elems = UINT64_MAX;
+    }
+    uint64_t r;
+    if (mul_ovf(elems, elem_size, &r) || mul_ovf(r, 2u, &r)) return UINT64_MAX;
+    return r;
+}
+
+int vfkv_guard_kv_precision(int is_gemma4_moe, uint32_t dtype, int force) {
+    if (!is_gemma4_moe || dtype == VFKV_F8E4M3) return VFKV_OK;
+    if (force) {
+        fprintf(stderr, "vfkv: warning: gemma-4-MoE with %s KV is known-broken in the reference; proceeding (forced)\n",
+                dtype == VFKV_F16 ? "FP16" : "FP32");
+        return VFKV_OK;
+    }
+    return fail(VFKV_ERR_UNSUPPORTED,
+                "gemma-4-MoE requires an FP8 (E4M3) KV cache; %s KV is known-broken for this model",
+                dtype == VFKV_F16 ? "FP16" : "FP32");
+}
+
+uint32_t vfkv_kv_start_decode(uint32_t position, uint32_t sliding_window) {
+    const uint64_t seq = (uint64_t)position + 1u;
+    return seq > sliding_window ? (uint32_t)(seq - sliding_window) : 0u;
+}
+
+uint32_t vfkv_kv_start_batch(uint32_t base_pos, uint32_t seq_len, uint32_t window) {
+    if (window == 0u) return 0u;
+    const uint64_t end = (uint64_t)base_pos + seq_len;
+    return end > window ? (uint32_t)(end - window) : 0u;
+}
+
+// ---- append / expansion ----------------------------------------------------------------------------
+static int append_one(uint32_t dtype, const float* src, void* dst, uint32_t n, uint64_t off, vfkv_stream stream,
+                      const char* what) {
+    if (n == 0) return VFKV_OK;
+    if (!src || !dst) return fail(VFKV_ERR_INVALID_ARG, "%s: NULL buffer", what);
+    if (off % 4u != 0u) return fail(VFKV_ERR_ALIGNMENT, "%s: dst_byte_offset must be uint-aligned (got %llu)", what, (unsigned long long)off);
+    if ((((uintptr_t)dst) & 3u) != 0u || (((uintptr_t)src) & 3u) != 0u)
+        return fail(VFKV_ERR_ALIGNMENT, "%s: buffers must be 4-byte aligned", what);
+    char* d = (char*)dst + off;
+    VFKV_HIP(vfkv::launch_kv_append(dtype, src, src, d, d, n, 1, S(stream)));
+    return VFKV_OK;
+}
+
+int vfkv_store_fp8(const float* src, void* dst, uint32_t n_elements, uint64_t dst_byte_offset, vfkv_stream stream) {
+    return append_one(vfkv::kF8, src, dst, n_elements, dst_byte_offset, stream, "kv_store_fp8");
+}
+
+int vfkv_copy_fp16(const float* src, void* dst, uint32_t n_elements, uint64_t dst_byte_offset, vfkv_stream stream) {
+    return append_one(vfkv::kF16, src, dst, n_elements, dst_byte_offset, stream, "kv_copy_fp16");
+}
+
+int vfkv_fp8_to_f16(const void* src, void* dst_f16, uint64_t n_elems, vfkv_stream stream) {
+    if (n_elems == 0) return VFKV_OK;
+    if (!src || !dst_f16) return fail(VFKV_ERR_INVALID_ARG, "kv_fp8_to_f16: NULL buffer");
+    if ((((uintptr_t)dst_f16) & 1u) != 0u) return fail(VFKV_ERR_ALIGNMENT, "kv_fp8_to_f16: dst must be 2-byte aligned");
+    VFKV_HIP(vfkv::launch_fp8_to_f16(src, dst_f16, n_elems, S(stream)));
+    return VFKV_OK;
+}
+
+int vfkv_kv_write(vfkv_cache* c, uint32_t layer, uint32_t pos, uint32_t n_tokens, const float* k_src,
+                  const float* v_src, vfkv_stream stream) {
+    if (!c || !c->k || !c->v) return fail(VFKV_ERR_INVALID_ARG, "kv_write: cache has no buffers");
+    if (layer >= c->n_layers) return fail(VFKV_ERR_INVALID_ARG, "kv_write: layer %u out of range", layer);
+    if (n_tokens == 0) return VFKV_OK;
+    if (!k_src || !v_src) return fail(VFKV_ERR_INVALID_ARG, "kv_write: NULL source");
+    if ((uint64_t)pos + n_tokens > c->max_seq_len)
+        return fail(VFKV_ERR_INVALID_ARG, "kv_write: positions [%u, %llu) exceed max_seq_len %u", pos,
+                    (unsigned long long)pos + n_tokens, c->max_seq_len);
+    const uint64_t kv_dim = (uint64_t)kvh_for(c, layer) * hd_for(c, layer);
+    const uint64_t n = kv_dim * n_tokens;
+    if (n > UINT32_MAX) return fail(VFKV_ERR_OVERFLOW, "kv_write: %llu elements exceed the u32 element count", (unsigned long long)n);
+    const uint64_t off = layer_off(c, layer) + (uint64_t)pos * row_b(c, layer);
+    if (off % 4u != 0u) return fail(VFKV_ERR_ALIGNMENT, "kv_write: dst_byte_offset must be uint-aligned (got %llu)", (unsigned long long)off);
+    VFKV_HIP(vfkv::launch_kv_append(c->dtype, k_src, v_src, (char*)c->k + off, (char*)c->v + off, (uint32_t)n, 2, S(stream)));
+    return VFKV_OK;
+}
+
+// ---- decode attention ----------------------------------------------------------------------------------
+int vfkv_flash_attn_split(const float* q, const void* k_layer, const void* v_layer, uint32_t kv_dtype,
+                          float* scratch_out, float* scratch_max, float* scratch_sum, const vfkv_split_params* p,
+                          uint32_t tile, float softcap, vfkv_stream stream) {
+    if (!p) return fail(VFKV_ERR_INVALID_ARG, "flash_attn_split: params is NULL");
+    if (!q || !k_layer || !v_layer || !scratch_out || !scratch_max || !scratch_sum)
+        return fail(VFKV_ERR_INVALID_ARG, "flash_attn_split: NULL buffer");
+    if (kv_dtype > VFKV_F8E4M3) return fail(VFKV_ERR_INVALID_ARG, "flash_attn_split: unknown kv dtype %u", kv_dtype);
+    int rc = check_attn_dims(p->n_heads, p->n_kv_heads, p->head_dim);
+    if (rc != VFKV_OK) return rc;
+    if (p->seq_len == 0) return fail(VFKV_ERR_INVALID_ARG, "flash_attn_split: seq_len must be > 0");
+    if (tile == 0 || tile % 16u != 0u || tile > 65536u)
+        return fail(VFKV_ERR_INVALID_ARG, "flash_attn_split: tile must be a multiple of 16 in [16, 65536] (got %u)", tile);
+    const uint32_t need = (p->seq_len + tile - 1u) / tile;
+    if (p->n_tiles != need)
+        return fail(VFKV_ERR_INVALID_ARG, "flash_attn_split: n_tiles (%u) != ceil(seq_len / tile) (%u)", p->n_tiles, need);
+    if (!(softcap >= 0.f)) return fail(VFKV_ERR_INVALID_ARG, "flash_attn_split: softcap must be >= 0");
+    vfkv::SplitLaunch L;
+    L.q = q; L.k = k_layer; L.v = v_layer;
+    L.scratch_out = scratch_out; L.scratch_max = scratch_max; L.scratch_sum = scratch_sum;
+    L.dtype = kv_dtype; L.n_heads = p->n_heads; L.n_kv_heads = p->n_kv_heads; L.head_dim = p->head_dim;
+    L.seq_len = p->seq_len; L.kv_start = p->kv_start; L.tile = tile; L.tile_first = 0; L.n_tiles = p->n_tiles;
+    L.scale = p->scale; L.softcap = softcap;
+    VFKV_HIP(vfkv::launch_split(L, S(stream)));
+    return VFKV_OK;
+}
+
+int vfkv_flash_attn_reduce(const float* scratch_out, const float* scratch_max, const float* scratch_sum, float* o,
+                           uint32_t n_heads, uint32_t head_dim, uint32_t n_tiles, vfkv_stream stream) {
+    if (!scratch_out || !scratch_max || !scratch_sum || !o) return fail(VFKV_ERR_INVALID_ARG, "flash_attn_reduce: NULL buffer");
+    if (n_heads == 0 || head_dim == 0 || n_tiles == 0)
+        return fail(VFKV_ERR_INVALID_ARG, "flash_attn_reduce: n_heads, head_dim and n_tiles must be > 0");
+    if (head_dim > 512) return fail(VFKV_ERR_UNSUPPORTED, "flash_attn_reduce: head_dim %u > 512", head_dim);
+    VFKV_HIP(vfkv::launch_reduce(scratch_out, scratch_max, scratch_sum, o, n_heads, head_dim, n_tiles, S(stream)));
+    return VFKV_OK;
+}
+
+int vfkv_workspace_create(uint32_t n_heads, uint32_t head_dim, uint32_t max_seq_len, vfkv_workspace** out) {
+    if (!out) return fail(VFKV_ERR_INVALID_ARG, "out is NULL");
+    *out = nullptr;
+    if (n_heads == 0 || head_dim == 0 || max_seq_len == 0)
+        return fail(VFKV_ERR_INVALID_ARG, "workspace: n_heads, head_dim and max_seq_len must be > 0");
+    vfkv_workspace* w = new (std::nothrow) vfkv_workspace();
+    if (!w) return fail(VFKV_ERR_HIP, "host allocation failed");
+    w->n_heads = n_heads;
+    w->head_dim = head_dim;
+    w->max_tiles = (max_seq_len + 63u) / 64u;   // setup.rs:208-230
+    uint64_t n_out;
+    if (mul_ovf((uint64_t)n_heads * w->max_tiles, head_dim, &n_out) || n_out > (UINT64_MAX / 8)) {
+        delete w;
+        return fail(VFKV_ERR_OVERFLOW, "workspace size overflow");
+    }
+    const uint64_t n_ml = (uint64_t)n_heads * w->max_tiles;
+    // one allocation: [out | max | sum], each 256-byte aligned
+    const uint64_t out_b = (n_out * 4u + 255u) & ~255ull, ml_b = (n_ml * 4u + 255u) & ~255ull;
+    void* base = nullptr;
+    hipError_t e = hipMalloc(&base, out_b + 2u * ml_b);
+    if (e != hipSuccess) { delete w; return hip_fail(e, "hipMalloc(workspace)"); }
+    w->scratch_out = (float*)base;
+    w->scratch_max = (float*)((char*)base + out_b);
+    w->scratch_sum = (float*)((char*)base + out_b + ml_b);
+    *out = w;
+    return VFKV_OK;
+}
+
+void vfkv_workspace_destroy(vfkv_workspace* w) {
+    if (!w) return;
+    if (w->scratch_out) (void)hipFree(w->scratch_out);
+    delete w;
+}
+
+// Tile length for the convenience path: enough workgroups to cover the 256 CUs about twice, tiles a
+// multiple of 64 keys (so they never exceed the workspace's ceil(max_seq / 64) rows).
+static uint32_t choose_tile(uint32_t span, uint32_t n_kv_heads, uint32_t groups) {
+    static const uint32_t forced = [] {
+        const char* e = getenv("VFKV_DECODE_TILE");
+        return e ? (uint32_t)strtoul(e, nullptr, 10) : 0u;
+    }();
+    if (forced >= 64u && forced % 64u == 0u) return forced;
+    const uint32_t target_wgs = 512u;
+    uint32_t tiles = (target_wgs + n_kv_heads * groups - 1u) / (n_kv_heads * groups);
+    if (tiles == 0u) tiles = 1u;
+    uint32_t tile = (span + tiles - 1u) / tiles;
+    tile = ((tile + 63u) / 64u) * 64u;
+    if (tile < 64u) tile = 64u;
+    return tile;
+}
+
+uint32_t vfkv_decode_tile_for(uint32_t span, uint32_t n_heads, uint32_t n_kv_heads) {
+    if (span == 0u || n_kv_heads == 0u || n_heads == 0u || n_heads % n_kv_heads != 0u) return 0u;
+    const uint32_t g = n_heads / n_kv_heads;
+    const uint32_t groups = (g % 4u == 0u) ? g / 4u : (g % 2u == 0u) ? g / 2u : g;
+    return choose_tile(span, n_kv_heads, groups);
+}
+
+int vfkv_decode_attention(vfkv_cache* c, uint32_t layer, uint32_t kv_layer, uint32_t n_heads, const float* q, float* o,
+                          uint32_t position, uint32_t kv_start, float scale, float softcap, vfkv_workspace* ws,
+                          vfkv_stream stream) {
+    if (!c || !c->k || !c->v) return fail(VFKV_ERR_INVALID_ARG, "decode_attention: cache has no buffers");
+    if (!ws) return fail(VFKV_ERR_INVALID_ARG, "decode_attention: workspace is NULL");
+    if (!q || !o) return fail(VFKV_ERR_INVALID_ARG, "decode_attention: NULL buffer");
+    if (layer >= c->n_layers || kv_layer >= c->n_layers)
+        return fail(VFKV_ERR_INVALID_ARG, "decode_attention: layer %u / kv_layer %u out of range", layer, kv_layer);
+    if (position >= c->max_seq_len)
+        return fail(VFKV_ERR_INVALID_ARG, "decode_attention: position %u >= max_seq_len %u", position, c->max_seq_len);
+    if (!(softcap >= 0.f)) return fail(VFKV_ERR_INVALID_ARG, "decode_attention: softcap must be >= 0");
+    const uint32_t hd = hd_for(c, layer), kvh = kvh_for(c, layer);
+    int rc = check_attn_dims(n_heads, kvh, hd);
+    if (rc != VFKV_OK) return rc;
+    const uint32_t seq_len = position + 1u;
+    if (kv_start >= seq_len) return fail(VFKV_ERR_INVALID_ARG, "decode_attention: kv_start %u leaves no visible key (seq_len %u)", kv_start, seq_len);
+    if (n_heads > ws->n_heads || hd > ws->head_dim)
+        return fail(VFKV_ERR_WORKSPACE, "decode_attention: workspace built for %u heads x %u dims, need %u x %u",
+                    ws->n_heads, ws->head_dim, n_heads, hd);
+    const uint32_t tile = vfkv_decode_tile_for(seq_len - kv_start, n_heads, kvh);
+    const uint32_t first = kv_start / tile;
+    const uint32_t n_tiles = (seq_len + tile - 1u) / tile - first;
+    if (n_tiles > ws->max_tiles) return fail(VFKV_ERR_WORKSPACE, "decode_attention: %u tiles > workspace capacity %u", n_tiles, ws->max_tiles);
+    const uint64_t off = layer_off(c, kv_layer);
+    vfkv::SplitLaunch L;
+    L.q = q; L.k = (char*)c->k + off; L.v = (char*)c->v + off;
+    L.scratch_out = ws->scratch_out; L.scratch_max = ws->scratch_max; L.scratch_sum = ws->scratch_sum;
+    L.dtype = c->dtype; L.n_heads = n_heads; L.n_kv_heads = kvh; L.head_dim = hd;
+    L.seq_len = seq_len; L.kv_start = kv_start; L.tile = tile; L.tile_first = first; L.n_tiles = n_tiles;
+    L.scale = scale; L.softcap = softcap;
+    VFKV_HIP(vfkv::launch_split(L, S(stream)));
+    VFKV_HIP(vfkv::launch_reduce(ws->scratch_out, ws->scratch_max, ws->scratch_sum, o, n_heads, hd, n_tiles, S(stream)));
+    return VFKV_OK;
+}
+
+// ---- prefill attention -------------------------------------------------------------------------------
+int vfkv_flash_attn_batch(const float* q, const void* k_layer, const void* v_layer, uint32_t kv_dtype, float* o,
+                          const vfkv_batch_params* p, float softcap, vfkv_stream stream) {
+    if (!p) return fail(VFKV_ERR_INVALID_ARG, "flash_attn_batch: params is NULL");
+    if (!q || !k_layer || !v_layer || !o) return fail(VFKV_ERR_INVALID_ARG, "flash_attn_batch: NULL buffer");
+    if (kv_dtype > VFKV_F8E4M3) return fail(VFKV_ERR_INVALID_ARG, "flash_attn_batch: unknown kv dtype %u", kv_dtype);
+    int rc = check_attn_dims(p->n_heads, p->n_kv_heads, p->head_dim);
+    if (rc != VFKV_OK) return rc;
+    if (p->m == 0) return VFKV_OK;
+    if (p->n_kv == 0) return fail(VFKV_ERR_INVALID_ARG, "flash_attn_batch: n_kv must be > 0");
+    if (!(softcap >= 0.f)) return fail(VFKV_ERR_INVALID_ARG, "flash_attn_batch: softcap must be >= 0");
+    const uint64_t first_len = (uint64_t)p->q_start + 1u;
+    const uint64_t vis0 = first_len < p->n_kv ? first_len : p->n_kv;
+    if (p->kv_start >= vis0)
+        return fail(VFKV_ERR_INVALID_ARG, "flash_attn_batch: kv_start %u leaves query 0 without a visible key", p->kv_start);
+    vfkv::BatchLaunch L;
+    L.q = q; L.k = k_layer; L.v = v_layer; L.o = o;
+    L.dtype = kv_dtype; L.n_heads = p->n_heads; L.n_kv_heads = p->n_kv_heads; L.head_dim = p->head_dim;
+    L.m = p->m; L.n_kv = p->n_kv; L.q_start = p->q_start; L.kv_start = p->kv_start;
+    L.scale = p->scale; L.softcap = softcap;
+    VFKV_HIP(vfkv::launch_batch(L, S(stream)));
+    return VFKV_OK;
+}
+
+int vfkv_prefill_attention(vfkv_cache* c, uint32_t layer, uint32_t kv_layer, uint32_t n_heads, const float* q, float* o,
+                           uint32_t m, uint32_t base_pos, uint32_t window, float scale, float softcap,
+                           vfkv_stream stream) {
+    if (!c || !c->k || !c->v) return fail(VFKV_ERR_INVALID_ARG, "prefill_attention: cache has no buffers");
+    if (layer >= c->n_layers || kv_layer >= c->n_layers)
+        return fail(VFKV_ERR_INVALID_ARG, "prefill_attention: layer %u / kv_layer %u out of range", layer, kv_layer);
+    if ((uint64_t)base_pos + m > c->max_seq_len)
+        return fail(VFKV_ERR_INVALID_ARG, "prefill_attention: positions [%u, %llu) exceed max_seq_len %u", base_pos,
+                    (unsigned long long)base_pos + m, c->max_seq_len);
+    vfkv_batch_params p;
+    p.n_heads = n_heads;
+    p.n_kv_heads = kvh_for(c, layer);
+    p.head_dim = hd_for(c, layer);
+    p.m = m;
+    p.n_kv = base_pos + m;
+    p.q_start = base_pos;
+    p.scale = scale;
+    p.kv_start = vfkv_kv_start_batch(base_pos, m, window);
+    const uint64_t off = layer_off(c, kv_layer);
+    return vfkv_flash_attn_batch(q, (char*)c->k + off, (char*)c->v + off, c->dtype, o, &p, softcap, stream);
+}
+
+}  // extern "C"

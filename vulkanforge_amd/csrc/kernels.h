@@ -1,0 +1,47 @@
+// Internal launch interface between the C ABI (api.cpp) and the gfx950 kernels.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace vfkv {
+
+// ---- kv_append.hip ----
+hipError_t launch_kv_append(uint32_t dtype, const float* k_src, const float* v_src, void* k_dst, void* v_dst,
+                            uint32_t n_elements, int n_tensors, hipStream_t stream);
+hipError_t launch_fp8_to_f16(const void* src, void* dst, uint64_t n, hipStream_t stream);
+
+// ---- attn_decode.hip ----
+struct SplitLaunch {
+    const float* q;        // [n_heads, head_dim] f32
+    const void* k;         // layer slab, [pos][kv_head][d] in `dtype`
+    const void* v;
+    float* scratch_out;    // [(h * n_tiles + j) * head_dim + d]
+    float* scratch_max;    // [h * n_tiles + j]
+    float* scratch_sum;
+    uint32_t dtype, n_heads, n_kv_heads, head_dim;
+    uint32_t seq_len, kv_start;
+    uint32_t tile;         // keys per tile
+    uint32_t tile_first;   // absolute index of the first tile launched
+    uint32_t n_tiles;      // tiles launched == row length of the scratch arrays
+    float scale, softcap;
+};
+// Returns hipErrorInvalidValue when no kernel covers the shape.
+hipError_t launch_split(const SplitLaunch& a, hipStream_t stream);
+hipError_t launch_reduce(const float* scratch_out, const float* scratch_max, const float* scratch_sum, float* o,
+                         uint32_t n_heads, uint32_t head_dim, uint32_t n_tiles, hipStream_t stream);
+// Smallest tile granule (keys) the split kernel for this shape works in; 0 if unsupported.
+uint32_t split_tile_granule(uint32_t dtype, uint32_t head_dim);
+
+// ---- attn_prefill.hip ----
+struct BatchLaunch {
+    const float* q;   // [m, n_heads, head_dim] f32
+    const void* k;
+    const void* v;
+    float* o;         // [m, n_heads, head_dim] f32
+    uint32_t dtype, n_heads, n_kv_heads, head_dim;
+    uint32_t m, n_kv, q_start, kv_start;
+    float scale, softcap;
+};
+hipError_t launch_batch(const BatchLaunch& a, hipStream_t stream);
+
+}  // namespace vfkv

@@ -1,0 +1,115 @@
+// KV append and expansion kernels for gfx950.
+//
+//   kv_store_fp8   f32 -> E4M3FN bytes      (vk_shaders/kv_store_fp8.comp:42-67)
+//   kv_copy_fp16   f32 -> f16               (vk_shaders/kv_copy_fp16.comp:39-51)
+//   kv_copy_f32    f32 -> f32               (the vkCmdCopyBuffer branch, executor/attention.rs:575-581)
+//   kv_fp8_to_f16  E4M3FN bytes -> f16      (vk_shaders/kv_fp8_to_f16.comp:28-33)
+//
+// All are pure streaming kernels (HBM bound).  One thread converts one 32-bit destination word
+// for the two append kernels -- 16-byte coalesced loads, 4-byte coalesced stores -- so the only
+// alignment the destination needs is the 4 bytes the reference also demands.  K and V of one
+// append go out in a single launch (blockIdx.y selects the tensor).
+#include "device_utils.h"
+#include "kernels.h"
+
+namespace vfkv {
+
+struct AppendArgs {
+    const float* src[2];
+    uint8_t* dst[2];   // already offset by dst_byte_offset
+    uint32_t n;        // elements per tensor
+};
+
+// mode: 0 = fp8, 1 = f16, 2 = f32 copy
+template <int MODE>
+__global__ __launch_bounds__(256) void kv_append_kernel(AppendArgs a) {
+    const float* __restrict__ src = a.src[blockIdx.y];
+    uint8_t* __restrict__ dst = a.dst[blockIdx.y];
+    constexpr uint32_t EPW = MODE == 0 ? 4u : MODE == 1 ? 2u : 1u;  // elements per 32-bit word
+    const uint32_t n = a.n;
+    const uint32_t n_words = (n + EPW - 1u) / EPW;
+    const bool src16 = (((uintptr_t)src) & 15u) == 0u;
+    for (uint32_t w = blockIdx.x * blockDim.x + threadIdx.x; w < n_words; w += gridDim.x * blockDim.x) {
+        const uint32_t e0 = w * EPW;
+        float v[4] = {0.f, 0.f, 0.f, 0.f};
+        if (MODE == 0 && src16 && e0 + 4u <= n) {
+            const float4 f = *reinterpret_cast<const float4*>(src + e0);
+            v[0] = f.x; v[1] = f.y; v[2] = f.z; v[3] = f.w;
+        } else {
+#pragma unroll
+            for (uint32_t j = 0; j < EPW; ++j)
+                if (e0 + j < n) v[j] = src[e0 + j];  // ragged tail is zero-padded to the word
+        }
+        uint32_t out;
+        if (MODE == 0) {
+            out = pack4_e4m3(v[0], v[1], v[2], v[3]);
+        } else if (MODE == 1) {
+            out = f32_to_h16_bits(v[0]) | (f32_to_h16_bits(v[1]) << 16);
+        } else {
+            out = __builtin_bit_cast(uint32_t, v[0]);
+        }
+        reinterpret_cast<uint32_t*>(dst)[w] = out;
+    }
+}
+
+template <int MODE>
+static hipError_t launch_append(const float* k_src, const float* v_src, void* k_dst, void* v_dst, uint32_t n,
+                                int n_tensors, hipStream_t stream) {
+    if (n == 0) return hipSuccess;
+    AppendArgs a;
+    a.src[0] = k_src; a.src[1] = v_src;
+    a.dst[0] = (uint8_t*)k_dst; a.dst[1] = (uint8_t*)v_dst;
+    a.n = n;
+    constexpr uint32_t EPW = MODE == 0 ? 4u : MODE == 1 ? 2u : 1u;
+    const uint32_t n_words = (n + EPW - 1u) / EPW;
+    uint32_t blocks = (n_words + 255u) / 256u;
+    if (blocks > 4096u) blocks = 4096u;
+    hipLaunchKernelGGL(kv_append_kernel<MODE>, dim3(blocks, n_tensors), dim3(256), 0, stream, a);
+    return hipGetLastError();
+}
+
+hipError_t launch_kv_append(uint32_t dtype, const float* k_src, const float* v_src, void* k_dst, void* v_dst,
+                            uint32_t n, int n_tensors, hipStream_t stream) {
+    if (dtype == kF8) return launch_append<0>(k_src, v_src, k_dst, v_dst, n, n_tensors, stream);
+    if (dtype == kF16) return launch_append<1>(k_src, v_src, k_dst, v_dst, n, n_tensors, stream);
+    return launch_append<2>(k_src, v_src, k_dst, v_dst, n, n_tensors, stream);
+}
+
+// ---- E4M3 -> f16 expansion -------------------------------------------------------------------
+// 16 codes per thread: one 16-byte load, eight packed conversions, two 16-byte stores.
+__global__ __launch_bounds__(256) void kv_fp8_to_f16_kernel(const uint8_t* __restrict__ src,
+                                                            uint16_t* __restrict__ dst, uint64_t n, int vec_ok) {
+    const uint64_t n_vec = vec_ok ? n / 16u : 0u;
+    const uint64_t stride = (uint64_t)gridDim.x * blockDim.x;
+    const uint64_t tid = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    for (uint64_t i = tid; i < n_vec; i += stride) {
+        const uint4 w = reinterpret_cast<const uint4*>(src)[i];
+        const uint32_t in[4] = {w.x, w.y, w.z, w.w};
+        uint32_t out[8];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            half2_t lo, hi;
+            e4m3x4_to_h2(in[j], lo, hi);
+            out[2 * j] = __builtin_bit_cast(uint32_t, lo);
+            out[2 * j + 1] = __builtin_bit_cast(uint32_t, hi);
+        }
+        uint4* d = reinterpret_cast<uint4*>(dst) + 2u * i;
+        d[0] = make_uint4(out[0], out[1], out[2], out[3]);
+        d[1] = make_uint4(out[4], out[5], out[6], out[7]);
+    }
+    for (uint64_t i = n_vec * 16u + tid; i < n; i += stride)
+        dst[i] = (uint16_t)f32_to_h16_bits(__builtin_amdgcn_cvt_f32_fp8((int)src[i], 0));
+}
+
+hipError_t launch_fp8_to_f16(const void* src, void* dst, uint64_t n, hipStream_t stream) {
+    if (n == 0) return hipSuccess;
+    const int vec_ok = ((((uintptr_t)src) | ((uintptr_t)dst)) & 15u) == 0u;
+    uint64_t work = vec_ok ? (n + 15u) / 16u : n;
+    uint64_t blocks = (work + 255u) / 256u;
+    if (blocks > 8192u) blocks = 8192u;
+    hipLaunchKernelGGL(kv_fp8_to_f16_kernel, dim3((uint32_t)blocks), dim3(256), 0, stream,
+                       (const uint8_t*)src, (uint16_t*)dst, n, vec_ok);
+    return hipGetLastError();
+}
+
+}  // namespace vfkv

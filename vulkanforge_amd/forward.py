@@ -1,0 +1,147 @@
+"""Host mirror of the reference's dispatch helpers for this path (``Forward::run_*`` in
+src/backend/vulkan/forward/runs.rs and the four executor steps in forward/executor/attention.rs).
+
+Arguments are PyTorch CUDA(HIP) tensors or raw device pointers; PyTorch only supplies memory and
+the stream.  Every method enqueues on ``stream`` (default: torch's current stream) and returns
+without synchronising, like the reference records into an open command buffer.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import math
+
+from . import _ffi
+from .kv_cache import KvCache, KvDtype
+
+FA_TILE = 64  # runs.rs:766, flash_attn_split.comp:23-24
+
+
+def _ptr(x) -> int:
+    if x is None:
+        return 0
+    if isinstance(x, int):
+        return x
+    if not x.is_cuda:
+        raise ValueError("expected a device tensor: this path has no CPU implementation")
+    if not x.is_contiguous():
+        raise ValueError("expected a contiguous tensor")
+    return x.data_ptr()
+
+
+def _stream(stream) -> int:
+    if stream is None:
+        import torch
+        return torch.cuda.current_stream().cuda_stream
+    if isinstance(stream, int):
+        return stream
+    return stream.cuda_stream
+
+
+class Workspace:
+    """fa_scratch_out / max / sum (forward/setup.rs:203-230)."""
+
+    def __init__(self, n_heads: int, head_dim: int, max_seq_len: int):
+        h = C.c_void_p()
+        _ffi.check(_ffi.lib().vfkv_workspace_create(n_heads, head_dim, max_seq_len, C.byref(h)))
+        self._h = h
+
+    def destroy(self):
+        if getattr(self, "_h", None):
+            _ffi.lib().vfkv_workspace_destroy(self._h)
+            self._h = None
+
+    def __del__(self):
+        try:
+            self.destroy()
+        except Exception:
+            pass
+
+
+class Forward:
+    """The part of the reference's ``Forward`` that this path needs: a cache, a workspace, the head
+    geometry, and the default ``attn_scale = 1/sqrt(head_dim)`` (forward/setup.rs:786)."""
+
+    def __init__(self, kv_cache: KvCache, n_heads: int, workspace: Workspace | None = None):
+        self.kv_cache = kv_cache
+        self.n_heads = n_heads
+        cfg = kv_cache.config
+        max_hd = max(cfg.per_layer_head_dim) if cfg.per_layer_head_dim else cfg.head_dim
+        self.workspace = workspace or Workspace(n_heads, max_hd, cfg.max_seq_len)
+        self.attn_scale = 1.0 / math.sqrt(cfg.head_dim)
+
+    # ---- KV append (runs.rs:2389-2478) ----
+    @staticmethod
+    def run_kv_store_fp8(src, dst, n_elements: int, dst_byte_offset: int, stream=None) -> None:
+        _ffi.check(_ffi.lib().vfkv_store_fp8(_ptr(src), _ptr(dst), n_elements, dst_byte_offset, _stream(stream)))
+
+    @staticmethod
+    def run_kv_copy_fp16(src, dst, n_elements: int, dst_byte_offset: int, stream=None) -> None:
+        _ffi.check(_ffi.lib().vfkv_copy_fp16(_ptr(src), _ptr(dst), n_elements, dst_byte_offset, _stream(stream)))
+
+    @staticmethod
+    def run_kv_fp8_to_f16(src, dst, n_elems: int, stream=None) -> None:
+        """The conversion pass of run_flash_attn_cm_gemma_rs (runs.rs:1105-1137)."""
+        _ffi.check(_ffi.lib().vfkv_fp8_to_f16(_ptr(src), _ptr(dst), n_elems, _stream(stream)))
+
+    def step_kv_write(self, layer: int, position: int, k_src, v_src, stream=None) -> None:
+        """executor/attention.rs:546-597 (one token)."""
+        _ffi.check(_ffi.lib().vfkv_kv_write(self.kv_cache.handle, layer, position, 1, _ptr(k_src), _ptr(v_src),
+                                            _stream(stream)))
+
+    def b_step_kv_write(self, layer: int, base_pos: int, seq_len: int, batch_k, batch_v, stream=None) -> None:
+        """executor/attention.rs:2134-2190 (seq_len tokens in one launch)."""
+        _ffi.check(_ffi.lib().vfkv_kv_write(self.kv_cache.handle, layer, base_pos, seq_len, _ptr(batch_k),
+                                            _ptr(batch_v), _stream(stream)))
+
+    # ---- decode attention (runs.rs:722-822, 1463-1571) ----
+    @staticmethod
+    def run_flash_attn_split(q, k_layer, v_layer, kv_dtype, scratch_out, scratch_max, scratch_sum, n_heads,
+                             n_kv_heads, head_dim, seq_len, scale, kv_start=0, tile=FA_TILE, softcap=0.0,
+                             max_seq=0, stream=None) -> int:
+        n_tiles = (seq_len + tile - 1) // tile
+        p = _ffi.SplitParams(n_heads, n_kv_heads, head_dim, seq_len, max_seq, scale, n_tiles, kv_start)
+        _ffi.check(_ffi.lib().vfkv_flash_attn_split(_ptr(q), _ptr(k_layer), _ptr(v_layer), int(kv_dtype),
+                                                    _ptr(scratch_out), _ptr(scratch_max), _ptr(scratch_sum),
+                                                    C.byref(p), tile, softcap, _stream(stream)))
+        return n_tiles
+
+    @staticmethod
+    def run_flash_attn_reduce(scratch_out, scratch_max, scratch_sum, o, n_heads, head_dim, n_tiles,
+                              stream=None) -> None:
+        _ffi.check(_ffi.lib().vfkv_flash_attn_reduce(_ptr(scratch_out), _ptr(scratch_max), _ptr(scratch_sum),
+                                                     _ptr(o), n_heads, head_dim, n_tiles, _stream(stream)))
+
+    def run_scalar_attn(self, layer: int, position: int, q, o, kv_layer: int | None = None, kv_start: int = 0,
+                        scale: float | None = None, softcap: float = 0.0, stream=None) -> None:
+        """Decode router (runs.rs:722-822); scale defaults to 1/sqrt(head_dim_for(layer))."""
+        if scale is None:
+            hd = self.kv_cache.head_dim_for(layer)
+            scale = self.attn_scale if hd == self.kv_cache.config.head_dim else 1.0 / math.sqrt(hd)
+        _ffi.check(_ffi.lib().vfkv_decode_attention(self.kv_cache.handle, layer,
+                                                    layer if kv_layer is None else kv_layer, self.n_heads,
+                                                    _ptr(q), _ptr(o), position, kv_start, scale, softcap,
+                                                    self.workspace._h, _stream(stream)))
+
+    step_attention = run_scalar_attn  # executor/attention.rs:599-625
+
+    # ---- prefill attention (runs.rs:933-1010, executor/attention.rs:2192-2390) ----
+    @staticmethod
+    def run_flash_attn_batch(q, k_layer, v_layer, kv_dtype, o, n_heads, n_kv_heads, head_dim, m, q_start, n_kv,
+                             scale, kv_start=0, softcap=0.0, stream=None) -> None:
+        p = _ffi.BatchParams(n_heads, n_kv_heads, head_dim, m, n_kv, q_start, scale, kv_start)
+        _ffi.check(_ffi.lib().vfkv_flash_attn_batch(_ptr(q), _ptr(k_layer), _ptr(v_layer), int(kv_dtype), _ptr(o),
+                                                    C.byref(p), softcap, _stream(stream)))
+
+    def b_step_attention(self, layer: int, base_pos: int, seq_len: int, q, o, kv_layer: int | None = None,
+                         kv_start_window: int = 0, scale: float | None = None, softcap: float = 0.0,
+                         stream=None) -> None:
+        if scale is None:
+            hd = self.kv_cache.head_dim_for(layer)
+            scale = self.attn_scale if hd == self.kv_cache.config.head_dim else 1.0 / math.sqrt(hd)
+        _ffi.check(_ffi.lib().vfkv_prefill_attention(self.kv_cache.handle, layer,
+                                                     layer if kv_layer is None else kv_layer, self.n_heads,
+                                                     _ptr(q), _ptr(o), seq_len, base_pos, kv_start_window, scale,
+                                                     softcap, _stream(stream)))
+
+
+__all__ = ["Forward", "Workspace", "KvDtype", "FA_TILE"]

@@ -1,0 +1,78 @@
+"""The benchmark configurations of this path (geometry and synthetic-input recipes) and their
+algorithmic work, so tests and the benchmark agree on shapes and byte counts."""
+from __future__ import annotations
+
+from dataclasses import dataclass
+
+from .kv_cache import KvDtype
+
+
+@dataclass(frozen=True)
+class DecodeWorkload:
+    name: str
+    n_layers: int
+    n_heads: int
+    n_kv_heads: int
+    head_dim: int
+    context: int            # keys visible to the decode query (after the append, if any)
+    dtype: KvDtype
+    append: bool            # append one token per layer inside the step
+    softcap: float = 0.0
+    window: int = 0         # sliding window of the sliding layers (0 = none)
+    sliding_pattern: int = 0  # k sliding layers followed by one global layer, repeated
+
+    def layer_window(self, layer: int) -> int:
+        if not self.window or not self.sliding_pattern:
+            return 0
+        return 0 if (layer % (self.sliding_pattern + 1)) == self.sliding_pattern else self.window
+
+    def kv_bytes_layer(self, layer: int) -> int:
+        win = self.layer_window(layer)
+        keys = min(self.context, win) if win else self.context
+        return 2 * keys * self.n_kv_heads * self.head_dim * self.dtype.element_size()
+
+    def kv_bytes_step(self) -> int:
+        """Algorithmic KV bytes one decode step must read (K and V of every visible key once)."""
+        return sum(self.kv_bytes_layer(i) for i in range(self.n_layers))
+
+
+@dataclass(frozen=True)
+class PrefillWorkload:
+    name: str
+    n_layers: int
+    n_heads: int
+    n_kv_heads: int
+    head_dim: int
+    base_pos: int
+    m: int
+    dtype: KvDtype
+
+    def pairs_per_head(self) -> int:
+        return sum(self.base_pos + i + 1 for i in range(self.m))
+
+    def flops_layer(self) -> int:
+        """4 * head_dim flop per (query, key) pair and head, causal-exact."""
+        return self.pairs_per_head() * self.n_heads * 4 * self.head_dim
+
+    def kv_bytes_layer(self) -> int:
+        return 2 * (self.base_pos + self.m) * self.n_kv_heads * self.head_dim * self.dtype.element_size()
+
+
+DECODE = {
+    "decode_f16_2k_1layer": DecodeWorkload("decode_f16_2k_1layer", 1, 32, 8, 128, 2049, KvDtype.F16, True),
+    "decode_fp8_8k_32layers": DecodeWorkload("decode_fp8_8k_32layers", 32, 32, 8, 128, 8193, KvDtype.F8, True),
+    "decode_fp8_32k_32layers": DecodeWorkload("decode_fp8_32k_32layers", 32, 32, 8, 128, 32768, KvDtype.F8, False),
+    "decode_f16_hd256_sliding_12layers": DecodeWorkload("decode_f16_hd256_sliding_12layers", 12, 16, 8, 256, 16384,
+                                                        KvDtype.F16, False, softcap=50.0, window=4096,
+                                                        sliding_pattern=5),
+}
+PREFILL = {
+    "prefill_fp8_512x4608_32layers": PrefillWorkload("prefill_fp8_512x4608_32layers", 32, 32, 8, 128, 4096, 512,
+                                                     KvDtype.F8),
+}
+
+assert DECODE["decode_f16_2k_1layer"].kv_bytes_step() == 8_392_704
+assert DECODE["decode_fp8_8k_32layers"].kv_bytes_step() == 536_936_448
+assert DECODE["decode_fp8_32k_32layers"].kv_bytes_step() == 2_147_483_648
+assert DECODE["decode_f16_hd256_sliding_12layers"].kv_bytes_step() == 603_979_776
+assert PREFILL["prefill_fp8_512x4608_32layers"].flops_layer() == 36_511_416_320

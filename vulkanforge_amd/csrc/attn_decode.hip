@@ -1,16 +1,25 @@
 // Split-K decode attention for gfx950: worker (flash_attn_split.comp:82-162) and log-sum-exp
 // merge (flash_attn_reduce.comp:35-81), re-designed around the HBM stream.
 //
-// Worker layout.  One workgroup (4 wavefronts) owns one (tile of keys, KV head, group of GT query
-// heads).  A K or V row of one KV head is D*elem bytes; LPR = D*elem/16 lanes cover it with one
-// 16-byte load each, so a wavefront load instruction fetches RPI = 64/LPR complete rows and every
-// byte of the row is requested exactly once per KV head -- the GT query heads of the GQA group are
-// all served from the same registers.  Lane (r, c) keeps the c-th 16-byte slice of Q for each of the
-// GT heads in registers, accumulates GT partial dot products per K row, and the LPR lanes of a row
-// combine them with a butterfly.  Scores of a block of BI row-iterations stay in registers; the
-// block maximum is made wavefront-uniform, weights are exponentiated once, and the same lanes then
-// stream the V rows and accumulate GT x (16/elem) outputs each.  Row groups, wavefronts and finally
-// workgroups are merged by log-sum-exp weights.  All arithmetic after the element decode is f32.
+// Worker.  One workgroup (NW wavefronts) owns one (tile of keys, KV head, group of GT query heads);
+// every K / V byte of the tile is requested from memory once and serves all GT heads of the GQA
+// group.  Each wavefront walks its share of the tile in runs of 64 rows:
+//
+//   K phase   LPRK lanes x 16 B cover a row, so one load instruction fetches 64/LPRK whole rows.
+//             Each lane keeps its 16-byte slice of Q for the GT heads in registers as f16 pairs,
+//             multiplies with v_dot2_f32_f16 (products of two f16 values are exact in f32) and the
+//             lanes of a row combine their partial sums with DPP butterflies.  The row's GT scores
+//             go to LDS.  When Q is not exactly representable in f16 the run is swept a second time
+//             with the rounding remainders of Q, which restores f32 accuracy.
+//   softmax   one lane per row: scale, optional soft-cap, mask, wavefront maximum through DPP row
+//             broadcasts, one exp2 per score; the weights go back to LDS.
+//   V phase   LPRV lanes x VB bytes cover a row; every lane accumulates GT x VE outputs in f32.
+//
+// K and V rows travel through two small register rings that are refilled immediately after use
+// with the rows needed one ring-length later (of this run or of the wavefront's next run), so the
+// loads of one phase are in flight during the other.  Loads are raw buffer loads whose descriptor
+// ends at the last populated row: rows past it read as zero without touching memory, which is also
+// how the ring is "refilled" when there is no next run.
 #include "device_utils.h"
 #include "kernels.h"
 
@@ -32,203 +41,331 @@ struct SplitArgs {
 template <int DT>
 struct ElemBytes { static constexpr int value = DT == kF32 ? 4 : DT == kF16 ? 2 : 1; };
 
-// Decode the 16 bytes a lane loaded into EPL floats.
-template <int DT>
-__device__ __forceinline__ void decode16(const uint4& raw, float* out) {
-    const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
-    if (DT == kF8) {
+template <int GT> struct RowVec;
+template <> struct RowVec<4> { typedef float4_t T; };
+template <> struct RowVec<2> { typedef float2_t T; };
+template <> struct RowVec<1> { typedef float T; };
+template <int GT> __device__ __forceinline__ float rv_get(const typename RowVec<GT>::T& v, int g) { return v[g]; }
+template <> __device__ __forceinline__ float rv_get<1>(const float& v, int) { return v; }
+template <int GT> __device__ __forceinline__ void rv_set(typename RowVec<GT>::T& v, int g, float x) { v[g] = x; }
+template <> __device__ __forceinline__ void rv_set<1>(float& v, int, float x) { v = x; }
+
+constexpr uint32_t kOOB = 0x80000000u;   // byte offset beyond any slab (slabs are < 2 GiB): the buffer load returns zeros, no memory access
+constexpr int kRun = 64;                 // rows per run: one softmax row per lane
+
+template <int DT, int D, int GT, int NW, bool CAP>
+__global__ __launch_bounds__(NW * 64) void split_kernel(SplitArgs a) {
+  constexpr int ES = ElemBytes<DT>::value;
+  constexpr int KE = 16 / ES;
+  constexpr int QR = DT == kF32 ? KE : KE / 2;
+  constexpr int LPRK = D / KE, RPK = 64 / LPRK, KI = kRun / RPK;     // K loads per run
+  constexpr int VB0 = (ES == 1 && GT > 2) ? 8 : 16;          // keeps GT x VE accumulators at <= 32 registers
+  constexpr int VB = (D * ES / VB0 < 8) ? D * ES / 8 : VB0;    // at least 8 lanes per V row
+  constexpr int VE = VB / ES;
+  constexpr int LPRV = D * ES / VB, RPV = 64 / LPRV, VI = kRun / RPV;  // V loads per run
+  constexpr int PFK = KI < 8 ? KI : 8;                                // registers in the K ring
+  constexpr int PFV = VB == 8 ? (VI < 16 ? VI : 16) : (VI < 8 ? VI : 8);
+  constexpr bool SPLITQ = DT != kF32;
+  static_assert(LPRK >= 4 && LPRK <= 64 && LPRV >= 8 && LPRV <= 64, "unsupported row shape");
+  static_assert(KI % PFK == 0 && VI % PFV == 0, "rings must tile a run");
+  typedef typename RowVec<GT>::T rowvec_t;
+
+  __shared__ rowvec_t lds_s[NW][kRun];
+  constexpr int QN = SPLITQ ? D / 2 : D;
+  __shared__ uint32_t lds_q[2][GT][QN];
+  __shared__ float lds_o[NW][GT][D];
+  __shared__ float lds_m[NW][GT], lds_l[NW][GT];
+  __shared__ int lds_haslo;
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int ck = lane % LPRK, rk = lane / LPRK;
+  const int cv = lane % LPRV, rv = lane / LPRV;
+  const uint32_t jl = blockIdx.x, kvh = blockIdx.y;
+  const uint32_t h0 = kvh * (a.n_heads / a.n_kv_heads) + blockIdx.z * GT;
+  const uint32_t tile_base = (a.tile_first + jl) * a.tile;
+  uint32_t tile_end = tile_base + a.tile; if (tile_end > a.seq_len) tile_end = a.seq_len;
+  const uint32_t lo = tile_base > a.kv_start ? tile_base : a.kv_start;
+
+  // ---- Q -> LDS once per workgroup ----
+  if (tid == 0) lds_haslo = 0;
+  __syncthreads();
+  {
+    bool any_lo = false;
+    if (SPLITQ) {
+      for (int idx = tid; idx < GT * D / 2; idx += NW * 64) {
+        const int g = idx / (D / 2), pr = idx % (D / 2);
+        const float2 f = *reinterpret_cast<const float2*>(a.q + (size_t)(h0 + g) * D + 2 * pr);
+        const _Float16 hx = (_Float16)f.x, hy = (_Float16)f.y;
+        const _Float16 lx = (_Float16)(f.x - (float)hx), ly = (_Float16)(f.y - (float)hy);
+        lds_q[0][g][pr] = __builtin_bit_cast(uint32_t, half2_t{hx, hy});
+        lds_q[1][g][pr] = __builtin_bit_cast(uint32_t, half2_t{lx, ly});
+        any_lo |= (lx != (_Float16)0) | (ly != (_Float16)0);
+      }
+      if (any_lo) lds_haslo = 1;
+    } else {
+      for (int idx = tid; idx < GT * D; idx += NW * 64) {
+        const int g = idx / D, d = idx % D;
+        lds_q[0][g][d] = __builtin_bit_cast(uint32_t, a.q[(size_t)(h0 + g) * D + d]);
+      }
+    }
+  }
+  __syncthreads();
+  const int npass = (SPLITQ && __builtin_amdgcn_readfirstlane(lds_haslo) != 0) ? 2 : 1;
+  uint32_t qh[GT][QR];
+  auto load_q = [&](int part) {
 #pragma unroll
-        for (int j = 0; j < 4; ++j) e4m3x4_to_f32(w[j], out + 4 * j);
-    } else if (DT == kF16) {
+    for (int g = 0; g < GT; ++g)
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            out[2 * j] = h16_bits_to_f32(w[j] & 0xFFFFu);
-            out[2 * j + 1] = h16_bits_to_f32(w[j] >> 16);
+      for (int j = 0; j < QR; ++j) qh[g][j] = lds_q[part][g][ck * QR + j];
+  };
+  load_q(0);
+
+  float m_run[GT], l_run[GT], acc[GT][VE];
+#pragma unroll
+  for (int g = 0; g < GT; ++g) { m_run[g] = kMasked; l_run[g] = 0.f;
+#pragma unroll
+    for (int e = 0; e < VE; ++e) acc[g][e] = 0.f; }
+
+  const uint32_t row_stride = a.n_kv_heads * D * ES;
+  const __amdgpu_buffer_rsrc_t krsrc = __builtin_amdgcn_make_buffer_rsrc((void*)a.k, 0, a.seq_len * row_stride, 0x00020000);
+  const __amdgpu_buffer_rsrc_t vrsrc = __builtin_amdgcn_make_buffer_rsrc((void*)a.v, 0, a.seq_len * row_stride, 0x00020000);
+  const uint32_t lane_koff = rk * row_stride + kvh * D * ES + ck * 16;
+  const uint32_t lane_voff = rv * row_stride + kvh * D * ES + cv * VB;
+  const float scale_l2 = a.scale * 1.44269504088896f;
+  const float cap_l2 = a.softcap * 1.44269504088896f;
+
+  // runs of this wavefront: w, w + NW, ... counted from the first run that reaches the window
+  const uint32_t first_run = (lo - tile_base) / kRun;
+  const uint32_t n_runs = tile_end > tile_base ? (tile_end - tile_base + kRun - 1) / kRun : 0;
+  auto run_off = [&](uint32_t r) -> uint32_t {   // byte offset of a run's first row, or out of bounds when there is none
+    return r < n_runs ? (tile_base + r * kRun) * row_stride : kOOB;
+  };
+
+  u32x4 kreg[PFK];
+  u32x4 vreg4[VB == 16 ? PFV : 1];
+  u32x2 vreg2[VB == 8 ? PFV : 1];
+  // lane part in the VGPR offset, uniform part in the scalar offset; the range check covers their sum
+  auto issue_k = [&](int j, uint32_t off) { kreg[j] = __builtin_amdgcn_raw_buffer_load_b128(krsrc, lane_koff, off, 0); };
+  auto issue_v = [&](int j, uint32_t off) {
+    if (VB == 16) vreg4[j] = __builtin_amdgcn_raw_buffer_load_b128(vrsrc, lane_voff, off, 0);
+    else vreg2[j] = __builtin_amdgcn_raw_buffer_load_b64(vrsrc, lane_voff, off, 0);
+  };
+
+  uint32_t r = first_run + w;
+  if (lo < tile_end && r < n_runs) {
+    {
+      const uint32_t off = run_off(r);
+#pragma unroll
+      for (int j = 0; j < PFK; ++j) issue_k(j, off + (uint32_t)(j * RPK) * row_stride);
+#pragma unroll
+      for (int j = 0; j < PFV; ++j) issue_v(j, off + (uint32_t)(j * RPV) * row_stride);
+    }
+    for (; r < n_runs; r += NW) {
+      const uint32_t off = run_off(r), noff = run_off(r + NW);
+      const uint32_t rb = tile_base + r * kRun;
+      // ---------------- K phase ----------------
+      // (vector elements are copied to scalars before __builtin_bit_cast: bit-casting the element
+      // expression directly was observed to read element 0)
+      auto dot = [&](int j, float (&s)[GT]) {
+        if (DT == kF8) {
+          half2_t kh[8];
+#pragma unroll
+          for (int x = 0; x < 4; ++x) e4m3x4_to_h2(kreg[j][x], kh[2 * x], kh[2 * x + 1]);
+#pragma unroll
+          for (int g = 0; g < GT; ++g) {
+            float d2 = 0.f;
+#pragma unroll
+            for (int x = 0; x < 8; ++x) d2 = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2_t, qh[g][x % QR]), kh[x], d2, false);
+            s[g] = d2;
+          }
+        } else if (DT == kF16) {
+#pragma unroll
+          for (int g = 0; g < GT; ++g) {
+            float d2 = 0.f;
+#pragma unroll
+            for (int x = 0; x < 4; ++x) { const uint32_t kw = kreg[j][x]; d2 = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2_t, qh[g][x % QR]), __builtin_bit_cast(half2_t, kw), d2, false); }
+            s[g] = d2;
+          }
+        } else {
+#pragma unroll
+          for (int g = 0; g < GT; ++g) {
+            float d2 = 0.f;
+#pragma unroll
+            for (int x = 0; x < 4; ++x) { const uint32_t kw = kreg[j][x]; d2 = fmaf(__builtin_bit_cast(float, qh[g][x % QR]), __builtin_bit_cast(float, kw), d2); }
+            s[g] = d2;
+          }
         }
+      };
+      auto put_scores = [&](int i, float (&s)[GT], bool accumulate) {
+        rowvec_t sv;
+#pragma unroll
+        for (int g = 0; g < GT; ++g) rv_set<GT>(sv, g, group_sum<LPRK>(s[g]));
+        if (ck == 0) {
+          if (accumulate) { rowvec_t old = lds_s[w][i * RPK + rk]; lds_s[w][i * RPK + rk] = old + sv; }
+          else lds_s[w][i * RPK + rk] = sv;
+        }
+      };
+      // Q = hi + lo (only when some lo != 0): the run is swept once per part, Q swapped through LDS; the
+      // second sweep re-reads the same K rows (cache hits) through the same ring.
+#pragma unroll 1
+      for (int pass = 0; pass < npass; ++pass) {
+        if (npass == 2) load_q(pass);
+        const uint32_t wrap = (pass + 1 < npass) ? off : noff;
+#pragma unroll
+        for (int i = 0; i < KI; ++i) {
+          float s[GT];
+          dot(i % PFK, s);
+          issue_k(i % PFK, i + PFK < KI ? off + (uint32_t)((i + PFK) * RPK) * row_stride : wrap + (uint32_t)((i + PFK - KI) * RPK) * row_stride);
+          put_scores(i, s, pass > 0);
+        }
+      }
+      if (npass == 2) load_q(0);
+      __builtin_amdgcn_wave_barrier();
+      // ---------------- softmax: lane = row ----------------
+      {
+        const uint32_t t = rb + lane;
+        const bool valid = t < tile_end && t >= lo;
+        rowvec_t sv = lds_s[w][lane];
+        float x[GT];
+        bool changed = false;
+        float mnew[GT];
+#pragma unroll
+        for (int g = 0; g < GT; ++g) {
+          float y = rv_get<GT>(sv, g) * scale_l2;
+          if (CAP) y = cap_l2 * tanhf(y / cap_l2);
+          y = valid ? y : kMasked;
+          x[g] = y;
+          mnew[g] = fmaxf(m_run[g], wave_max_uniform(y));
+          changed |= mnew[g] > m_run[g];
+        }
+        if (changed) {
+#pragma unroll
+          for (int g = 0; g < GT; ++g) {
+            const float alpha = exp2f(m_run[g] - mnew[g]);
+            l_run[g] *= alpha;
+#pragma unroll
+            for (int e = 0; e < VE; ++e) acc[g][e] *= alpha;
+            m_run[g] = mnew[g];
+          }
+        }
+#pragma unroll
+        for (int g = 0; g < GT; ++g) {
+          const float p = valid ? exp2f(x[g] - m_run[g]) : 0.f;
+          l_run[g] += p;
+          rv_set<GT>(sv, g, p);
+        }
+        lds_s[w][lane] = sv;
+      }
+      __builtin_amdgcn_wave_barrier();
+      // ---------------- V phase ----------------
+#pragma unroll
+      for (int i = 0; i < VI; ++i) {
+        const int j = i % PFV;
+        float vf[VE];
+        if (DT == kF8) {
+          if (VB == 8) { e4m3x4_to_f32(vreg2[j].x, vf); e4m3x4_to_f32(vreg2[j].y, vf + 4 % VE); }
+          else {
+#pragma unroll
+            for (int q4 = 0; q4 < 4; ++q4) e4m3x4_to_f32(vreg4[j][q4], vf + (4 * q4) % VE);
+          }
+        } else if (DT == kF16) {
+#pragma unroll
+          for (int q4 = 0; q4 < 4; ++q4) { vf[(2 * q4) % VE] = h16_bits_to_f32(vreg4[j][q4] & 0xFFFFu); vf[(2 * q4 + 1) % VE] = h16_bits_to_f32(vreg4[j][q4] >> 16); }
+        } else {
+#pragma unroll
+          for (int q4 = 0; q4 < 4; ++q4) { const uint32_t vw = vreg4[j][q4]; vf[q4 % VE] = __builtin_bit_cast(float, vw); }
+        }
+        issue_v(j, (i + PFV < VI ? off + (uint32_t)((i + PFV) * RPV) * row_stride : noff + (uint32_t)((i + PFV - VI) * RPV) * row_stride));
+        const rowvec_t pv = lds_s[w][i * RPV + rv];
+#pragma unroll
+        for (int g = 0; g < GT; ++g) {
+          const float p = rv_get<GT>(pv, g);
+#pragma unroll
+          for (int e = 0; e < VE; ++e) acc[g][e] = fmaf(p, vf[e], acc[g][e]);
+        }
+      }
+      __builtin_amdgcn_wave_barrier();
+    }
+  }
+
+  // ---------------- wave-level merge of the RPV row groups, then workgroup merge ----------------
+#pragma unroll
+  for (int g = 0; g < GT; ++g) l_run[g] = wave_sum_uniform(l_run[g]);
+  constexpr int G1 = (LPRV <= 32 && GT >= 2) ? GT / 2 : GT;
+  float r1[G1][VE];
+  int head_off = 0;
+  if (LPRV <= 32) {
+    if (GT >= 2) {
+#pragma unroll
+      for (int g = 0; g < G1; ++g)
+#pragma unroll
+        for (int e = 0; e < VE; ++e) { float x = acc[g][e], y = acc[g + G1][e]; swap32(x, y); r1[g][e] = x + y; }
+      head_off += (lane >> 5) * G1;
     } else {
 #pragma unroll
-        for (int j = 0; j < 4; ++j) out[j] = __builtin_bit_cast(float, w[j]);
+      for (int e = 0; e < VE; ++e) r1[0][e] = xor32_sum(acc[0][e]);
     }
+  } else {
+#pragma unroll
+    for (int g = 0; g < G1; ++g)
+#pragma unroll
+      for (int e = 0; e < VE; ++e) r1[g][e] = acc[g][e];
+  }
+  constexpr int G2 = (LPRV <= 16 && G1 >= 2) ? G1 / 2 : G1;
+  float r2[G2][VE];
+  if (LPRV <= 16) {
+    if (G1 >= 2) {
+#pragma unroll
+      for (int g = 0; g < G2; ++g)
+#pragma unroll
+        for (int e = 0; e < VE; ++e) { float x = r1[g][e], y = r1[g + G2][e]; swap16(x, y); r2[g][e] = x + y; }
+      head_off += ((lane >> 4) & 1) * G2;
+    } else {
+#pragma unroll
+      for (int e = 0; e < VE; ++e) r2[0][e] = xor16_sum(r1[0][e]);
+    }
+  } else {
+#pragma unroll
+    for (int g = 0; g < G2; ++g)
+#pragma unroll
+      for (int e = 0; e < VE; ++e) r2[g][e] = r1[g][e];
+  }
+  if (LPRV <= 8) {
+#pragma unroll
+    for (int g = 0; g < G2; ++g)
+#pragma unroll
+      for (int e = 0; e < VE; ++e) r2[g][e] += dpp_f<kDppRor8>(r2[g][e]);
+  }
+  bool writer = true;
+  if (LPRV <= 8) writer = writer && ((lane & 8) == 0);
+  if (LPRV <= 16 && G1 < 2) writer = writer && ((lane & 16) == 0);
+  if (LPRV <= 32 && GT < 2) writer = writer && ((lane & 32) == 0);
+  if (writer) {
+#pragma unroll
+    for (int g = 0; g < G2; ++g)
+#pragma unroll
+      for (int e = 0; e < VE; ++e) lds_o[w][head_off + g][cv * VE + e] = r2[g][e];
+  }
+  if (lane == 0) {
+#pragma unroll
+    for (int g = 0; g < GT; ++g) { lds_m[w][g] = m_run[g]; lds_l[w][g] = l_run[g]; }
+  }
+  __syncthreads();
+  for (int idx = tid; idx < GT * D; idx += NW * 64) {
+    const int g = idx / D, d = idx - g * D;
+    float M = lds_m[0][g];
+#pragma unroll
+    for (int ww = 1; ww < NW; ++ww) M = fmaxf(M, lds_m[ww][g]);
+    float o = 0.f, l = 0.f;
+#pragma unroll
+    for (int ww = 0; ww < NW; ++ww) { const float f = exp2f(lds_m[ww][g] - M); o = fmaf(f, lds_o[ww][g][d], o); l = fmaf(f, lds_l[ww][g], l); }
+    const size_t pidx = (size_t)(h0 + g) * a.n_tiles + jl;
+    a.so[pidx * D + d] = o;
+    if (d == 0) { a.sm[pidx] = M > -1e29f ? M * 0.693147180559945f : kMasked; a.ss[pidx] = l; }
+  }
 }
 
-constexpr int kSplitWaves = 4;
-
-template <int DT, int D, int GT, int BI>
-__global__ __launch_bounds__(kSplitWaves * kWave) void split_kernel(SplitArgs a) {
-    constexpr int ES = ElemBytes<DT>::value;
-    constexpr int EPL = 16 / ES;        // elements per lane per row
-    constexpr int LPR = D / EPL;        // lanes per row
-    constexpr int RPI = kWave / LPR;    // rows per wavefront load
-    constexpr int NW = kSplitWaves;
-    constexpr int ROWS_WG = NW * RPI;   // rows per workgroup iteration
-    static_assert(LPR >= 1 && LPR <= kWave && (LPR & (LPR - 1)) == 0, "row must map onto a power-of-two lane group");
-
-    __shared__ float lds_o[NW][GT][D];
-    __shared__ float lds_m[NW][GT];
-    __shared__ float lds_l[NW][GT];
-
-    const int tid = threadIdx.x;
-    const int lane = tid & (kWave - 1);
-    const int w = tid >> 6;
-    const int c = lane % LPR;
-    const int r = lane / LPR;
-
-    const uint32_t jl = blockIdx.x;                 // tile index local to this launch
-    const uint32_t kvh = blockIdx.y;
-    const uint32_t g_per_kv = a.n_heads / a.n_kv_heads;
-    const uint32_t h0 = kvh * g_per_kv + blockIdx.z * GT;
-
-    const uint32_t tile_base = (a.tile_first + jl) * a.tile;
-    uint32_t tile_end = tile_base + a.tile;
-    if (tile_end > a.seq_len) tile_end = a.seq_len;
-    const uint32_t lo = tile_base > a.kv_start ? tile_base : a.kv_start;
-
-    // Q slice of this lane for each head of the group.
-    float qf[GT][EPL];
-#pragma unroll
-    for (int g = 0; g < GT; ++g) {
-        const float4* qp = reinterpret_cast<const float4*>(a.q + (size_t)(h0 + g) * D + c * EPL);
-#pragma unroll
-        for (int e4 = 0; e4 < EPL / 4; ++e4) {
-            const float4 f = qp[e4];
-            qf[g][4 * e4 + 0] = f.x; qf[g][4 * e4 + 1] = f.y; qf[g][4 * e4 + 2] = f.z; qf[g][4 * e4 + 3] = f.w;
-        }
-    }
-
-    float m_run[GT], l_run[GT], acc[GT][EPL];
-#pragma unroll
-    for (int g = 0; g < GT; ++g) {
-        m_run[g] = kMasked;
-        l_run[g] = 0.f;
-#pragma unroll
-        for (int e = 0; e < EPL; ++e) acc[g][e] = 0.f;
-    }
-
-    const size_t row_stride = (size_t)a.n_kv_heads * D * ES;   // bytes between consecutive positions
-    const size_t head_byte = (size_t)kvh * D * ES + (size_t)c * 16;
-    const uint32_t last_row = a.seq_len - 1u;
-
-    if (lo < tile_end) {
-        for (uint32_t blk = tile_base; blk < tile_end; blk += BI * ROWS_WG) {
-            if (blk + BI * ROWS_WG <= lo) continue;          // block entirely below the window
-            uint4 kraw[BI], vraw[BI];
-            uint32_t valid_bits = 0u;
-#pragma unroll
-            for (int i = 0; i < BI; ++i) {
-                const uint32_t t = blk + i * ROWS_WG + w * RPI + r;
-                const uint32_t tc = t < last_row ? t : last_row;   // stay inside the populated slab
-                if (t < tile_end && t >= lo) valid_bits |= (1u << i);
-                kraw[i] = *reinterpret_cast<const uint4*>(a.k + (size_t)tc * row_stride + head_byte);
-            }
-#pragma unroll
-            for (int i = 0; i < BI; ++i) {
-                const uint32_t t = blk + i * ROWS_WG + w * RPI + r;
-                const uint32_t tc = t < last_row ? t : last_row;
-                vraw[i] = *reinterpret_cast<const uint4*>(a.v + (size_t)tc * row_stride + head_byte);
-            }
-
-            // ---- scores of the block ----
-            float s[BI][GT];
-            float bmax[GT];
-#pragma unroll
-            for (int g = 0; g < GT; ++g) bmax[g] = kMasked;
-#pragma unroll
-            for (int i = 0; i < BI; ++i) {
-                float kd[EPL];
-                decode16<DT>(kraw[i], kd);
-                const bool valid = (valid_bits >> i) & 1u;
-#pragma unroll
-                for (int g = 0; g < GT; ++g) {
-                    float p = 0.f;
-#pragma unroll
-                    for (int e = 0; e < EPL; ++e) p = fmaf(qf[g][e], kd[e], p);
-                    p = group_sum<LPR>(p) * a.scale;
-                    if (a.softcap > 0.f) p = a.softcap * tanhf(p / a.softcap);
-                    p = valid ? p : kMasked;
-                    s[i][g] = p;
-                    bmax[g] = fmaxf(bmax[g], p);
-                }
-            }
-            // wavefront-uniform running maximum, rescale what has been accumulated so far
-#pragma unroll
-            for (int g = 0; g < GT; ++g) {
-                float bm = bmax[g];
-#pragma unroll
-                for (int off = LPR; off < kWave; off <<= 1) bm = fmaxf(bm, __shfl_xor(bm, off, kWave));
-                const float m_new = fmaxf(m_run[g], bm);
-                if (m_new > m_run[g]) {   // wavefront-uniform
-                    const float alpha = __expf(m_run[g] - m_new);
-                    l_run[g] *= alpha;
-#pragma unroll
-                    for (int e = 0; e < EPL; ++e) acc[g][e] *= alpha;
-                    m_run[g] = m_new;
-                }
-            }
-            // ---- weights and V accumulation ----
-#pragma unroll
-            for (int i = 0; i < BI; ++i) {
-                float vd[EPL];
-                decode16<DT>(vraw[i], vd);
-                const bool valid = (valid_bits >> i) & 1u;
-#pragma unroll
-                for (int g = 0; g < GT; ++g) {
-                    const float p = valid ? __expf(s[i][g] - m_run[g]) : 0.f;
-                    l_run[g] += p;
-#pragma unroll
-                    for (int e = 0; e < EPL; ++e) acc[g][e] = fmaf(p, vd[e], acc[g][e]);
-                }
-            }
-        }
-    }
-
-    // ---- merge the RPI row groups of the wavefront (all share m_run) ----
-#pragma unroll
-    for (int off = LPR; off < kWave; off <<= 1) {
-#pragma unroll
-        for (int g = 0; g < GT; ++g) {
-            l_run[g] += __shfl_xor(l_run[g], off, kWave);
-#pragma unroll
-            for (int e = 0; e < EPL; ++e) acc[g][e] += __shfl_xor(acc[g][e], off, kWave);
-        }
-    }
-    if (r == 0) {
-#pragma unroll
-        for (int g = 0; g < GT; ++g) {
-#pragma unroll
-            for (int e = 0; e < EPL; ++e) lds_o[w][g][c * EPL + e] = acc[g][e];
-        }
-    }
-    if (lane == 0) {
-#pragma unroll
-        for (int g = 0; g < GT; ++g) {
-            lds_m[w][g] = m_run[g];
-            lds_l[w][g] = l_run[g];
-        }
-    }
-    __syncthreads();
-
-    // ---- merge the wavefronts and write the tile partial ----
-    for (int idx = tid; idx < GT * D; idx += NW * kWave) {
-        const int g = idx / D;
-        const int d = idx - g * D;
-        float M = lds_m[0][g];
-#pragma unroll
-        for (int ww = 1; ww < NW; ++ww) M = fmaxf(M, lds_m[ww][g]);
-        float o = 0.f, l = 0.f;
-#pragma unroll
-        for (int ww = 0; ww < NW; ++ww) {
-            const float f = __expf(lds_m[ww][g] - M);
-            o = fmaf(f, lds_o[ww][g][d], o);
-            l = fmaf(f, lds_l[ww][g], l);
-        }
-        const size_t pidx = (size_t)(h0 + g) * a.n_tiles + jl;
-        a.so[pidx * D + d] = o;
-        if (d == 0) {
-            a.sm[pidx] = M;
-            a.ss[pidx] = l;
-        }
-    }
-}
 
 // ---- generic worker: any head_dim <= 512, any dtype; one wavefront per (tile, head) -----------
 // Lanes walk the keys of the tile 64 at a time (one key per lane, serial dot over d), then walk the
@@ -264,11 +401,11 @@ __global__ __launch_bounds__(kWave) void split_generic_kernel(SplitArgs a, uint3
             if (a.softcap > 0.f) s = a.softcap * tanhf(s / a.softcap);
             sc = s;
         }
-        const float bm = group_max<kWave>(sc);
+        const float bm = wave_max_all(sc);
         const float m_new = fmaxf(m_run, bm);
         const float alpha = __expf(m_run - m_new);
         const float p = valid ? __expf(sc - m_new) : 0.f;
-        l_run = l_run * alpha + group_sum<kWave>(p);
+        l_run = l_run * alpha + wave_sum_all(p);
         m_run = m_new;
         __syncthreads();
         p_lds[lane] = p;
@@ -317,7 +454,7 @@ __global__ __launch_bounds__(kReduceThreads) void reduce_kernel(const float* __r
 
     float M = kMasked;
     for (uint32_t j = tid; j < n_tiles; j += kReduceThreads) M = fmaxf(M, hm[j]);
-    M = group_max<kWave>(M);
+    M = wave_max_all(M);
     if ((tid & (kWave - 1)) == 0) red[tid >> 6] = M;
     __syncthreads();
     M = red[0];
@@ -327,7 +464,7 @@ __global__ __launch_bounds__(kReduceThreads) void reduce_kernel(const float* __r
 
     float L = 0.f;
     for (uint32_t j = tid; j < n_tiles; j += kReduceThreads) L += __expf(hm[j] - M) * hs[j];
-    L = group_sum<kWave>(L);
+    L = wave_sum_all(L);
     if ((tid & (kWave - 1)) == 0) red[tid >> 6] = L;
     __syncthreads();
     L = 0.f;
@@ -380,20 +517,15 @@ __global__ __launch_bounds__(kWave) void reduce_generic_kernel(const float* __re
 }
 
 // ---- dispatch -----------------------------------------------------------------------------------
-template <int DT, int D>
-struct SplitTraits {
-    static constexpr int ES = ElemBytes<DT>::value;
-    static constexpr int LPR = D * ES / 16;
-    static constexpr int RPI = kWave / LPR;
-    static constexpr int BI = 8;
-    static constexpr uint32_t granule = kSplitWaves * RPI;   // rows per workgroup iteration
-};
+constexpr int kSplitWaves = 4;
 
 template <int DT, int D, int GT>
 static hipError_t launch_split_t(const SplitArgs& a, uint32_t groups, hipStream_t stream) {
-    constexpr int BI = SplitTraits<DT, D>::BI;
     dim3 grid(a.n_tiles, a.n_kv_heads, groups);
-    hipLaunchKernelGGL((split_kernel<DT, D, GT, BI>), grid, dim3(kSplitWaves * kWave), 0, stream, a);
+    if (a.softcap > 0.f)
+        hipLaunchKernelGGL((split_kernel<DT, D, GT, kSplitWaves, true>), grid, dim3(kSplitWaves * kWave), 0, stream, a);
+    else
+        hipLaunchKernelGGL((split_kernel<DT, D, GT, kSplitWaves, false>), grid, dim3(kSplitWaves * kWave), 0, stream, a);
     return hipGetLastError();
 }
 
@@ -411,9 +543,7 @@ static bool fast_shape(uint32_t dtype, uint32_t D) {
 
 uint32_t split_tile_granule(uint32_t dtype, uint32_t D) {
     if (dtype > kF8 || D == 0u || D > 512u) return 0u;
-    if (!fast_shape(dtype, D)) return (uint32_t)kWave;
-    const uint32_t lpr = D * elem_size(dtype) / 16u;
-    return kSplitWaves * (kWave / lpr);
+    return (uint32_t)kRun;
 }
 
 hipError_t launch_split(const SplitLaunch& L, hipStream_t stream) {
@@ -428,7 +558,9 @@ hipError_t launch_split(const SplitLaunch& L, hipStream_t stream) {
     a.scale = L.scale; a.softcap = L.softcap;
     const uint32_t g = L.n_heads / L.n_kv_heads;
     const bool aligned = ((((uintptr_t)L.k) | ((uintptr_t)L.v) | ((uintptr_t)L.q)) & 15u) == 0u;
-    if (fast_shape(L.dtype, L.head_dim) && aligned) {
+    // the register-tiled worker addresses the slab with 32-bit byte offsets below 2 GiB
+    const uint64_t slab_bytes = (uint64_t)L.seq_len * L.n_kv_heads * L.head_dim * elem_size(L.dtype);
+    if (fast_shape(L.dtype, L.head_dim) && aligned && slab_bytes < 0x7FFF0000ull) {
 #define VFKV_CASE(DT, DD) \
     if (L.dtype == DT && L.head_dim == DD) return launch_split_d<DT, DD>(a, g, stream);
         VFKV_CASE(kF8, 64) VFKV_CASE(kF8, 128) VFKV_CASE(kF8, 256) VFKV_CASE(kF8, 512)

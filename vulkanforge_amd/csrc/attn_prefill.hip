@@ -47,11 +47,11 @@ __global__ __launch_bounds__(kWave) void batch_generic_kernel(BatchArgs a) {
             if (a.softcap > 0.f) s = a.softcap * tanhf(s / a.softcap);
             sc = s;
         }
-        const float bm = group_max<kWave>(sc);
+        const float bm = wave_max_all(sc);
         const float m_new = fmaxf(m_run, bm);
         const float alpha = __expf(m_run - m_new);
         const float p = valid ? __expf(sc - m_new) : 0.f;
-        l_run = l_run * alpha + group_sum<kWave>(p);
+        l_run = l_run * alpha + wave_sum_all(p);
         m_run = m_new;
         __syncthreads();
         p_lds[lane] = p;

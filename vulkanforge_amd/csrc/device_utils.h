@@ -11,6 +11,8 @@ typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
 typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
 typedef float float4_t __attribute__((ext_vector_type(4)));
 typedef float float16_t __attribute__((ext_vector_type(16)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 
 constexpr int kWave = 64;
 constexpr float kMasked = -1e30f;  // the reference's "minus infinity" (flash_attn_split.comp:102)
@@ -23,15 +25,21 @@ __host__ __device__ constexpr uint32_t elem_size(uint32_t dtype) { return dtype 
 // Saturating round-to-nearest-even E4M3FN with the reference's corner cases
 // (src/backend/vulkan/fp8_ext.rs:126-186): NaN -> 0x7F (sign dropped), |x| >= 448 and +-Inf ->
 // sign|0x7E.  v_cvt_pk_fp8_f32 rounds to nearest even including subnormals; the clamp supplies
-// the saturation and the select canonicalises NaN before the conversion.
-__device__ __forceinline__ float e4m3_presat(float x) {
-    float c = __builtin_amdgcn_fmed3f(x, -448.0f, 448.0f);
-    return (x != x) ? __builtin_bit_cast(float, 0x7FC00000u) : c;
-}
+// the saturation (it also maps +-Inf to +-448).  The instruction encodes a NaN input as 0xFF, so
+// NaN lanes are converted as zero and their byte is then set to the reference's 0x7F.
 __device__ __forceinline__ uint32_t pack4_e4m3(float a, float b, float c, float d) {
-    int w = __builtin_amdgcn_cvt_pk_fp8_f32(e4m3_presat(a), e4m3_presat(b), 0, false);
-    w = __builtin_amdgcn_cvt_pk_fp8_f32(e4m3_presat(c), e4m3_presat(d), w, true);
-    return (uint32_t)w;
+    const float in[4] = {a, b, c, d};
+    float s[4];
+    uint32_t nan_bytes = 0u;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const bool is_nan = in[j] != in[j];
+        s[j] = is_nan ? 0.0f : __builtin_amdgcn_fmed3f(in[j], -448.0f, 448.0f);
+        nan_bytes |= is_nan ? (0x7Fu << (8 * j)) : 0u;
+    }
+    int w = __builtin_amdgcn_cvt_pk_fp8_f32(s[0], s[1], 0, false);
+    w = __builtin_amdgcn_cvt_pk_fp8_f32(s[2], s[3], w, true);
+    return (uint32_t)w | nan_bytes;
 }
 
 // ---- E4M3FN decode -------------------------------------------------------------------------
@@ -68,26 +76,73 @@ __device__ __forceinline__ float load_kv_elem(const void* base, uint32_t dtype, 
     return __builtin_amdgcn_cvt_f32_fp8((int)((const uint8_t*)base)[idx], 0);
 }
 
-// ---- wavefront reductions ------------------------------------------------------------------
-template <int WIDTH>
-__device__ __forceinline__ float group_sum(float v) {  // all lanes of each aligned WIDTH-group get the sum
-#pragma unroll
-    for (int off = WIDTH / 2; off >= 1; off >>= 1) v += __shfl_xor(v, off, kWave);
-    return v;
+// ---- wavefront (64-lane) data movement -----------------------------------------------------
+// DPP controls (gfx9 encoding): quad permutes for lane^1 / lane^2, mirrors for the 8- and 16-lane
+// steps, row broadcasts for the cross-row steps of a full-wave reduction.
+template <int CTRL>
+__device__ __forceinline__ float dpp_f(float x) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), CTRL, 0xf, 0xf, true));
 }
-template <int WIDTH>
-__device__ __forceinline__ float group_max(float v) {
-#pragma unroll
-    for (int off = WIDTH / 2; off >= 1; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, kWave));
-    return v;
+template <int CTRL, int ROWMASK>
+__device__ __forceinline__ float dpp_keep(float old, float x) {   // lanes of rows outside ROWMASK receive `old`
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(__builtin_bit_cast(int, old), __builtin_bit_cast(int, x),
+                                                                 CTRL, ROWMASK, 0xf, false));
 }
+constexpr int kDppXor1 = 0xB1, kDppXor2 = 0x4E, kDppHalfMirror = 0x141, kDppMirror = 0x140, kDppRor8 = 0x128;
+constexpr int kDppBcast15 = 0x142, kDppBcast31 = 0x143;
 
-__device__ __forceinline__ float softcap_apply(float s, float cap) {
-    // cap * tanh(s / cap); tanh(x) = 1 - 2 / (exp(2x) + 1) stays finite for large |x|
-    float x = s / cap;
-    float e = __expf(2.0f * x);
-    float t = 1.0f - 2.0f / (e + 1.0f);
-    return cap * t;
+// In-place lane swaps of gfx950.  The instructions are issued directly: the two-result compiler
+// builtins were observed to return the first result twice.  Both operands are read and written.
+__device__ __forceinline__ void swap32(float& a, float& b) {   // a.lanes[32..63] <-> b.lanes[0..31]
+    asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
+}
+__device__ __forceinline__ void swap16(float& a, float& b) {   // odd 16-lane rows of a <-> even rows of b
+    asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
+}
+__device__ __forceinline__ float xor16_sum(float x) { float y = x; swap16(x, y); return x + y; }
+__device__ __forceinline__ float xor32_sum(float x) { float y = x; swap32(x, y); return x + y; }
+
+// Sum over each aligned group of W lanes; every lane of the group gets the result.
+template <int W>
+__device__ __forceinline__ float group_sum(float x) {
+    if (W >= 2) x += dpp_f<kDppXor1>(x);
+    if (W >= 4) x += dpp_f<kDppXor2>(x);
+    if (W >= 8) x += dpp_f<kDppHalfMirror>(x);
+    if (W >= 16) x += dpp_f<kDppMirror>(x);
+    if (W >= 32) x = xor16_sum(x);
+    if (W >= 64) x = xor32_sum(x);
+    return x;
+}
+// Wavefront-wide max / sum as a uniform (scalar register) value: in-row butterflies, then the two
+// row broadcasts leave the total in lane 63.
+__device__ __forceinline__ float wave_max_uniform(float x) {
+    x = fmaxf(x, dpp_f<kDppXor1>(x));
+    x = fmaxf(x, dpp_f<kDppXor2>(x));
+    x = fmaxf(x, dpp_f<kDppHalfMirror>(x));
+    x = fmaxf(x, dpp_f<kDppMirror>(x));
+    x = fmaxf(x, dpp_keep<kDppBcast15, 0xa>(x, x));
+    x = fmaxf(x, dpp_keep<kDppBcast31, 0xc>(x, x));
+    return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, x), 63));
+}
+__device__ __forceinline__ float wave_sum_uniform(float x) {
+    x += dpp_f<kDppXor1>(x);
+    x += dpp_f<kDppXor2>(x);
+    x += dpp_f<kDppHalfMirror>(x);
+    x += dpp_f<kDppMirror>(x);
+    x += dpp_keep<kDppBcast15, 0xa>(0.f, x);
+    x += dpp_keep<kDppBcast31, 0xc>(0.f, x);
+    return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, x), 63));
+}
+// Shuffle-based all-lane variants for the generic kernels (vector result in every lane).
+__device__ __forceinline__ float wave_sum_all(float v) {
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) v += __shfl_xor(v, off, kWave);
+    return v;
+}
+__device__ __forceinline__ float wave_max_all(float v) {
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, kWave));
+    return v;
 }
 
 }  // namespace vfkv

@@ -283,9 +283,10 @@ def bench_prefill(args, wl):
 
         import oracle
         threads = len(os.sched_getaffinity(0))
-        kh = kbuf[:per_layer].cpu().numpy().view(oracle.NP_DTYPE[int(wl.dtype)]).reshape(max_seq, Hkv, D)
-        vh = vbuf[:per_layer].cpu().numpy().view(oracle.NP_DTYPE[int(wl.dtype)]).reshape(max_seq, Hkv, D)
-        ms = 8                       # the last `ms` query rows of layer 0, repeated until the time target
+        last = (L - 1) * per_layer   # `o` holds the output of the last layer of the step
+        kh = kbuf[last:last + per_layer].cpu().numpy().view(oracle.NP_DTYPE[int(wl.dtype)]).reshape(max_seq, Hkv, D)
+        vh = vbuf[last:last + per_layer].cpu().numpy().view(oracle.NP_DTYPE[int(wl.dtype)]).reshape(max_seq, Hkv, D)
+        ms = 8                       # the last `ms` query rows of that layer, repeated until the time target
         qs = wl.base_pos + wl.m - ms
         qh = q[wl.m - ms:].cpu().numpy()
         flops_sample = sum(qs + i + 1 for i in range(ms)) * H * 4 * D
@@ -300,7 +301,7 @@ def bench_prefill(args, wl):
         result["config"]["max_abs_err_vs_oracle_last_rows"] = err
         result["cpu_baseline"] = {"value": flops_sample * reps / spent / 1e12, "unit": "TFLOP/s", "cores": threads,
                                   "kind": "port",
-                                  "sample": f"last {ms} of {wl.m} query rows of layer 0, {reps} repetitions, CPU "
+                                  "sample": f"last {ms} of {wl.m} query rows of one layer, {reps} repetitions, CPU "
                                             f"oracle (attn_batch_ref, f64), {spent:.1f} s"}
     cache.destroy()
     return result

@@ -52,6 +52,10 @@ CASES = [
     (vf.KvDtype.F16, 4, 1, 512, 10, 70, 0, 0.0),
     (vf.KvDtype.F32, 12, 4, 64, 30, 90, 5, 0.0),
     (vf.KvDtype.F8, 6, 2, 80, 19, 45, 0, 0.0),
+    (vf.KvDtype.F8, 64, 8, 128, 21, 77, 0, 0.0),      # G = 8
+    (vf.KvDtype.F8, 4, 4, 64, 100, 30, 0, 0.0),       # G = 1, head_dim 64
+    (vf.KvDtype.F16, 8, 8, 64, 17, 200, 190, 0.0),
+    (vf.KvDtype.F16, 48, 4, 128, 5, 40, 0, 0.0),      # G = 12
 ]
 
 
@@ -71,6 +75,21 @@ def test_batch_matches_oracle(dtype, heads, hkv, d, m, q_start, kv_start, cap):
     assert np.isfinite(o).all()
     err = np.abs(o - ref).max()
     assert err < TOL[dtype], err
+
+
+@pytest.mark.parametrize("dtype", (vf.KvDtype.F8, vf.KvDtype.F16))
+def test_batch_with_f32_queries_keeps_f32_accuracy(dtype):
+    # Q values that are not representable in f16: the kernel must not lose them (hi + lo split)
+    heads, hkv, d, m, q_start = 16, 4, 128, 40, 500
+    r = rng(91)
+    n_kv = q_start + m
+    q = (r.standard_normal((m, heads, d)) * 3).astype(np.float32)
+    k = encode_np(fp16_normal(r, (n_kv, hkv, d)), dtype)
+    v = encode_np(fp16_normal(r, (n_kv, hkv, d)), dtype)
+    scale = float(1.0 / np.sqrt(d))
+    o = gpu_batch(q, k, v, dtype, heads, hkv, d, m, q_start, n_kv, scale)
+    ref = oracle.attn_batch_ref(q, k, v, int(dtype), m, n_kv, heads, hkv, d, q_start, scale)
+    assert np.abs(o - ref).max() < 1e-3
 
 
 def test_config5_chunk_append_then_prefill_fp8_one_layer():

@@ -87,6 +87,47 @@ __global__ __launch_bounds__(NW * 64) void split_kernel(SplitArgs a) {
   uint32_t tile_end = tile_base + a.tile; if (tile_end > a.seq_len) tile_end = a.seq_len;
   const uint32_t lo = tile_base > a.kv_start ? tile_base : a.kv_start;
 
+  float m_run[GT], l_run[GT], acc[GT][VE];
+#pragma unroll
+  for (int g = 0; g < GT; ++g) { m_run[g] = kMasked; l_run[g] = 0.f;
+#pragma unroll
+    for (int e = 0; e < VE; ++e) acc[g][e] = 0.f; }
+
+  const uint32_t row_stride = a.n_kv_heads * D * ES;
+  const __amdgpu_buffer_rsrc_t krsrc = __builtin_amdgcn_make_buffer_rsrc((void*)a.k, 0, a.seq_len * row_stride, 0x00020000);
+  const __amdgpu_buffer_rsrc_t vrsrc = __builtin_amdgcn_make_buffer_rsrc((void*)a.v, 0, a.seq_len * row_stride, 0x00020000);
+  const uint32_t lane_koff = rk * row_stride + kvh * D * ES + ck * 16;
+  const uint32_t lane_voff = rv * row_stride + kvh * D * ES + cv * VB;
+  const float scale_l2 = a.scale * 1.44269504088896f;
+  const float cap_l2 = a.softcap * 1.44269504088896f;
+
+  // runs of this wavefront: w, w + NW, ... counted from the first run that reaches the window
+  const uint32_t first_run = (lo - tile_base) / kRun;
+  const uint32_t n_runs = tile_end > tile_base ? (tile_end - tile_base + kRun - 1) / kRun : 0;
+  auto run_off = [&](uint32_t r) -> uint32_t {   // byte offset of a run's first row, or out of bounds when there is none
+    return r < n_runs ? (tile_base + r * kRun) * row_stride : kOOB;
+  };
+
+  u32x4 kreg[PFK];
+  u32x4 vreg4[VB == 16 ? PFV : 1];
+  u32x2 vreg2[VB == 8 ? PFV : 1];
+  // lane part in the VGPR offset, uniform part in the scalar offset; the range check covers their sum
+  auto issue_k = [&](int j, uint32_t off) { kreg[j] = __builtin_amdgcn_raw_buffer_load_b128(krsrc, lane_koff, off, 0); };
+  auto issue_v = [&](int j, uint32_t off) {
+    if (VB == 16) vreg4[j] = __builtin_amdgcn_raw_buffer_load_b128(vrsrc, lane_voff, off, 0);
+    else vreg2[j] = __builtin_amdgcn_raw_buffer_load_b64(vrsrc, lane_voff, off, 0);
+  };
+
+  uint32_t r = first_run + w;
+  const bool active = lo < tile_end && r < n_runs;
+  {   // fill both rings first: these loads do not depend on Q and fly while Q is staged
+    const uint32_t off = active ? run_off(r) : kOOB;
+#pragma unroll
+    for (int j = 0; j < PFK; ++j) issue_k(j, off + (uint32_t)(j * RPK) * row_stride);
+#pragma unroll
+    for (int j = 0; j < PFV; ++j) issue_v(j, off + (uint32_t)(j * RPV) * row_stride);
+  }
+
   // ---- Q -> LDS once per workgroup ----
   if (tid == 0) lds_haslo = 0;
   __syncthreads();
@@ -121,46 +162,7 @@ __global__ __launch_bounds__(NW * 64) void split_kernel(SplitArgs a) {
   };
   load_q(0);
 
-  float m_run[GT], l_run[GT], acc[GT][VE];
-#pragma unroll
-  for (int g = 0; g < GT; ++g) { m_run[g] = kMasked; l_run[g] = 0.f;
-#pragma unroll
-    for (int e = 0; e < VE; ++e) acc[g][e] = 0.f; }
-
-  const uint32_t row_stride = a.n_kv_heads * D * ES;
-  const __amdgpu_buffer_rsrc_t krsrc = __builtin_amdgcn_make_buffer_rsrc((void*)a.k, 0, a.seq_len * row_stride, 0x00020000);
-  const __amdgpu_buffer_rsrc_t vrsrc = __builtin_amdgcn_make_buffer_rsrc((void*)a.v, 0, a.seq_len * row_stride, 0x00020000);
-  const uint32_t lane_koff = rk * row_stride + kvh * D * ES + ck * 16;
-  const uint32_t lane_voff = rv * row_stride + kvh * D * ES + cv * VB;
-  const float scale_l2 = a.scale * 1.44269504088896f;
-  const float cap_l2 = a.softcap * 1.44269504088896f;
-
-  // runs of this wavefront: w, w + NW, ... counted from the first run that reaches the window
-  const uint32_t first_run = (lo - tile_base) / kRun;
-  const uint32_t n_runs = tile_end > tile_base ? (tile_end - tile_base + kRun - 1) / kRun : 0;
-  auto run_off = [&](uint32_t r) -> uint32_t {   // byte offset of a run's first row, or out of bounds when there is none
-    return r < n_runs ? (tile_base + r * kRun) * row_stride : kOOB;
-  };
-
-  u32x4 kreg[PFK];
-  u32x4 vreg4[VB == 16 ? PFV : 1];
-  u32x2 vreg2[VB == 8 ? PFV : 1];
-  // lane part in the VGPR offset, uniform part in the scalar offset; the range check covers their sum
-  auto issue_k = [&](int j, uint32_t off) { kreg[j] = __builtin_amdgcn_raw_buffer_load_b128(krsrc, lane_koff, off, 0); };
-  auto issue_v = [&](int j, uint32_t off) {
-    if (VB == 16) vreg4[j] = __builtin_amdgcn_raw_buffer_load_b128(vrsrc, lane_voff, off, 0);
-    else vreg2[j] = __builtin_amdgcn_raw_buffer_load_b64(vrsrc, lane_voff, off, 0);
-  };
-
-  uint32_t r = first_run + w;
-  if (lo < tile_end && r < n_runs) {
-    {
-      const uint32_t off = run_off(r);
-#pragma unroll
-      for (int j = 0; j < PFK; ++j) issue_k(j, off + (uint32_t)(j * RPK) * row_stride);
-#pragma unroll
-      for (int j = 0; j < PFV; ++j) issue_v(j, off + (uint32_t)(j * RPV) * row_stride);
-    }
+  if (active) {
     for (; r < n_runs; r += NW) {
       const uint32_t off = run_off(r), noff = run_off(r + NW);
       const uint32_t rb = tile_base + r * kRun;
@@ -437,60 +439,88 @@ __global__ __launch_bounds__(kWave) void split_generic_kernel(SplitArgs a, uint3
 
 // ---- log-sum-exp merge of the tile partials (flash_attn_reduce.comp:35-81) ---------------------
 // One workgroup per head.  The global maximum over tiles is taken first so that the weighted sums
-// have no serial dependency; mathematically this is the reference's running merge.
+// have no serial dependency; mathematically this is the reference's running merge.  Every load a
+// thread needs (its tiles' max / sum and its slice of the partial outputs) is issued before the
+// first reduction, so the kernel costs about one memory round trip.
 constexpr int kReduceThreads = 256;
+constexpr int kReduceChunk = 8;      // partial-output rows a thread holds in registers at a time
 __global__ __launch_bounds__(kReduceThreads) void reduce_kernel(const float* __restrict__ so,
                                                                 const float* __restrict__ sm,
                                                                 const float* __restrict__ ss,
                                                                 float* __restrict__ o, uint32_t D,
                                                                 uint32_t n_tiles) {
-    extern __shared__ float lds[];   // [parts][D] partial sums, then [parts] partial L
-    __shared__ float red[kReduceThreads / kWave];
+    extern __shared__ float lds[];   // [n_tiles] weights, then [parts][D] partial sums
+    __shared__ float red[2][kReduceThreads / kWave];
     const uint32_t h = blockIdx.x;
     const int tid = threadIdx.x;
     const float* hm = sm + (size_t)h * n_tiles;
     const float* hs = ss + (size_t)h * n_tiles;
     const float* ho = so + (size_t)h * n_tiles * D;
+    float* wts = lds;
+    float* psum = lds + n_tiles;
 
+    const uint32_t d4n = D / 4u;                       // D is a multiple of 4 on this path
+    const uint32_t parts = kReduceThreads / d4n;       // >= 1 because D <= 1024
+    const uint32_t part = tid / d4n, d4 = tid % d4n;
+    const bool has_slice = part < parts;
+
+    // first chunk of partial outputs, in flight during the max / sum reductions
+    float4 x[kReduceChunk];
+#pragma unroll
+    for (int c = 0; c < kReduceChunk; ++c) {
+        const uint32_t j = part + c * parts;
+        x[c] = (has_slice && j < n_tiles) ? *reinterpret_cast<const float4*>(ho + (size_t)j * D + 4u * d4)
+                                          : make_float4(0.f, 0.f, 0.f, 0.f);
+    }
     float M = kMasked;
     for (uint32_t j = tid; j < n_tiles; j += kReduceThreads) M = fmaxf(M, hm[j]);
-    M = wave_max_all(M);
-    if ((tid & (kWave - 1)) == 0) red[tid >> 6] = M;
+    M = wave_max_uniform(M);
+    if ((tid & (kWave - 1)) == 0) red[0][tid >> 6] = M;
     __syncthreads();
-    M = red[0];
+    M = red[0][0];
 #pragma unroll
-    for (int i = 1; i < kReduceThreads / kWave; ++i) M = fmaxf(M, red[i]);
-    __syncthreads();
+    for (int i = 1; i < kReduceThreads / kWave; ++i) M = fmaxf(M, red[0][i]);
 
     float L = 0.f;
-    for (uint32_t j = tid; j < n_tiles; j += kReduceThreads) L += __expf(hm[j] - M) * hs[j];
-    L = wave_sum_all(L);
-    if ((tid & (kWave - 1)) == 0) red[tid >> 6] = L;
+    for (uint32_t j = tid; j < n_tiles; j += kReduceThreads) {
+        const float wj = __expf(hm[j] - M);
+        wts[j] = wj;
+        L = fmaf(wj, hs[j], L);
+    }
+    L = wave_sum_uniform(L);
+    if ((tid & (kWave - 1)) == 0) red[1][tid >> 6] = L;
     __syncthreads();
     L = 0.f;
 #pragma unroll
-    for (int i = 0; i < kReduceThreads / kWave; ++i) L += red[i];
+    for (int i = 0; i < kReduceThreads / kWave; ++i) L += red[1][i];
 
-    // threads = (part, d4): each sums its share of the tiles for four consecutive d
-    const uint32_t d4n = D / 4u;                       // D is a multiple of 4 on this path
-    const uint32_t parts = kReduceThreads / d4n > 0 ? kReduceThreads / d4n : 1u;
-    const uint32_t part = tid / d4n, d4 = tid % d4n;
     float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
-    if (part < parts) {
-        for (uint32_t j = part; j < n_tiles; j += parts) {
-            const float wj = __expf(hm[j] - M);
-            const float4 x = *reinterpret_cast<const float4*>(ho + (size_t)j * D + 4u * d4);
-            acc.x = fmaf(wj, x.x, acc.x); acc.y = fmaf(wj, x.y, acc.y);
-            acc.z = fmaf(wj, x.z, acc.z); acc.w = fmaf(wj, x.w, acc.w);
+    if (has_slice) {
+        for (uint32_t j0 = part; j0 < n_tiles; j0 += kReduceChunk * parts) {
+            if (j0 != part) {
+#pragma unroll
+                for (int c = 0; c < kReduceChunk; ++c) {
+                    const uint32_t j = j0 + c * parts;
+                    x[c] = j < n_tiles ? *reinterpret_cast<const float4*>(ho + (size_t)j * D + 4u * d4)
+                                       : make_float4(0.f, 0.f, 0.f, 0.f);
+                }
+            }
+#pragma unroll
+            for (int c = 0; c < kReduceChunk; ++c) {
+                const uint32_t j = j0 + c * parts;
+                const float wj = j < n_tiles ? wts[j] : 0.f;
+                acc.x = fmaf(wj, x[c].x, acc.x); acc.y = fmaf(wj, x[c].y, acc.y);
+                acc.z = fmaf(wj, x[c].z, acc.z); acc.w = fmaf(wj, x[c].w, acc.w);
+            }
         }
-        float* dst = lds + (size_t)part * D + 4u * d4;
+        float* dst = psum + (size_t)part * D + 4u * d4;
         dst[0] = acc.x; dst[1] = acc.y; dst[2] = acc.z; dst[3] = acc.w;
     }
     __syncthreads();
     const float inv = 1.0f / L;
     for (uint32_t d = tid; d < D; d += kReduceThreads) {
         float sum = 0.f;
-        for (uint32_t p = 0; p < parts; ++p) sum += lds[(size_t)p * D + d];
+        for (uint32_t p = 0; p < parts; ++p) sum += psum[(size_t)p * D + d];
         o[(size_t)h * D + d] = sum * inv;
     }
 }
@@ -576,12 +606,12 @@ hipError_t launch_split(const SplitLaunch& L, hipStream_t stream) {
 hipError_t launch_reduce(const float* so, const float* sm, const float* ss, float* o, uint32_t n_heads,
                          uint32_t D, uint32_t n_tiles, hipStream_t stream) {
     if (n_heads == 0u || D == 0u || n_tiles == 0u) return hipErrorInvalidValue;
-    const bool vec = (D % 4u == 0u) && (D / 4u <= (uint32_t)kReduceThreads) &&
+    const bool vec = (D % 4u == 0u) && (D / 4u <= (uint32_t)kReduceThreads) && n_tiles <= 8192u &&
                      ((((uintptr_t)so) & 15u) == 0u);
     if (vec) {
         const uint32_t d4n = D / 4u;
         const uint32_t parts = kReduceThreads / d4n;
-        const size_t lds = (size_t)parts * D * sizeof(float);
+        const size_t lds = ((size_t)parts * D + n_tiles) * sizeof(float);
         hipLaunchKernelGGL(reduce_kernel, dim3(n_heads), dim3(kReduceThreads), lds, stream, so, sm, ss, o, D, n_tiles);
     } else {
         hipLaunchKernelGGL(reduce_generic_kernel, dim3(n_heads), dim3(kWave), 0, stream, so, sm, ss, o, D, n_tiles);

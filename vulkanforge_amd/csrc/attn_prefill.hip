@@ -1,6 +1,7 @@
 // Chunked-prefill causal attention over the cache (flash_attn_batch.comp:105-208) for gfx950.
 //
-// batch_generic_kernel: one wavefront per (query, head); covers every dtype and head_dim <= 512.
+// batch_mfma_kernel    (attn_prefill_mfma.h) f16 matrix-core tiles for FP8 / F16 caches, head_dim 64/128/256.
+// batch_generic_kernel one wavefront per (query, head); covers every dtype and head_dim <= 512.
 #include "device_utils.h"
 #include "kernels.h"
 
@@ -16,6 +17,10 @@ struct BatchArgs {
     float scale, softcap;
     uint32_t dtype;
 };
+
+}  // namespace vfkv
+#include "attn_prefill_mfma.h"
+namespace vfkv {
 
 __global__ __launch_bounds__(kWave) void batch_generic_kernel(BatchArgs a) {
     __shared__ float p_lds[kWave];
@@ -86,6 +91,30 @@ hipError_t launch_batch(const BatchLaunch& L, hipStream_t stream) {
     a.n_heads = L.n_heads; a.n_kv_heads = L.n_kv_heads; a.head_dim = L.head_dim;
     a.m = L.m; a.n_kv = L.n_kv; a.q_start = L.q_start; a.kv_start = L.kv_start;
     a.scale = L.scale; a.softcap = L.softcap; a.dtype = L.dtype;
+    const uint32_t g = L.n_heads / L.n_kv_heads;
+    const uint64_t slab_bytes = (uint64_t)L.n_kv * L.n_kv_heads * L.head_dim * elem_size(L.dtype);
+    const bool aligned = ((((uintptr_t)L.k) | ((uintptr_t)L.v) | ((uintptr_t)L.q) | ((uintptr_t)L.o)) & 15u) == 0u;
+    if ((L.dtype == kF8 || L.dtype == kF16) && g <= 16u && aligned && slab_bytes < 0x7FFF0000ull &&
+        (L.head_dim == 64u || L.head_dim == 128u || L.head_dim == 256u)) {
+        // two key splits per workgroup while that still leaves two wavefronts per SIMD worth of registers
+        const uint32_t nsplit = g <= 4u ? 2u : 1u;
+        const dim3 grid((L.m + 15u) / 16u, L.n_kv_heads), block(g * nsplit * kWave);
+        const size_t vbytes = (size_t)nsplit * 2 * 32 * (L.head_dim + 16) * sizeof(_Float16);
+        const size_t mbytes = (size_t)(nsplit - 1) * g * 64 * (L.head_dim / 4 + 2) * sizeof(float);
+        const size_t lds = vbytes > mbytes ? vbytes : mbytes;
+#define VFKV_PF2(DT, DD, CAPV, MT, NS) hipLaunchKernelGGL((batch_mfma_kernel<DT, DD, CAPV, MT, NS>), grid, block, lds, stream, a)
+#define VFKV_PF(DT, DD)                                                                   \
+    if (L.dtype == DT && L.head_dim == DD) {                                              \
+        const bool cap = L.softcap > 0.f;                                                 \
+        if (g <= 4u) { if (cap) VFKV_PF2(DT, DD, true, 512, 2); else VFKV_PF2(DT, DD, false, 512, 2); }     \
+        else if (g <= 8u) { if (cap) VFKV_PF2(DT, DD, true, 512, 1); else VFKV_PF2(DT, DD, false, 512, 1); } \
+        else { if (cap) VFKV_PF2(DT, DD, true, 1024, 1); else VFKV_PF2(DT, DD, false, 1024, 1); }           \
+        return hipGetLastError();                                                         \
+    }
+        VFKV_PF(kF8, 64) VFKV_PF(kF8, 128) VFKV_PF(kF8, 256) VFKV_PF(kF16, 64) VFKV_PF(kF16, 128) VFKV_PF(kF16, 256)
+#undef VFKV_PF2
+#undef VFKV_PF
+    }
     hipLaunchKernelGGL(batch_generic_kernel, dim3(L.n_heads, L.m), dim3(kWave), 0, stream, a);
     return hipGetLastError();
 }

@@ -116,7 +116,7 @@ def bench_decode(args, wl):
     fill_cache(torch, vf, fwd, wl, max_seq, args.seed, outliers)
 
     g = torch.Generator(device="cuda").manual_seed(args.seed + 1)
-    q = torch.randn((L, H, D), device=dev, generator=g).half().float()
+    q = torch.randn((L, H, D), device=dev, generator=g)
     o = torch.zeros((L, H, D), device=dev)
     k_new = torch.randn((L, Hkv * D), device=dev, generator=g).half().float()
     v_new = torch.randn((L, Hkv * D), device=dev, generator=g).half().float()
@@ -134,36 +134,52 @@ def bench_decode(args, wl):
     sec_per_step = time_steps(torch, step, args)
     bytes_step = wl.kv_bytes_step()
 
-    # ---- replay with HIP events around every launch of the split worker (the dominant kernel) ----
+    # ---- duration of the split worker (the dominant kernel): its launches of one step, back to back on
+    # the benchmark's stream, bracketed by one pair of HIP events; repeated and averaged.  (Events around
+    # every single launch would add their own packets between kernels and overstate the duration.)
     stream = torch.cuda.current_stream()
     lib = _ffi.lib()
     max_tiles = (max_seq + 63) // 64
     so = torch.empty((H * max_tiles * D,), device=dev)
     sm = torch.empty((H * max_tiles,), device=dev)
     ss = torch.empty((H * max_tiles,), device=dev)
-    n_ev = min(args.steps, 20)
-    pairs = []
-    for _ in range(n_ev):
+
+    def split_only():
         for layer in range(L):
             span = wl.context - starts[layer]
             tile = lib.vfkv_decode_tile_for(span, H, Hkv)
             klay = cache.k_ptr + cache.layer_offset_bytes(layer)
             vlay = cache.v_ptr + cache.layer_offset_bytes(layer)
-            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            e0.record(stream)
-            nt = fwd.run_flash_attn_split(q[layer], klay, vlay, wl.dtype, so, sm, ss, H, Hkv, D, wl.context, scale,
-                                          kv_start=starts[layer], tile=tile, softcap=wl.softcap)
-            e1.record(stream)
-            fwd.run_flash_attn_reduce(so, sm, ss, o[layer], H, D, nt)
-            pairs.append((layer, e0, e1))
+            fwd.run_flash_attn_split(q[layer], klay, vlay, wl.dtype, so, sm, ss, H, Hkv, D, wl.context, scale,
+                                     kv_start=starts[layer], tile=tile, softcap=wl.softcap)
+
+    run_split = split_only
+    if not args.no_graph:
+        split_only()
+        torch.cuda.synchronize()
+        g2 = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g2):
+            split_only()
+        run_split = g2.replay
+    run_split()
     torch.cuda.synchronize()
-    # byte-weighted: total algorithmic bytes / total kernel time == bytes per launch / mean duration
-    split_ms = sum(e0.elapsed_time(e1) for _l, e0, e1 in pairs)
-    launches = len(pairs)
-    bytes_launch = bytes_step / L
+    n_ev = min(max(args.steps, 5), 20)
+    pairs = []
+    for _ in range(n_ev):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record(stream)
+        run_split()
+        e1.record(stream)
+        pairs.append((e0, e1))
+    torch.cuda.synchronize()
+    split_ms = sum(e0.elapsed_time(e1) for e0, e1 in pairs)
+    launches = n_ev * L
+    bytes_launch = bytes_step / L          # mean over the layers of the step
     avg_ms = split_ms / launches
     achieved = bytes_launch / (avg_ms * 1e-3) / 1e9
 
+    mfma_worker = os.environ.get("VFKV_DECODE_WORKER", "m")[:1] != "v" and D <= 128 and wl.dtype.label() != "FP32"
+    worker_name = "split_mfma_kernel" if mfma_worker else "split_kernel"
     result = {
         "metric": "kv_read_GBps_decode_step",
         "value": bytes_step / sec_per_step / 1e9,
@@ -179,11 +195,11 @@ def bench_decode(args, wl):
         "dtype": "f32",
         "kv_dtype": wl.dtype.label(),
         "launch": "eager" if args.no_graph else "hip_graph",
-        "data": "synthetic (seeded N(0,1) rounded to fp16; cache written by the append kernels)",
+        "data": "synthetic (seeded N(0,1) f32 queries; K/V rows N(0,1) written through the append kernels)",
         "config": {"workload": wl.name, "n_layers": L, "n_heads": H, "n_kv_heads": Hkv, "head_dim": D,
                    "context": wl.context, "append_per_step": wl.append, "kv_bytes_per_step": bytes_step,
                    "pct_of_hbm_peak": 100.0 * bytes_step / sec_per_step / 1e9 / HBM_PEAK_GBPS},
-        "roofline": {"bound": "hbm", "kernel": "split_kernel", "achieved": achieved, "peak": HBM_PEAK_GBPS,
+        "roofline": {"bound": "hbm", "kernel": worker_name, "achieved": achieved, "peak": HBM_PEAK_GBPS,
                      "unit": "GB/s", "frac": achieved / HBM_PEAK_GBPS, "traffic": None,
                      "avg_launch_us": avg_ms * 1e3, "launches_timed": launches,
                      "algorithmic_bytes_per_launch": bytes_launch},
@@ -240,7 +256,7 @@ def bench_prefill(args, wl):
         n_layers = L
     fill_cache(torch, vf, fwd, _W, wl.base_pos, args.seed, False)
     g = torch.Generator(device="cuda").manual_seed(args.seed + 1)
-    q = torch.randn((wl.m, H, D), device=dev, generator=g).half().float()
+    q = torch.randn((wl.m, H, D), device=dev, generator=g)
     kn = torch.randn((wl.m, Hkv * D), device=dev, generator=g).half().float()
     vn = torch.randn((wl.m, Hkv * D), device=dev, generator=g).half().float()
     o = torch.zeros((wl.m, H, D), device=dev)
@@ -271,7 +287,7 @@ def bench_prefill(args, wl):
         "unit": "TFLOP/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": sec_per_step * 1e3,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f16", "kv_dtype": wl.dtype.label(),
-        "data": "synthetic (seeded N(0,1) rounded to fp16)",
+        "data": "synthetic (seeded N(0,1) f32 queries; K/V rows N(0,1) written through the append kernels)",
         "config": {"workload": wl.name, "n_layers": L, "n_heads": H, "n_kv_heads": Hkv, "head_dim": D,
                    "m": wl.m, "q_start": wl.base_pos, "n_kv": max_seq, "flop_per_step": flops_step},
         "roofline": {"bound": "mfma", "kernel": "flash_attn_batch", "achieved": achieved, "peak": MFMA_F16_PEAK_TFLOPS,
@@ -307,6 +323,23 @@ def bench_prefill(args, wl):
     return result
 
 
+def copy_calibration(args):
+    """Plain device-to-device copy of a known size, launched `steps` times: the reference point for the
+    FETCH_SIZE / WRITE_SIZE counters (what they read for a kernel whose HBM traffic is known)."""
+    import torch
+    n = 64 << 20
+    src = torch.empty(n, dtype=torch.uint8, device="cuda").random_(0, 255)
+    bufs = [torch.empty_like(src) for _ in range(8)]      # rotate destinations so nothing stays cached
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        bufs[i % len(bufs)].copy_(src)
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    return {"metric": "copy_calibration", "bytes_read_per_launch": n, "bytes_written_per_launch": n,
+            "launches": args.steps, "value": 2 * n * args.steps / dt / 1e9, "unit": "GB/s", "n_gpus": 1}
+
+
 def main():
     args = parse_args()
     if args.gpus != 1:
@@ -318,8 +351,10 @@ def main():
         res = bench_decode(args, workloads.DECODE[args.workload])
     elif args.workload in workloads.PREFILL:
         res = bench_prefill(args, workloads.PREFILL[args.workload])
+    elif args.workload == "copy_calibration":
+        res = copy_calibration(args)
     else:
-        print("unknown workload; choose from: " + ", ".join(list(workloads.DECODE) + list(workloads.PREFILL)),
+        print("unknown workload; choose from: " + ", ".join(list(workloads.DECODE) + list(workloads.PREFILL) + ["copy_calibration"]),
               file=sys.stderr)
         sys.exit(2)
     print(json.dumps(res))

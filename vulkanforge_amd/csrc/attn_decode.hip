@@ -546,8 +546,29 @@ __global__ __launch_bounds__(kWave) void reduce_generic_kernel(const float* __re
     }
 }
 
+}  // namespace vfkv
+#include "attn_decode_mfma.h"
+namespace vfkv {
+
 // ---- dispatch -----------------------------------------------------------------------------------
 constexpr int kSplitWaves = 4;
+
+template <int DT, int D, int RUN>
+static hipError_t launch_split_mfma(const SplitArgs& a, uint32_t g, hipStream_t stream) {
+    const uint32_t gt = g < 8u ? g : 8u;
+    dim3 grid(a.n_tiles, a.n_kv_heads, (g + gt - 1u) / gt);
+    if (a.softcap > 0.f)
+        hipLaunchKernelGGL((split_mfma_kernel<DT, D, RUN, kSplitWaves, true>), grid, dim3(kSplitWaves * kWave), 0, stream, a, gt);
+    else
+        hipLaunchKernelGGL((split_mfma_kernel<DT, D, RUN, kSplitWaves, false>), grid, dim3(kSplitWaves * kWave), 0, stream, a, gt);
+    return hipGetLastError();
+}
+
+// VFKV_DECODE_WORKER=valu keeps the vector-ALU worker for every shape (for comparisons).
+static bool mfma_worker_enabled() {
+    static const bool on = [] { const char* e = getenv("VFKV_DECODE_WORKER"); return !(e && e[0] == 'v'); }();
+    return on;
+}
 
 template <int DT, int D, int GT>
 static hipError_t launch_split_t(const SplitArgs& a, uint32_t groups, hipStream_t stream) {
@@ -590,6 +611,12 @@ hipError_t launch_split(const SplitLaunch& L, hipStream_t stream) {
     const bool aligned = ((((uintptr_t)L.k) | ((uintptr_t)L.v) | ((uintptr_t)L.q)) & 15u) == 0u;
     // the register-tiled worker addresses the slab with 32-bit byte offsets below 2 GiB
     const uint64_t slab_bytes = (uint64_t)L.seq_len * L.n_kv_heads * L.head_dim * elem_size(L.dtype);
+    if (aligned && slab_bytes < 0x7FFF0000ull && mfma_worker_enabled()) {
+        if (L.dtype == kF8 && L.head_dim == 64u) return launch_split_mfma<kF8, 64, 64>(a, g, stream);
+        if (L.dtype == kF8 && L.head_dim == 128u) return launch_split_mfma<kF8, 128, 64>(a, g, stream);
+        if (L.dtype == kF16 && L.head_dim == 64u) return launch_split_mfma<kF16, 64, 64>(a, g, stream);
+        if (L.dtype == kF16 && L.head_dim == 128u) return launch_split_mfma<kF16, 128, 32>(a, g, stream);
+    }
     if (fast_shape(L.dtype, L.head_dim) && aligned && slab_bytes < 0x7FFF0000ull) {
 #define VFKV_CASE(DT, DD) \
     if (L.dtype == DT && L.head_dim == DD) return launch_split_d<DT, DD>(a, g, stream);

@@ -1,0 +1,282 @@
+// Matrix-core worker of the split-K decode attention (flash_attn_split.comp:82-162) for gfx950;
+// included by attn_decode.hip.
+//
+// One workgroup (NW wavefronts) owns one (tile of keys, KV head, slice of up to 8 query heads of the
+// GQA group); every K / V byte of the tile is requested from memory once and serves all heads of the
+// slice.  Each wavefront walks its share of the tile in runs of RUN rows and keeps both products on
+// v_mfma_f32_16x16x32_f16 (f32 accumulation), so the vector ALU only converts FP8, does the softmax
+// and packs the weights:
+//
+//   S^T[row, col]  = K[row, :] . Q[col, :]     A = K rows straight from global memory (each lane owns a
+//                                              contiguous quarter of a row; FP8 widens to f16 exactly),
+//                                              B = Q^T, resident in registers.  The 16 columns are
+//                                              cols 0..7 = f16(q) of head col, cols 8..15 = f16(q - f16(q))
+//                                              of head col-8: adding column c+8 to column c (one DPP
+//                                              rotate) gives scores of f32-level accuracy for any f32 Q.
+//   softmax        in the accumulator layout: a lane owns 4 rows per 16-row tile of ONE column, so the
+//                  running maximum needs two cross-row lane swaps per run and the weights are already
+//                  where the second product wants its B operand.
+//   O^T[d, col]   += V^T[d, row] . P[row, col]  A = V^T through a row-major f16 copy of the run in LDS read
+//                                              with the transposing LDS load, B = P: columns 0..7 carry
+//                                              f16(p), columns 8..15 carry f16(p - f16(p)); the two halves
+//                                              of O^T are added once, at the end of the tile.
+//
+// K and V rows of the next run are requested as soon as the registers of the current run are consumed,
+// through raw buffer loads whose descriptor ends at the last populated row (rows past it read as zero
+// without touching memory, which is also how the prefetch is fed when there is no next run).
+#pragma once
+
+namespace vfkv {
+
+template <int DT, int D, int RUN, int NW, bool CAP>
+__global__ __launch_bounds__(NW * 64) void split_mfma_kernel(SplitArgs a, uint32_t gt) {
+    constexpr int ES = DT == kF16 ? 2 : 1;
+    constexpr int RT = RUN / 16;                 // 16-row tiles per run
+    constexpr int PKS = RUN / 32;                // k-steps (32 rows) of the second product
+    constexpr int KS = D / 32;                   // k-steps of the first product
+    constexpr int DTILES = D / 16;
+    constexpr int SEG = D / 4, SEGB = SEG * ES;  // a lane group's quarter of a K row
+    constexpr int KLD = SEGB / 16;               // 16-byte loads per lane per K row
+    constexpr int VPITCH = D + 16;               // halves per V row in LDS (+32 B against bank conflicts)
+    constexpr int VCHUNK_ROW = D * ES / 16;      // 16-byte chunks per V row
+    constexpr int VLD = RUN * VCHUNK_ROW / 64;   // V loads per lane per run
+    constexpr int VROWS = 64 / VCHUNK_ROW;       // rows covered by one V load of the wavefront
+    static_assert(D % 32 == 0 && SEGB % 16 == 0 && RUN % 32 == 0 && VCHUNK_ROW <= 64 && VLD >= 1, "unsupported shape");
+    static_assert(NW * RUN * VPITCH * 2 >= NW * 8 * D * 4, "merge buffer must fit in the V staging area");
+
+    __shared__ __attribute__((aligned(16))) _Float16 vlds[NW][RUN * VPITCH];
+    __shared__ float lds_m[NW][8], lds_l[NW][8];
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int n16 = lane & 15, kg = lane >> 4;
+    const int col = n16 & 7;
+    const bool is_lo = n16 >= 8;
+    const uint32_t jl = blockIdx.x, kvh = blockIdx.y;
+    const uint32_t g_all = a.n_heads / a.n_kv_heads;
+    const uint32_t hz = blockIdx.z * gt;
+    const uint32_t gcount = g_all - hz < gt ? g_all - hz : gt;
+    const uint32_t h0 = kvh * g_all + hz;
+    const uint32_t tile_base = (a.tile_first + jl) * a.tile;
+    uint32_t tile_end = tile_base + a.tile; if (tile_end > a.seq_len) tile_end = a.seq_len;
+    const uint32_t lo = tile_base > a.kv_start ? tile_base : a.kv_start;
+
+    // ---- Q^T operands: lane (column n16, group kg) holds q[kg*SEG + c*8 + j], j < 8, per k-step c ----
+    float4 qraw[KS][2];
+    {
+        const bool col_ok = (uint32_t)col < gcount;
+        const float* qp = a.q + (size_t)(h0 + (col_ok ? col : 0)) * D + kg * SEG;
+#pragma unroll
+        for (int c = 0; c < KS; ++c)
+#pragma unroll
+            for (int j4 = 0; j4 < 2; ++j4) {
+                qraw[c][j4] = *reinterpret_cast<const float4*>(qp + c * 8 + j4 * 4);
+                if (!col_ok) qraw[c][j4] = make_float4(0.f, 0.f, 0.f, 0.f);
+            }
+    }
+
+    const uint32_t row_stride = a.n_kv_heads * D * ES;
+    const __amdgpu_buffer_rsrc_t krsrc = __builtin_amdgcn_make_buffer_rsrc((void*)a.k, 0, a.seq_len * row_stride, 0x00020000);
+    const __amdgpu_buffer_rsrc_t vrsrc = __builtin_amdgcn_make_buffer_rsrc((void*)a.v, 0, a.seq_len * row_stride, 0x00020000);
+    const uint32_t head_b = kvh * D * ES;
+    const uint32_t lane_koff = n16 * row_stride + head_b + kg * SEGB;
+    const int vrow = lane / VCHUNK_ROW, vcol = lane % VCHUNK_ROW;
+    const uint32_t lane_voff = vrow * row_stride + head_b + vcol * 16;
+    const float scale_l2 = a.scale * 1.44269504088896f;
+    const float cap_l2 = a.softcap * 1.44269504088896f;
+
+    // runs of this wavefront: w, w + NW, ... counted from the first run that reaches the window
+    const uint32_t first_run = (lo - tile_base) / RUN;
+    const uint32_t n_runs = tile_end > tile_base ? (tile_end - tile_base + RUN - 1) / RUN : 0;
+    auto run_off = [&](uint32_t r) -> uint32_t {   // byte offset of a run's first row, or out of bounds when there is none
+        return r < n_runs ? (tile_base + r * RUN) * row_stride : kOOB;
+    };
+
+    u32x4 kraw[RT][KLD];
+    u32x4 vraw[VLD];
+    auto issue_k = [&](int t, uint32_t off) {
+#pragma unroll
+        for (int x = 0; x < KLD; ++x)
+            kraw[t][x] = __builtin_amdgcn_raw_buffer_load_b128(krsrc, lane_koff + x * 16, off + (uint32_t)(t * 16) * row_stride, 0);
+    };
+    auto issue_v = [&](int c, uint32_t off) {
+        vraw[c] = __builtin_amdgcn_raw_buffer_load_b128(vrsrc, lane_voff, off + (uint32_t)(c * VROWS) * row_stride, 0);
+    };
+
+    uint32_t r = first_run + w;
+    const bool active = lo < tile_end && r < n_runs;
+    {
+        const uint32_t off = active ? run_off(r) : kOOB;
+#pragma unroll
+        for (int t = 0; t < RT; ++t) issue_k(t, off);
+#pragma unroll
+        for (int c = 0; c < VLD; ++c) issue_v(c, off);
+    }
+
+    half8_t qb[KS];
+#pragma unroll
+    for (int c = 0; c < KS; ++c)
+#pragma unroll
+        for (int j4 = 0; j4 < 2; ++j4) {
+            const float v4[4] = {qraw[c][j4].x, qraw[c][j4].y, qraw[c][j4].z, qraw[c][j4].w};
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const _Float16 hv = (_Float16)v4[j];
+                const _Float16 lv = (_Float16)(v4[j] - (float)hv);
+                qb[c][j4 * 4 + j] = is_lo ? lv : hv;
+            }
+        }
+
+    float4_t oacc[DTILES];
+#pragma unroll
+    for (int dt = 0; dt < DTILES; ++dt) oacc[dt] = float4_t{0.f, 0.f, 0.f, 0.f};
+    float m_run = kMasked, l_run = 0.f;
+    _Float16* const vb = &vlds[w][0];
+
+    if (active) {
+        for (; r < n_runs; r += NW) {
+            const uint32_t noff = run_off(r + NW);
+            const uint32_t rb = tile_base + r * RUN;
+            // ---------------- S^T = K Q^T ----------------
+            float4_t s[RT];
+#pragma unroll
+            for (int t = 0; t < RT; ++t) {
+                half8_t ka[KS];
+#pragma unroll
+                for (int c = 0; c < KS; ++c) {
+                    if (DT == kF8) {
+                        const uint32_t w0 = kraw[t][c / 2][(c % 2) * 2], w1 = kraw[t][c / 2][(c % 2) * 2 + 1];
+                        half2_t p0, p1, p2, p3;
+                        e4m3x4_to_h2(w0, p0, p1);
+                        e4m3x4_to_h2(w1, p2, p3);
+                        ka[c][0] = p0[0]; ka[c][1] = p0[1]; ka[c][2] = p1[0]; ka[c][3] = p1[1];
+                        ka[c][4] = p2[0]; ka[c][5] = p2[1]; ka[c][6] = p3[0]; ka[c][7] = p3[1];
+                    } else {
+                        const u32x4 wv = kraw[t][c % KLD];
+                        ka[c] = __builtin_bit_cast(half8_t, wv);
+                    }
+                }
+                issue_k(t, noff);
+                s[t] = float4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int c = 0; c < KS; ++c) s[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ka[c], qb[c], s[t], 0, 0, 0);
+            }
+            // ---------------- softmax: this lane owns rows rb + t*16 + kg*4 + i of column n16 ----------------
+            const bool interior = rb >= lo && rb + RUN <= tile_end;      // wavefront-uniform
+            float x[RT][4];
+            float tmax = kMasked;
+#pragma unroll
+            for (int t = 0; t < RT; ++t)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    float y = s[t][i];
+                    y += dpp_f<kDppRor8>(y);                             // f16(q) part + remainder part
+                    y *= scale_l2;
+                    if (CAP) y = cap_l2 * tanhf(y / cap_l2);
+                    x[t][i] = y;
+                }
+            if (!interior) {
+#pragma unroll
+                for (int t = 0; t < RT; ++t)
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        const uint32_t row = rb + t * 16 + kg * 4 + i;
+                        x[t][i] = (row >= lo && row < tile_end) ? x[t][i] : kMasked;
+                    }
+            }
+#pragma unroll
+            for (int t = 0; t < RT; ++t)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) tmax = fmaxf(tmax, x[t][i]);
+            { float y = tmax; swap16(tmax, y); tmax = fmaxf(tmax, y); y = tmax; swap32(tmax, y); tmax = fmaxf(tmax, y); }
+            const float m_new = fmaxf(m_run, tmax);
+            if (__builtin_amdgcn_ballot_w64(m_new > m_run) != 0ull) {
+                const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
+                l_run *= alpha;
+#pragma unroll
+                for (int dt = 0; dt < DTILES; ++dt) oacc[dt] *= alpha;
+                m_run = m_new;
+            }
+            half8_t pb[PKS];
+#pragma unroll
+            for (int t = 0; t < RT; ++t)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    float p = __builtin_amdgcn_exp2f(x[t][i] - m_run);
+                    if (!interior) p = x[t][i] > -1e29f ? p : 0.f;
+                    l_run += p;
+                    const _Float16 ph = (_Float16)p;
+                    const _Float16 pl = (_Float16)(p - (float)ph);
+                    pb[t / 2][(t % 2) * 4 + i] = is_lo ? pl : ph;
+                }
+            // ---------------- V run -> f16 row-major in LDS ----------------
+#pragma unroll
+            for (int c = 0; c < VLD; ++c) {
+                _Float16* dst = vb + (c * VROWS + vrow) * VPITCH + vcol * (16 / ES);
+                if (DT == kF8) {
+                    uint32_t out[8];
+#pragma unroll
+                    for (int q4 = 0; q4 < 4; ++q4) {
+                        const uint32_t wd = vraw[c][q4];
+                        half2_t lo2, hi2;
+                        e4m3x4_to_h2(wd, lo2, hi2);
+                        out[2 * q4] = __builtin_bit_cast(uint32_t, lo2);
+                        out[2 * q4 + 1] = __builtin_bit_cast(uint32_t, hi2);
+                    }
+                    reinterpret_cast<u32x4*>(dst)[0] = u32x4{out[0], out[1], out[2], out[3]};
+                    reinterpret_cast<u32x4*>(dst)[1] = u32x4{out[4], out[5], out[6], out[7]};
+                } else {
+                    *reinterpret_cast<u32x4*>(dst) = vraw[c];
+                }
+                issue_v(c, noff);
+            }
+            // ---------------- O^T += V^T P ----------------
+#pragma unroll
+            for (int ks = 0; ks < PKS; ++ks)
+#pragma unroll
+                for (int dt = 0; dt < DTILES; ++dt) {
+                    // supplier lane s of a 16-lane group points at V[row = ks*32 + 4*kg + s/4 (+16)][d = dt*16 + 4*(s%4)]
+                    const _Float16* p0 = vb + (ks * 32 + kg * 4 + n16 / 4) * VPITCH + dt * 16 + 4 * (n16 % 4);
+                    const half4_t v0 = lds_read_tr16(p0);
+                    const half4_t v1 = lds_read_tr16(p0 + 16 * VPITCH);
+                    half8_t va;
+                    va[0] = v0[0]; va[1] = v0[1]; va[2] = v0[2]; va[3] = v0[3]; va[4] = v1[0]; va[5] = v1[1]; va[6] = v1[2]; va[7] = v1[3];
+                    oacc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(va, pb[ks], oacc[dt], 0, 0, 0);
+                }
+        }
+    }
+
+    // ---------------- wavefront totals, then the workgroup merge through LDS ----------------
+    l_run = xor32_sum(xor16_sum(l_run));
+#pragma unroll
+    for (int dt = 0; dt < DTILES; ++dt)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) { const float y = oacc[dt][i]; oacc[dt][i] = y + dpp_f<kDppRor8>(y); }
+    __syncthreads();                                   // every wavefront is done with its V staging area
+    float* lds_o = reinterpret_cast<float*>(&vlds[0][0]);     // [NW][8][D]
+    if (!is_lo) {
+#pragma unroll
+        for (int dt = 0; dt < DTILES; ++dt)
+            *reinterpret_cast<float4_t*>(lds_o + (size_t)(w * 8 + col) * D + dt * 16 + kg * 4) = oacc[dt];
+        if (kg == 0) { lds_m[w][col] = m_run; lds_l[w][col] = l_run; }
+    }
+    __syncthreads();
+    for (int idx = tid; idx < (int)gcount * D; idx += NW * 64) {
+        const int g = idx / D, d = idx - g * D;
+        float M = lds_m[0][g];
+#pragma unroll
+        for (int ww = 1; ww < NW; ++ww) M = fmaxf(M, lds_m[ww][g]);
+        float o = 0.f, l = 0.f;
+#pragma unroll
+        for (int ww = 0; ww < NW; ++ww) {
+            const float f = __builtin_amdgcn_exp2f(lds_m[ww][g] - M);
+            o = fmaf(f, lds_o[(size_t)(ww * 8 + g) * D + d], o);
+            l = fmaf(f, lds_l[ww][g], l);
+        }
+        const size_t pidx = (size_t)(h0 + g) * a.n_tiles + jl;
+        a.so[pidx * D + d] = o;
+        if (d == 0) { a.sm[pidx] = M > -1e29f ? M * 0.693147180559945f : kMasked; a.ss[pidx] = l; }
+    }
+}
+
+}  // namespace vfkv

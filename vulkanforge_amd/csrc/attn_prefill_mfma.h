@@ -29,16 +29,6 @@
 
 namespace vfkv {
 
-typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
-typedef short short4_t __attribute__((ext_vector_type(4)));
-
-// Transposing LDS read: within each group of 16 lanes, lane i receives element i%4 of the four
-// 4-element (8-byte) chunks addressed by lanes i/4, i/4+4, i/4+8 and i/4+12 of the group.
-__device__ __forceinline__ half4_t lds_read_tr16(const _Float16* p) {
-    const short4_t r = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) short4_t*)p);
-    return __builtin_bit_cast(half4_t, r);
-}
-
 template <int DT, int D, bool CAP, int MAXT, int NSPLIT>
 __global__ __launch_bounds__(MAXT) void batch_mfma_kernel(BatchArgs a) {
     constexpr int ES = DT == kF16 ? 2 : 1;

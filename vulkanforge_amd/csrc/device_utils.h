@@ -133,6 +133,15 @@ __device__ __forceinline__ float wave_sum_uniform(float x) {
     x += dpp_keep<kDppBcast31, 0xc>(0.f, x);
     return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, x), 63));
 }
+// Transposing LDS read (ds_read_b64_tr_b16): within each group of 16 lanes, lane i receives element
+// i%4 of the four 4-element (8-byte) chunks addressed by lanes i/4, i/4+4, i/4+8 and i/4+12 of the group.
+typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
+typedef short short4_t __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ half4_t lds_read_tr16(const _Float16* p) {
+    const short4_t r = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) short4_t*)p);
+    return __builtin_bit_cast(half4_t, r);
+}
+
 // Shuffle-based all-lane variants for the generic kernels (vector result in every lane).
 __device__ __forceinline__ float wave_sum_all(float v) {
 #pragma unroll

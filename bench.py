@@ -31,6 +31,15 @@ HBM_PEAK_GBPS = 8000.0       # MI355X HBM3E, published
 MFMA_F16_PEAK_TFLOPS = 2500.0
 
 
+# HBM bytes per launch of the dominant kernel, measured with rocprofv3 --pmc FETCH_SIZE and --pmc WRITE_SIZE
+# (two runs) and scaled by what the same counters read for a plain 64 MiB device copy
+# (FETCH_SIZE x 1.9991, WRITE_SIZE x 1.0 to KiB).  Only the workloads that were profiled have an entry.
+MEASURED_TRAFFIC_BYTES = {
+    "decode_fp8_32k_32layers": (65781 + 1152) * 1024,
+    "prefill_fp8_512x4608_32layers": (81245 + 8192) * 1024,
+}
+
+
 def parse_args():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -40,6 +49,8 @@ def parse_args():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="target CPU time of the baseline sample")
     ap.add_argument("--seed", type=int, default=1234)
+    ap.add_argument("--f32-queries", action="store_true",
+                    help="leave the queries as general f32 values instead of casting them to fp16 first")
     ap.add_argument("--no-graph", action="store_true",
                     help="launch every kernel from Python instead of replaying one captured HIP graph per step")
     return ap.parse_args()
@@ -117,6 +128,8 @@ def bench_decode(args, wl):
 
     g = torch.Generator(device="cuda").manual_seed(args.seed + 1)
     q = torch.randn((L, H, D), device=dev, generator=g)
+    if not args.f32_queries:
+        q = q.half().float()
     o = torch.zeros((L, H, D), device=dev)
     k_new = torch.randn((L, Hkv * D), device=dev, generator=g).half().float()
     v_new = torch.randn((L, Hkv * D), device=dev, generator=g).half().float()
@@ -195,12 +208,12 @@ def bench_decode(args, wl):
         "dtype": "f32",
         "kv_dtype": wl.dtype.label(),
         "launch": "eager" if args.no_graph else "hip_graph",
-        "data": "synthetic (seeded N(0,1) f32 queries; K/V rows N(0,1) written through the append kernels)",
+        "data": "synthetic, seeded N(0,1); queries " + ("general f32" if args.f32_queries else "cast to fp16 as the configuration states") + "; K/V rows cast to fp16 and written through the append kernels",
         "config": {"workload": wl.name, "n_layers": L, "n_heads": H, "n_kv_heads": Hkv, "head_dim": D,
                    "context": wl.context, "append_per_step": wl.append, "kv_bytes_per_step": bytes_step,
                    "pct_of_hbm_peak": 100.0 * bytes_step / sec_per_step / 1e9 / HBM_PEAK_GBPS},
         "roofline": {"bound": "hbm", "kernel": worker_name, "achieved": achieved, "peak": HBM_PEAK_GBPS,
-                     "unit": "GB/s", "frac": achieved / HBM_PEAK_GBPS, "traffic": None,
+                     "unit": "GB/s", "frac": achieved / HBM_PEAK_GBPS, "traffic": MEASURED_TRAFFIC_BYTES.get(wl.name),
                      "avg_launch_us": avg_ms * 1e3, "launches_timed": launches,
                      "algorithmic_bytes_per_launch": bytes_launch},
     }
@@ -257,6 +270,8 @@ def bench_prefill(args, wl):
     fill_cache(torch, vf, fwd, _W, wl.base_pos, args.seed, False)
     g = torch.Generator(device="cuda").manual_seed(args.seed + 1)
     q = torch.randn((wl.m, H, D), device=dev, generator=g)
+    if not args.f32_queries:
+        q = q.half().float()
     kn = torch.randn((wl.m, Hkv * D), device=dev, generator=g).half().float()
     vn = torch.randn((wl.m, Hkv * D), device=dev, generator=g).half().float()
     o = torch.zeros((wl.m, H, D), device=dev)
@@ -287,11 +302,11 @@ def bench_prefill(args, wl):
         "unit": "TFLOP/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": sec_per_step * 1e3,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f16", "kv_dtype": wl.dtype.label(),
-        "data": "synthetic (seeded N(0,1) f32 queries; K/V rows N(0,1) written through the append kernels)",
+        "data": "synthetic, seeded N(0,1); queries " + ("general f32" if args.f32_queries else "cast to fp16 as the configuration states") + "; K/V rows cast to fp16 and written through the append kernels",
         "config": {"workload": wl.name, "n_layers": L, "n_heads": H, "n_kv_heads": Hkv, "head_dim": D,
                    "m": wl.m, "q_start": wl.base_pos, "n_kv": max_seq, "flop_per_step": flops_step},
         "roofline": {"bound": "mfma", "kernel": "flash_attn_batch", "achieved": achieved, "peak": MFMA_F16_PEAK_TFLOPS,
-                     "unit": "TFLOP/s", "frac": achieved / MFMA_F16_PEAK_TFLOPS, "traffic": None,
+                     "unit": "TFLOP/s", "frac": achieved / MFMA_F16_PEAK_TFLOPS, "traffic": MEASURED_TRAFFIC_BYTES.get(wl.name),
                      "avg_launch_us": avg_ms * 1e3},
     }
     if not args.no_cpu_baseline:

@@ -35,7 +35,7 @@ MFMA_F16_PEAK_TFLOPS = 2500.0
 # (two runs) and scaled by what the same counters read for a plain 64 MiB device copy
 # (FETCH_SIZE x 1.9991, WRITE_SIZE x 1.0 to KiB).  Only the workloads that were profiled have an entry.
 MEASURED_TRAFFIC_BYTES = {
-    "decode_fp8_32k_32layers": (65781 + 1152) * 1024,
+    "decode_fp8_32k_32layers": (65607 + 520) * 1024,
     "prefill_fp8_512x4608_32layers": (81245 + 8192) * 1024,
 }
 
@@ -160,7 +160,7 @@ def bench_decode(args, wl):
     def split_only():
         for layer in range(L):
             span = wl.context - starts[layer]
-            tile = lib.vfkv_decode_tile_for(span, H, Hkv)
+            tile = lib.vfkv_decode_tile_for(span, H, Hkv, D, int(wl.dtype))
             klay = cache.k_ptr + cache.layer_offset_bytes(layer)
             vlay = cache.v_ptr + cache.layer_offset_bytes(layer)
             fwd.run_flash_attn_split(q[layer], klay, vlay, wl.dtype, so, sm, ss, H, Hkv, D, wl.context, scale,

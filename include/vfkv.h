@@ -177,7 +177,8 @@ void vfkv_workspace_destroy(vfkv_workspace* w);
  * counterpart in the reference, which hard-codes 64 (runs.rs:766); exposed so that callers who
  * drive vfkv_flash_attn_split / _reduce themselves can reproduce the same launch.  The
  * environment variable VFKV_DECODE_TILE (a multiple of 64) overrides the choice. */
-uint32_t vfkv_decode_tile_for(uint32_t span, uint32_t n_heads, uint32_t n_kv_heads);
+uint32_t vfkv_decode_tile_for(uint32_t span, uint32_t n_heads, uint32_t n_kv_heads, uint32_t head_dim,
+                              uint32_t kv_dtype);
 
 /* Forward::run_scalar_attn (forward/runs.rs:722-822) == step_attention's body
  * (executor/attention.rs:599-625): one decode query per head over keys [kv_start, position].

@@ -392,13 +392,12 @@ void vfkv_workspace_destroy(vfkv_workspace* w) {
 
 // Tile length for the convenience path: enough workgroups to cover the 256 CUs about twice, tiles a
 // multiple of 64 keys (so they never exceed the workspace's ceil(max_seq / 64) rows).
-static uint32_t choose_tile(uint32_t span, uint32_t n_kv_heads, uint32_t groups) {
+static uint32_t choose_tile(uint32_t span, uint32_t n_kv_heads, uint32_t groups, uint32_t target_wgs) {
     static const uint32_t forced = [] {
         const char* e = getenv("VFKV_DECODE_TILE");
         return e ? (uint32_t)strtoul(e, nullptr, 10) : 0u;
     }();
     if (forced >= 64u && forced % 64u == 0u) return forced;
-    const uint32_t target_wgs = 512u;
     uint32_t tiles = (target_wgs + n_kv_heads * groups - 1u) / (n_kv_heads * groups);
     if (tiles == 0u) tiles = 1u;
     uint32_t tile = (span + tiles - 1u) / tiles;
@@ -407,11 +406,15 @@ static uint32_t choose_tile(uint32_t span, uint32_t n_kv_heads, uint32_t groups)
     return tile;
 }
 
-uint32_t vfkv_decode_tile_for(uint32_t span, uint32_t n_heads, uint32_t n_kv_heads) {
+uint32_t vfkv_decode_tile_for(uint32_t span, uint32_t n_heads, uint32_t n_kv_heads, uint32_t head_dim, uint32_t kv_dtype) {
     if (span == 0u || n_kv_heads == 0u || n_heads == 0u || n_heads % n_kv_heads != 0u) return 0u;
     const uint32_t g = n_heads / n_kv_heads;
+    // The matrix-core worker (1- and 2-byte caches, head_dim 64 / 128) runs best with one workgroup per CU and
+    // serves up to 8 heads of a group per workgroup; the vector-ALU worker wants two and serves up to 4.
+    const bool mfma = (kv_dtype == VFKV_F8E4M3 || kv_dtype == VFKV_F16) && (head_dim == 64u || head_dim == 128u);
+    if (mfma) return choose_tile(span, n_kv_heads, (g + 7u) / 8u, 256u);
     const uint32_t groups = (g % 4u == 0u) ? g / 4u : (g % 2u == 0u) ? g / 2u : g;
-    return choose_tile(span, n_kv_heads, groups);
+    return choose_tile(span, n_kv_heads, groups, 512u);
 }
 
 int vfkv_decode_attention(vfkv_cache* c, uint32_t layer, uint32_t kv_layer, uint32_t n_heads, const float* q, float* o,
@@ -433,7 +436,7 @@ int vfkv_decode_attention(vfkv_cache* c, uint32_t layer, uint32_t kv_layer, uint
     if (n_heads > ws->n_heads || hd > ws->head_dim)
         return fail(VFKV_ERR_WORKSPACE, "decode_attention: workspace built for %u heads x %u dims, need %u x %u",
                     ws->n_heads, ws->head_dim, n_heads, hd);
-    const uint32_t tile = vfkv_decode_tile_for(seq_len - kv_start, n_heads, kvh);
+    const uint32_t tile = vfkv_decode_tile_for(seq_len - kv_start, n_heads, kvh, hd, c->dtype);
     const uint32_t first = kv_start / tile;
     const uint32_t n_tiles = (seq_len + tile - 1u) / tile - first;
     if (n_tiles > ws->max_tiles) return fail(VFKV_ERR_WORKSPACE, "decode_attention: %u tiles > workspace capacity %u", n_tiles, ws->max_tiles);

@@ -553,14 +553,32 @@ namespace vfkv {
 // ---- dispatch -----------------------------------------------------------------------------------
 constexpr int kSplitWaves = 4;
 
-template <int DT, int D, int RUN>
+// Build-time tuning of the matrix-core worker: rows per run for 1-byte / 2-byte caches, wavefronts per workgroup.
+#ifndef VFKV_MFMA_RUN_F8
+#define VFKV_MFMA_RUN_F8 32
+#endif
+#ifndef VFKV_MFMA_PF_F8
+#define VFKV_MFMA_PF_F8 1
+#endif
+#ifndef VFKV_MFMA_PF_F16
+#define VFKV_MFMA_PF_F16 1
+#endif
+#ifndef VFKV_MFMA_RUN_F16
+#define VFKV_MFMA_RUN_F16 32
+#endif
+#ifndef VFKV_MFMA_WAVES
+#define VFKV_MFMA_WAVES 4
+#endif
+
+template <int DT, int D, int RUN, int PF>
 static hipError_t launch_split_mfma(const SplitArgs& a, uint32_t g, hipStream_t stream) {
+    constexpr int NW = VFKV_MFMA_WAVES;
     const uint32_t gt = g < 8u ? g : 8u;
-    dim3 grid(a.n_tiles, a.n_kv_heads, (g + gt - 1u) / gt);
+    dim3 grid(a.n_kv_heads, a.n_tiles, (g + gt - 1u) / gt);
     if (a.softcap > 0.f)
-        hipLaunchKernelGGL((split_mfma_kernel<DT, D, RUN, kSplitWaves, true>), grid, dim3(kSplitWaves * kWave), 0, stream, a, gt);
+        hipLaunchKernelGGL((split_mfma_kernel<DT, D, RUN, PF, NW, true>), grid, dim3(NW * kWave), 0, stream, a, gt);
     else
-        hipLaunchKernelGGL((split_mfma_kernel<DT, D, RUN, kSplitWaves, false>), grid, dim3(kSplitWaves * kWave), 0, stream, a, gt);
+        hipLaunchKernelGGL((split_mfma_kernel<DT, D, RUN, PF, NW, false>), grid, dim3(NW * kWave), 0, stream, a, gt);
     return hipGetLastError();
 }
 
@@ -612,10 +630,10 @@ hipError_t launch_split(const SplitLaunch& L, hipStream_t stream) {
     // the register-tiled worker addresses the slab with 32-bit byte offsets below 2 GiB
     const uint64_t slab_bytes = (uint64_t)L.seq_len * L.n_kv_heads * L.head_dim * elem_size(L.dtype);
     if (aligned && slab_bytes < 0x7FFF0000ull && mfma_worker_enabled()) {
-        if (L.dtype == kF8 && L.head_dim == 64u) return launch_split_mfma<kF8, 64, 64>(a, g, stream);
-        if (L.dtype == kF8 && L.head_dim == 128u) return launch_split_mfma<kF8, 128, 64>(a, g, stream);
-        if (L.dtype == kF16 && L.head_dim == 64u) return launch_split_mfma<kF16, 64, 64>(a, g, stream);
-        if (L.dtype == kF16 && L.head_dim == 128u) return launch_split_mfma<kF16, 128, 32>(a, g, stream);
+        if (L.dtype == kF8 && L.head_dim == 64u) return launch_split_mfma<kF8, 64, 64, 1>(a, g, stream);
+        if (L.dtype == kF8 && L.head_dim == 128u) return launch_split_mfma<kF8, 128, VFKV_MFMA_RUN_F8, VFKV_MFMA_PF_F8>(a, g, stream);
+        if (L.dtype == kF16 && L.head_dim == 64u) return launch_split_mfma<kF16, 64, 64, 1>(a, g, stream);
+        if (L.dtype == kF16 && L.head_dim == 128u) return launch_split_mfma<kF16, 128, VFKV_MFMA_RUN_F16, VFKV_MFMA_PF_F16>(a, g, stream);
     }
     if (fast_shape(L.dtype, L.head_dim) && aligned && slab_bytes < 0x7FFF0000ull) {
 #define VFKV_CASE(DT, DD) \

@@ -25,10 +25,11 @@
 // through raw buffer loads whose descriptor ends at the last populated row (rows past it read as zero
 // without touching memory, which is also how the prefetch is fed when there is no next run).
 #pragma once
+#include <type_traits>
 
 namespace vfkv {
 
-template <int DT, int D, int RUN, int NW, bool CAP>
+template <int DT, int D, int RUN, int PF, int NW, bool CAP>
 __global__ __launch_bounds__(NW * 64) void split_mfma_kernel(SplitArgs a, uint32_t gt) {
     constexpr int ES = DT == kF16 ? 2 : 1;
     constexpr int RT = RUN / 16;                 // 16-row tiles per run
@@ -46,13 +47,14 @@ __global__ __launch_bounds__(NW * 64) void split_mfma_kernel(SplitArgs a, uint32
 
     __shared__ __attribute__((aligned(16))) _Float16 vlds[NW][RUN * VPITCH];
     __shared__ float lds_m[NW][8], lds_l[NW][8];
+    __shared__ __attribute__((aligned(16))) _Float16 qlds[16][D + 8];   // rows 0-7: f16(q) per head, rows 8-15: remainders
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int n16 = lane & 15, kg = lane >> 4;
     const int col = n16 & 7;
     const bool is_lo = n16 >= 8;
-    const uint32_t jl = blockIdx.x, kvh = blockIdx.y;
+    const uint32_t kvh = blockIdx.x, jl = blockIdx.y;     // KV head fastest: the workgroups of one tile start together
     const uint32_t g_all = a.n_heads / a.n_kv_heads;
     const uint32_t hz = blockIdx.z * gt;
     const uint32_t gcount = g_all - hz < gt ? g_all - hz : gt;
@@ -60,20 +62,6 @@ __global__ __launch_bounds__(NW * 64) void split_mfma_kernel(SplitArgs a, uint32
     const uint32_t tile_base = (a.tile_first + jl) * a.tile;
     uint32_t tile_end = tile_base + a.tile; if (tile_end > a.seq_len) tile_end = a.seq_len;
     const uint32_t lo = tile_base > a.kv_start ? tile_base : a.kv_start;
-
-    // ---- Q^T operands: lane (column n16, group kg) holds q[kg*SEG + c*8 + j], j < 8, per k-step c ----
-    float4 qraw[KS][2];
-    {
-        const bool col_ok = (uint32_t)col < gcount;
-        const float* qp = a.q + (size_t)(h0 + (col_ok ? col : 0)) * D + kg * SEG;
-#pragma unroll
-        for (int c = 0; c < KS; ++c)
-#pragma unroll
-            for (int j4 = 0; j4 < 2; ++j4) {
-                qraw[c][j4] = *reinterpret_cast<const float4*>(qp + c * 8 + j4 * 4);
-                if (!col_ok) qraw[c][j4] = make_float4(0.f, 0.f, 0.f, 0.f);
-            }
-    }
 
     const uint32_t row_stride = a.n_kv_heads * D * ES;
     const __amdgpu_buffer_rsrc_t krsrc = __builtin_amdgcn_make_buffer_rsrc((void*)a.k, 0, a.seq_len * row_stride, 0x00020000);
@@ -92,40 +80,69 @@ __global__ __launch_bounds__(NW * 64) void split_mfma_kernel(SplitArgs a, uint32
         return r < n_runs ? (tile_base + r * RUN) * row_stride : kOOB;
     };
 
-    u32x4 kraw[RT][KLD];
-    u32x4 vraw[VLD];
-    auto issue_k = [&](int t, uint32_t off) {
+    u32x4 kraw[PF][RT][KLD];             // PF runs in flight per wavefront
+    u32x4 vraw[PF][VLD];
+    auto issue_k = [&](int b, int t, uint32_t off) {
 #pragma unroll
         for (int x = 0; x < KLD; ++x)
-            kraw[t][x] = __builtin_amdgcn_raw_buffer_load_b128(krsrc, lane_koff + x * 16, off + (uint32_t)(t * 16) * row_stride, 0);
+            kraw[b][t][x] = __builtin_amdgcn_raw_buffer_load_b128(krsrc, lane_koff + x * 16, off + (uint32_t)(t * 16) * row_stride, 0);
     };
-    auto issue_v = [&](int c, uint32_t off) {
-        vraw[c] = __builtin_amdgcn_raw_buffer_load_b128(vrsrc, lane_voff, off + (uint32_t)(c * VROWS) * row_stride, 0);
+    auto issue_v = [&](int b, int c, uint32_t off) {
+        vraw[b][c] = __builtin_amdgcn_raw_buffer_load_b128(vrsrc, lane_voff, off + (uint32_t)(c * VROWS) * row_stride, 0);
     };
 
     uint32_t r = first_run + w;
     const bool active = lo < tile_end && r < n_runs;
-    {
-        const uint32_t off = active ? run_off(r) : kOOB;
+    const uint32_t off0 = active ? run_off(r) : kOOB;
 #pragma unroll
-        for (int t = 0; t < RT; ++t) issue_k(t, off);
-#pragma unroll
-        for (int c = 0; c < VLD; ++c) issue_v(c, off);
-    }
+    for (int t = 0; t < RT; ++t) issue_k(0, t, off0);
 
-    half8_t qb[KS];
+    // ---- Q^T operands.  The workgroup converts its heads' queries once (coalesced 16-byte loads) into f16 value /
+    // remainder planes in LDS; lane (column n16, group kg) then holds q[kg*SEG + c*8 + j], j < 8, per k-step c.
+    // The query load sits between the K and the V requests: loads return in order, so the wait for it covers K only.
+    constexpr int QLD = (8 * D / 4 + NW * 64 - 1) / (NW * 64);      // 16-byte query loads per thread (<= 8 heads)
+    const int nq4 = (int)gcount * D / 4;
+    float4 qf[QLD];
 #pragma unroll
-    for (int c = 0; c < KS; ++c)
+    for (int i = 0; i < QLD; ++i) {
+        const int idx = tid + i * NW * 64;
+        qf[i] = *reinterpret_cast<const float4*>(a.q + (size_t)h0 * D + (idx < nq4 ? idx : 0) * 4);
+    }
 #pragma unroll
-        for (int j4 = 0; j4 < 2; ++j4) {
-            const float v4[4] = {qraw[c][j4].x, qraw[c][j4].y, qraw[c][j4].z, qraw[c][j4].w};
+    for (int c = 0; c < VLD; ++c) issue_v(0, c, off0);
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                const _Float16 hv = (_Float16)v4[j];
-                const _Float16 lv = (_Float16)(v4[j] - (float)hv);
-                qb[c][j4 * 4 + j] = is_lo ? lv : hv;
-            }
+    for (int b = 1; b < PF; ++b) {
+        const uint32_t offb = active ? run_off(r + b * NW) : kOOB;
+#pragma unroll
+        for (int t = 0; t < RT; ++t) issue_k(b, t, offb);
+#pragma unroll
+        for (int c = 0; c < VLD; ++c) issue_v(b, c, offb);
+    }
+    {
+#pragma unroll
+        for (int i = 0; i < QLD; ++i) {
+            const int idx = tid + i * NW * 64;
+            if (idx >= nq4) continue;
+            const float4 f = qf[i];
+            const int g = (idx * 4) / D, d = (idx * 4) % D;
+            const float v4[4] = {f.x, f.y, f.z, f.w};
+            _Float16 hv[4], lv[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) { hv[j] = (_Float16)v4[j]; lv[j] = (_Float16)(v4[j] - (float)hv[j]); }
+            *reinterpret_cast<half4_t*>(&qlds[g][d]) = half4_t{hv[0], hv[1], hv[2], hv[3]};
+            *reinterpret_cast<half4_t*>(&qlds[8 + g][d]) = half4_t{lv[0], lv[1], lv[2], lv[3]};
         }
+    }
+    __syncthreads();
+    half8_t qb[KS];
+    {
+        const bool col_ok = (uint32_t)col < gcount;
+#pragma unroll
+        for (int c = 0; c < KS; ++c) {
+            const u32x4 raw = *reinterpret_cast<const u32x4*>(&qlds[col_ok ? n16 : 0][kg * SEG + c * 8]);
+            qb[c] = __builtin_bit_cast(half8_t, col_ok ? raw : u32x4{0u, 0u, 0u, 0u});
+        }
+    }
 
     float4_t oacc[DTILES];
 #pragma unroll
@@ -134,9 +151,13 @@ __global__ __launch_bounds__(NW * 64) void split_mfma_kernel(SplitArgs a, uint32
     _Float16* const vb = &vlds[w][0];
 
     if (active) {
-        for (; r < n_runs; r += NW) {
-            const uint32_t noff = run_off(r + NW);
-            const uint32_t rb = tile_base + r * RUN;
+        for (; r < n_runs; r += PF * NW) {
+#pragma unroll
+          for (int b = 0; b < PF; ++b) {
+            const uint32_t rr = r + (uint32_t)(b * NW);
+            if (rr >= n_runs) break;                                     // wavefront-uniform
+            const uint32_t noff = run_off(rr + PF * NW);
+            const uint32_t rb = tile_base + rr * RUN;
             // ---------------- S^T = K Q^T ----------------
             float4_t s[RT];
 #pragma unroll
@@ -145,70 +166,75 @@ __global__ __launch_bounds__(NW * 64) void split_mfma_kernel(SplitArgs a, uint32
 #pragma unroll
                 for (int c = 0; c < KS; ++c) {
                     if (DT == kF8) {
-                        const uint32_t w0 = kraw[t][c / 2][(c % 2) * 2], w1 = kraw[t][c / 2][(c % 2) * 2 + 1];
+                        const uint32_t w0 = kraw[b][t][c / 2][(c % 2) * 2], w1 = kraw[b][t][c / 2][(c % 2) * 2 + 1];
                         half2_t p0, p1, p2, p3;
                         e4m3x4_to_h2(w0, p0, p1);
                         e4m3x4_to_h2(w1, p2, p3);
                         ka[c][0] = p0[0]; ka[c][1] = p0[1]; ka[c][2] = p1[0]; ka[c][3] = p1[1];
                         ka[c][4] = p2[0]; ka[c][5] = p2[1]; ka[c][6] = p3[0]; ka[c][7] = p3[1];
                     } else {
-                        const u32x4 wv = kraw[t][c % KLD];
+                        const u32x4 wv = kraw[b][t][c % KLD];
                         ka[c] = __builtin_bit_cast(half8_t, wv);
                     }
                 }
-                issue_k(t, noff);
+                issue_k(b, t, noff);
                 s[t] = float4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
                 for (int c = 0; c < KS; ++c) s[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ka[c], qb[c], s[t], 0, 0, 0);
             }
             // ---------------- softmax: this lane owns rows rb + t*16 + kg*4 + i of column n16 ----------------
             const bool interior = rb >= lo && rb + RUN <= tile_end;      // wavefront-uniform
-            float x[RT][4];
-            float tmax = kMasked;
-#pragma unroll
-            for (int t = 0; t < RT; ++t)
-#pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    float y = s[t][i];
-                    y += dpp_f<kDppRor8>(y);                             // f16(q) part + remainder part
-                    y *= scale_l2;
-                    if (CAP) y = cap_l2 * tanhf(y / cap_l2);
-                    x[t][i] = y;
-                }
-            if (!interior) {
+            u32x4 pbits[PKS];
+            auto softmax = [&](auto masked_tag) {
+                constexpr bool MASKED = decltype(masked_tag)::value;
+                float x[RT][4];
+                float tmax = kMasked;
 #pragma unroll
                 for (int t = 0; t < RT; ++t)
 #pragma unroll
                     for (int i = 0; i < 4; ++i) {
-                        const uint32_t row = rb + t * 16 + kg * 4 + i;
-                        x[t][i] = (row >= lo && row < tile_end) ? x[t][i] : kMasked;
+                        float y = s[t][i];
+                        y += dpp_f<kDppRor8>(y);                         // f16(q) part + remainder part
+                        y *= scale_l2;
+                        if (CAP) y = cap_l2 * tanhf(y / cap_l2);
+                        if (MASKED) {
+                            const uint32_t row = rb + t * 16 + kg * 4 + i;
+                            y = (row >= lo && row < tile_end) ? y : kMasked;
+                        }
+                        x[t][i] = y;
+                        tmax = fmaxf(tmax, y);
                     }
-            }
+                { float y = tmax; swap16(tmax, y); tmax = fmaxf(tmax, y); y = tmax; swap32(tmax, y); tmax = fmaxf(tmax, y); }
+                const float m_new = fmaxf(m_run, tmax);
+                if (__builtin_amdgcn_ballot_w64(m_new > m_run) != 0ull) {
+                    const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
+                    l_run *= alpha;
 #pragma unroll
-            for (int t = 0; t < RT; ++t)
+                    for (int dt = 0; dt < DTILES; ++dt) oacc[dt] *= alpha;
+                    m_run = m_new;
+                }
+                // weights as f16 value (columns 0-7) or f16 remainder (columns 8-15), two rows per register
 #pragma unroll
-                for (int i = 0; i < 4; ++i) tmax = fmaxf(tmax, x[t][i]);
-            { float y = tmax; swap16(tmax, y); tmax = fmaxf(tmax, y); y = tmax; swap32(tmax, y); tmax = fmaxf(tmax, y); }
-            const float m_new = fmaxf(m_run, tmax);
-            if (__builtin_amdgcn_ballot_w64(m_new > m_run) != 0ull) {
-                const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
-                l_run *= alpha;
+                for (int t = 0; t < RT; ++t)
 #pragma unroll
-                for (int dt = 0; dt < DTILES; ++dt) oacc[dt] *= alpha;
-                m_run = m_new;
-            }
+                    for (int i2 = 0; i2 < 2; ++i2) {
+                        float2_t pp;
+#pragma unroll
+                        for (int e = 0; e < 2; ++e) {
+                            float pv = __builtin_amdgcn_exp2f(x[t][2 * i2 + e] - m_run);
+                            if (MASKED) pv = x[t][2 * i2 + e] > -1e29f ? pv : 0.f;
+                            pp[e] = pv;
+                        }
+                        l_run += pp[0] + pp[1];
+                        const half2_t ph = __builtin_convertvector(pp, half2_t);
+                        const half2_t pl = __builtin_convertvector(pp - __builtin_convertvector(ph, float2_t), half2_t);
+                        pbits[t / 2][(t % 2) * 2 + i2] = is_lo ? __builtin_bit_cast(uint32_t, pl) : __builtin_bit_cast(uint32_t, ph);
+                    }
+            };
+            if (interior) softmax(std::false_type{}); else softmax(std::true_type{});
             half8_t pb[PKS];
 #pragma unroll
-            for (int t = 0; t < RT; ++t)
-#pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    float p = __builtin_amdgcn_exp2f(x[t][i] - m_run);
-                    if (!interior) p = x[t][i] > -1e29f ? p : 0.f;
-                    l_run += p;
-                    const _Float16 ph = (_Float16)p;
-                    const _Float16 pl = (_Float16)(p - (float)ph);
-                    pb[t / 2][(t % 2) * 4 + i] = is_lo ? pl : ph;
-                }
+            for (int ks = 0; ks < PKS; ++ks) pb[ks] = __builtin_bit_cast(half8_t, pbits[ks]);
             // ---------------- V run -> f16 row-major in LDS ----------------
 #pragma unroll
             for (int c = 0; c < VLD; ++c) {
@@ -217,7 +243,7 @@ __global__ __launch_bounds__(NW * 64) void split_mfma_kernel(SplitArgs a, uint32
                     uint32_t out[8];
 #pragma unroll
                     for (int q4 = 0; q4 < 4; ++q4) {
-                        const uint32_t wd = vraw[c][q4];
+                        const uint32_t wd = vraw[b][c][q4];
                         half2_t lo2, hi2;
                         e4m3x4_to_h2(wd, lo2, hi2);
                         out[2 * q4] = __builtin_bit_cast(uint32_t, lo2);
@@ -226,9 +252,9 @@ __global__ __launch_bounds__(NW * 64) void split_mfma_kernel(SplitArgs a, uint32
                     reinterpret_cast<u32x4*>(dst)[0] = u32x4{out[0], out[1], out[2], out[3]};
                     reinterpret_cast<u32x4*>(dst)[1] = u32x4{out[4], out[5], out[6], out[7]};
                 } else {
-                    *reinterpret_cast<u32x4*>(dst) = vraw[c];
+                    *reinterpret_cast<u32x4*>(dst) = vraw[b][c];
                 }
-                issue_v(c, noff);
+                issue_v(b, c, noff);
             }
             // ---------------- O^T += V^T P ----------------
 #pragma unroll
@@ -243,6 +269,7 @@ __global__ __launch_bounds__(NW * 64) void split_mfma_kernel(SplitArgs a, uint32
                     va[0] = v0[0]; va[1] = v0[1]; va[2] = v0[2]; va[3] = v0[3]; va[4] = v1[0]; va[5] = v1[1]; va[6] = v1[2]; va[7] = v1[3];
                     oacc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(va, pb[ks], oacc[dt], 0, 0, 0);
                 }
+          }
         }
     }
 

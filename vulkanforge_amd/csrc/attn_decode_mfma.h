@@ -91,9 +91,19 @@ __global__ __launch_bounds__(NW * 64) void split_mfma_kernel(SplitArgs a, uint32
         vraw[b][c] = __builtin_amdgcn_raw_buffer_load_b128(vrsrc, lane_voff, off + (uint32_t)(c * VROWS) * row_stride, 0);
     };
 
-    uint32_t r = first_run + w;
-    const bool active = lo < tile_end && r < n_runs;
-    const uint32_t off0 = active ? run_off(r) : kOOB;
+    // This wavefront's runs are r0, r0 + NW, ...; it walks them cyclically from a starting point that depends on the
+    // KV head, so that the workgroups reading the same position rows are not all at the same rows at the same time.
+    const uint32_t r0 = first_run + w;
+    const uint32_t n_mine = (lo < tile_end && r0 < n_runs) ? (n_runs - r0 + NW - 1) / NW : 0u;
+    const bool active = n_mine != 0u;
+    const uint32_t rot = active ? (kvh * 3u) % n_mine : 0u;
+    auto nth_run = [&](uint32_t i) -> uint32_t {   // i-th run of this wavefront; n_runs (= none) past the last
+        if (i >= n_mine) return n_runs;
+        uint32_t ii = i + rot;
+        if (ii >= n_mine) ii -= n_mine;
+        return r0 + ii * NW;
+    };
+    const uint32_t off0 = run_off(nth_run(0));
 #pragma unroll
     for (int t = 0; t < RT; ++t) issue_k(0, t, off0);
 
@@ -112,7 +122,7 @@ __global__ __launch_bounds__(NW * 64) void split_mfma_kernel(SplitArgs a, uint32
     for (int c = 0; c < VLD; ++c) issue_v(0, c, off0);
 #pragma unroll
     for (int b = 1; b < PF; ++b) {
-        const uint32_t offb = active ? run_off(r + b * NW) : kOOB;
+        const uint32_t offb = run_off(nth_run(b));
 #pragma unroll
         for (int t = 0; t < RT; ++t) issue_k(b, t, offb);
 #pragma unroll
@@ -151,12 +161,12 @@ __global__ __launch_bounds__(NW * 64) void split_mfma_kernel(SplitArgs a, uint32
     _Float16* const vb = &vlds[w][0];
 
     if (active) {
-        for (; r < n_runs; r += PF * NW) {
+        for (uint32_t it = 0; it < n_mine; it += PF) {
 #pragma unroll
           for (int b = 0; b < PF; ++b) {
-            const uint32_t rr = r + (uint32_t)(b * NW);
-            if (rr >= n_runs) break;                                     // wavefront-uniform
-            const uint32_t noff = run_off(rr + PF * NW);
+            if (it + b >= n_mine) break;                                 // wavefront-uniform
+            const uint32_t rr = nth_run(it + b);
+            const uint32_t noff = run_off(nth_run(it + b + PF));
             const uint32_t rb = tile_base + rr * RUN;
             // ---------------- S^T = K Q^T ----------------
             float4_t s[RT];

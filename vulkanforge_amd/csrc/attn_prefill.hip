@@ -20,6 +20,7 @@ struct BatchArgs {
 
 }  // namespace vfkv
 #include "attn_prefill_mfma.h"
+#include "attn_prefill_mfma2.h"
 namespace vfkv {
 
 __global__ __launch_bounds__(kWave) void batch_generic_kernel(BatchArgs a) {
@@ -94,15 +95,51 @@ hipError_t launch_batch(const BatchLaunch& L, hipStream_t stream) {
     const uint32_t g = L.n_heads / L.n_kv_heads;
     const uint64_t slab_bytes = (uint64_t)L.n_kv * L.n_kv_heads * L.head_dim * elem_size(L.dtype);
     const bool aligned = ((((uintptr_t)L.k) | ((uintptr_t)L.v) | ((uintptr_t)L.q) | ((uintptr_t)L.o)) & 15u) == 0u;
-    if ((L.dtype == kF8 || L.dtype == kF16) && g <= 16u && aligned && slab_bytes < 0x7FFF0000ull &&
-        (L.head_dim == 64u || L.head_dim == 128u || L.head_dim == 256u)) {
+    const bool mfma_ok = (L.dtype == kF8 || L.dtype == kF16) && aligned && slab_bytes < 0x7FFF0000ull &&
+                         (L.head_dim == 64u || L.head_dim == 128u || L.head_dim == 256u);
+    // Second-generation kernel: NCB heads per wavefront, private tiles per wavefront, no barrier in the loop.
+    static const bool v2_on = [] { const char* e = getenv("VFKV_PREFILL_KERNEL"); return !(e && e[0] == '1'); }();
+    if (mfma_ok && v2_on && L.head_dim <= 128u) {
+        // two heads per wavefront where the registers allow it
+        static const int force_ncb = [] { const char* e = getenv("VFKV_PREFILL_NCB"); return e ? atoi(e) : 0; }();
+        uint32_t ncb = (g % 2u == 0u && (L.head_dim == 64u || (L.head_dim == 128u && L.dtype == kF8))) ? 2u : 1u;
+        if (force_ncb == 1) ncb = 1u;
+        const uint32_t hp = g / ncb;
+        if (hp <= 8u) {
+            const uint32_t max_waves = ncb == 1u ? 12u : 8u;  // one head per wavefront needs fewer registers: three wavefronts per SIMD
+            const uint32_t ns = max_waves / hp;               // key splits: fill the workgroup
+            const uint32_t nwaves = hp * ns;
+            const dim3 grid((L.m + 15u) / 16u, L.n_kv_heads), block(nwaves * kWave);
+            const size_t vbytes = (size_t)nwaves * 32 * (L.head_dim + 16) * sizeof(_Float16) +
+                                  (size_t)2 * g * 16 * (L.head_dim + 8) * sizeof(_Float16);
+            const size_t mbytes = (size_t)(ns - 1) * hp * ncb * 64 * (L.head_dim / 4 + 2) * sizeof(float);
+            const size_t lds = vbytes > mbytes ? vbytes : mbytes;
+            const bool cap = L.softcap > 0.f;
+            bool launched = true;
+#define VFKV_P2(DT, DD, NCBV, PFDV)                                                                         \
+    if (L.dtype == DT && L.head_dim == DD && ncb == NCBV) {                                                 \
+        if (cap) hipLaunchKernelGGL((batch_mfma2_kernel<DT, DD, NCBV, PFDV, true>), grid, block, lds, stream, a, (int)hp, (int)ns);  \
+        else hipLaunchKernelGGL((batch_mfma2_kernel<DT, DD, NCBV, PFDV, false>), grid, block, lds, stream, a, (int)hp, (int)ns);      \
+    } else
+            VFKV_P2(kF8, 64, 2, 2) VFKV_P2(kF8, 64, 1, 2) VFKV_P2(kF8, 128, 2, 2) VFKV_P2(kF8, 128, 1, 2)
+            VFKV_P2(kF16, 64, 2, 2) VFKV_P2(kF16, 64, 1, 2) VFKV_P2(kF16, 128, 1, 1)
+            { launched = false; }
+#undef VFKV_P2
+            if (launched) return hipGetLastError();
+        }
+    }
+    if (mfma_ok && g <= 16u) {
         // two key splits per workgroup while that still leaves two wavefronts per SIMD worth of registers
         const uint32_t nsplit = g <= 4u ? 2u : 1u;
         const dim3 grid((L.m + 15u) / 16u, L.n_kv_heads), block(g * nsplit * kWave);
         const size_t vbytes = (size_t)nsplit * 2 * 32 * (L.head_dim + 16) * sizeof(_Float16);
         const size_t mbytes = (size_t)(nsplit - 1) * g * 64 * (L.head_dim / 4 + 2) * sizeof(float);
         const size_t lds = vbytes > mbytes ? vbytes : mbytes;
-#define VFKV_PF2(DT, DD, CAPV, MT, NS) hipLaunchKernelGGL((batch_mfma_kernel<DT, DD, CAPV, MT, NS>), grid, block, lds, stream, a)
+// tiles in flight per key split: deeper for the shapes whose registers allow it
+#ifndef VFKV_PREFILL_PFD
+#define VFKV_PREFILL_PFD 3
+#endif
+#define VFKV_PF2(DT, DD, CAPV, MT, NS) hipLaunchKernelGGL((batch_mfma_kernel<DT, DD, CAPV, MT, NS, (DD <= 128 && MT <= 512 && DT == kF8) ? VFKV_PREFILL_PFD : 1>), grid, block, lds, stream, a)
 #define VFKV_PF(DT, DD)                                                                   \
     if (L.dtype == DT && L.head_dim == DD) {                                              \
         const bool cap = L.softcap > 0.f;                                                 \

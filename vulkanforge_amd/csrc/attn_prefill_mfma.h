@@ -29,7 +29,7 @@
 
 namespace vfkv {
 
-template <int DT, int D, bool CAP, int MAXT, int NSPLIT>
+template <int DT, int D, bool CAP, int MAXT, int NSPLIT, int PFD>
 __global__ __launch_bounds__(MAXT) void batch_mfma_kernel(BatchArgs a) {
     constexpr int ES = DT == kF16 ? 2 : 1;
     constexpr int KT = 32;                       // keys per tile
@@ -99,18 +99,19 @@ __global__ __launch_bounds__(MAXT) void batch_mfma_kernel(BatchArgs a) {
     constexpr int VCHUNK_ROW = D * ES / 16;                     // chunks per key row
     constexpr int VCHUNKS = KT * VCHUNK_ROW;
     constexpr int VMAX = (VCHUNKS + 63) / 64;                   // chunks per thread when G == 1 (fewer for larger G)
-    u32x4 vstage[VMAX];
-    auto v_issue = [&](uint32_t tbase) {
+    constexpr uint32_t kNoTile = 0x80000000u;                   // byte offset past any slab: the load returns zeros, no memory access
+    u32x4 vstage[PFD][VMAX];                                    // PFD tiles in flight per split
+    auto v_issue = [&](int slot, uint32_t toff) {               // toff: byte offset of the tile's first row (or kNoTile)
 #pragma unroll
         for (int c = 0; c < VMAX; ++c) {
             const int chunk = stid + c * nthreads;
             if (chunk < VCHUNKS) {
                 const int row = chunk / VCHUNK_ROW, col = chunk % VCHUNK_ROW;
-                vstage[c] = __builtin_amdgcn_raw_buffer_load_b128(vrsrc, row * row_stride + head_b + col * 16, tbase * row_stride, 0);
+                vstage[slot][c] = __builtin_amdgcn_raw_buffer_load_b128(vrsrc, row * row_stride + head_b + col * 16, toff, 0);
             }
         }
     };
-    auto v_commit = [&](int buf) {                              // widen to f16 and store row-major
+    auto v_commit = [&](int buf, int slot) {                    // widen to f16 and store row-major
         _Float16* base = vlds + (size_t)(sp * 2 + buf) * KT * VPITCH;
 #pragma unroll
         for (int c = 0; c < VMAX; ++c) {
@@ -121,7 +122,7 @@ __global__ __launch_bounds__(MAXT) void batch_mfma_kernel(BatchArgs a) {
                     uint32_t out[8];
 #pragma unroll
                     for (int x = 0; x < 4; ++x) {
-                        const uint32_t wd = vstage[c][x];
+                        const uint32_t wd = vstage[slot][c][x];
                         half2_t lo2, hi2;
                         e4m3x4_to_h2(wd, lo2, hi2);
                         out[2 * x] = __builtin_bit_cast(uint32_t, lo2);
@@ -131,31 +132,31 @@ __global__ __launch_bounds__(MAXT) void batch_mfma_kernel(BatchArgs a) {
                     dst[0] = u32x4{out[0], out[1], out[2], out[3]};
                     dst[1] = u32x4{out[4], out[5], out[6], out[7]};
                 } else {
-                    *reinterpret_cast<u32x4*>(base + row * VPITCH + col * 8) = vstage[c];
+                    *reinterpret_cast<u32x4*>(base + row * VPITCH + col * 8) = vstage[slot][c];
                 }
             }
         }
     };
 
     // K operands of one tile: [half of the tile][16-byte piece of this lane's quarter row]
-    u32x4 kraw[2][KLD];
-    auto k_issue = [&](uint32_t tbase) {
+    u32x4 kraw[PFD][2][KLD];
+    auto k_issue = [&](int slot, uint32_t toff) {
 #pragma unroll
         for (int kt = 0; kt < 2; ++kt)
 #pragma unroll
             for (int x = 0; x < KLD; ++x)
-                kraw[kt][x] = __builtin_amdgcn_raw_buffer_load_b128(krsrc, lane_koff + x * 16, (tbase + kt * 16) * row_stride, 0);
+                kraw[slot][kt][x] = __builtin_amdgcn_raw_buffer_load_b128(krsrc, lane_koff + x * 16, toff + (uint32_t)(kt * 16) * row_stride, 0);
     };
-    auto k_operand = [&](int kt, int c) -> half8_t {            // 8 consecutive d of this lane's quarter, k-step c
+    auto k_operand = [&](int slot, int kt, int c) -> half8_t {            // 8 consecutive d of this lane's quarter, k-step c
         half8_t r;
         if (DT == kF8) {
-            const uint32_t w0 = kraw[kt][c / 2][(c % 2) * 2], w1 = kraw[kt][c / 2][(c % 2) * 2 + 1];
+            const uint32_t w0 = kraw[slot][kt][c / 2][(c % 2) * 2], w1 = kraw[slot][kt][c / 2][(c % 2) * 2 + 1];
             half2_t p0, p1, p2, p3;
             e4m3x4_to_h2(w0, p0, p1);
             e4m3x4_to_h2(w1, p2, p3);
             r[0] = p0[0]; r[1] = p0[1]; r[2] = p1[0]; r[3] = p1[1]; r[4] = p2[0]; r[5] = p2[1]; r[6] = p3[0]; r[7] = p3[1];
         } else {
-            const u32x4 wv = kraw[kt][c];
+            const u32x4 wv = kraw[slot][kt][c];
             r = __builtin_bit_cast(half8_t, wv);
         }
         return r;
@@ -169,20 +170,29 @@ __global__ __launch_bounds__(MAXT) void batch_mfma_kernel(BatchArgs a) {
     if (t_first < kmax) {
         const uint32_t step = KT * NSPLIT;
         uint32_t tb = t_first + sp * KT;                        // this split's first tile (may already be past the end)
-        if (tb < kmax) { v_issue(tb); k_issue(tb); }
+        auto tile_off = [&](uint32_t t) -> uint32_t { return t < kmax ? t * row_stride : kNoTile; };
+#pragma unroll
+        for (int sl = 0; sl < PFD; ++sl) { v_issue(sl, tile_off(tb + sl * step)); k_issue(sl, tile_off(tb + sl * step)); }
         int buf = 0;
-        for (uint32_t round = t_first; round < kmax; round += step, tb += step, buf ^= 1) {
-            const bool live = tb < kmax;                        // wavefront-uniform; every wavefront still meets the barrier
-            if (live) v_commit(buf);
+        for (uint32_t round = t_first; round < kmax; round += PFD * step, tb += PFD * step) {
+#pragma unroll
+          for (int sl = 0; sl < PFD; ++sl) {
+            if (round + sl * step >= kmax) break;               // workgroup-uniform
+            const uint32_t tcur = tb + sl * step;
+            const bool live = tcur < kmax;                      // wavefront-uniform; every wavefront still meets the barrier
+            if (live) v_commit(buf, sl);
             __syncthreads();                                    // V tiles visible; the other buffers are free again
+            const int cbuf = buf;
+            buf ^= 1;
             if (!live) continue;
-            // operands of this tile, then prefetch the next tile while computing
+            // operands of this tile, then request the tile PFD steps ahead into the freed registers
             half8_t ka[2][KS];
 #pragma unroll
             for (int kt = 0; kt < 2; ++kt)
 #pragma unroll
-                for (int c = 0; c < KS; ++c) ka[kt][c] = k_operand(kt, c);
-            if (tb + step < kmax) { v_issue(tb + step); k_issue(tb + step); }
+                for (int c = 0; c < KS; ++c) ka[kt][c] = k_operand(sl, kt, c);
+            { const uint32_t noff = tile_off(tcur + PFD * step); v_issue(sl, noff); k_issue(sl, noff); }
+            const uint32_t tbk = tcur;                          // first key of this tile
 
             float4_t s[2] = {float4_t{0.f, 0.f, 0.f, 0.f}, float4_t{0.f, 0.f, 0.f, 0.f}};
 #pragma unroll
@@ -202,7 +212,7 @@ __global__ __launch_bounds__(MAXT) void batch_mfma_kernel(BatchArgs a) {
             for (int kt = 0; kt < 2; ++kt)
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
-                    const uint32_t t = tb + kt * 16 + kg * 4 + i;
+                    const uint32_t t = tbk + kt * 16 + kg * 4 + i;
                     float y = s[kt][i] * scale_l2;
                     if (CAP) y = cap_l2 * tanhf(y / cap_l2);
                     y = (t < my_len && t >= a.kv_start) ? y : kMasked;
@@ -229,7 +239,7 @@ __global__ __launch_bounds__(MAXT) void batch_mfma_kernel(BatchArgs a) {
                 for (int dt = 0; dt < DTILES; ++dt) oacc[dt] *= alpha;
             }
             // ---- O^T += V^T P^T ----
-            const _Float16* vb = vlds + (size_t)(sp * 2 + buf) * KT * VPITCH;
+            const _Float16* vb = vlds + (size_t)(sp * 2 + cbuf) * KT * VPITCH;
 #pragma unroll
             for (int dt = 0; dt < DTILES; ++dt) {
                 // supplier lane s of a 16-lane group points at V[key = 4*kg + s/4 (+16)][d = dt*16 + 4*(s%4)]
@@ -241,6 +251,7 @@ __global__ __launch_bounds__(MAXT) void batch_mfma_kernel(BatchArgs a) {
                 oacc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(va, pb, oacc[dt], 0, 0, 0);
                 oacc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(va, pl, oacc[dt], 0, 0, 0);
             }
+          }
         }
     }
     l_run = xor32_sum(xor16_sum(l_run));                        // every lane of a query column now has its split's sum

@@ -1,0 +1,338 @@
+// Matrix-core kernel of the chunked-prefill attention (flash_attn_batch.comp:105-208) for gfx950, second
+// generation; included by attn_prefill.hip.
+//
+// Workgroup = one KV head x 16 consecutive queries.  Its wavefronts are (head slice hp, key split sp): a
+// wavefront serves NCB query heads of the GQA group (NCB column blocks of 16 queries each) over the key tiles
+// sp, sp + NS, ... of 32 keys.  Nothing is shared between wavefronts inside the loop -- each one converts its own
+// K rows, stages its own V tile in a private LDS area and walks at its own pace -- so there is no workgroup
+// barrier until the key splits are merged at the end.  Per tile, with v_mfma_f32_16x16x32_f16:
+//
+//   S^T[key, query] = K[key, :] . Q[query, :]      A = K rows straight from global memory (a lane owns a contiguous
+//                                                  quarter row; FP8 widens to f16 exactly), converted once and
+//                                                  reused for the NCB heads; B = Q^T, resident in registers
+//   softmax (online) in the accumulator layout: a lane owns 8 scores of ONE query, so max / sum need two
+//                                                  lane swaps per tile and head; tiles that every query of the
+//                                                  block sees completely take a path without any compare
+//   O^T[d, query]  += V^T[d, key] . P^T[key, query]  A = V^T through a row-major f16 copy of the tile in LDS and
+//                                                  the transposing LDS read, read once for the NCB heads;
+//                                                  B = P^T as f16(p) and f16(p - f16(p)) (two products)
+//
+// Q is used as f16(q); when some q of the workgroup is not exactly representable the first product is
+// repeated with f16(q - f16(q)) kept in LDS, which restores f32-level accuracy.
+#pragma once
+#include <type_traits>
+
+namespace vfkv {
+
+template <int DT, int D, int NCB, int PFD, bool CAP>
+__global__ __launch_bounds__(NCB == 1 ? 768 : 512) void batch_mfma2_kernel(BatchArgs a, int HP, int NS) {
+    constexpr int ES = DT == kF16 ? 2 : 1;
+    constexpr int KT = 32;                       // keys per tile
+    constexpr int KS = D / 32;                   // MFMA k-steps of the first product
+    constexpr int DTILES = D / 16;
+    constexpr int SEG = D / 4, SEGB = SEG * ES;  // a lane group's quarter of a key row
+    constexpr int KLD = SEGB / 16;
+    constexpr int VPITCH = D + 16;               // halves per V row in LDS
+    constexpr int VCHUNK_ROW = D * ES / 16;      // 16-byte chunks per V row
+    constexpr int VLD = KT * VCHUNK_ROW / 64;    // V loads per lane per tile
+    constexpr int VROWS = 64 / VCHUNK_ROW;
+    constexpr uint32_t kNoTile = 0x80000000u;    // byte offset past any slab: the load returns zeros, no memory access
+    static_assert(D % 32 == 0 && SEGB % 16 == 0 && VLD >= 1, "unsupported head_dim");
+
+    extern __shared__ __attribute__((aligned(16))) _Float16 lds[];      // [waves][KT][VPITCH] V tiles | [G][16][D + 8] f16(q) | [G][16][D + 8] remainders
+    __shared__ int lds_haslo;
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int nwaves = HP * NS;
+    const int hp = w % HP, sp = w / HP;
+    const int n16 = lane & 15, kg = lane >> 4;
+    const int G = a.n_heads / a.n_kv_heads;
+    const uint32_t kvh = blockIdx.y;
+    const uint32_t q0 = blockIdx.x * 16;
+    const uint32_t qi = q0 + n16;                               // this lane's query (column of S^T)
+    const bool q_ok = qi < a.m;
+    const uint32_t row_stride = a.n_kv_heads * D * ES;
+    const int g0 = hp * NCB;                                    // first head (inside the group) of this wavefront
+
+    _Float16* const vb = lds + (size_t)w * KT * VPITCH;
+    constexpr int QPITCH = D + 8;
+    _Float16* const qhi_lds = lds + (size_t)nwaves * KT * VPITCH;   // [G][16][D + 8] f16(q)
+    _Float16* const qlo_lds = qhi_lds + (size_t)G * 16 * QPITCH;    // [G][16][D + 8] f16(q - f16(q))
+
+    // ---- key range ----
+    uint32_t kmax = a.q_start + q0 + 16;                        // one past the last key any of the 16 queries sees
+    if (kmax > a.n_kv) kmax = a.n_kv;
+    const uint32_t my_len = q_ok ? (a.q_start + qi + 1 < a.n_kv ? a.q_start + qi + 1 : a.n_kv) : 0;   // causal_len of this lane's query
+    uint32_t full_len = a.q_start + q0 + 1;                     // keys every query of the block sees
+    if (full_len > a.n_kv) full_len = a.n_kv;
+    const uint32_t t_first = (a.kv_start / KT) * KT;
+    const float scale_l2 = a.scale * 1.44269504088896f;
+    const float cap_l2 = a.softcap * 1.44269504088896f;
+
+    const __amdgpu_buffer_rsrc_t krsrc = __builtin_amdgcn_make_buffer_rsrc((void*)a.k, 0, a.n_kv * row_stride, 0x00020000);
+    const __amdgpu_buffer_rsrc_t vrsrc = __builtin_amdgcn_make_buffer_rsrc((void*)a.v, 0, a.n_kv * row_stride, 0x00020000);
+    const uint32_t head_b = kvh * D * ES;
+    const uint32_t lane_koff = n16 * row_stride + head_b + kg * SEGB;
+    const int vrow = lane / VCHUNK_ROW, vcol = lane % VCHUNK_ROW;
+    const uint32_t lane_voff = vrow * row_stride + head_b + vcol * 16;
+
+    u32x4 kraw[PFD][2][KLD];
+    u32x4 vraw[PFD][VLD];
+    auto issue = [&](int slot, uint32_t toff) {
+#pragma unroll
+        for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+            for (int x = 0; x < KLD; ++x)
+                kraw[slot][kt][x] = __builtin_amdgcn_raw_buffer_load_b128(krsrc, lane_koff + x * 16, toff + (uint32_t)(kt * 16) * row_stride, 0);
+#pragma unroll
+        for (int c = 0; c < VLD; ++c)
+            vraw[slot][c] = __builtin_amdgcn_raw_buffer_load_b128(vrsrc, lane_voff, toff + (uint32_t)(c * VROWS) * row_stride, 0);
+    };
+    const uint32_t step = KT * NS;
+    const uint32_t tb0 = t_first + sp * KT;                     // this wavefront's first tile (may already be past the end)
+    auto tile_off = [&](uint32_t t) -> uint32_t { return t < kmax ? t * row_stride : kNoTile; };
+#pragma unroll
+    for (int sl = 0; sl < PFD; ++sl) issue(sl, tile_off(tb0 + sl * step));
+
+    // ---- Q^T as B operands: lane (query n16, group kg) holds q[kg*SEG + c*8 + j], j < 8, per k-step c and head ----
+    if (tid == 0) lds_haslo = 0;
+    __syncthreads();
+    {
+        bool any_lo = false;
+#pragma unroll
+        for (int cb = 0; cb < NCB; ++cb) {
+            const uint32_t h = kvh * G + g0 + cb;
+            const float* qp = a.q + ((size_t)(q_ok ? qi : 0) * a.n_heads + h) * D + kg * SEG;
+            _Float16* lo_row = qlo_lds + ((size_t)(g0 + cb) * 16 + n16) * QPITCH + kg * SEG;
+            _Float16* hi_row = qhi_lds + ((size_t)(g0 + cb) * 16 + n16) * QPITCH + kg * SEG;
+#pragma unroll
+            for (int c = 0; c < KS; ++c) {
+                half8_t lo8, hi8;
+#pragma unroll
+                for (int j4 = 0; j4 < 2; ++j4) {
+                    float4 f = *reinterpret_cast<const float4*>(qp + c * 8 + j4 * 4);
+                    if (!q_ok) f = make_float4(0.f, 0.f, 0.f, 0.f);
+                    const float v[4] = {f.x, f.y, f.z, f.w};
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        const _Float16 hv = (_Float16)v[j];
+                        const _Float16 lv = (_Float16)(v[j] - (float)hv);
+                        hi8[j4 * 4 + j] = hv;
+                        lo8[j4 * 4 + j] = lv;
+                        any_lo |= lv != (_Float16)0;
+                    }
+                }
+                *reinterpret_cast<half8_t*>(lo_row + c * 8) = lo8;
+                *reinterpret_cast<half8_t*>(hi_row + c * 8) = hi8;
+            }
+        }
+        if (any_lo) lds_haslo = 1;
+    }
+    __syncthreads();
+    const bool has_lo = __builtin_amdgcn_readfirstlane(lds_haslo) != 0;   // workgroup-uniform
+
+    float4_t oacc[NCB][DTILES];
+#pragma unroll
+    for (int cb = 0; cb < NCB; ++cb)
+#pragma unroll
+        for (int dt = 0; dt < DTILES; ++dt) oacc[cb][dt] = float4_t{0.f, 0.f, 0.f, 0.f};
+    float m_run[NCB], l_run[NCB];
+#pragma unroll
+    for (int cb = 0; cb < NCB; ++cb) { m_run[cb] = kMasked; l_run[cb] = 0.f; }
+
+    for (uint32_t tb = tb0; tb < kmax; tb += PFD * step) {
+#pragma unroll
+        for (int sl = 0; sl < PFD; ++sl) {
+            const uint32_t tcur = tb + sl * step;
+            if (tcur >= kmax) break;                            // wavefront-uniform
+            const uint32_t noff = tile_off(tcur + PFD * step);
+            // ---------------- V tile -> f16 row-major in this wavefront's LDS area (first: the writes complete behind the first product and the softmax) ----------------
+#pragma unroll
+            for (int c = 0; c < VLD; ++c) {
+                _Float16* dst = vb + (c * VROWS + vrow) * VPITCH + vcol * (16 / ES);
+                if (DT == kF8) {
+                    uint32_t out[8];
+#pragma unroll
+                    for (int q4 = 0; q4 < 4; ++q4) {
+                        const uint32_t wd = vraw[sl][c][q4];
+                        half2_t lo2, hi2;
+                        e4m3x4_to_h2(wd, lo2, hi2);
+                        out[2 * q4] = __builtin_bit_cast(uint32_t, lo2);
+                        out[2 * q4 + 1] = __builtin_bit_cast(uint32_t, hi2);
+                    }
+                    reinterpret_cast<u32x4*>(dst)[0] = u32x4{out[0], out[1], out[2], out[3]};
+                    reinterpret_cast<u32x4*>(dst)[1] = u32x4{out[4], out[5], out[6], out[7]};
+                } else {
+                    *reinterpret_cast<u32x4*>(dst) = vraw[sl][c];
+                }
+                vraw[sl][c] = __builtin_amdgcn_raw_buffer_load_b128(vrsrc, lane_voff, noff + (uint32_t)(c * VROWS) * row_stride, 0);
+            }
+            // ---------------- S^T = K Q^T for the NCB heads (Q operands re-read from LDS every tile) ----------------
+            float4_t s[NCB][2];
+            half8_t qhi[NCB][KS];
+#pragma unroll
+            for (int cb = 0; cb < NCB; ++cb)
+#pragma unroll
+                for (int c = 0; c < KS; ++c)
+                    qhi[cb][c] = *reinterpret_cast<const half8_t*>(qhi_lds + ((size_t)(g0 + cb) * 16 + n16) * QPITCH + kg * SEG + c * 8);
+#pragma unroll
+            for (int kt = 0; kt < 2; ++kt) {
+                half8_t ka[KS];
+#pragma unroll
+                for (int c = 0; c < KS; ++c) {
+                    if (DT == kF8) {
+                        const uint32_t w0 = kraw[sl][kt][c / 2][(c % 2) * 2], w1 = kraw[sl][kt][c / 2][(c % 2) * 2 + 1];
+                        half2_t p0, p1, p2, p3;
+                        e4m3x4_to_h2(w0, p0, p1);
+                        e4m3x4_to_h2(w1, p2, p3);
+                        ka[c][0] = p0[0]; ka[c][1] = p0[1]; ka[c][2] = p1[0]; ka[c][3] = p1[1];
+                        ka[c][4] = p2[0]; ka[c][5] = p2[1]; ka[c][6] = p3[0]; ka[c][7] = p3[1];
+                    } else {
+                        const u32x4 wv = kraw[sl][kt][c % KLD];
+                        ka[c] = __builtin_bit_cast(half8_t, wv);
+                    }
+                }
+#pragma unroll
+                for (int x = 0; x < KLD; ++x)
+                    kraw[sl][kt][x] = __builtin_amdgcn_raw_buffer_load_b128(krsrc, lane_koff + x * 16, noff + (uint32_t)(kt * 16) * row_stride, 0);
+#pragma unroll
+                for (int cb = 0; cb < NCB; ++cb) {
+                    s[cb][kt] = float4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                    for (int c = 0; c < KS; ++c) s[cb][kt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ka[c], qhi[cb][c], s[cb][kt], 0, 0, 0);
+                }
+                if (has_lo) {
+#pragma unroll
+                    for (int cb = 0; cb < NCB; ++cb) {
+                        const _Float16* lo_row = qlo_lds + ((size_t)(g0 + cb) * 16 + n16) * QPITCH + kg * SEG;
+#pragma unroll
+                        for (int c = 0; c < KS; ++c) {
+                            const half8_t ql = *reinterpret_cast<const half8_t*>(lo_row + c * 8);
+                            s[cb][kt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ka[c], ql, s[cb][kt], 0, 0, 0);
+                        }
+                    }
+                }
+            }
+            // ---------------- online softmax: this lane owns keys tcur + kt*16 + kg*4 + i of query n16 ----------------
+            u32x4 phi[NCB], plo[NCB];
+            auto softmax = [&](auto masked_tag) {
+                constexpr bool MASKED = decltype(masked_tag)::value;
+#pragma unroll
+                for (int cb = 0; cb < NCB; ++cb) {
+                    float x[8];
+                    float tmax = kMasked;
+#pragma unroll
+                    for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) {
+                            float y = s[cb][kt][i] * scale_l2;
+                            if (CAP) y = cap_l2 * tanhf(y / cap_l2);
+                            if (MASKED) {
+                                const uint32_t t = tcur + kt * 16 + kg * 4 + i;
+                                y = (t < my_len && t >= a.kv_start) ? y : kMasked;
+                            }
+                            x[kt * 4 + i] = y;
+                            tmax = fmaxf(tmax, y);
+                        }
+                    { float y = tmax; swap16(tmax, y); tmax = fmaxf(tmax, y); y = tmax; swap32(tmax, y); tmax = fmaxf(tmax, y); }
+                    const float m_new = fmaxf(m_run[cb], tmax);
+                    if (__builtin_amdgcn_ballot_w64(m_new > m_run[cb]) != 0ull) {
+                        const float alpha = __builtin_amdgcn_exp2f(m_run[cb] - m_new);
+                        l_run[cb] *= alpha;
+#pragma unroll
+                        for (int dt = 0; dt < DTILES; ++dt) oacc[cb][dt] *= alpha;
+                        m_run[cb] = m_new;
+                    }
+#pragma unroll
+                    for (int j2 = 0; j2 < 4; ++j2) {
+                        float2_t pp;
+#pragma unroll
+                        for (int e = 0; e < 2; ++e) {
+                            float pv = __builtin_amdgcn_exp2f(x[2 * j2 + e] - m_run[cb]);
+                            if (MASKED) pv = x[2 * j2 + e] > -1e29f ? pv : 0.f;
+                            pp[e] = pv;
+                        }
+                        l_run[cb] += pp[0] + pp[1];
+                        const half2_t ph = __builtin_convertvector(pp, half2_t);
+                        const half2_t pl = __builtin_convertvector(pp - __builtin_convertvector(ph, float2_t), half2_t);
+                        phi[cb][j2] = __builtin_bit_cast(uint32_t, ph);
+                        plo[cb][j2] = __builtin_bit_cast(uint32_t, pl);
+                    }
+                }
+            };
+            const bool interior = tcur >= a.kv_start && tcur + KT <= full_len;   // every query of the block sees the whole tile
+            if (interior) softmax(std::false_type{}); else softmax(std::true_type{});
+            // ---------------- O^T += V^T P^T for the NCB heads ----------------
+#pragma unroll
+            for (int dt = 0; dt < DTILES; ++dt) {
+                // supplier lane s of a 16-lane group points at V[key = 4*kg + s/4 (+16)][d = dt*16 + 4*(s%4)]
+                const _Float16* p0 = vb + (kg * 4 + n16 / 4) * VPITCH + dt * 16 + 4 * (n16 % 4);
+                const half4_t v0 = lds_read_tr16(p0);
+                const half4_t v1 = lds_read_tr16(p0 + 16 * VPITCH);
+                half8_t va;
+                va[0] = v0[0]; va[1] = v0[1]; va[2] = v0[2]; va[3] = v0[3]; va[4] = v1[0]; va[5] = v1[1]; va[6] = v1[2]; va[7] = v1[3];
+#pragma unroll
+                for (int cb = 0; cb < NCB; ++cb)
+                    oacc[cb][dt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(va, __builtin_bit_cast(half8_t, phi[cb]), oacc[cb][dt], 0, 0, 0);
+#pragma unroll
+                for (int cb = 0; cb < NCB; ++cb)
+                    oacc[cb][dt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(va, __builtin_bit_cast(half8_t, plo[cb]), oacc[cb][dt], 0, 0, 0);
+            }
+        }
+    }
+#pragma unroll
+    for (int cb = 0; cb < NCB; ++cb) l_run[cb] = xor32_sum(xor16_sum(l_run[cb]));   // every lane of a query column has its wavefront's sum
+
+    // ---- merge the key splits through LDS (split 0 collects), normalise and store ----
+    constexpr int REC = DTILES * 4 + 2;
+    if (NS > 1) {
+        __syncthreads();                                        // every wavefront is done with its V area
+        float* mbuf = reinterpret_cast<float*>(lds);            // [NS-1][HP][NCB][64][REC]
+        if (sp > 0) {
+#pragma unroll
+            for (int cb = 0; cb < NCB; ++cb) {
+                float* rec = mbuf + ((size_t)(((sp - 1) * HP + hp) * NCB + cb) * 64 + lane) * REC;
+#pragma unroll
+                for (int dt = 0; dt < DTILES; ++dt)
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) rec[dt * 4 + i] = oacc[cb][dt][i];
+                rec[DTILES * 4] = m_run[cb];
+                rec[DTILES * 4 + 1] = l_run[cb];
+            }
+        }
+        __syncthreads();
+        if (sp > 0) return;
+#pragma unroll 1
+        for (int s2 = 1; s2 < NS; ++s2) {
+#pragma unroll
+            for (int cb = 0; cb < NCB; ++cb) {
+                const float* rec = mbuf + ((size_t)(((s2 - 1) * HP + hp) * NCB + cb) * 64 + lane) * REC;
+                const float m2 = rec[DTILES * 4], l2 = rec[DTILES * 4 + 1];
+                const float mm = fmaxf(m_run[cb], m2);
+                const float f1 = __builtin_amdgcn_exp2f(m_run[cb] - mm), f2 = __builtin_amdgcn_exp2f(m2 - mm);
+#pragma unroll
+                for (int dt = 0; dt < DTILES; ++dt)
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) oacc[cb][dt][i] = oacc[cb][dt][i] * f1 + rec[dt * 4 + i] * f2;
+                l_run[cb] = l_run[cb] * f1 + l2 * f2;
+                m_run[cb] = mm;
+            }
+        }
+    }
+    if (q_ok) {
+#pragma unroll
+        for (int cb = 0; cb < NCB; ++cb) {
+            const uint32_t h = kvh * G + g0 + cb;
+            const float inv = 1.0f / l_run[cb];
+            float* op = a.o + ((size_t)qi * a.n_heads + h) * D + kg * 4;      // lane (query n16) holds d = dt*16 + kg*4 + i
+#pragma unroll
+            for (int dt = 0; dt < DTILES; ++dt) {
+                const float4_t r = oacc[cb][dt] * inv;
+                *reinterpret_cast<float4*>(op + dt * 16) = make_float4(r[0], r[1], r[2], r[3]);
+            }
+        }
+    }
+}
+
+}  // namespace vfkv

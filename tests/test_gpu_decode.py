@@ -61,6 +61,10 @@ CASES = [
     (vf.KvDtype.F8, 16, 2, 256, 600, 128, 0, 0.0),
     (vf.KvDtype.F8, 8, 2, 512, 300, 64, 100, 0.0),
     (vf.KvDtype.F8, 16, 4, 64, 900, 320, 0, 0.0),
+    (vf.KvDtype.F8, 32, 2, 128, 700, 1024, 0, 0.0),   # G = 16: two slices of 8 heads, one ragged tile
+    (vf.KvDtype.F8, 24, 2, 128, 1300, 448, 5, 0.0),   # G = 12: slices of 8 and 4 heads
+    (vf.KvDtype.F8, 32, 8, 128, 3000, 1024, 1900, 0.0),  # window starting inside a tile, several runs per wavefront
+    (vf.KvDtype.F16, 20, 4, 128, 1111, 320, 0, 20.0), # G = 5 with soft-cap
     (vf.KvDtype.F16, 32, 8, 128, 2049, 512, 0, 0.0),
     (vf.KvDtype.F16, 16, 8, 256, 1500, 256, 0, 50.0),
     (vf.KvDtype.F16, 16, 8, 256, 1500, 64, 1100, 50.0),

@@ -56,6 +56,10 @@ CASES = [
     (vf.KvDtype.F8, 4, 4, 64, 100, 30, 0, 0.0),       # G = 1, head_dim 64
     (vf.KvDtype.F16, 8, 8, 64, 17, 200, 190, 0.0),
     (vf.KvDtype.F16, 48, 4, 128, 5, 40, 0, 0.0),      # G = 12
+    (vf.KvDtype.F8, 24, 8, 128, 40, 1000, 0, 0.0),    # G = 3: one head per wavefront, four key splits
+    (vf.KvDtype.F8, 12, 2, 128, 23, 2100, 1500, 0.0), # G = 6: three head pairs, two key splits, window
+    (vf.KvDtype.F8, 16, 8, 64, 70, 600, 0, 30.0),     # G = 2: one head pair, eight key splits, soft-cap
+    (vf.KvDtype.F16, 16, 2, 128, 33, 900, 0, 0.0),    # G = 8 on a 2-byte cache
 ]
 
 

@@ -634,6 +634,8 @@ hipError_t launch_split(const SplitLaunch& L, hipStream_t stream) {
         if (L.dtype == kF8 && L.head_dim == 128u) return launch_split_mfma<kF8, 128, VFKV_MFMA_RUN_F8, VFKV_MFMA_PF_F8>(a, g, stream);
         if (L.dtype == kF16 && L.head_dim == 64u) return launch_split_mfma<kF16, 64, 64, 1>(a, g, stream);
         if (L.dtype == kF16 && L.head_dim == 128u) return launch_split_mfma<kF16, 128, VFKV_MFMA_RUN_F16, VFKV_MFMA_PF_F16>(a, g, stream);
+        if (L.dtype == kF8 && L.head_dim == 256u) return launch_split_mfma<kF8, 256, 32, 1>(a, g, stream);
+        if (L.dtype == kF16 && L.head_dim == 256u) return launch_split_mfma<kF16, 256, 32, 1>(a, g, stream);
     }
     if (fast_shape(L.dtype, L.head_dim) && aligned && slab_bytes < 0x7FFF0000ull) {
 #define VFKV_CASE(DT, DD) \

@@ -35,8 +35,8 @@ MFMA_F16_PEAK_TFLOPS = 2500.0
 # (two runs) and scaled by what the same counters read for a plain 64 MiB device copy
 # (FETCH_SIZE x 1.9991, WRITE_SIZE x 1.0 to KiB).  Only the workloads that were profiled have an entry.
 MEASURED_TRAFFIC_BYTES = {
-    "decode_fp8_32k_32layers": (65607 + 520) * 1024,
-    "prefill_fp8_512x4608_32layers": (81245 + 8192) * 1024,
+    "decode_fp8_32k_32layers": (65604 + 520) * 1024,
+    "prefill_fp8_512x4608_32layers": (81365 + 8192) * 1024,
 }
 
 
@@ -191,7 +191,7 @@ def bench_decode(args, wl):
     avg_ms = split_ms / launches
     achieved = bytes_launch / (avg_ms * 1e-3) / 1e9
 
-    mfma_worker = os.environ.get("VFKV_DECODE_WORKER", "m")[:1] != "v" and D <= 128 and wl.dtype.label() != "FP32"
+    mfma_worker = os.environ.get("VFKV_DECODE_WORKER", "m")[:1] != "v" and D <= 256 and wl.dtype.label() != "FP32"
     worker_name = "split_mfma_kernel" if mfma_worker else "split_kernel"
     result = {
         "metric": "kv_read_GBps_decode_step",
@@ -305,7 +305,7 @@ def bench_prefill(args, wl):
         "data": "synthetic, seeded N(0,1); queries " + ("general f32" if args.f32_queries else "cast to fp16 as the configuration states") + "; K/V rows cast to fp16 and written through the append kernels",
         "config": {"workload": wl.name, "n_layers": L, "n_heads": H, "n_kv_heads": Hkv, "head_dim": D,
                    "m": wl.m, "q_start": wl.base_pos, "n_kv": max_seq, "flop_per_step": flops_step},
-        "roofline": {"bound": "mfma", "kernel": "flash_attn_batch", "achieved": achieved, "peak": MFMA_F16_PEAK_TFLOPS,
+        "roofline": {"bound": "mfma", "kernel": "batch_mfma2_kernel", "achieved": achieved, "peak": MFMA_F16_PEAK_TFLOPS,
                      "unit": "TFLOP/s", "frac": achieved / MFMA_F16_PEAK_TFLOPS, "traffic": MEASURED_TRAFFIC_BYTES.get(wl.name),
                      "avg_launch_us": avg_ms * 1e3},
     }

@@ -92,43 +92,43 @@ __global__ __launch_bounds__(NCB == 1 ? 768 : 512) void batch_mfma2_kernel(Batch
     const uint32_t step = KT * NS;
     const uint32_t tb0 = t_first + sp * KT;                     // this wavefront's first tile (may already be past the end)
     auto tile_off = [&](uint32_t t) -> uint32_t { return t < kmax ? t * row_stride : kNoTile; };
-#pragma unroll
-    for (int sl = 0; sl < PFD; ++sl) issue(sl, tile_off(tb0 + sl * step));
-
-    // ---- Q^T as B operands: lane (query n16, group kg) holds q[kg*SEG + c*8 + j], j < 8, per k-step c and head ----
+    // ---- Q block of the workgroup: 16 queries x G heads x D floats, loaded once with coalesced 16-byte loads (before the
+    // K / V requests, so waiting for it does not wait for them) and kept in LDS as an f16 value plane and a remainder plane
+    constexpr int QLD = 4;                                      // query loads per thread and round
+    const int nthreads = nwaves * 64;
+    const int q4_total = 16 * G * (D / 4);
     if (tid == 0) lds_haslo = 0;
-    __syncthreads();
-    {
-        bool any_lo = false;
+    bool any_lo = false;
+    for (int base = 0; base < q4_total; base += QLD * nthreads) {
+        float4 qf[QLD];
 #pragma unroll
-        for (int cb = 0; cb < NCB; ++cb) {
-            const uint32_t h = kvh * G + g0 + cb;
-            const float* qp = a.q + ((size_t)(q_ok ? qi : 0) * a.n_heads + h) * D + kg * SEG;
-            _Float16* lo_row = qlo_lds + ((size_t)(g0 + cb) * 16 + n16) * QPITCH + kg * SEG;
-            _Float16* hi_row = qhi_lds + ((size_t)(g0 + cb) * 16 + n16) * QPITCH + kg * SEG;
-#pragma unroll
-            for (int c = 0; c < KS; ++c) {
-                half8_t lo8, hi8;
-#pragma unroll
-                for (int j4 = 0; j4 < 2; ++j4) {
-                    float4 f = *reinterpret_cast<const float4*>(qp + c * 8 + j4 * 4);
-                    if (!q_ok) f = make_float4(0.f, 0.f, 0.f, 0.f);
-                    const float v[4] = {f.x, f.y, f.z, f.w};
-#pragma unroll
-                    for (int j = 0; j < 4; ++j) {
-                        const _Float16 hv = (_Float16)v[j];
-                        const _Float16 lv = (_Float16)(v[j] - (float)hv);
-                        hi8[j4 * 4 + j] = hv;
-                        lo8[j4 * 4 + j] = lv;
-                        any_lo |= lv != (_Float16)0;
-                    }
-                }
-                *reinterpret_cast<half8_t*>(lo_row + c * 8) = lo8;
-                *reinterpret_cast<half8_t*>(hi_row + c * 8) = hi8;
-            }
+        for (int i = 0; i < QLD; ++i) {
+            const int idx = base + tid + i * nthreads;
+            const int qq = idx / (G * (D / 4)), rem = idx - qq * (G * (D / 4));
+            const bool ok = idx < q4_total && q0 + qq < a.m;
+            qf[i] = *reinterpret_cast<const float4*>(a.q + ((size_t)(ok ? q0 + qq : 0) * a.n_heads + kvh * G) * D + (ok ? rem * 4 : 0));
+            if (!ok) qf[i] = make_float4(0.f, 0.f, 0.f, 0.f);
         }
-        if (any_lo) lds_haslo = 1;
+        if (base == 0) {
+#pragma unroll
+            for (int sl = 0; sl < PFD; ++sl) issue(sl, tile_off(tb0 + sl * step));
+        }
+#pragma unroll
+        for (int i = 0; i < QLD; ++i) {
+            const int idx = base + tid + i * nthreads;
+            if (idx >= q4_total) continue;
+            const int qq = idx / (G * (D / 4)), rem = idx - qq * (G * (D / 4));
+            const int g = rem / (D / 4), d = (rem - g * (D / 4)) * 4;
+            const float v[4] = {qf[i].x, qf[i].y, qf[i].z, qf[i].w};
+            _Float16 hv[4], lv[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) { hv[j] = (_Float16)v[j]; lv[j] = (_Float16)(v[j] - (float)hv[j]); any_lo |= lv[j] != (_Float16)0; }
+            *reinterpret_cast<half4_t*>(qhi_lds + ((size_t)g * 16 + qq) * QPITCH + d) = half4_t{hv[0], hv[1], hv[2], hv[3]};
+            *reinterpret_cast<half4_t*>(qlo_lds + ((size_t)g * 16 + qq) * QPITCH + d) = half4_t{lv[0], lv[1], lv[2], lv[3]};
+        }
     }
+    __syncthreads();                                            // lds_haslo cleared, planes written
+    if (any_lo) lds_haslo = 1;
     __syncthreads();
     const bool has_lo = __builtin_amdgcn_readfirstlane(lds_haslo) != 0;   // workgroup-uniform
 
@@ -141,6 +141,12 @@ __global__ __launch_bounds__(NCB == 1 ? 768 : 512) void batch_mfma2_kernel(Batch
 #pragma unroll
     for (int cb = 0; cb < NCB; ++cb) { m_run[cb] = kMasked; l_run[cb] = 0.f; }
 
+#ifdef VFKV_X_STAGGER
+    if (w >= nwaves / 2) __builtin_amdgcn_s_sleep(VFKV_X_STAGGER);
+#endif
+#ifdef VFKV_X_PRIO
+    if (w >= nwaves / 2) __builtin_amdgcn_s_setprio(VFKV_X_PRIO);
+#endif
     for (uint32_t tb = tb0; tb < kmax; tb += PFD * step) {
 #pragma unroll
         for (int sl = 0; sl < PFD; ++sl) {

@@ -141,12 +141,6 @@ __global__ __launch_bounds__(NCB == 1 ? 768 : 512) void batch_mfma2_kernel(Batch
 #pragma unroll
     for (int cb = 0; cb < NCB; ++cb) { m_run[cb] = kMasked; l_run[cb] = 0.f; }
 
-#ifdef VFKV_X_STAGGER
-    if (w >= nwaves / 2) __builtin_amdgcn_s_sleep(VFKV_X_STAGGER);
-#endif
-#ifdef VFKV_X_PRIO
-    if (w >= nwaves / 2) __builtin_amdgcn_s_setprio(VFKV_X_PRIO);
-#endif
     for (uint32_t tb = tb0; tb < kmax; tb += PFD * step) {
 #pragma unroll
         for (int sl = 0; sl < PFD; ++sl) {

@@ -139,10 +139,12 @@ def bench_decode(args, wl):
 
     def step():
         for layer in range(L):
-            if wl.append:
-                fwd.step_kv_write(layer, pos, k_new[layer], v_new[layer])
-            fwd.run_scalar_attn(layer, pos, q[layer], o[layer], kv_start=starts[layer], scale=scale,
-                                softcap=wl.softcap)
+            if wl.append:       # step_kv_write + step_attention of the new token, issued as one call
+                fwd.step_kv_write_attention(layer, pos, q[layer], k_new[layer], v_new[layer], o[layer],
+                                            kv_start=starts[layer], scale=scale, softcap=wl.softcap)
+            else:
+                fwd.run_scalar_attn(layer, pos, q[layer], o[layer], kv_start=starts[layer], scale=scale,
+                                    softcap=wl.softcap)
 
     sec_per_step = time_steps(torch, step, args)
     bytes_step = wl.kv_bytes_step()

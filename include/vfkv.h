@@ -192,6 +192,17 @@ int vfkv_decode_attention(vfkv_cache* c, uint32_t layer, uint32_t kv_layer, uint
                           const float* q, float* o, uint32_t position, uint32_t kv_start, float scale,
                           float softcap, vfkv_workspace* ws, vfkv_stream stream);
 
+/* step_kv_write followed by step_attention for the same layer and token, as the executor issues them
+ * back to back (executor/attention.rs:546-625): appends the token's K and V rows (f32,
+ * kv_heads_for(layer) * head_dim_for(layer) elements each) at `position`, then attends over keys
+ * [kv_start, position].  Where the decode worker can, the workgroups that own `position` write the
+ * rows themselves before reading them, which saves the append launch; otherwise this is exactly
+ * vfkv_kv_write + vfkv_decode_attention.  The cache bytes and the output are the same either way. */
+int vfkv_kv_write_decode_attention(vfkv_cache* c, uint32_t layer, uint32_t n_heads, const float* q,
+                                   const float* k_src, const float* v_src, float* o, uint32_t position,
+                                   uint32_t kv_start, float scale, float softcap, vfkv_workspace* ws,
+                                   vfkv_stream stream);
+
 /* ------------------------------------------------------------------------------------------ */
 /* Chunked-prefill causal attention over the cache.                                           */
 /* ------------------------------------------------------------------------------------------ */

@@ -221,6 +221,50 @@ def test_config2_fp8_outliers_append_then_decode_two_layers():
         assert err < 5e-3 and err < TIGHT * 40, err
 
 
+@pytest.mark.parametrize("dtype,heads,hkv,d,ctx,window", [
+    (vf.KvDtype.F8, 32, 8, 128, 8192, 0),       # configuration 2 geometry: the worker writes the row itself
+    (vf.KvDtype.F8, 32, 8, 128, 1000, 300),     # new position in a ragged last tile, sliding window
+    (vf.KvDtype.F16, 16, 8, 256, 777, 0),       # 2-byte cache, head_dim 256
+    (vf.KvDtype.F16, 8, 8, 64, 64, 0),          # the new row opens a tile of its own
+    (vf.KvDtype.F8, 24, 2, 128, 500, 0),        # GQA group of 12: two head slices, separate append launch
+    (vf.KvDtype.F32, 8, 2, 128, 300, 0),        # 4-byte cache: separate append launch
+])
+def test_kv_write_attention_in_one_call_matches_the_two_calls(dtype, heads, hkv, d, ctx, window):
+    # step_kv_write + step_attention (executor/attention.rs:546-625) through the single entry point: cache bytes and
+    # output must equal what the two separate calls produce, bit for bit, and match the oracle
+    from gpu_util import read_device
+    fill = outlier_normal if dtype == vf.KvDtype.F8 else fp16_normal
+    esz = dtype.element_size()
+    r = rng(77 + ctx)
+    k_new, v_new, q = fill(r, (1, hkv * d)), fill(r, (1, hkv * d)), fp16_normal(r, (heads, d))
+    kv_start = max(0, ctx + 1 - window) if window else 0
+    outs, rows = [], []
+    for fused in (False, True):
+        cache, hist = _cache_with_history(dtype, 1, hkv, d, ctx + 1, fill, 70 + ctx)
+        fwd = vf.Forward(cache, heads)
+        o = torch.full((heads, d), float("nan"), device=DEV)
+        print(f"case dtype={dtype.label()} H={heads} Hkv={hkv} D={d} ctx={ctx} window={window} fused={fused}", flush=True)
+        if fused:
+            fwd.step_kv_write_attention(0, ctx, to_dev(q), to_dev(k_new), to_dev(v_new), o, kv_start=kv_start)
+        else:
+            fwd.step_kv_write(0, ctx, to_dev(k_new), to_dev(v_new))
+            fwd.run_scalar_attn(0, ctx, to_dev(q), o, kv_start=kv_start)
+        torch.cuda.synchronize()
+        off = cache.pos_offset_bytes(0, ctx)
+        rows.append((read_device(cache.k_ptr + off, hkv * d * esz).copy(), read_device(cache.v_ptr + off, hkv * d * esz).copy()))
+        outs.append(to_np(o).copy())
+        cache.destroy()
+    assert (rows[0][0] == rows[1][0]).all() and (rows[0][1] == rows[1][1]).all()
+    assert np.array_equal(outs[0], outs[1])
+    k_all, v_all = hist[0][0].copy(), hist[0][1].copy()
+    k_all[ctx], v_all[ctx] = k_new[0], v_new[0]
+    ke, ve = encode_np(k_all, dtype), encode_np(v_all, dtype)
+    assert (rows[1][0].view(ke.dtype) == ke[ctx].reshape(-1)).all()
+    ref = oracle.attn_decode_ref(q, ke.reshape(-1, hkv, d), ve.reshape(-1, hkv, d), int(dtype), heads, hkv, d, ctx + 1,
+                                 1.0 / np.sqrt(d), kv_start=kv_start)
+    assert np.abs(outs[1] - ref).max() < TOL[dtype]
+
+
 def test_config4_hd256_sliding_window_softcap_f16():
     # BASELINE config 4 geometry: 16/8/256, F16 KV, window 4096 at context 16384, soft-cap 50;
     # layer 0 sliding, layer 1 global

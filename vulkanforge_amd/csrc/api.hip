@@ -417,29 +417,29 @@ uint32_t vfkv_decode_tile_for(uint32_t span, uint32_t n_heads, uint32_t n_kv_hea
     return choose_tile(span, n_kv_heads, groups, 512u);
 }
 
-int vfkv_decode_attention(vfkv_cache* c, uint32_t layer, uint32_t kv_layer, uint32_t n_heads, const float* q, float* o,
-                          uint32_t position, uint32_t kv_start, float scale, float softcap, vfkv_workspace* ws,
-                          vfkv_stream stream) {
-    if (!c || !c->k || !c->v) return fail(VFKV_ERR_INVALID_ARG, "decode_attention: cache has no buffers");
-    if (!ws) return fail(VFKV_ERR_INVALID_ARG, "decode_attention: workspace is NULL");
-    if (!q || !o) return fail(VFKV_ERR_INVALID_ARG, "decode_attention: NULL buffer");
+static int decode_attention_impl(vfkv_cache* c, uint32_t layer, uint32_t kv_layer, uint32_t n_heads, const float* q, float* o,
+                                 uint32_t position, uint32_t kv_start, float scale, float softcap, vfkv_workspace* ws,
+                                 const float* k_new, const float* v_new, vfkv_stream stream, const char* who) {
+    if (!c || !c->k || !c->v) return fail(VFKV_ERR_INVALID_ARG, "%s: cache has no buffers", who);
+    if (!ws) return fail(VFKV_ERR_INVALID_ARG, "%s: workspace is NULL", who);
+    if (!q || !o) return fail(VFKV_ERR_INVALID_ARG, "%s: NULL buffer", who);
     if (layer >= c->n_layers || kv_layer >= c->n_layers)
-        return fail(VFKV_ERR_INVALID_ARG, "decode_attention: layer %u / kv_layer %u out of range", layer, kv_layer);
+        return fail(VFKV_ERR_INVALID_ARG, "%s: layer %u / kv_layer %u out of range", who, layer, kv_layer);
     if (position >= c->max_seq_len)
-        return fail(VFKV_ERR_INVALID_ARG, "decode_attention: position %u >= max_seq_len %u", position, c->max_seq_len);
-    if (!(softcap >= 0.f)) return fail(VFKV_ERR_INVALID_ARG, "decode_attention: softcap must be >= 0");
+        return fail(VFKV_ERR_INVALID_ARG, "%s: position %u >= max_seq_len %u", who, position, c->max_seq_len);
+    if (!(softcap >= 0.f)) return fail(VFKV_ERR_INVALID_ARG, "%s: softcap must be >= 0", who);
     const uint32_t hd = hd_for(c, layer), kvh = kvh_for(c, layer);
     int rc = check_attn_dims(n_heads, kvh, hd);
     if (rc != VFKV_OK) return rc;
     const uint32_t seq_len = position + 1u;
-    if (kv_start >= seq_len) return fail(VFKV_ERR_INVALID_ARG, "decode_attention: kv_start %u leaves no visible key (seq_len %u)", kv_start, seq_len);
+    if (kv_start >= seq_len) return fail(VFKV_ERR_INVALID_ARG, "%s: kv_start %u leaves no visible key (seq_len %u)", who, kv_start, seq_len);
     if (n_heads > ws->n_heads || hd > ws->head_dim)
-        return fail(VFKV_ERR_WORKSPACE, "decode_attention: workspace built for %u heads x %u dims, need %u x %u",
+        return fail(VFKV_ERR_WORKSPACE, "%s: workspace built for %u heads x %u dims, need %u x %u", who,
                     ws->n_heads, ws->head_dim, n_heads, hd);
     const uint32_t tile = vfkv_decode_tile_for(seq_len - kv_start, n_heads, kvh, hd, c->dtype);
     const uint32_t first = kv_start / tile;
     const uint32_t n_tiles = (seq_len + tile - 1u) / tile - first;
-    if (n_tiles > ws->max_tiles) return fail(VFKV_ERR_WORKSPACE, "decode_attention: %u tiles > workspace capacity %u", n_tiles, ws->max_tiles);
+    if (n_tiles > ws->max_tiles) return fail(VFKV_ERR_WORKSPACE, "%s: %u tiles > workspace capacity %u", who, n_tiles, ws->max_tiles);
     const uint64_t off = layer_off(c, kv_layer);
     vfkv::SplitLaunch L;
     L.q = q; L.k = (char*)c->k + off; L.v = (char*)c->v + off;
@@ -447,9 +447,34 @@ int vfkv_decode_attention(vfkv_cache* c, uint32_t layer, uint32_t kv_layer, uint
     L.dtype = c->dtype; L.n_heads = n_heads; L.n_kv_heads = kvh; L.head_dim = hd;
     L.seq_len = seq_len; L.kv_start = kv_start; L.tile = tile; L.tile_first = first; L.n_tiles = n_tiles;
     L.scale = scale; L.softcap = softcap;
+    if (k_new) {
+        L.k_new = k_new; L.v_new = v_new; L.append_pos = position;
+        if (!vfkv::split_appends(L)) {          // this shape's worker cannot write the row itself: append in its own launch
+            L.k_new = nullptr; L.v_new = nullptr;
+            rc = vfkv_kv_write(c, layer, position, 1, k_new, v_new, stream);
+            if (rc != VFKV_OK) return rc;
+        }
+    }
     VFKV_HIP(vfkv::launch_split(L, S(stream)));
     VFKV_HIP(vfkv::launch_reduce(ws->scratch_out, ws->scratch_max, ws->scratch_sum, o, n_heads, hd, n_tiles, S(stream)));
     return VFKV_OK;
+}
+
+int vfkv_decode_attention(vfkv_cache* c, uint32_t layer, uint32_t kv_layer, uint32_t n_heads, const float* q, float* o,
+                          uint32_t position, uint32_t kv_start, float scale, float softcap, vfkv_workspace* ws,
+                          vfkv_stream stream) {
+    return decode_attention_impl(c, layer, kv_layer, n_heads, q, o, position, kv_start, scale, softcap, ws, nullptr, nullptr,
+                                 stream, "decode_attention");
+}
+
+int vfkv_kv_write_decode_attention(vfkv_cache* c, uint32_t layer, uint32_t n_heads, const float* q, const float* k_src,
+                                   const float* v_src, float* o, uint32_t position, uint32_t kv_start, float scale,
+                                   float softcap, vfkv_workspace* ws, vfkv_stream stream) {
+    if (!k_src || !v_src) return fail(VFKV_ERR_INVALID_ARG, "kv_write_decode_attention: NULL source row");
+    if (c && layer < c->n_layers && (layer_off(c, layer) + (uint64_t)position * row_b(c, layer)) % 4u != 0u)
+        return fail(VFKV_ERR_ALIGNMENT, "kv_write_decode_attention: dst_byte_offset must be uint-aligned");
+    return decode_attention_impl(c, layer, layer, n_heads, q, o, position, kv_start, scale, softcap, ws, k_src, v_src, stream,
+                                 "kv_write_decode_attention");
 }
 
 // ---- prefill attention -------------------------------------------------------------------------------

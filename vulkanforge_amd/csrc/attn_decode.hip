@@ -32,6 +32,9 @@ struct SplitArgs {
     float* so;
     float* sm;
     float* ss;
+    const float* k_new;   // optional: one token row [n_kv_heads * D] f32 to append at row `append_pos` first (matrix-core worker)
+    const float* v_new;
+    uint32_t append_pos;
     uint32_t n_heads, n_kv_heads;
     uint32_t seq_len, kv_start;
     uint32_t tile, tile_first, n_tiles;
@@ -615,6 +618,18 @@ uint32_t split_tile_granule(uint32_t dtype, uint32_t D) {
     return (uint32_t)kRun;
 }
 
+// True when launch_split would write the token row (k_new, v_new) itself: the matrix-core worker with a single head
+// slice, where one workgroup per KV head owns the new row and can store it before anything reads it.
+bool split_appends(const SplitLaunch& L) {
+    if (!L.k_new || !L.v_new || L.n_kv_heads == 0u) return false;
+    const uint32_t g = L.n_heads / L.n_kv_heads;
+    const bool aligned = ((((uintptr_t)L.k) | ((uintptr_t)L.v) | ((uintptr_t)L.q) | ((uintptr_t)L.k_new) | ((uintptr_t)L.v_new)) & 15u) == 0u;
+    const uint64_t slab_bytes = (uint64_t)L.seq_len * L.n_kv_heads * L.head_dim * elem_size(L.dtype);
+    const bool mfma_shape = (L.dtype == kF8 || L.dtype == kF16) && (L.head_dim == 64u || L.head_dim == 128u || L.head_dim == 256u);
+    return aligned && slab_bytes < 0x7FFF0000ull && mfma_worker_enabled() && mfma_shape && g <= 8u &&
+           L.append_pos < L.seq_len && L.append_pos >= L.kv_start;
+}
+
 hipError_t launch_split(const SplitLaunch& L, hipStream_t stream) {
     if (L.dtype > kF8 || L.head_dim == 0u || L.head_dim > 512u) return hipErrorInvalidValue;
     if (L.n_tiles == 0u) return hipSuccess;
@@ -625,10 +640,15 @@ hipError_t launch_split(const SplitLaunch& L, hipStream_t stream) {
     a.seq_len = L.seq_len; a.kv_start = L.kv_start;
     a.tile = L.tile; a.tile_first = L.tile_first; a.n_tiles = L.n_tiles;
     a.scale = L.scale; a.softcap = L.softcap;
+    a.k_new = nullptr; a.v_new = nullptr; a.append_pos = 0u;
     const uint32_t g = L.n_heads / L.n_kv_heads;
     const bool aligned = ((((uintptr_t)L.k) | ((uintptr_t)L.v) | ((uintptr_t)L.q)) & 15u) == 0u;
     // the register-tiled worker addresses the slab with 32-bit byte offsets below 2 GiB
     const uint64_t slab_bytes = (uint64_t)L.seq_len * L.n_kv_heads * L.head_dim * elem_size(L.dtype);
+    if (L.k_new && L.v_new) {
+        if (!split_appends(L)) return hipErrorInvalidValue;      // the caller asked for a fused append this worker cannot do
+        a.k_new = L.k_new; a.v_new = L.v_new; a.append_pos = L.append_pos;
+    }
     if (aligned && slab_bytes < 0x7FFF0000ull && mfma_worker_enabled()) {
         if (L.dtype == kF8 && L.head_dim == 64u) return launch_split_mfma<kF8, 64, 64, 1>(a, g, stream);
         if (L.dtype == kF8 && L.head_dim == 128u) return launch_split_mfma<kF8, 128, VFKV_MFMA_RUN_F8, VFKV_MFMA_PF_F8>(a, g, stream);

@@ -91,6 +91,34 @@ __global__ __launch_bounds__(NW * 64) void split_mfma_kernel(SplitArgs a, uint32
         vraw[b][c] = __builtin_amdgcn_raw_buffer_load_b128(vrsrc, lane_voff, off + (uint32_t)(c * VROWS) * row_stride, 0);
     };
 
+    // ---- optional fused append (step_kv_write, executor/attention.rs:546): the workgroup whose tile holds the new
+    // position converts and stores this KV head's slice of the new K and V rows before anything reads them.  The
+    // stores are complete (vmcnt == 0) and the workgroup has met at the barrier before the first load is issued;
+    // the lines were not touched by this workgroup before, so the loads fetch them from L2, where the stores went.
+    if (a.k_new != nullptr && a.append_pos >= tile_base && a.append_pos < tile_end) {
+        constexpr int EPW = 4 / ES;                              // elements per 32-bit word of the cache
+        if (tid < D / EPW) {
+            const size_t src = (size_t)kvh * D + (size_t)tid * EPW;
+            const size_t dst = ((size_t)a.append_pos * a.n_kv_heads + kvh) * D * ES + (size_t)tid * 4;
+            uint32_t kw, vw;
+            if (DT == kF8) {
+                const float4 kf = *reinterpret_cast<const float4*>(a.k_new + src);
+                const float4 vf = *reinterpret_cast<const float4*>(a.v_new + src);
+                kw = pack4_e4m3(kf.x, kf.y, kf.z, kf.w);
+                vw = pack4_e4m3(vf.x, vf.y, vf.z, vf.w);
+            } else {
+                const float2 kf = *reinterpret_cast<const float2*>(a.k_new + src);
+                const float2 vf = *reinterpret_cast<const float2*>(a.v_new + src);
+                kw = f32_to_h16_bits(kf.x) | (f32_to_h16_bits(kf.y) << 16);
+                vw = f32_to_h16_bits(vf.x) | (f32_to_h16_bits(vf.y) << 16);
+            }
+            *reinterpret_cast<uint32_t*>(const_cast<uint8_t*>(a.k) + dst) = kw;
+            *reinterpret_cast<uint32_t*>(const_cast<uint8_t*>(a.v) + dst) = vw;
+        }
+        __builtin_amdgcn_s_waitcnt(0);
+        __syncthreads();
+    }
+
     // This wavefront's runs are r0, r0 + NW, ...; it walks them cyclically from a starting point that depends on the
     // KV head, so that the workgroups reading the same position rows are not all at the same rows at the same time.
     const uint32_t r0 = first_run + w;

@@ -124,6 +124,17 @@ class Forward:
 
     step_attention = run_scalar_attn  # executor/attention.rs:599-625
 
+    def step_kv_write_attention(self, layer: int, position: int, q, k_src, v_src, o, kv_start: int = 0,
+                                scale: float | None = None, softcap: float = 0.0, stream=None) -> None:
+        """step_kv_write + step_attention of one token (executor/attention.rs:546-625) as one call: where the
+        decode worker can, it writes the new rows itself and the append launch disappears."""
+        if scale is None:
+            hd = self.kv_cache.head_dim_for(layer)
+            scale = self.attn_scale if hd == self.kv_cache.config.head_dim else 1.0 / math.sqrt(hd)
+        _ffi.check(_ffi.lib().vfkv_kv_write_decode_attention(self.kv_cache.handle, layer, self.n_heads, _ptr(q),
+                                                             _ptr(k_src), _ptr(v_src), _ptr(o), position, kv_start,
+                                                             scale, softcap, self.workspace._h, _stream(stream)))
+
     # ---- prefill attention (runs.rs:933-1010, executor/attention.rs:2192-2390) ----
     @staticmethod
     def run_flash_attn_batch(q, k_layer, v_layer, kv_dtype, o, n_heads, n_kv_heads, head_dim, m, q_start, n_kv,

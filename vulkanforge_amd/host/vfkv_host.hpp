@@ -151,6 +151,13 @@ public:
     void step_attention(uint32_t layer, uint32_t position, const float* q, float* attn_out) {   // attention.rs:599-625
         run_scalar_attn(layer, position, q, attn_out, layer, 0);
     }
+    // step_kv_write + step_attention of one token (attention.rs:546-625) in one call; the decode worker writes the
+    // new rows itself where it can
+    void step_kv_write_attention(uint32_t layer, uint32_t position, const float* q, const float* k_src, const float* v_src,
+                                 float* attn_out, uint32_t kv_start = 0, float softcap = 0.f) {
+        check(vfkv_kv_write_decode_attention(kv_cache.handle(), layer, n_heads, q, k_src, v_src, attn_out, position, kv_start,
+                                             scale_for(layer), softcap, ws_, stream));
+    }
     // runs.rs:933-1010
     void run_flash_attn_batch(uint32_t layer, const float* q_buf, float* o_buf, uint32_t m, uint32_t q_start, uint32_t n_kv,
                               uint32_t kv_layer, uint32_t kv_start, float softcap = 0.f) {

@@ -265,6 +265,23 @@ def test_kv_write_attention_in_one_call_matches_the_two_calls(dtype, heads, hkv,
     assert np.abs(outs[1] - ref).max() < TOL[dtype]
 
 
+@pytest.mark.parametrize("dtype,heads,hkv,d,seq", [(vf.KvDtype.F8, 32, 8, 128, 200), (vf.KvDtype.F8, 16, 2, 256, 256),
+                                                  (vf.KvDtype.F16, 12, 4, 64, 129), (vf.KvDtype.F8, 40, 2, 128, 255)])
+def test_spans_of_one_tile_skip_the_merge_launch(dtype, heads, hkv, d, seq):
+    # up to 256 visible keys the convenience path uses one tile per KV head and the worker writes the output itself
+    fill = outlier_normal if dtype == vf.KvDtype.F8 else fp16_normal
+    cache, hist = _cache_with_history(dtype, 1, hkv, d, seq, fill, 90 + seq)
+    fwd = vf.Forward(cache, heads)
+    q = fp16_normal(rng(91), (heads, d))
+    o = torch.full((heads, d), float("nan"), device=DEV)
+    print(f"case dtype={dtype.label()} H={heads} Hkv={hkv} D={d} seq={seq}", flush=True)
+    fwd.run_scalar_attn(0, seq - 1, to_dev(q), o)
+    torch.cuda.synchronize()
+    ke, ve = (encode_np(x, dtype).reshape(seq, hkv, d) for x in hist[0])
+    ref = oracle.attn_decode_ref(q, ke, ve, int(dtype), heads, hkv, d, seq, 1.0 / np.sqrt(d))
+    assert np.abs(to_np(o) - ref).max() < TOL[dtype]
+
+
 def test_config4_hd256_sliding_window_softcap_f16():
     # BASELINE config 4 geometry: 16/8/256, F16 KV, window 4096 at context 16384, soft-cap 50;
     # layer 0 sliding, layer 1 global
@@ -311,7 +328,7 @@ def test_short_context_goes_through_the_same_path():
     fwd = vf.Forward(cache, heads)
     q = fp16_normal(rng(52), (heads, d))
     ke, ve = (encode_np(x, vf.KvDtype.F16).reshape(64, hkv, d) for x in hist[0])
-    for pos in (0, 1, 17, 63):
+    for pos in (0, 1, 17, 63):   # one tile: the worker writes the normalised output itself, no merge launch
         o = torch.full((heads, d), float("nan"), device=DEV)
         fwd.run_scalar_attn(0, pos, to_dev(q), o)
         torch.cuda.synchronize()

@@ -412,7 +412,12 @@ uint32_t vfkv_decode_tile_for(uint32_t span, uint32_t n_heads, uint32_t n_kv_hea
     // The matrix-core worker (1- and 2-byte caches, head_dim 64 / 128) runs best with one workgroup per CU and
     // serves up to 8 heads of a group per workgroup; the vector-ALU worker wants two and serves up to 4.
     const bool mfma = (kv_dtype == VFKV_F8E4M3 || kv_dtype == VFKV_F16) && (head_dim == 64u || head_dim == 128u || head_dim == 256u);
-    if (mfma) return choose_tile(span, n_kv_heads, (g + 7u) / 8u, 256u);
+    if (mfma) {
+        // short spans: one tile, so the worker writes the output itself and no merge launch follows
+        static const bool forced = getenv("VFKV_DECODE_TILE") != nullptr;
+        if (span <= 256u && !forced) return 256u;
+        return choose_tile(span, n_kv_heads, (g + 7u) / 8u, 256u);
+    }
     const uint32_t groups = (g % 4u == 0u) ? g / 4u : (g % 2u == 0u) ? g / 2u : g;
     return choose_tile(span, n_kv_heads, groups, 512u);
 }
@@ -454,6 +459,11 @@ static int decode_attention_impl(vfkv_cache* c, uint32_t layer, uint32_t kv_laye
             rc = vfkv_kv_write(c, layer, position, 1, k_new, v_new, stream);
             if (rc != VFKV_OK) return rc;
         }
+    }
+    if (vfkv::split_writes_output(L)) {         // one tile sees every key: the worker normalises and writes o itself
+        L.o_direct = o;
+        VFKV_HIP(vfkv::launch_split(L, S(stream)));
+        return VFKV_OK;
     }
     VFKV_HIP(vfkv::launch_split(L, S(stream)));
     VFKV_HIP(vfkv::launch_reduce(ws->scratch_out, ws->scratch_max, ws->scratch_sum, o, n_heads, hd, n_tiles, S(stream)));

@@ -32,6 +32,7 @@ struct SplitArgs {
     float* so;
     float* sm;
     float* ss;
+    float* o_direct;      // optional, single-tile launches of the matrix-core worker: final output [n_heads][D], no partials
     const float* k_new;   // optional: one token row [n_kv_heads * D] f32 to append at row `append_pos` first (matrix-core worker)
     const float* v_new;
     uint32_t append_pos;
@@ -630,6 +631,15 @@ bool split_appends(const SplitLaunch& L) {
            L.append_pos < L.seq_len && L.append_pos >= L.kv_start;
 }
 
+// True when a launch of one tile can write the normalised output itself (matrix-core worker shapes).
+bool split_writes_output(const SplitLaunch& L) {
+    if (L.n_tiles != 1u || L.n_kv_heads == 0u) return false;
+    const bool aligned = ((((uintptr_t)L.k) | ((uintptr_t)L.v) | ((uintptr_t)L.q)) & 15u) == 0u;
+    const uint64_t slab_bytes = (uint64_t)L.seq_len * L.n_kv_heads * L.head_dim * elem_size(L.dtype);
+    const bool mfma_shape = (L.dtype == kF8 || L.dtype == kF16) && (L.head_dim == 64u || L.head_dim == 128u || L.head_dim == 256u);
+    return aligned && slab_bytes < 0x7FFF0000ull && mfma_worker_enabled() && mfma_shape;
+}
+
 hipError_t launch_split(const SplitLaunch& L, hipStream_t stream) {
     if (L.dtype > kF8 || L.head_dim == 0u || L.head_dim > 512u) return hipErrorInvalidValue;
     if (L.n_tiles == 0u) return hipSuccess;
@@ -640,7 +650,11 @@ hipError_t launch_split(const SplitLaunch& L, hipStream_t stream) {
     a.seq_len = L.seq_len; a.kv_start = L.kv_start;
     a.tile = L.tile; a.tile_first = L.tile_first; a.n_tiles = L.n_tiles;
     a.scale = L.scale; a.softcap = L.softcap;
-    a.k_new = nullptr; a.v_new = nullptr; a.append_pos = 0u;
+    a.k_new = nullptr; a.v_new = nullptr; a.append_pos = 0u; a.o_direct = nullptr;
+    if (L.o_direct) {
+        if (!split_writes_output(L)) return hipErrorInvalidValue;
+        a.o_direct = L.o_direct;
+    }
     const uint32_t g = L.n_heads / L.n_kv_heads;
     const bool aligned = ((((uintptr_t)L.k) | ((uintptr_t)L.v) | ((uintptr_t)L.q)) & 15u) == 0u;
     // the register-tiled worker addresses the slab with 32-bit byte offsets below 2 GiB

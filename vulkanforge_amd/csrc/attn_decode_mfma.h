@@ -338,6 +338,12 @@ __global__ __launch_bounds__(NW * 64) void split_mfma_kernel(SplitArgs a, uint32
             o = fmaf(f, lds_o[(size_t)(ww * 8 + g) * D + d], o);
             l = fmaf(f, lds_l[ww][g], l);
         }
+        if (a.o_direct != nullptr) {
+            // a single tile covers every visible key (the reference's single-workgroup shader for seq <= 64,
+            // forward/runs.rs:776-821): the merge is a plain normalisation, done here, and no merge launch follows
+            a.o_direct[(size_t)(h0 + g) * D + d] = o / l;
+            continue;
+        }
         const size_t pidx = (size_t)(h0 + g) * a.n_tiles + jl;
         a.so[pidx * D + d] = o;
         if (d == 0) { a.sm[pidx] = M > -1e29f ? M * 0.693147180559945f : kMasked; a.ss[pidx] = l; }

@@ -28,11 +28,15 @@ struct SplitLaunch {
     const float* k_new = nullptr;
     const float* v_new = nullptr;
     uint32_t append_pos = 0;
+    // optional, launches of a single tile: final output [n_heads, head_dim]; the worker normalises itself and writes
+    // no partials (only when split_writes_output() is true)
+    float* o_direct = nullptr;
 };
 // Returns hipErrorInvalidValue when no kernel covers the shape (or when k_new / v_new are given although
 // split_appends() is false: then the caller appends the row with launch_kv_append and leaves them NULL).
 hipError_t launch_split(const SplitLaunch& a, hipStream_t stream);
 bool split_appends(const SplitLaunch& a);
+bool split_writes_output(const SplitLaunch& a);
 hipError_t launch_reduce(const float* scratch_out, const float* scratch_max, const float* scratch_sum, float* o,
                          uint32_t n_heads, uint32_t head_dim, uint32_t n_tiles, hipStream_t stream);
 // Smallest tile granule (keys) the split kernel for this shape works in; 0 if unsupported.

@@ -529,6 +529,31 @@ __global__ __launch_bounds__(kReduceThreads) void reduce_kernel(const float* __r
     }
 }
 
+// Few tiles (<= MAXT <= 64): one wavefront per (head, 64 output dimensions), no LDS and no barrier.  Lane j owns tile
+// j's max / sum and turns them into its merge weight; every lane also owns one output dimension and loads that
+// dimension of all partial outputs before the first reduction, so the kernel costs one memory round trip.
+template <int MAXT>
+__global__ __launch_bounds__(kWave) void reduce_direct_kernel(const float* __restrict__ so, const float* __restrict__ sm,
+                                                              const float* __restrict__ ss, float* __restrict__ o,
+                                                              uint32_t D, uint32_t n_tiles) {
+    const uint32_t h = blockIdx.y, lane = threadIdx.x;
+    const uint32_t d = blockIdx.x * kWave + lane;
+    const float* ho = so + (size_t)h * n_tiles * D + d;
+    float x[MAXT];
+#pragma unroll
+    for (int j = 0; j < MAXT; ++j) x[j] = ho[(size_t)((uint32_t)j < n_tiles ? j : 0) * D];
+    const float mj = lane < n_tiles ? sm[(size_t)h * n_tiles + lane] : kMasked;
+    const float sj = lane < n_tiles ? ss[(size_t)h * n_tiles + lane] : 0.f;
+    const float M = wave_max_uniform(mj);
+    const float wj = lane < n_tiles ? __expf(mj - M) : 0.f;
+    const float L = wave_sum_uniform(wj * sj);
+    float acc = 0.f;
+#pragma unroll
+    for (int j = 0; j < MAXT; ++j)
+        acc = fmaf(__builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, wj), j)), x[j], acc);
+    o[(size_t)h * D + d] = acc * (1.0f / L);
+}
+
 // scalar variant for head_dim not a multiple of 4 (or > 1024 threads' worth): one thread per d
 __global__ __launch_bounds__(kWave) void reduce_generic_kernel(const float* __restrict__ so,
                                                                const float* __restrict__ sm,
@@ -689,7 +714,11 @@ hipError_t launch_reduce(const float* so, const float* sm, const float* ss, floa
     if (n_heads == 0u || D == 0u || n_tiles == 0u) return hipErrorInvalidValue;
     const bool vec = (D % 4u == 0u) && (D / 4u <= (uint32_t)kReduceThreads) && n_tiles <= 8192u &&
                      ((((uintptr_t)so) & 15u) == 0u);
-    if (vec) {
+    if (n_tiles <= 64u && D % (uint32_t)kWave == 0u) {
+        const dim3 grid(D / kWave, n_heads);
+        if (n_tiles <= 32u) hipLaunchKernelGGL(reduce_direct_kernel<32>, grid, dim3(kWave), 0, stream, so, sm, ss, o, D, n_tiles);
+        else hipLaunchKernelGGL(reduce_direct_kernel<64>, grid, dim3(kWave), 0, stream, so, sm, ss, o, D, n_tiles);
+    } else if (vec) {
         const uint32_t d4n = D / 4u;
         const uint32_t parts = kReduceThreads / d4n;
         const size_t lds = ((size_t)parts * D + n_tiles) * sizeof(float);

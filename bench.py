@@ -80,6 +80,11 @@ def fill_cache(torch, vf, fwd, wl, n_tokens, seed, outliers):
     torch.cuda.synchronize()
 
 
+# The V buffer starts 256 bytes into its allocation, as in the caches vfkv_cache_create allocates itself: K and V
+# of one row then differ in address bits 7-8 (see the comment there).
+V_SKEW = int(os.environ.get("VFKV_BENCH_V_SKEW", "256"))
+
+
 def time_steps(torch, step, args):
     """W untimed steps, then exactly K timed steps between two device synchronisations.  One step's
     launches are captured once into a HIP graph and replayed, so the host's per-launch cost (Python
@@ -119,7 +124,7 @@ def bench_decode(args, wl):
     es = wl.dtype.element_size()
     nbytes = L * max_seq * Hkv * D * es
     kbuf = torch.empty(nbytes, dtype=torch.uint8, device=dev)
-    vbuf = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+    vbuf = torch.empty(nbytes + V_SKEW, dtype=torch.uint8, device=dev)[V_SKEW:]
     cache = vf.KvCache(vf.KvCacheConfig(L, Hkv, D, max_seq, dtype=wl.dtype), k_buffer=kbuf.data_ptr(),
                        v_buffer=vbuf.data_ptr())
     fwd = vf.Forward(cache, H)
@@ -262,7 +267,7 @@ def bench_prefill(args, wl):
     es = wl.dtype.element_size()
     per_layer = max_seq * Hkv * D * es
     kbuf = torch.empty(L * per_layer, dtype=torch.uint8, device=dev)
-    vbuf = torch.empty(L * per_layer, dtype=torch.uint8, device=dev)
+    vbuf = torch.empty(L * per_layer + V_SKEW, dtype=torch.uint8, device=dev)[V_SKEW:]
     cache = vf.KvCache(vf.KvCacheConfig(L, Hkv, D, max_seq, dtype=wl.dtype), k_buffer=kbuf.data_ptr(),
                        v_buffer=vbuf.data_ptr())
     fwd = vf.Forward(cache, H)

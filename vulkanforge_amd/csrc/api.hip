@@ -460,6 +460,9 @@ static int decode_attention_impl(vfkv_cache* c, uint32_t layer, uint32_t kv_laye
     L.dtype = c->dtype; L.n_heads = n_heads; L.n_kv_heads = kvh; L.head_dim = hd;
     L.seq_len = seq_len; L.kv_start = kv_start; L.tile = tile; L.tile_first = first; L.n_tiles = n_tiles;
     L.scale = scale; L.softcap = softcap;
+    // the partials stay inside the workspace, so they need not correspond to tiles (VFKV_DECODE_INTERLEAVE=0: they do)
+    static const bool interleave = [] { const char* e = getenv("VFKV_DECODE_INTERLEAVE"); return !(e && e[0] == '0'); }();
+    L.interleave = interleave;
     if (k_new) {
         L.k_new = k_new; L.v_new = v_new; L.append_pos = position;
         if (!vfkv::split_appends(L)) {          // this shape's worker cannot write the row itself: append in its own launch

@@ -39,6 +39,8 @@ struct SplitArgs {
     uint32_t n_heads, n_kv_heads;
     uint32_t seq_len, kv_start;
     uint32_t tile, tile_first, n_tiles;
+    uint32_t group;          // n_heads / n_kv_heads
+    uint32_t interleave;     // matrix-core worker: deal the runs of the launched span round-robin instead of by tile
     float scale, softcap;
 };
 
@@ -671,11 +673,12 @@ hipError_t launch_split(const SplitLaunch& L, hipStream_t stream) {
     SplitArgs a;
     a.q = L.q; a.k = (const uint8_t*)L.k; a.v = (const uint8_t*)L.v;
     a.so = L.scratch_out; a.sm = L.scratch_max; a.ss = L.scratch_sum;
-    a.n_heads = L.n_heads; a.n_kv_heads = L.n_kv_heads;
+    a.n_heads = L.n_heads; a.n_kv_heads = L.n_kv_heads; a.group = L.n_heads / L.n_kv_heads;
     a.seq_len = L.seq_len; a.kv_start = L.kv_start;
     a.tile = L.tile; a.tile_first = L.tile_first; a.n_tiles = L.n_tiles;
     a.scale = L.scale; a.softcap = L.softcap;
     a.k_new = nullptr; a.v_new = nullptr; a.append_pos = 0u; a.o_direct = nullptr;
+    a.interleave = L.interleave ? 1u : 0u;
     if (L.o_direct) {
         if (!split_writes_output(L)) return hipErrorInvalidValue;
         a.o_direct = L.o_direct;

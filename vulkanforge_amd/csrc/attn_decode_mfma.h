@@ -55,12 +55,18 @@ __global__ __launch_bounds__(NW * 64) void split_mfma_kernel(SplitArgs a, uint32
     const int col = n16 & 7;
     const bool is_lo = n16 >= 8;
     const uint32_t kvh = blockIdx.x, jl = blockIdx.y;     // KV head fastest: the workgroups of one tile start together
-    const uint32_t g_all = a.n_heads / a.n_kv_heads;
+    const uint32_t g_all = a.group;                        // n_heads / n_kv_heads, divided on the host
     const uint32_t hz = blockIdx.z * gt;
     const uint32_t gcount = g_all - hz < gt ? g_all - hz : gt;
     const uint32_t h0 = kvh * g_all + hz;
-    const uint32_t tile_base = (a.tile_first + jl) * a.tile;
-    uint32_t tile_end = tile_base + a.tile; if (tile_end > a.seq_len) tile_end = a.seq_len;
+    // Two ways to hand the visible rows to the workgroups.  Contiguous: workgroup jl owns tile jl (the reference's
+    // split, partial jl = tile jl).  Interleaved (a.interleave): the rows from the first launched tile to seq_len are
+    // one sequence of runs dealt round-robin to all wavefronts of the KV head, so at any moment the whole chip reads
+    // one narrow band of position rows front to back -- measurably faster than n_tiles separate streams -- and the
+    // partial of workgroup jl covers a comb of runs (the merge does not care which rows a partial covers).
+    const bool il = a.interleave != 0u;
+    const uint32_t tile_base = il ? a.tile_first * a.tile : (a.tile_first + jl) * a.tile;
+    uint32_t tile_end = tile_base + a.tile; if (il || tile_end > a.seq_len) tile_end = a.seq_len;
     const uint32_t lo = tile_base > a.kv_start ? tile_base : a.kv_start;
 
     const uint32_t row_stride = a.n_kv_heads * D * ES;
@@ -95,7 +101,11 @@ __global__ __launch_bounds__(NW * 64) void split_mfma_kernel(SplitArgs a, uint32
     // position converts and stores this KV head's slice of the new K and V rows before anything reads them.  The
     // stores are complete (vmcnt == 0) and the workgroup has met at the barrier before the first load is issued;
     // the lines were not touched by this workgroup before, so the loads fetch them from L2, where the stores went.
-    if (a.k_new != nullptr && a.append_pos >= tile_base && a.append_pos < tile_end) {
+    bool owns_new_row = false;
+    if (a.k_new != nullptr)
+        owns_new_row = il ? ((((a.append_pos - tile_base) / RUN - first_run) / NW) % a.n_tiles == jl)
+                          : (a.append_pos >= tile_base && a.append_pos < tile_end);
+    if (owns_new_row) {
         constexpr int EPW = 4 / ES;                              // elements per 32-bit word of the cache
         if (tid < D / EPW) {
             const size_t src = (size_t)kvh * D + (size_t)tid * EPW;
@@ -119,16 +129,22 @@ __global__ __launch_bounds__(NW * 64) void split_mfma_kernel(SplitArgs a, uint32
         __syncthreads();
     }
 
-    // This wavefront's runs are r0, r0 + NW, ...; it walks them cyclically from a starting point that depends on the
-    // KV head, so that the workgroups reading the same position rows are not all at the same rows at the same time.
-    const uint32_t r0 = first_run + w;
-    const uint32_t n_mine = (lo < tile_end && r0 < n_runs) ? (n_runs - r0 + NW - 1) / NW : 0u;
-    const bool active = n_mine != 0u;
-    const uint32_t rot = active ? (kvh * 3u) % n_mine : 0u;
+    // This wavefront's runs are r0, r0 + rs, ...  In a contiguous tile it walks them cyclically from a starting point
+    // that depends on the KV head, so that the workgroups reading the same position rows are not all at the same rows
+    // at the same time (with separate streams per tile that helps; the interleaved walk is better off without).
+    // (No division by a run-time value on the way to the first load: the rotation is taken modulo the largest power
+    // of two that fits, and the interleaved walk needs no count of its runs.)
+    const uint32_t rs = il ? NW * a.n_tiles : NW;                     // distance between two runs of a wavefront
+    const uint32_t r0 = first_run + (il ? jl * NW : 0u) + w;
+    const bool active = lo < tile_end && r0 < n_runs;
+    const uint32_t n_cyc = (active && !il) ? (n_runs - r0 + NW - 1) / NW : 0u;   // runs walked cyclically (contiguous tile)
+    const uint32_t rot = n_cyc != 0u ? (kvh * 3u) & ((1u << (31 - __builtin_clz(n_cyc))) - 1u) : 0u;
     auto nth_run = [&](uint32_t i) -> uint32_t {   // i-th run of this wavefront; n_runs (= none) past the last
-        if (i >= n_mine) return n_runs;
+        if (!active) return n_runs;
+        if (il) { const uint32_t r = r0 + i * rs; return r < n_runs ? r : n_runs; }
+        if (i >= n_cyc) return n_runs;
         uint32_t ii = i + rot;
-        if (ii >= n_mine) ii -= n_mine;
+        if (ii >= n_cyc) ii -= n_cyc;
         return r0 + ii * NW;
     };
     const uint32_t off0 = run_off(nth_run(0));
@@ -189,11 +205,11 @@ __global__ __launch_bounds__(NW * 64) void split_mfma_kernel(SplitArgs a, uint32
     _Float16* const vb = &vlds[w][0];
 
     if (active) {
-        for (uint32_t it = 0; it < n_mine; it += PF) {
+        for (uint32_t it = 0; nth_run(it) < n_runs; it += PF) {
 #pragma unroll
           for (int b = 0; b < PF; ++b) {
-            if (it + b >= n_mine) break;                                 // wavefront-uniform
             const uint32_t rr = nth_run(it + b);
+            if (rr >= n_runs) break;                                     // wavefront-uniform
             const uint32_t noff = run_off(nth_run(it + b + PF));
             const uint32_t rb = tile_base + rr * RUN;
             // ---------------- S^T = K Q^T ----------------

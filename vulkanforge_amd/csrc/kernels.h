@@ -31,6 +31,9 @@ struct SplitLaunch {
     // optional, launches of a single tile: final output [n_heads, head_dim]; the worker normalises itself and writes
     // no partials (only when split_writes_output() is true)
     float* o_direct = nullptr;
+    // partial j need not be tile j: the matrix-core worker then deals the rows of the launched tiles to its
+    // workgroups in interleaved runs (other workers ignore the flag); the merge is the same either way
+    bool interleave = false;
 };
 // Returns hipErrorInvalidValue when no kernel covers the shape (or when k_new / v_new are given although
 // split_appends() is false: then the caller appends the row with launch_kv_append and leaves them NULL).

@@ -471,7 +471,7 @@ static int decode_attention_impl(vfkv_cache* c, uint32_t layer, uint32_t kv_laye
             if (rc != VFKV_OK) return rc;
         }
     }
-    if (vfkv::split_writes_output(L)) {         // one tile sees every key: the worker normalises and writes o itself
+    if (vfkv::split_writes_output(L) && ((uintptr_t)o & 15u) == 0u) {   // one tile sees every key: the worker normalises and writes o itself
         L.o_direct = o;
         VFKV_HIP(vfkv::launch_split(L, S(stream)));
         return VFKV_OK;

@@ -651,7 +651,8 @@ uint32_t split_tile_granule(uint32_t dtype, uint32_t D) {
 bool split_appends(const SplitLaunch& L) {
     if (!L.k_new || !L.v_new || L.n_kv_heads == 0u) return false;
     const uint32_t g = L.n_heads / L.n_kv_heads;
-    const bool aligned = ((((uintptr_t)L.k) | ((uintptr_t)L.v) | ((uintptr_t)L.q) | ((uintptr_t)L.k_new) | ((uintptr_t)L.v_new)) & 15u) == 0u;
+    const bool aligned = ((((uintptr_t)L.k) | ((uintptr_t)L.v) | ((uintptr_t)L.q) | ((uintptr_t)L.k_new) | ((uintptr_t)L.v_new) |
+                           ((uintptr_t)L.scratch_out)) & 15u) == 0u;
     const uint64_t slab_bytes = (uint64_t)L.seq_len * L.n_kv_heads * L.head_dim * elem_size(L.dtype);
     const bool mfma_shape = (L.dtype == kF8 || L.dtype == kF16) && (L.head_dim == 64u || L.head_dim == 128u || L.head_dim == 256u);
     return aligned && slab_bytes < 0x7FFF0000ull && mfma_worker_enabled() && mfma_shape && g <= 8u &&
@@ -661,7 +662,7 @@ bool split_appends(const SplitLaunch& L) {
 // True when a launch of one tile can write the normalised output itself (matrix-core worker shapes).
 bool split_writes_output(const SplitLaunch& L) {
     if (L.n_tiles != 1u || L.n_kv_heads == 0u) return false;
-    const bool aligned = ((((uintptr_t)L.k) | ((uintptr_t)L.v) | ((uintptr_t)L.q)) & 15u) == 0u;
+    const bool aligned = ((((uintptr_t)L.k) | ((uintptr_t)L.v) | ((uintptr_t)L.q) | ((uintptr_t)L.scratch_out)) & 15u) == 0u;
     const uint64_t slab_bytes = (uint64_t)L.seq_len * L.n_kv_heads * L.head_dim * elem_size(L.dtype);
     const bool mfma_shape = (L.dtype == kF8 || L.dtype == kF16) && (L.head_dim == 64u || L.head_dim == 128u || L.head_dim == 256u);
     return aligned && slab_bytes < 0x7FFF0000ull && mfma_worker_enabled() && mfma_shape;
@@ -680,7 +681,7 @@ hipError_t launch_split(const SplitLaunch& L, hipStream_t stream) {
     a.k_new = nullptr; a.v_new = nullptr; a.append_pos = 0u; a.o_direct = nullptr;
     a.interleave = L.interleave ? 1u : 0u;
     if (L.o_direct) {
-        if (!split_writes_output(L)) return hipErrorInvalidValue;
+        if (!split_writes_output(L) || ((uintptr_t)L.o_direct & 15u) != 0u) return hipErrorInvalidValue;
         a.o_direct = L.o_direct;
     }
     const uint32_t g = L.n_heads / L.n_kv_heads;
@@ -691,7 +692,9 @@ hipError_t launch_split(const SplitLaunch& L, hipStream_t stream) {
         if (!split_appends(L)) return hipErrorInvalidValue;      // the caller asked for a fused append this worker cannot do
         a.k_new = L.k_new; a.v_new = L.v_new; a.append_pos = L.append_pos;
     }
-    if (aligned && slab_bytes < 0x7FFF0000ull && mfma_worker_enabled()) {
+    // the matrix-core worker also stores its partials (or the output) 16 bytes at a time
+    const bool out_aligned = ((((uintptr_t)L.scratch_out) | ((uintptr_t)L.o_direct)) & 15u) == 0u;
+    if (aligned && out_aligned && slab_bytes < 0x7FFF0000ull && mfma_worker_enabled()) {
         if (L.dtype == kF8 && L.head_dim == 64u) return launch_split_mfma<kF8, 64, 64, 1>(a, g, stream);
         if (L.dtype == kF8 && L.head_dim == 128u) return launch_split_mfma<kF8, 128, VFKV_MFMA_RUN_F8, VFKV_MFMA_PF_F8>(a, g, stream);
         if (L.dtype == kF16 && L.head_dim == 64u) return launch_split_mfma<kF16, 64, 64, 1>(a, g, stream);

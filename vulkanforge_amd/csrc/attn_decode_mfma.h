@@ -43,7 +43,7 @@ __global__ __launch_bounds__(NW * 64) void split_mfma_kernel(SplitArgs a, uint32
     constexpr int VLD = RUN * VCHUNK_ROW / 64;   // V loads per lane per run
     constexpr int VROWS = 64 / VCHUNK_ROW;       // rows covered by one V load of the wavefront
     static_assert(D % 32 == 0 && SEGB % 16 == 0 && RUN % 32 == 0 && VCHUNK_ROW <= 64 && VLD >= 1, "unsupported shape");
-    static_assert(NW * RUN * VPITCH * 2 >= NW * 8 * D * 4, "merge buffer must fit in the V staging area");
+    static_assert(NW * RUN * VPITCH * 2 >= NW * (D / 16) * 64 * 16, "merge buffer must fit in the V staging area");
 
     __shared__ __attribute__((aligned(16))) _Float16 vlds[NW][RUN * VPITCH];
     __shared__ float lds_m[NW][8], lds_l[NW][8];
@@ -328,41 +328,51 @@ __global__ __launch_bounds__(NW * 64) void split_mfma_kernel(SplitArgs a, uint32
     }
 
     // ---------------- wavefront totals, then the workgroup merge through LDS ----------------
+    // Every wavefront parks its accumulators in LDS in register order (lane-major: conflict-free 16-byte accesses),
+    // then wavefront w merges the d-tiles w, w + NW, ... of all wavefronts and stores them straight from registers.
     l_run = xor32_sum(xor16_sum(l_run));
 #pragma unroll
     for (int dt = 0; dt < DTILES; ++dt)
 #pragma unroll
         for (int i = 0; i < 4; ++i) { const float y = oacc[dt][i]; oacc[dt][i] = y + dpp_f<kDppRor8>(y); }
     __syncthreads();                                   // every wavefront is done with its V staging area
-    float* lds_o = reinterpret_cast<float*>(&vlds[0][0]);     // [NW][8][D]
-    if (!is_lo) {
+    float4_t* const slot = reinterpret_cast<float4_t*>(&vlds[0][0]);     // [NW][DTILES][64 lanes]
 #pragma unroll
-        for (int dt = 0; dt < DTILES; ++dt)
-            *reinterpret_cast<float4_t*>(lds_o + (size_t)(w * 8 + col) * D + dt * 16 + kg * 4) = oacc[dt];
-        if (kg == 0) { lds_m[w][col] = m_run; lds_l[w][col] = l_run; }
-    }
+    for (int dt = 0; dt < DTILES; ++dt) slot[(w * DTILES + dt) * 64 + lane] = oacc[dt];
+    if (kg == 0 && !is_lo) { lds_m[w][col] = m_run; lds_l[w][col] = l_run; }
     __syncthreads();
-    for (int idx = tid; idx < (int)gcount * D; idx += NW * 64) {
-        const int g = idx / D, d = idx - g * D;
-        float M = lds_m[0][g];
+    float fw[NW];
+    float M = lds_m[0][col];
 #pragma unroll
-        for (int ww = 1; ww < NW; ++ww) M = fmaxf(M, lds_m[ww][g]);
-        float o = 0.f, l = 0.f;
+    for (int ww = 1; ww < NW; ++ww) M = fmaxf(M, lds_m[ww][col]);
+    float l = 0.f;
 #pragma unroll
-        for (int ww = 0; ww < NW; ++ww) {
-            const float f = __builtin_amdgcn_exp2f(lds_m[ww][g] - M);
-            o = fmaf(f, lds_o[(size_t)(ww * 8 + g) * D + d], o);
-            l = fmaf(f, lds_l[ww][g], l);
-        }
+    for (int ww = 0; ww < NW; ++ww) {
+        fw[ww] = __builtin_amdgcn_exp2f(lds_m[ww][col] - M);
+        l = fmaf(fw[ww], lds_l[ww][col], l);
+    }
+    const bool writer = !is_lo && (uint32_t)col < gcount;
+    const size_t pidx = (size_t)(h0 + col) * a.n_tiles + jl;
+    const float inv_l = a.o_direct != nullptr ? 1.0f / l : 1.0f;
+#pragma unroll
+    for (int dt0 = 0; dt0 < DTILES; dt0 += NW) {
+        const int dt = dt0 + w;
+        if (dt >= DTILES) break;                       // wavefront-uniform (only when DTILES < NW)
+        float4_t o = float4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int ww = 0; ww < NW; ++ww) o += fw[ww] * slot[(ww * DTILES + dt) * 64 + lane];
+        if (!writer) continue;
         if (a.o_direct != nullptr) {
             // a single tile covers every visible key (the reference's single-workgroup shader for seq <= 64,
             // forward/runs.rs:776-821): the merge is a plain normalisation, done here, and no merge launch follows
-            a.o_direct[(size_t)(h0 + g) * D + d] = o / l;
-            continue;
+            *reinterpret_cast<float4_t*>(a.o_direct + (size_t)(h0 + col) * D + dt * 16 + kg * 4) = o * inv_l;
+        } else {
+            *reinterpret_cast<float4_t*>(a.so + pidx * D + dt * 16 + kg * 4) = o;
         }
-        const size_t pidx = (size_t)(h0 + g) * a.n_tiles + jl;
-        a.so[pidx * D + d] = o;
-        if (d == 0) { a.sm[pidx] = M > -1e29f ? M * 0.693147180559945f : kMasked; a.ss[pidx] = l; }
+    }
+    if (writer && w == 0 && kg == 0 && a.o_direct == nullptr) {
+        a.sm[pidx] = M > -1e29f ? M * 0.693147180559945f : kMasked;
+        a.ss[pidx] = l;
     }
 }
 

@@ -341,34 +341,44 @@ __global__ __launch_bounds__(NW * 64) void split_mfma_kernel(SplitArgs a, uint32
     for (int dt = 0; dt < DTILES; ++dt) slot[(w * DTILES + dt) * 64 + lane] = oacc[dt];
     if (kg == 0 && !is_lo) { lds_m[w][col] = m_run; lds_l[w][col] = l_run; }
     __syncthreads();
-    float fw[NW];
-    float M = lds_m[0][col];
+    // all LDS reads of the merge are issued before the first use, so their latencies overlap
+    constexpr int MT = DTILES / NW;                    // d-tiles merged and stored by each wavefront
+    static_assert(DTILES % NW == 0, "d-tiles must divide evenly among the wavefronts");
+    float mw[NW], lw[NW];
+    float4_t part[MT][NW];
 #pragma unroll
-    for (int ww = 1; ww < NW; ++ww) M = fmaxf(M, lds_m[ww][col]);
+    for (int ww = 0; ww < NW; ++ww) { mw[ww] = lds_m[ww][col]; lw[ww] = lds_l[ww][col]; }
+#pragma unroll
+    for (int t = 0; t < MT; ++t)
+#pragma unroll
+        for (int ww = 0; ww < NW; ++ww) part[t][ww] = slot[(ww * DTILES + t * NW + w) * 64 + lane];
+    float M = mw[0];
+#pragma unroll
+    for (int ww = 1; ww < NW; ++ww) M = fmaxf(M, mw[ww]);
+    float fw[NW];
     float l = 0.f;
 #pragma unroll
     for (int ww = 0; ww < NW; ++ww) {
-        fw[ww] = __builtin_amdgcn_exp2f(lds_m[ww][col] - M);
-        l = fmaf(fw[ww], lds_l[ww][col], l);
+        fw[ww] = __builtin_amdgcn_exp2f(mw[ww] - M);
+        l = fmaf(fw[ww], lw[ww], l);
     }
     const bool writer = !is_lo && (uint32_t)col < gcount;
     const size_t pidx = (size_t)(h0 + col) * a.n_tiles + jl;
-    const float inv_l = a.o_direct != nullptr ? 1.0f / l : 1.0f;
+    // a single tile covers every visible key (the reference's single-workgroup shader for seq <= 64,
+    // forward/runs.rs:776-821): the merge is a plain normalisation, done here, and no merge launch follows
+    const bool direct = a.o_direct != nullptr;
+    const float inv_l = direct ? __builtin_amdgcn_rcpf(l) : 1.0f;
+    float* const obase = direct ? a.o_direct + (size_t)(h0 + col) * D : a.so + pidx * D;
 #pragma unroll
-    for (int dt0 = 0; dt0 < DTILES; dt0 += NW) {
-        const int dt = dt0 + w;
-        if (dt >= DTILES) break;                       // wavefront-uniform (only when DTILES < NW)
-        float4_t o = float4_t{0.f, 0.f, 0.f, 0.f};
+    for (int t = 0; t < MT; ++t) {
+        float4_t o = fw[0] * part[t][0];
 #pragma unroll
-        for (int ww = 0; ww < NW; ++ww) o += fw[ww] * slot[(ww * DTILES + dt) * 64 + lane];
-        if (!writer) continue;
-        if (a.o_direct != nullptr) {
-            // a single tile covers every visible key (the reference's single-workgroup shader for seq <= 64,
-            // forward/runs.rs:776-821): the merge is a plain normalisation, done here, and no merge launch follows
-            *reinterpret_cast<float4_t*>(a.o_direct + (size_t)(h0 + col) * D + dt * 16 + kg * 4) = o * inv_l;
-        } else {
-            *reinterpret_cast<float4_t*>(a.so + pidx * D + dt * 16 + kg * 4) = o;
+        for (int ww = 1; ww < NW; ++ww) o += fw[ww] * part[t][ww];
+        if (direct) {                                  // one Newton step brings the reciprocal to f32 accuracy
+            const float r = inv_l * (2.0f - l * inv_l);
+            o *= r;
         }
+        if (writer) *reinterpret_cast<float4_t*>(obase + (t * NW + w) * 16 + kg * 4) = o;
     }
     if (writer && w == 0 && kg == 0 && a.o_direct == nullptr) {
         a.sm[pidx] = M > -1e29f ? M * 0.693147180559945f : kMasked;

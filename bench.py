@@ -35,7 +35,7 @@ MFMA_F16_PEAK_TFLOPS = 2500.0
 # (two runs) and scaled by what the same counters read for a plain 64 MiB device copy
 # (FETCH_SIZE x 1.9991, WRITE_SIZE x 1.0 to KiB).  Only the workloads that were profiled have an entry.
 MEASURED_TRAFFIC_BYTES = {
-    "decode_fp8_32k_32layers": (65604 + 520) * 1024,
+    "decode_fp8_32k_32layers": (65635 + 520) * 1024,
     "prefill_fp8_512x4608_32layers": (81365 + 8192) * 1024,
 }
 
@@ -171,7 +171,7 @@ def bench_decode(args, wl):
             klay = cache.k_ptr + cache.layer_offset_bytes(layer)
             vlay = cache.v_ptr + cache.layer_offset_bytes(layer)
             fwd.run_flash_attn_split(q[layer], klay, vlay, wl.dtype, so, sm, ss, H, Hkv, D, wl.context, scale,
-                                     kv_start=starts[layer], tile=tile, softcap=wl.softcap)
+                                     kv_start=starts[layer], tile=tile, softcap=wl.softcap, interleaved=True)
 
     run_split = split_only
     if not args.no_graph:

@@ -160,6 +160,16 @@ int vfkv_flash_attn_split(const float* q, const void* k_layer, const void* v_lay
                           const vfkv_split_params* p, uint32_t tile, float softcap,
                           vfkv_stream stream);
 
+/* Same arguments and the same number of partials as vfkv_flash_attn_split, for callers that only ever
+ * hand the partials to vfkv_flash_attn_reduce: partial j is then not tile j.  Where the matrix-core
+ * worker serves the shape, the rows are dealt to the n_tiles workgroups in interleaved runs (what
+ * vfkv_decode_attention launches); elsewhere this is vfkv_flash_attn_split.  The merged output is the
+ * same either way (forward/runs.rs:1463-1571 as a whole; no single counterpart in the reference). */
+int vfkv_flash_attn_split_interleaved(const float* q, const void* k_layer, const void* v_layer,
+                                      uint32_t kv_dtype, float* scratch_out, float* scratch_max,
+                                      float* scratch_sum, const vfkv_split_params* p, uint32_t tile,
+                                      float softcap, vfkv_stream stream);
+
 /* Forward::run_flash_attn_split_reduce, reducer half (forward/runs.rs:1543-1571) +
  * flash_attn_reduce.comp:35-81 (FlashAttnReducePushConstants, pipeline.rs:573-580). */
 int vfkv_flash_attn_reduce(const float* scratch_out, const float* scratch_max,

@@ -61,7 +61,7 @@ def read_device(ptr, nbytes):
 
 
 def gpu_split_reduce(q, k_enc, v_enc, dtype, H, Hkv, D, seq, scale, tile=64, kv_start=0, softcap=0.0,
-                     poison=True):
+                     poison=True, interleaved=False):
     """Runs vfkv_flash_attn_split + vfkv_flash_attn_reduce; returns (o, scratch_out, max, sum)."""
     n_tiles = (seq + tile - 1) // tile
     fill = float("nan") if poison else 0.0
@@ -71,7 +71,7 @@ def gpu_split_reduce(q, k_enc, v_enc, dtype, H, Hkv, D, seq, scale, tile=64, kv_
     o = torch.full((H, D), fill, device=DEV, dtype=torch.float32)
     qd, kd, vd = to_dev(q), to_dev(k_enc), to_dev(v_enc)
     nt = vf.Forward.run_flash_attn_split(qd, kd, vd, dtype, so, sm, ss, H, Hkv, D, seq, scale, kv_start=kv_start,
-                                         tile=tile, softcap=softcap)
+                                         tile=tile, softcap=softcap, interleaved=interleaved)
     assert nt == n_tiles
     vf.Forward.run_flash_attn_reduce(so, sm, ss, o, H, D, n_tiles)
     torch.cuda.synchronize()

@@ -104,6 +104,30 @@ def test_split_reduce_matches_oracle(dtype, heads, hkv, d, seq, tile, kv_start, 
         assert (sm[:, :dead] == np.float32(-1e30)).all() and (ss[:, :dead] == 0).all() and (so[:, :dead] == 0).all()
 
 
+@pytest.mark.parametrize("dtype,heads,hkv,d,seq,tile,kv_start,cap", CASES)
+def test_interleaved_split_reduce_matches_oracle(dtype, heads, hkv, d, seq, tile, kv_start, cap):
+    # vfkv_flash_attn_split_interleaved: the partials are combs of rows rather than tiles, so only the merged
+    # output is compared; the same launch with contiguous tiles must agree to rounding
+    r = rng(hash((int(dtype), heads, hkv, d, seq, tile, 7)) % (1 << 31))
+    q = fp16_normal(r, (heads, d))
+    kf = outlier_normal(r, (seq, hkv, d)) if dtype == vf.KvDtype.F8 else fp16_normal(r, (seq, hkv, d))
+    vfl = outlier_normal(r, (seq, hkv, d)) if dtype == vf.KvDtype.F8 else fp16_normal(r, (seq, hkv, d))
+    k, v = encode_np(kf, dtype), encode_np(vfl, dtype)
+    scale = float(1.0 / np.sqrt(d))
+    print(f"case interleaved dtype={dtype.label()} H={heads} Hkv={hkv} D={d} seq={seq} tile={tile} "
+          f"kv_start={kv_start} cap={cap}", flush=True)
+    o, so, sm, ss = gpu_split_reduce(q, k, v, dtype, heads, hkv, d, seq, scale, tile=tile, kv_start=kv_start,
+                                     softcap=cap, interleaved=True)
+    o_tiles, *_ = gpu_split_reduce(q, k, v, dtype, heads, hkv, d, seq, scale, tile=tile, kv_start=kv_start,
+                                   softcap=cap)
+    ref = oracle.attn_decode_ref(q, k, v, int(dtype), heads, hkv, d, seq, scale, kv_start=kv_start, softcap=cap)
+    assert np.isfinite(o).all() and np.isfinite(so).all() and np.isfinite(sm).all() and np.isfinite(ss).all()
+    err = np.abs(o - ref).max()
+    assert err < TOL[dtype], err
+    assert err < TIGHT * max(1.0, np.abs(ref).max()), err
+    assert np.abs(o - o_tiles).max() < TIGHT * max(1.0, np.abs(ref).max())
+
+
 def test_tile_invariance_and_linearity_full_size_fp8():
     # size-independent properties at the benchmark's largest single-layer shape (32768 keys, FP8)
     seq, heads, hkv, d = 32768, 32, 8, 128

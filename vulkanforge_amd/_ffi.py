@@ -76,6 +76,7 @@ SIGNATURES = {
     "vfkv_fp8_to_f16": (C.c_int, [_vp, _vp, _u64, _vp]),
     "vfkv_kv_write": (C.c_int, [_vp, _u32, _u32, _u32, _vp, _vp, _vp]),
     "vfkv_flash_attn_split": (C.c_int, [_vp, _vp, _vp, _u32, _vp, _vp, _vp, C.POINTER(SplitParams), _u32, _f, _vp]),
+    "vfkv_flash_attn_split_interleaved": (C.c_int, [_vp, _vp, _vp, _u32, _vp, _vp, _vp, C.POINTER(SplitParams), _u32, _f, _vp]),
     "vfkv_flash_attn_reduce": (C.c_int, [_vp, _vp, _vp, _vp, _u32, _u32, _u32, _vp]),
     "vfkv_workspace_create": (C.c_int, [_u32, _u32, _u32, C.POINTER(_vp)]),
     "vfkv_workspace_destroy": (None, [_vp]),

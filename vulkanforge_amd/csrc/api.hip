@@ -328,9 +328,9 @@ int vfkv_kv_write(vfkv_cache* c, uint32_t layer, uint32_t pos, uint32_t n_tokens
 }
 
 // ---- decode attention ----------------------------------------------------------------------------------
-int vfkv_flash_attn_split(const float* q, const void* k_layer, const void* v_layer, uint32_t kv_dtype,
-                          float* scratch_out, float* scratch_max, float* scratch_sum, const vfkv_split_params* p,
-                          uint32_t tile, float softcap, vfkv_stream stream) {
+static int flash_attn_split_impl(const float* q, const void* k_layer, const void* v_layer, uint32_t kv_dtype,
+                                 float* scratch_out, float* scratch_max, float* scratch_sum, const vfkv_split_params* p,
+                                 uint32_t tile, float softcap, bool interleave, vfkv_stream stream) {
     if (!p) return fail(VFKV_ERR_INVALID_ARG, "flash_attn_split: params is NULL");
     if (!q || !k_layer || !v_layer || !scratch_out || !scratch_max || !scratch_sum)
         return fail(VFKV_ERR_INVALID_ARG, "flash_attn_split: NULL buffer");
@@ -349,9 +349,23 @@ int vfkv_flash_attn_split(const float* q, const void* k_layer, const void* v_lay
     L.scratch_out = scratch_out; L.scratch_max = scratch_max; L.scratch_sum = scratch_sum;
     L.dtype = kv_dtype; L.n_heads = p->n_heads; L.n_kv_heads = p->n_kv_heads; L.head_dim = p->head_dim;
     L.seq_len = p->seq_len; L.kv_start = p->kv_start; L.tile = tile; L.tile_first = 0; L.n_tiles = p->n_tiles;
-    L.scale = p->scale; L.softcap = softcap;
+    L.scale = p->scale; L.softcap = softcap; L.interleave = interleave;
     VFKV_HIP(vfkv::launch_split(L, S(stream)));
     return VFKV_OK;
+}
+
+int vfkv_flash_attn_split(const float* q, const void* k_layer, const void* v_layer, uint32_t kv_dtype,
+                          float* scratch_out, float* scratch_max, float* scratch_sum, const vfkv_split_params* p,
+                          uint32_t tile, float softcap, vfkv_stream stream) {
+    return flash_attn_split_impl(q, k_layer, v_layer, kv_dtype, scratch_out, scratch_max, scratch_sum, p, tile, softcap,
+                                 false, stream);
+}
+
+int vfkv_flash_attn_split_interleaved(const float* q, const void* k_layer, const void* v_layer, uint32_t kv_dtype,
+                                      float* scratch_out, float* scratch_max, float* scratch_sum,
+                                      const vfkv_split_params* p, uint32_t tile, float softcap, vfkv_stream stream) {
+    return flash_attn_split_impl(q, k_layer, v_layer, kv_dtype, scratch_out, scratch_max, scratch_sum, p, tile, softcap,
+                                 true, stream);
 }
 
 int vfkv_flash_attn_reduce(const float* scratch_out, const float* scratch_max, const float* scratch_sum, float* o,

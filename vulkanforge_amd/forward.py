@@ -97,12 +97,14 @@ class Forward:
     @staticmethod
     def run_flash_attn_split(q, k_layer, v_layer, kv_dtype, scratch_out, scratch_max, scratch_sum, n_heads,
                              n_kv_heads, head_dim, seq_len, scale, kv_start=0, tile=FA_TILE, softcap=0.0,
-                             max_seq=0, stream=None) -> int:
+                             max_seq=0, stream=None, interleaved=False) -> int:
+        """``interleaved=True`` calls vfkv_flash_attn_split_interleaved: same partial count, but partial j is
+        not tile j (only the merged output is meaningful)."""
         n_tiles = (seq_len + tile - 1) // tile
         p = _ffi.SplitParams(n_heads, n_kv_heads, head_dim, seq_len, max_seq, scale, n_tiles, kv_start)
-        _ffi.check(_ffi.lib().vfkv_flash_attn_split(_ptr(q), _ptr(k_layer), _ptr(v_layer), int(kv_dtype),
-                                                    _ptr(scratch_out), _ptr(scratch_max), _ptr(scratch_sum),
-                                                    C.byref(p), tile, softcap, _stream(stream)))
+        fn = _ffi.lib().vfkv_flash_attn_split_interleaved if interleaved else _ffi.lib().vfkv_flash_attn_split
+        _ffi.check(fn(_ptr(q), _ptr(k_layer), _ptr(v_layer), int(kv_dtype), _ptr(scratch_out), _ptr(scratch_max),
+                      _ptr(scratch_sum), C.byref(p), tile, softcap, _stream(stream)))
         return n_tiles
 
     @staticmethod

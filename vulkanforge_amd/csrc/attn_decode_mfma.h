@@ -241,6 +241,7 @@ __global__ __launch_bounds__(NW * 64) void split_mfma_kernel(SplitArgs a, uint32
             u32x4 pbits[PKS];
             auto softmax = [&](auto masked_tag) {
                 constexpr bool MASKED = decltype(masked_tag)::value;
+                constexpr bool FOLD = !MASKED && !CAP;                   // scores stay unscaled until the exponent
                 float x[RT][4];
                 float tmax = kMasked;
 #pragma unroll
@@ -249,7 +250,7 @@ __global__ __launch_bounds__(NW * 64) void split_mfma_kernel(SplitArgs a, uint32
                     for (int i = 0; i < 4; ++i) {
                         float y = s[t][i];
                         y += dpp_f<kDppRor8>(y);                         // f16(q) part + remainder part
-                        y *= scale_l2;
+                        if (!FOLD) y *= scale_l2;                        // FOLD: the scale rides in the exponent's FMA
                         if (CAP) y = cap_l2 * tanhf(y / cap_l2);
                         if (MASKED) {
                             const uint32_t row = rb + t * 16 + kg * 4 + i;
@@ -259,6 +260,7 @@ __global__ __launch_bounds__(NW * 64) void split_mfma_kernel(SplitArgs a, uint32
                         tmax = fmaxf(tmax, y);
                     }
                 { float y = tmax; swap16(tmax, y); tmax = fmaxf(tmax, y); y = tmax; swap32(tmax, y); tmax = fmaxf(tmax, y); }
+                if (FOLD) tmax *= scale_l2;
                 const float m_new = fmaxf(m_run, tmax);
                 if (__builtin_amdgcn_ballot_w64(m_new > m_run) != 0ull) {
                     const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
@@ -275,14 +277,15 @@ __global__ __launch_bounds__(NW * 64) void split_mfma_kernel(SplitArgs a, uint32
                         float2_t pp;
 #pragma unroll
                         for (int e = 0; e < 2; ++e) {
-                            float pv = __builtin_amdgcn_exp2f(x[t][2 * i2 + e] - m_run);
-                            if (MASKED) pv = x[t][2 * i2 + e] > -1e29f ? pv : 0.f;
+                            const float xe = x[t][2 * i2 + e];
+                            float pv = __builtin_amdgcn_exp2f(FOLD ? __builtin_fmaf(xe, scale_l2, -m_run) : xe - m_run);
+                            if (MASKED) pv = xe > -1e29f ? pv : 0.f;
                             pp[e] = pv;
                         }
                         l_run += pp[0] + pp[1];
-                        const half2_t ph = __builtin_convertvector(pp, half2_t);
-                        const half2_t pl = __builtin_convertvector(pp - __builtin_convertvector(ph, float2_t), half2_t);
-                        pbits[t / 2][(t % 2) * 2 + i2] = is_lo ? __builtin_bit_cast(uint32_t, pl) : __builtin_bit_cast(uint32_t, ph);
+                        const uint32_t ph = __builtin_bit_cast(uint32_t, __builtin_convertvector(pp, half2_t));
+                        const uint32_t pl = pack_f16_remainder(pp[0], pp[1], ph);
+                        pbits[t / 2][(t % 2) * 2 + i2] = is_lo ? pl : ph;
                     }
             };
             if (interior) softmax(std::false_type{}); else softmax(std::true_type{});

@@ -218,6 +218,7 @@ __global__ __launch_bounds__(NCB == 1 ? 768 : 512) void batch_mfma2_kernel(Batch
             u32x4 phi[NCB], plo[NCB];
             auto softmax = [&](auto masked_tag) {
                 constexpr bool MASKED = decltype(masked_tag)::value;
+                constexpr bool FOLD = !MASKED && !CAP;                   // scores stay unscaled until the exponent's FMA
 #pragma unroll
                 for (int cb = 0; cb < NCB; ++cb) {
                     float x[8];
@@ -226,7 +227,7 @@ __global__ __launch_bounds__(NCB == 1 ? 768 : 512) void batch_mfma2_kernel(Batch
                     for (int kt = 0; kt < 2; ++kt)
 #pragma unroll
                         for (int i = 0; i < 4; ++i) {
-                            float y = s[cb][kt][i] * scale_l2;
+                            float y = FOLD ? s[cb][kt][i] : s[cb][kt][i] * scale_l2;
                             if (CAP) y = cap_l2 * tanhf(y / cap_l2);
                             if (MASKED) {
                                 const uint32_t t = tcur + kt * 16 + kg * 4 + i;
@@ -236,6 +237,7 @@ __global__ __launch_bounds__(NCB == 1 ? 768 : 512) void batch_mfma2_kernel(Batch
                             tmax = fmaxf(tmax, y);
                         }
                     { float y = tmax; swap16(tmax, y); tmax = fmaxf(tmax, y); y = tmax; swap32(tmax, y); tmax = fmaxf(tmax, y); }
+                    if (FOLD) tmax *= scale_l2;
                     const float m_new = fmaxf(m_run[cb], tmax);
                     if (__builtin_amdgcn_ballot_w64(m_new > m_run[cb]) != 0ull) {
                         const float alpha = __builtin_amdgcn_exp2f(m_run[cb] - m_new);
@@ -249,15 +251,14 @@ __global__ __launch_bounds__(NCB == 1 ? 768 : 512) void batch_mfma2_kernel(Batch
                         float2_t pp;
 #pragma unroll
                         for (int e = 0; e < 2; ++e) {
-                            float pv = __builtin_amdgcn_exp2f(x[2 * j2 + e] - m_run[cb]);
-                            if (MASKED) pv = x[2 * j2 + e] > -1e29f ? pv : 0.f;
+                            const float xe = x[2 * j2 + e];
+                            float pv = __builtin_amdgcn_exp2f(FOLD ? __builtin_fmaf(xe, scale_l2, -m_run[cb]) : xe - m_run[cb]);
+                            if (MASKED) pv = xe > -1e29f ? pv : 0.f;
                             pp[e] = pv;
                         }
                         l_run[cb] += pp[0] + pp[1];
-                        const half2_t ph = __builtin_convertvector(pp, half2_t);
-                        const half2_t pl = __builtin_convertvector(pp - __builtin_convertvector(ph, float2_t), half2_t);
-                        phi[cb][j2] = __builtin_bit_cast(uint32_t, ph);
-                        plo[cb][j2] = __builtin_bit_cast(uint32_t, pl);
+                        phi[cb][j2] = __builtin_bit_cast(uint32_t, __builtin_convertvector(pp, half2_t));
+                        plo[cb][j2] = pack_f16_remainder(pp[0], pp[1], phi[cb][j2]);
                     }
                 }
             };

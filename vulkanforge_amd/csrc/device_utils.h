@@ -62,6 +62,17 @@ __device__ __forceinline__ void e4m3x4_to_h2(uint32_t w, half2_t& lo, half2_t& h
     hi = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8((int)w, 1.0f, true);
 }
 
+// Packed f16 remainders of two f32 values against their packed f16 roundings `h`: f16(p - f32(h)) per element.
+// One mixed-precision FMA per element (the f16 source is widened inside the instruction), bit-identical to
+// converting back, subtracting and converting again.
+__device__ __forceinline__ uint32_t pack_f16_remainder(float p0, float p1, uint32_t h) {
+    uint32_t r;
+    asm("v_fma_mixlo_f16 %0, %1, 1.0, -%3 op_sel:[0,0,0] op_sel_hi:[0,0,1]\n\t"
+        "v_fma_mixhi_f16 %0, %2, 1.0, -%3 op_sel:[0,0,1] op_sel_hi:[0,0,1]"
+        : "=&v"(r) : "v"(p0), "v"(p1), "v"(h));
+    return r;
+}
+
 __device__ __forceinline__ float h16_bits_to_f32(uint32_t bits16) {
     return (float)__builtin_bit_cast(_Float16, (uint16_t)bits16);
 }

@@ -345,6 +345,68 @@ def bench_prefill(args, wl):
     return result
 
 
+def bench_rope_append(args, wl):
+    """One step = for every layer one launch of K-norm + RoPE + append (K and V rows).  Also times the plain append
+    of the same rows (no norm, no rotation) so the cost of the fused arithmetic can be read off."""
+    import numpy as np
+    import torch
+
+    import vulkanforge_amd as vf
+
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    L, Hkv, D, T = wl.n_layers, wl.n_kv_heads, wl.head_dim, wl.n_tokens
+    cache = vf.KvCache(vf.KvCacheConfig(L, Hkv, D, wl.base_pos + T, dtype=wl.dtype))
+    fwd = vf.Forward(cache, Hkv)
+    g = torch.Generator(device="cuda").manual_seed(args.seed)
+    k = torch.randn((L, T, Hkv * D), device=dev, generator=g)
+    v = torch.randn((L, T, Hkv * D), device=dev, generator=g).half().float()
+    w = 1.0 + 0.1 * torch.randn((D,), device=dev, generator=g)
+    theta_scale = float((1.0 / 1e6) ** (2.0 / D))
+
+    def step():
+        for layer in range(L):
+            fwd.step_k_rope_kv_write(layer, wl.base_pos, T, k[layer], v[layer], D, theta_scale, k_norm_weight=w)
+
+    def plain():
+        for layer in range(L):
+            fwd.b_step_kv_write(layer, wl.base_pos, T, k[layer], v[layer])
+
+    sec = time_steps(torch, step, args)
+    sec_plain = time_steps(torch, plain, args)
+    step()
+    torch.cuda.synchronize()
+    result = {
+        "metric": "k_rope_append_GBps", "value": wl.bytes_step() / sec / 1e9, "unit": "GB/s", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": sec * 1e3, "us_per_launch": sec * 1e6 / L,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "kv_dtype": wl.dtype.label(),
+        "data": "synthetic, seeded N(0,1)",
+        "config": {"workload": wl.name, "n_layers": L, "n_kv_heads": Hkv, "head_dim": D, "tokens_per_layer": T,
+                   "base_pos": wl.base_pos, "bytes_per_step": wl.bytes_step(),
+                   "plain_append_us_per_launch": sec_plain * 1e6 / L},
+        "roofline": {"bound": "hbm", "kernel": "rope_append_kernel", "achieved": wl.bytes_step() / sec / 1e9,
+                     "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": wl.bytes_step() / sec / 1e9 / HBM_PEAK_GBPS,
+                     "traffic": None, "avg_launch_us": sec * 1e6 / L},
+    }
+    if not args.no_cpu_baseline:
+        import oracle
+        kk = k[0].cpu().numpy().reshape(T, Hkv, D)
+        pos = (wl.base_pos + np.arange(T)).astype(np.int32)
+        t0 = time.perf_counter()
+        reps = 0
+        while time.perf_counter() - t0 < min(args.cpu_seconds, 2.0):
+            ref = oracle.rms_norm_rope(kk, pos, D, D, theta_scale, weight=w.cpu().numpy(), eps=1e-6)
+            enc = oracle.f32_to_e4m3(ref.reshape(-1)) if wl.dtype == vf.KvDtype.F8 else ref
+            reps += 1
+        spent = time.perf_counter() - t0
+        result["cpu_baseline"] = {"value": wl.bytes_step() / L / 2 * reps / spent / 1e9, "unit": "GB/s",
+                                  "cores": oracle.default_threads(), "kind": "port",
+                                  "sample": f"K rows of one layer, {reps} repetitions, CPU oracle, {spent:.1f} s"}
+        del enc
+    cache.destroy()
+    return result
+
+
 def copy_calibration(args):
     """Plain device-to-device copy of a known size, launched `steps` times: the reference point for the
     FETCH_SIZE / WRITE_SIZE counters (what they read for a kernel whose HBM traffic is known)."""
@@ -373,10 +435,12 @@ def main():
         res = bench_decode(args, workloads.DECODE[args.workload])
     elif args.workload in workloads.PREFILL:
         res = bench_prefill(args, workloads.PREFILL[args.workload])
+    elif args.workload in workloads.ROPE_APPEND:
+        res = bench_rope_append(args, workloads.ROPE_APPEND[args.workload])
     elif args.workload == "copy_calibration":
         res = copy_calibration(args)
     else:
-        print("unknown workload; choose from: " + ", ".join(list(workloads.DECODE) + list(workloads.PREFILL) + ["copy_calibration"]),
+        print("unknown workload; choose from: " + ", ".join(list(workloads.DECODE) + list(workloads.PREFILL) + list(workloads.ROPE_APPEND) + ["copy_calibration"]),
               file=sys.stderr)
         sys.exit(2)
     print(json.dumps(res))

@@ -131,6 +131,36 @@ int vfkv_fp8_to_f16(const void* src, void* dst_f16, uint64_t n_elems, vfkv_strea
 int vfkv_kv_write(vfkv_cache* c, uint32_t layer, uint32_t pos, uint32_t n_tokens,
                   const float* k_src, const float* v_src, vfkv_stream stream);
 
+/* RoPE parameters as the reference's callers fill RopePushConstants (forward/runs.rs:2547-2580,
+ * 680-700): freq_scale = attn_factor = 1, ext_factor = 0 (the YaRN ramp of rope_funcs.glsl:17-37 is
+ * not built), no sections. */
+#define VFKV_ROPE_NORM 0u /* GGML_ROPE_TYPE_NORMAL: pairs (2p, 2p + 1)              (rope_funcs.glsl:39-76)  */
+#define VFKV_ROPE_NEOX 2u /* GGML_ROPE_TYPE_NEOX:   pairs (p, p + rotary_dim / 2)   (rope_funcs.glsl:78-112) */
+typedef struct {
+    uint32_t rope_mode;   /* VFKV_ROPE_NORM / VFKV_ROPE_NEOX (config.rope_variant, runs.rs:2532-2535) */
+    uint32_t rotary_dim;  /* n_dims: even, <= head_dim; elements beyond it pass through */
+    float theta_scale;    /* (1 / freq_base)^(2 / rotary_dim)  (forward/layer_plan.rs:532) */
+    float freq_scale;     /* 1.0 in the reference's callers */
+    float attn_factor;    /* 1.0 in the reference's callers */
+    float eps;            /* rms_norm epsilon (cfg.rms_norm_eps); used only with a norm weight */
+} vfkv_rope_params;
+
+/* `KNormRope` or `KRope` followed by `KvWrite` (forward/layer_plan.rs:119-137) in one launch:
+ * step_k_norm_rope / step_k_rope (executor/attention.rs:435-530; batch :2040-2075) =
+ * run_rms_norm_mul_rope (forward/runs.rs:2492-2600, rms_norm.comp:36-129 fused with
+ * rope_funcs.glsl:39-112) or run_rope_neox_with_pos_offset (runs.rs:647-720), then step_kv_write
+ * (attention.rs:546-597).  K rows [n_tokens, kv_heads * head_dim] f32 are RMS-normalised per head
+ * and multiplied by `k_norm_weight[head_dim]` (NULL: no norm, the plain `KRope`), rotated with
+ * theta = positions[t] * theta_scale^p / freq_factors[p] (positions NULL: pos + t, the values the
+ * reference writes to rope_pos_buf; freq_factors NULL: 1, has_ff = 0), and stored at position
+ * pos + t of `layer` in the cache dtype; V rows are stored as vfkv_kv_write stores them.  `k_out`
+ * (may be k_src, may be NULL) receives the rotated K as f32, which is what the reference leaves in
+ * k_buf. */
+int vfkv_k_rope_kv_write(vfkv_cache* c, uint32_t layer, uint32_t pos, uint32_t n_tokens,
+                         const float* k_src, const float* v_src, const float* k_norm_weight,
+                         const int32_t* positions, const float* freq_factors,
+                         const vfkv_rope_params* p, float* k_out, vfkv_stream stream);
+
 /* ------------------------------------------------------------------------------------------ */
 /* Decode attention: split-K worker + log-sum-exp merge.                                      */
 /* ------------------------------------------------------------------------------------------ */

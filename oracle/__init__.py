@@ -79,6 +79,8 @@ def _declare(L: C.CDLL) -> None:
         getattr(L, name).argtypes = ([C.c_void_p] * 3 + [C.c_uint32] * 8 + [C.c_float] * 2
                                      + [C.c_void_p, C.c_int])
         getattr(L, name).restype = None
+    L.vfo_rms_norm_rope.argtypes = [C.c_void_p] * 5 + [C.c_uint32] * 5 + [C.c_float] * 4
+    L.vfo_rms_norm_rope.restype = None
     L.vfo_max_threads.argtypes = []
     L.vfo_max_threads.restype = C.c_int
 
@@ -235,3 +237,28 @@ def attn_batch_shader(q, k, v, dtype, m, n_kv, n_heads, n_kv_heads, head_dim, q_
                       kv_start=0, softcap=0.0, threads=None) -> np.ndarray:
     return _batch(lib().vfo_attn_batch_shader, q, k, v, dtype, m, n_kv, n_heads, n_kv_heads, head_dim,
                   q_start, scale, kv_start, softcap, threads)
+
+
+ROPE_NORM, ROPE_NEOX = 0, 2
+
+
+def rope_theta_scale(freq_base: float, rotary_dim: int) -> np.float32:
+    """(1 / freq_base)^(2 / rotary_dim) in f32 (forward/layer_plan.rs:532)."""
+    return np.float32(np.float32(1.0) / np.float32(freq_base)) ** np.float32(np.float32(2.0) / np.float32(rotary_dim))
+
+
+def rms_norm_rope(x, pos, head_dim, n_dims, theta_scale, mode=ROPE_NEOX, weight=None, ff=None, freq_scale=1.0,
+                  attn_factor=1.0, eps=1e-6) -> np.ndarray:
+    """x: [m, heads, head_dim] f32, pos: [m] int32 -> rotated (optionally RMS-normed * weight) copy."""
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    m, heads = x.shape[0], x.shape[1]
+    assert x.shape[2] == head_dim
+    pos = np.ascontiguousarray(pos, dtype=np.int32)
+    assert pos.shape == (m,)
+    w = None if weight is None else np.ascontiguousarray(weight, dtype=np.float32)
+    f = None if ff is None else np.ascontiguousarray(ff, dtype=np.float32)
+    out = np.empty_like(x)
+    lib().vfo_rms_norm_rope(_p(x), _p(w) if w is not None else None, _p(pos), _p(f) if f is not None else None,
+                            _p(out), m, heads, head_dim, mode, n_dims, float(theta_scale), float(freq_scale),
+                            float(attn_factor), float(eps))
+    return out

@@ -28,6 +28,15 @@
  *                                 vk_shaders/flash_attn_reduce.comp:35-81          invariance, tests/flash_attn_tiled_ref.rs:279-295)
  *   vfo_attn_batch_ref            tests/correctness.rs:3016-3071                   scipy softmax per query; M=1 == decode; causal isolation
  *   vfo_attn_batch_shader         vk_shaders/flash_attn_batch.comp:105-208         == vfo_attn_batch_ref within 1e-4..5e-3 on the reference's cases
+ *   vfo_rms_norm_rope             vk_shaders/rms_norm.comp:36-129 (fusion path),   NEOX: the reference's generator case and f32 CPU formula at
+ *                                 vk_shaders/rope_funcs.glsl:17-112                positions 0 / 100 / 4096 with its thresholds
+ *                                                                                 (tests/correctness.rs:799-884); both modes: numpy complex-
+ *                                                                                 rotation formulation, pair-norm invariance, pos=0 identity,
+ *                                                                                 additivity of positions; norm: numpy x/sqrt(mean(x^2)+eps)*w
+ *                                                                                 (the CPU formula of tests/correctness.rs:665-700).
+ *                                                                                 NORM mode (adjacent pairs), partial rotary_dim and frequency
+ *                                                                                 factors have no reference test: parity unpinned by the
+ *                                                                                 reference, pinned by the formulations above only.
  *
  * Extensions that the reference does not implement (so no reference test can pin them):
  *   - `kv_start > 0` on every attention routine follows the shader text
@@ -532,6 +541,55 @@ void vfo_attn_batch_shader(const float* q, const void* k, const void* v, uint32_
         for (uint32_t d = 0; d < head_dim; ++d) o[d] = acc[d] * inv;
         free(acc);
     }
+}
+
+/* ------------------------------------------------------------------------------------------
+ * K (or Q) RMS-norm * weight followed by RoPE, the step in front of the KV append
+ * (rms_norm.comp:36-129 with RMS_NORM_ROPE_FUSION, rope_funcs.glsl:17-112; host: run_rms_norm_mul_rope
+ * runs.rs:2492-2600, run_rope_neox_with_pos_offset runs.rs:647-720).
+ *
+ * x, out: [m][heads][head_dim] f32 (out may alias x).  weight: [head_dim] or NULL (plain RoPE).
+ * pos: [m] token positions.  ff: [n_dims / 2] frequency factors or NULL.  mode 0 = NORM: pairs
+ * (i0, i0 + 1); mode 2 = NEOX: pairs (i0 / 2, i0 / 2 + n_dims / 2); dims >= n_dims pass through.
+ * The reference's callers pass freq_scale = 1, ext_factor = 0 (no YaRN ramp), attn_factor = 1; the
+ * ext_factor != 0 branch of rope_yarn is not restated.
+ *
+ * Arithmetic: the shader works in f32 (sum of squares by a tree, theta = pos * pow(theta_scale, i0/2),
+ * cos / sin of the GPU).  Here the sum of squares is accumulated in f64, theta is formed in f32 exactly
+ * as the shader writes it (so the angle is the same number), and the trigonometry and the rotation are
+ * evaluated in f64 and rounded once.
+ * ---------------------------------------------------------------------------------------- */
+void vfo_rms_norm_rope(const float* x, const float* weight, const int32_t* pos, const float* ff, float* out,
+                       uint32_t m, uint32_t heads, uint32_t head_dim, uint32_t mode, uint32_t n_dims,
+                       float theta_scale, float freq_scale, float attn_factor, float eps) {
+#pragma omp parallel for collapse(2) schedule(static)
+    for (uint32_t t = 0; t < m; ++t)
+        for (uint32_t h = 0; h < heads; ++h) {
+            const float* row = x + ((size_t)t * heads + h) * head_dim;
+            float* dst = out + ((size_t)t * heads + h) * head_dim;
+            float* y = (float*)malloc(sizeof(float) * head_dim);
+            if (weight) {                                   /* rms_norm.comp:61-112 */
+                double ss = 0.0;
+                for (uint32_t d = 0; d < head_dim; ++d) ss += (double)row[d] * (double)row[d];
+                const float mean = (float)(ss / (double)head_dim);
+                const float scale = (float)(1.0 / sqrt((double)mean + (double)eps));
+                for (uint32_t d = 0; d < head_dim; ++d) y[d] = (scale * row[d]) * weight[d];
+            } else {
+                for (uint32_t d = 0; d < head_dim; ++d) y[d] = row[d];
+            }
+            for (uint32_t d = 0; d < head_dim; ++d) dst[d] = y[d];          /* dims >= n_dims: rope_funcs.glsl:56-61,90-95 */
+            for (uint32_t i0 = 0; i0 + 1 < n_dims; i0 += 2) {
+                const float theta_base = (float)pos[t] * powf(theta_scale, (float)i0 / 2.0f);   /* :63,97 */
+                const float freq_factor = ff ? ff[i0 / 2] : 1.0f;                              /* :65,99 */
+                const float theta = freq_scale * (theta_base / freq_factor);                   /* rope_yarn :20-22 */
+                const double c = cos((double)theta) * (double)attn_factor, sn = sin((double)theta) * (double)attn_factor;
+                const uint32_t a = mode == 2u ? i0 / 2 : i0, b = mode == 2u ? i0 / 2 + n_dims / 2 : i0 + 1;
+                const double x0 = y[a], x1 = y[b];
+                dst[a] = (float)(x0 * c - x1 * sn);                                            /* :73-74, :107-108 */
+                dst[b] = (float)(x0 * sn + x1 * c);
+            }
+            free(y);
+        }
 }
 
 int vfo_max_threads(void) {

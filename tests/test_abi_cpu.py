@@ -167,3 +167,24 @@ def test_no_device_means_loud_failure():
     with pytest.raises(ValueError):
         import torch
         vf.Forward.run_kv_store_fp8(torch.zeros(8), torch.zeros(8, dtype=torch.uint8), 8, 0, stream=0)
+
+
+def test_k_rope_kv_write_rejects_bad_arguments():
+    # validation happens before any device work: the buffers below are never dereferenced
+    cache = vf.KvCache(vf.KvCacheConfig(2, 8, 128, 64, dtype=vf.KvDtype.F8), k_buffer=0x10000, v_buffer=0x20000)
+    L = _ffi.lib()
+    fake = 0x1000
+
+    def call(mode=_ffi.ROPE_NEOX, rot=128, fs=1.0, layer=0, pos=0, n=1, k=fake, v=fake, params=True):
+        p = _ffi.RopeParams(mode, rot, 0.9, fs, 1.0, 1e-6)
+        return L.vfkv_k_rope_kv_write(cache.handle, layer, pos, n, k, v, None, None, None,
+                                      C.byref(p) if params else None, None, None)
+
+    assert call(n=0) == 0                       # nothing to do
+    assert call(mode=8) == -4                   # MROPE / VISION are not built
+    assert b"rope_mode" in L.vfkv_last_error()
+    assert call(rot=127) == -1 and call(rot=130) == -1
+    assert call(layer=2) == -1 and call(pos=64) == -1 and call(pos=60, n=5) == -1
+    assert call(k=None) == -1 and call(v=None) == -1 and call(params=False) == -1
+    assert call(fs=0.0) == -1
+    cache.destroy()

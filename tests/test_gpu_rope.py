@@ -1,0 +1,190 @@
+"""GPU parity of vfkv_k_rope_kv_write (K RMS-norm * weight + RoPE + append of K and V in one launch) against the
+oracle, through the C ABI.
+
+Bars.  V bytes: bit-exact.  K with an F32 cache (and `k_out`): |gpu - oracle| <= max|k| * (5e-6 + pos * 2^-21) --
+the only slack is one ulp of the f32 angle theta <= pos * 2^-23 between two powf implementations, the same slack
+the reference grants its own GPU (tests/correctness.rs:799-815: 1e-5 / 1e-4 / 5e-4 at positions 0 / 100 / 4096
+for |x| <= 3.5).  K with an F16 / FP8 cache: the stored code must lie between the codes of (oracle - tol) and
+(oracle + tol), i.e. be a correct rounding of a value inside that band."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+import vulkanforge_amd as vf
+from vulkanforge_amd import _ffi
+from gpu_util import DEV, fp16_normal, read_device, rng, to_dev, to_np
+
+pytestmark = pytest.mark.gpu
+
+
+def k_tolerance(k_ref, pos):
+    return np.abs(k_ref).max() * (5e-6 + np.asarray(pos, np.float64) * 2.0 ** -21)
+
+
+def run_case(dtype, hkv, d, n_tok, pos0, rotary, mode, norm, use_pos_array, use_ff, freq_base=10000.0, k_out=True,
+             seed=0, max_seq=None):
+    r = rng(seed + d + n_tok + pos0)
+    max_seq = max_seq or pos0 + n_tok + 3
+    cache = vf.KvCache(vf.KvCacheConfig(2, hkv, d, max_seq, dtype=dtype))
+    cache.zero_fill()
+    fwd = vf.Forward(cache, hkv)
+    k = (r.standard_normal((n_tok, hkv, d)) * 1.5).astype(np.float32)
+    v = fp16_normal(r, (n_tok, hkv, d))
+    w = (1 + 0.2 * r.standard_normal(d)).astype(np.float32) if norm else None
+    ff = (1 + 2 * r.random(rotary // 2)).astype(np.float32) if use_ff else None
+    if use_pos_array:
+        positions = (pos0 + np.arange(n_tok) * 3 + (np.arange(n_tok) % 2) * 11).astype(np.int32)   # not pos0 + t on purpose
+    else:
+        positions = (pos0 + np.arange(n_tok)).astype(np.int32)
+    ts = float(oracle.rope_theta_scale(freq_base, rotary)) if rotary else 1.0
+    kd, vd = to_dev(k), to_dev(v)
+    kout = torch.full_like(kd, float("nan")) if k_out else None
+    layer = 1
+    fwd.step_k_rope_kv_write(layer, pos0, n_tok, kd, vd, rotary, ts, k_norm_weight=to_dev(w) if norm else None,
+                             positions=to_dev(positions) if use_pos_array else None,
+                             freq_factors=to_dev(ff) if use_ff else None, rope_mode=mode, eps=1e-6, k_out=kout)
+    torch.cuda.synchronize()
+    k_ref = oracle.rms_norm_rope(k, positions, d, rotary, ts, mode=mode, weight=w, ff=ff, eps=1e-6)
+    tol = k_tolerance(k_ref, positions)[:, None, None]
+    es = dtype.element_size()
+    off = cache.pos_offset_bytes(layer, pos0)
+    nbytes = n_tok * hkv * d * es
+    k_bytes = read_device(cache.k_ptr + off, nbytes)
+    v_bytes = read_device(cache.v_ptr + off, nbytes)
+    # ---- V: what vfkv_kv_write stores, bit for bit
+    v_exp = np.zeros(nbytes, np.uint8)
+    if dtype == vf.KvDtype.F8:
+        oracle.kv_store_fp8(v.reshape(-1), v_exp, v.size, 0)
+    elif dtype == vf.KvDtype.F16:
+        oracle.kv_copy_fp16(v.reshape(-1), v_exp, v.size, 0)
+    else:
+        v_exp = v.reshape(-1).view(np.uint8)
+    assert (v_bytes == v_exp).all()
+    # ---- K
+    if k_out:
+        ko = to_np(kout)
+        assert np.isfinite(ko).all()
+        assert (np.abs(ko - k_ref) <= tol).all(), float(np.abs(ko - k_ref).max())
+    if dtype == vf.KvDtype.F32:
+        got = k_bytes.view(np.float32).reshape(k_ref.shape)
+        assert (np.abs(got - k_ref) <= tol).all()
+        if k_out:
+            assert (got == ko).all()
+    else:
+        if dtype == vf.KvDtype.F8:
+            dec = lambda b: oracle.e4m3_to_f32(b)                                           # noqa: E731
+            enc = lambda x: oracle.f32_to_e4m3(x)                                           # noqa: E731
+            got = dec(k_bytes).reshape(k_ref.shape)
+        else:
+            dec = lambda b: oracle.f16_bits_to_f32(b)                                       # noqa: E731
+            enc = lambda x: oracle.f32_to_f16_bits(x)                                       # noqa: E731
+            got = dec(k_bytes.view(np.uint16)).reshape(k_ref.shape)
+        lo = dec(enc((k_ref - tol).astype(np.float32).reshape(-1))).reshape(k_ref.shape)
+        hi = dec(enc((k_ref + tol).astype(np.float32).reshape(-1))).reshape(k_ref.shape)
+        assert ((got >= lo) & (got <= hi)).all()
+        if k_out:                                   # the cache holds the conversion of exactly what k_out holds
+            assert (k_bytes.view(np.uint8 if dtype == vf.KvDtype.F8 else np.uint16) == enc(ko.reshape(-1))).all()
+    # rows outside [pos0, pos0 + n_tok) and the other layer stay zero
+    assert not read_device(cache.k_ptr, cache.pos_offset_bytes(layer, pos0)).any()
+    tail = cache.pos_offset_bytes(layer, pos0 + n_tok)
+    assert not read_device(cache.k_ptr + tail, cache.bytes_per_buffer() - tail).any()
+    cache.destroy()
+    return k_ref
+
+
+CASES = [
+    # dtype, hkv, d, n_tok, pos0, rotary, mode, norm, pos_array, ff
+    (vf.KvDtype.F8, 8, 128, 1, 8192, 128, _ffi.ROPE_NEOX, True, False, False),     # decode step, Qwen3-style K-norm
+    (vf.KvDtype.F8, 8, 128, 1, 100, 128, _ffi.ROPE_NEOX, False, False, False),     # plain KRope
+    (vf.KvDtype.F8, 8, 128, 512, 4096, 128, _ffi.ROPE_NEOX, True, False, False),   # prefill chunk
+    (vf.KvDtype.F16, 8, 256, 33, 1000, 256, _ffi.ROPE_NEOX, True, True, False),
+    (vf.KvDtype.F16, 2, 128, 7, 0, 64, _ffi.ROPE_NEOX, True, False, True),         # partial rotary, frequency factors
+    (vf.KvDtype.F32, 4, 128, 9, 50, 128, _ffi.ROPE_NORM, False, True, False),
+    (vf.KvDtype.F32, 4, 64, 9, 4000, 64, _ffi.ROPE_NORM, True, False, True),
+    (vf.KvDtype.F32, 1, 512, 3, 10, 128, _ffi.ROPE_NEOX, True, False, False),
+    (vf.KvDtype.F8, 3, 96, 5, 77, 32, _ffi.ROPE_NORM, True, True, False),
+    (vf.KvDtype.F8, 8, 128, 4, 32000, 128, _ffi.ROPE_NEOX, True, False, False),    # long context
+]
+
+
+@pytest.mark.parametrize("dtype,hkv,d,n_tok,pos0,rotary,mode,norm,pos_array,ff", CASES)
+def test_k_rope_kv_write_matches_oracle(dtype, hkv, d, n_tok, pos0, rotary, mode, norm, pos_array, ff):
+    print(f"case dtype={dtype.label()} hkv={hkv} D={d} tokens={n_tok} pos0={pos0} rotary={rotary} mode={mode} norm={norm} "
+          f"pos_array={pos_array} ff={ff}", flush=True)
+    run_case(dtype, hkv, d, n_tok, pos0, rotary, mode, norm, pos_array, ff)
+    run_case(dtype, hkv, d, n_tok, pos0, rotary, mode, norm, pos_array, ff, k_out=False, seed=1)
+
+
+@pytest.mark.parametrize("pos,threshold", ((0, 1e-5), (100, 1e-4), (4096, 5e-4)))
+def test_reference_rope_neox_fixture(pos, threshold):
+    # tests/correctness.rs:799-884: one head of 128, ramp input, NEOX, freq_base 1e6, the reference's thresholds
+    x = (np.float32(0.1) + np.float32(3.4) * np.arange(128, dtype=np.float32) / np.float32(127)).astype(np.float32)
+    half = 64
+    ts = np.float32(1.0) / np.float32(1e6) ** np.float32(2.0 / 128)
+    cpu = np.zeros(128, np.float32)
+    for i in range(half):
+        freq = np.float32(1.0)
+        for _ in range(i):
+            freq = np.float32(freq * ts)
+        theta = np.float32(pos) * freq
+        c, s = np.cos(theta, dtype=np.float32), np.sin(theta, dtype=np.float32)
+        cpu[i] = x[i] * c - x[i + half] * s
+        cpu[i + half] = x[i] * s + x[i + half] * c
+    cache = vf.KvCache(vf.KvCacheConfig(1, 1, 128, pos + 1, dtype=vf.KvDtype.F32))
+    fwd = vf.Forward(cache, 1)
+    kd = to_dev(x.reshape(1, 1, 128))
+    out = torch.empty_like(kd)
+    fwd.step_k_rope_kv_write(0, pos, 1, kd, kd, 128, float(ts), k_out=out)
+    torch.cuda.synchronize()
+    got = to_np(out).reshape(-1)
+    assert np.abs(got - cpu).max() < threshold
+    row = read_device(cache.k_ptr + cache.pos_offset_bytes(0, pos), 512).view(np.float32)
+    assert (row == got).all()
+    if pos == 0:
+        assert (got == x).all()
+    cache.destroy()
+
+
+def test_position_zero_is_the_plain_append_and_in_place_output():
+    # rotation by 0 is exact, so without a norm the K bytes are what vfkv_kv_write stores; k_out may alias k_src
+    r = rng(9)
+    hkv, d = 8, 128
+    k = fp16_normal(r, (1, hkv, d))
+    v = fp16_normal(r, (1, hkv, d))
+    for dtype in (vf.KvDtype.F8, vf.KvDtype.F16):
+        a = vf.KvCache(vf.KvCacheConfig(1, hkv, d, 4, dtype=dtype))
+        b = vf.KvCache(vf.KvCacheConfig(1, hkv, d, 4, dtype=dtype))
+        a.zero_fill(); b.zero_fill()
+        kd, vd = to_dev(k), to_dev(v)
+        vf.Forward(a, hkv).step_k_rope_kv_write(0, 0, 1, kd, vd, d, 0.9, k_out=kd)
+        vf.Forward(b, hkv).step_kv_write(0, 0, to_dev(k), vd)
+        torch.cuda.synchronize()
+        n = a.bytes_per_buffer()
+        assert (read_device(a.k_ptr, n) == read_device(b.k_ptr, n)).all()
+        assert (read_device(a.v_ptr, n) == read_device(b.v_ptr, n)).all()
+        assert (to_np(kd) == k).all()
+        a.destroy(); b.destroy()
+
+
+def test_rotated_keys_feed_decode_attention():
+    # the fused append followed by decode attention == oracle attention over oracle-rotated keys
+    r = rng(21)
+    h, hkv, d, seq = 32, 8, 128, 300
+    cache = vf.KvCache(vf.KvCacheConfig(1, hkv, d, seq, dtype=vf.KvDtype.F16))
+    fwd = vf.Forward(cache, h)
+    k = fp16_normal(r, (seq, hkv, d))
+    v = fp16_normal(r, (seq, hkv, d))
+    q = fp16_normal(r, (h, d))
+    w = (1 + 0.1 * r.standard_normal(d)).astype(np.float32)
+    ts = float(oracle.rope_theta_scale(10000.0, d))
+    fwd.step_k_rope_kv_write(0, 0, seq, to_dev(k), to_dev(v), d, ts, k_norm_weight=to_dev(w))
+    o = torch.empty((h, d), device=DEV)
+    fwd.run_scalar_attn(0, seq - 1, to_dev(q), o)
+    torch.cuda.synchronize()
+    k_rot = oracle.rms_norm_rope(k, np.arange(seq, dtype=np.int32), d, d, ts, weight=w)
+    k16 = oracle.f32_to_f16_bits(k_rot.reshape(-1)).reshape(seq, hkv, d)
+    v16 = oracle.f32_to_f16_bits(v.reshape(-1)).reshape(seq, hkv, d)
+    ref = oracle.attn_decode_ref(q, k16, v16, oracle.F16, h, hkv, d, seq, float(1 / np.sqrt(d)))
+    assert np.abs(to_np(o) - ref).max() < 2e-3
+    cache.destroy()

@@ -37,6 +37,13 @@ class BatchParams(C.Structure):
                 ("kv_start", C.c_uint32)]
 
 
+class RopeParams(C.Structure):
+    _fields_ = [("rope_mode", C.c_uint32), ("rotary_dim", C.c_uint32), ("theta_scale", C.c_float),
+                ("freq_scale", C.c_float), ("attn_factor", C.c_float), ("eps", C.c_float)]
+
+
+ROPE_NORM, ROPE_NEOX = 0, 2   # GGML_ROPE_TYPE_NORMAL / _NEOX (rms_norm.comp:25-26)
+
 assert C.sizeof(SplitParams) == 32 and C.sizeof(BatchParams) == 32  # pipeline.rs:569,611
 
 _u32, _u64, _vp, _f = C.c_uint32, C.c_uint64, C.c_void_p, C.c_float
@@ -75,6 +82,7 @@ SIGNATURES = {
     "vfkv_copy_fp16": (C.c_int, [_vp, _vp, _u32, _u64, _vp]),
     "vfkv_fp8_to_f16": (C.c_int, [_vp, _vp, _u64, _vp]),
     "vfkv_kv_write": (C.c_int, [_vp, _u32, _u32, _u32, _vp, _vp, _vp]),
+    "vfkv_k_rope_kv_write": (C.c_int, [_vp, _u32, _u32, _u32, _vp, _vp, _vp, _vp, _vp, C.POINTER(RopeParams), _vp, _vp]),
     "vfkv_flash_attn_split": (C.c_int, [_vp, _vp, _vp, _u32, _vp, _vp, _vp, C.POINTER(SplitParams), _u32, _f, _vp]),
     "vfkv_flash_attn_split_interleaved": (C.c_int, [_vp, _vp, _vp, _u32, _vp, _vp, _vp, C.POINTER(SplitParams), _u32, _f, _vp]),
     "vfkv_flash_attn_reduce": (C.c_int, [_vp, _vp, _vp, _vp, _u32, _u32, _u32, _vp]),

@@ -327,6 +327,36 @@ int vfkv_kv_write(vfkv_cache* c, uint32_t layer, uint32_t pos, uint32_t n_tokens
     return VFKV_OK;
 }
 
+int vfkv_k_rope_kv_write(vfkv_cache* c, uint32_t layer, uint32_t pos, uint32_t n_tokens, const float* k_src,
+                         const float* v_src, const float* k_norm_weight, const int32_t* positions,
+                         const float* freq_factors, const vfkv_rope_params* p, float* k_out, vfkv_stream stream) {
+    if (!c || !c->k || !c->v) return fail(VFKV_ERR_INVALID_ARG, "k_rope_kv_write: cache has no buffers");
+    if (!p) return fail(VFKV_ERR_INVALID_ARG, "k_rope_kv_write: params is NULL");
+    if (layer >= c->n_layers) return fail(VFKV_ERR_INVALID_ARG, "k_rope_kv_write: layer %u out of range", layer);
+    if (n_tokens == 0) return VFKV_OK;
+    if (!k_src || !v_src) return fail(VFKV_ERR_INVALID_ARG, "k_rope_kv_write: NULL source");
+    if ((uint64_t)pos + n_tokens > c->max_seq_len)
+        return fail(VFKV_ERR_INVALID_ARG, "k_rope_kv_write: positions [%u, %llu) exceed max_seq_len %u", pos,
+                    (unsigned long long)pos + n_tokens, c->max_seq_len);
+    const uint32_t hd = hd_for(c, layer), kvh = kvh_for(c, layer);
+    if (p->rope_mode != VFKV_ROPE_NORM && p->rope_mode != VFKV_ROPE_NEOX)
+        return fail(VFKV_ERR_UNSUPPORTED, "k_rope_kv_write: rope_mode %u (0 = NORM and 2 = NEOX are built)", p->rope_mode);
+    if (p->rotary_dim % 2u != 0u || p->rotary_dim > hd)
+        return fail(VFKV_ERR_INVALID_ARG, "k_rope_kv_write: rotary_dim %u must be even and <= head_dim %u", p->rotary_dim, hd);
+    if (hd > 512u || hd % 4u != 0u)
+        return fail(VFKV_ERR_UNSUPPORTED, "k_rope_kv_write: head_dim %u (multiples of 4 up to 512 are built)", hd);
+    if (!(p->freq_scale > 0.f)) return fail(VFKV_ERR_INVALID_ARG, "k_rope_kv_write: freq_scale must be > 0");
+    const uint64_t off = layer_off(c, layer) + (uint64_t)pos * row_b(c, layer);
+    vfkv::RopeAppendLaunch L;
+    L.k_src = k_src; L.v_src = v_src; L.weight = k_norm_weight; L.positions = positions; L.freq_factors = freq_factors;
+    L.k_out = k_out; L.k_dst = (char*)c->k + off; L.v_dst = (char*)c->v + off;
+    L.dtype = c->dtype; L.n_tokens = n_tokens; L.n_kv_heads = kvh; L.head_dim = hd; L.rotary_dim = p->rotary_dim;
+    L.mode = p->rope_mode; L.pos0 = pos; L.row_bytes = row_b(c, layer);
+    L.theta_scale = p->theta_scale; L.freq_scale = p->freq_scale; L.attn_factor = p->attn_factor; L.eps = p->eps;
+    VFKV_HIP(vfkv::launch_rope_append(L, S(stream)));
+    return VFKV_OK;
+}
+
 // ---- decode attention ----------------------------------------------------------------------------------
 static int flash_attn_split_impl(const float* q, const void* k_layer, const void* v_layer, uint32_t kv_dtype,
                                  float* scratch_out, float* scratch_max, float* scratch_sum, const vfkv_split_params* p,

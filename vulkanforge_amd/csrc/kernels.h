@@ -10,6 +10,24 @@ hipError_t launch_kv_append(uint32_t dtype, const float* k_src, const float* v_s
                             uint32_t n_elements, int n_tensors, hipStream_t stream);
 hipError_t launch_fp8_to_f16(const void* src, void* dst, uint64_t n, hipStream_t stream);
 
+// K RMS-norm * weight + RoPE + append of K and V rows in one launch (rope_append.hip).
+struct RopeAppendLaunch {
+    const float* k_src = nullptr;         // [n_tokens][n_kv_heads][head_dim]
+    const float* v_src = nullptr;         // same shape; NULL = K only
+    const float* weight = nullptr;        // [head_dim]; NULL = no RMS-norm
+    const int32_t* positions = nullptr;   // [n_tokens]; NULL = pos0 + token
+    const float* freq_factors = nullptr;  // [rotary_dim / 2]; NULL = 1
+    float* k_out = nullptr;               // rotated K as f32 (may alias k_src); NULL = not wanted
+    void* k_dst = nullptr;                // cache row of the first token (layer offset + pos0 * row_bytes applied)
+    void* v_dst = nullptr;
+    uint32_t dtype = 0, n_tokens = 0, n_kv_heads = 0, head_dim = 0, rotary_dim = 0;
+    uint32_t mode = 2;                    // 0 = NORM (adjacent pairs), 2 = NEOX (split halves)
+    uint32_t pos0 = 0;
+    uint64_t row_bytes = 0;
+    float theta_scale = 1.f, freq_scale = 1.f, attn_factor = 1.f, eps = 0.f;
+};
+hipError_t launch_rope_append(const RopeAppendLaunch& L, hipStream_t stream);
+
 // ---- attn_decode.hip ----
 struct SplitLaunch {
     const float* q;        // [n_heads, head_dim] f32

@@ -1,0 +1,145 @@
+// K RMS-norm * weight, RoPE and the KV append in one launch for gfx950.
+//
+// Replaces, per layer, the reference's `KNormRope` / `KRope` step followed by `KvWrite`
+// (forward/layer_plan.rs:119-137): rms_norm.comp:36-129 in its RMS_NORM_ROPE_FUSION form (or rope_neox.comp /
+// rope_norm.comp alone), rope_funcs.glsl:17-112, then kv_store_fp8.comp / kv_copy_fp16.comp for K and V.  The
+// rotated K row never makes the round trip through its f32 buffer (it is still written there when the caller asks
+// for it), and K and V go out in one launch.
+//
+// One wavefront per (token, tensor, KV head) row, four rows of a token per workgroup.  The angles depend on (token,
+// pair) only: the workgroup evaluates cos / sin once (accurate powf / sincosf: the arguments reach tens of thousands of
+// radians) into LDS while the rows and the norm weight are already in flight.  K: the sum of squares is a wavefront
+// reduction, the normalised row is parked in the wavefront's LDS row so that a lane can reach both elements of its
+// rotation pairs, rotated, and stored from LDS as whole 32-bit words of the cache dtype; V: plain conversion.
+// HBM / launch bound: 4 bytes read and 1, 2 or 4 written per element.
+#include "device_utils.h"
+#include "kernels.h"
+
+namespace vfkv {
+
+struct RopeAppendArgs {
+    const float* k_src;       // [n_tokens][n_kv_heads][head_dim]
+    const float* v_src;       // same shape, or NULL: K only
+    const float* weight;      // [head_dim] or NULL: no RMS-norm
+    const int32_t* positions; // [n_tokens] or NULL: pos0 + token
+    const float* freq_factors;// [rotary_dim / 2] or NULL
+    float* k_out;             // rotated K as f32 (may alias k_src) or NULL
+    uint8_t* k_dst;           // cache row of the first token, K
+    uint8_t* v_dst;
+    uint32_t n_kv_heads, head_dim, rotary_dim, mode, pos0, dtype;
+    uint64_t row_bytes;       // distance between two tokens' rows in the cache
+    float theta_scale, freq_scale, attn_factor, eps;
+};
+
+constexpr int kRopeMaxPerLane = 8;   // head_dim <= 512
+constexpr int kRopeWaves = 4;         // rows per workgroup, one per wavefront
+
+__global__ __launch_bounds__(kRopeWaves * kWave) void rope_append_kernel(RopeAppendArgs a) {
+    __shared__ float cs_lds[256], sn_lds[256];             // rotary_dim / 2 <= 256
+    __shared__ float rows[kRopeWaves][512];
+    const int tid = threadIdx.x, lane = tid & (kWave - 1);
+    const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const uint32_t tok = blockIdx.x;
+    const uint32_t D = a.head_dim;
+    const uint32_t half = a.rotary_dim / 2u;
+    const uint32_t n_units = a.v_src ? 2u * a.n_kv_heads : a.n_kv_heads;   // (tensor, head) rows of this token
+    const uint32_t u = blockIdx.y * kRopeWaves + w;                         // this wavefront's row
+    const bool active = u < n_units;
+    const bool is_v = u >= a.n_kv_heads;
+    const uint32_t kvh = is_v ? u - a.n_kv_heads : u;
+    const size_t src_off = ((size_t)tok * a.n_kv_heads + kvh) * D;
+    float* const row = rows[w];
+    // every global load of the wavefront (its row, the norm weight) is requested before the angles are computed, so the
+    // latencies overlap
+    float x[kRopeMaxPerLane], wt[kRopeMaxPerLane];
+    const bool normed = active && !is_v && a.weight != nullptr;
+    {
+        const float* src = (is_v ? a.v_src : a.k_src) + src_off;
+#pragma unroll
+        for (int j = 0; j < kRopeMaxPerLane; ++j) {
+            const uint32_t d = lane + j * kWave;
+            x[j] = (active && d < D) ? src[d] : 0.f;
+            wt[j] = (normed && d < D) ? a.weight[d] : 1.f;
+        }
+    }
+    // rope_funcs.glsl:63-67,97-101: theta = pos * theta_scale^p / freq_factor[p] * freq_scale, results scaled by attn_factor
+    if (blockIdx.y * kRopeWaves < a.n_kv_heads) {          // workgroup-uniform: workgroups that only hold V rows skip it
+        const float pos = (float)(a.positions ? a.positions[tok] : (int32_t)(a.pos0 + tok));
+        for (uint32_t p = tid; p < half; p += kRopeWaves * kWave) {
+            const float theta_base = pos * powf(a.theta_scale, (float)p);
+            const float ff = a.freq_factors ? a.freq_factors[p] : 1.0f;
+            const float theta = a.freq_scale * (theta_base / ff);
+            float sn, cs;
+            sincosf(theta, &sn, &cs);
+            cs_lds[p] = cs * a.attn_factor;
+            sn_lds[p] = sn * a.attn_factor;
+        }
+    }
+    __syncthreads();
+    if (!active) return;
+    if (normed) {                                          // rms_norm.comp:61-112: scale * x * w, f32
+        float ss = 0.f;
+#pragma unroll
+        for (int j = 0; j < kRopeMaxPerLane; ++j) ss = fmaf(x[j], x[j], ss);
+        ss = wave_sum_all(ss);
+        const float scale = 1.0f / sqrtf(ss / (float)D + a.eps);
+#pragma unroll
+        for (int j = 0; j < kRopeMaxPerLane; ++j) x[j] = (scale * x[j]) * wt[j];
+    }
+    // the LDS row is private to the wavefront and LDS operations of a wavefront execute in order, so the fences below only
+    // have to keep the compiler from moving accesses across them
+#pragma unroll
+    for (int j = 0; j < kRopeMaxPerLane; ++j) {
+        const uint32_t d = lane + j * kWave;
+        if (d < D) row[d] = x[j];
+    }
+    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+    if (!is_v) {
+        // rope_funcs.glsl:39-112: pair p of the rotary part is (2p, 2p + 1) in NORM mode, (p, p + n_dims / 2) in NEOX mode
+        for (uint32_t p = lane; p < half; p += kWave) {
+            const float cs = cs_lds[p], sn = sn_lds[p];
+            const uint32_t i0 = a.mode == 2u ? p : 2u * p, i1 = a.mode == 2u ? p + half : 2u * p + 1u;
+            const float x0 = row[i0], x1 = row[i1];
+            row[i0] = x0 * cs - x1 * sn;
+            row[i1] = x0 * sn + x1 * cs;
+        }
+        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+        if (a.k_out != nullptr)
+            for (uint32_t d = lane; d < D; d += kWave) a.k_out[src_off + d] = row[d];
+    }
+    // ---- the head's slice of the cache row as 32-bit words (kv_store_fp8.comp:42-67, kv_copy_fp16.comp:39-51)
+    uint8_t* dst = (is_v ? a.v_dst : a.k_dst) + (uint64_t)tok * a.row_bytes;
+    if (a.dtype == kF8) {
+        uint32_t* d32 = reinterpret_cast<uint32_t*>(dst + (size_t)kvh * D);
+        for (uint32_t e = lane; e < D / 4u; e += kWave)
+            d32[e] = pack4_e4m3(row[4 * e], row[4 * e + 1], row[4 * e + 2], row[4 * e + 3]);
+    } else if (a.dtype == kF16) {
+        uint32_t* d32 = reinterpret_cast<uint32_t*>(dst + (size_t)kvh * D * 2u);
+        for (uint32_t e = lane; e < D / 2u; e += kWave)
+            d32[e] = f32_to_h16_bits(row[2 * e]) | (f32_to_h16_bits(row[2 * e + 1]) << 16);
+    } else {
+        float* d32 = reinterpret_cast<float*>(dst + (size_t)kvh * D * 4u);
+        for (uint32_t d = lane; d < D; d += kWave) d32[d] = row[d];
+    }
+}
+
+hipError_t launch_rope_append(const RopeAppendLaunch& L, hipStream_t stream) {
+    if (L.n_tokens == 0u) return hipSuccess;
+    if (L.head_dim == 0u || L.head_dim > 512u || L.head_dim % 4u != 0u || L.rotary_dim > L.head_dim ||
+        L.rotary_dim % 2u != 0u || (L.mode != 0u && L.mode != 2u) || L.dtype > kF8 || L.n_kv_heads == 0u)
+        return hipErrorInvalidValue;
+    RopeAppendArgs a;
+    a.k_src = L.k_src; a.v_src = L.v_src; a.weight = L.weight; a.positions = L.positions;
+    a.freq_factors = L.freq_factors; a.k_out = L.k_out;
+    a.k_dst = (uint8_t*)L.k_dst; a.v_dst = (uint8_t*)L.v_dst;
+    a.n_kv_heads = L.n_kv_heads; a.head_dim = L.head_dim; a.rotary_dim = L.rotary_dim; a.mode = L.mode;
+    a.pos0 = L.pos0; a.dtype = L.dtype; a.row_bytes = L.row_bytes;
+    a.theta_scale = L.theta_scale; a.freq_scale = L.freq_scale; a.attn_factor = L.attn_factor; a.eps = L.eps;
+    const uint32_t n_units = L.v_src ? 2u * L.n_kv_heads : L.n_kv_heads;
+    if ((n_units + kRopeWaves - 1u) / kRopeWaves > 65535u) return hipErrorInvalidValue;
+    hipLaunchKernelGGL(rope_append_kernel, dim3(L.n_tokens, (n_units + kRopeWaves - 1u) / kRopeWaves), dim3(kRopeWaves * kWave),
+                       0, stream, a);
+    return hipGetLastError();
+}
+
+}  // namespace vfkv

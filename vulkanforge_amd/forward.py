@@ -93,6 +93,22 @@ class Forward:
         _ffi.check(_ffi.lib().vfkv_kv_write(self.kv_cache.handle, layer, base_pos, seq_len, _ptr(batch_k),
                                             _ptr(batch_v), _stream(stream)))
 
+    def step_k_rope_kv_write(self, layer: int, position: int, n_tokens: int, k_src, v_src, rotary_dim: int,
+                             theta_scale: float, k_norm_weight=None, positions=None, freq_factors=None,
+                             rope_mode: int = _ffi.ROPE_NEOX, freq_scale: float = 1.0, attn_factor: float = 1.0,
+                             eps: float = 1e-6, k_out=None, stream=None) -> None:
+        """step_k_norm_rope / step_k_rope followed by step_kv_write (executor/attention.rs:435-597; batch
+        :2040-2190) in one launch: K is RMS-normalised * ``k_norm_weight`` (None: plain RoPE), rotated and stored in
+        the cache dtype at ``position + t``; V is stored as ``step_kv_write`` stores it.  ``theta_scale`` =
+        (1 / freq_base)^(2 / rotary_dim) (layer_plan.rs:532).  ``k_out`` (may be ``k_src``) receives the rotated K."""
+        p = _ffi.RopeParams(rope_mode, rotary_dim, theta_scale, freq_scale, attn_factor, eps)
+        _ffi.check(_ffi.lib().vfkv_k_rope_kv_write(
+            self.kv_cache.handle, layer, position, n_tokens, _ptr(k_src), _ptr(v_src),
+            _ptr(k_norm_weight) if k_norm_weight is not None else None,
+            _ptr(positions) if positions is not None else None,
+            _ptr(freq_factors) if freq_factors is not None else None, C.byref(p),
+            _ptr(k_out) if k_out is not None else None, _stream(stream)))
+
     # ---- decode attention (runs.rs:722-822, 1463-1571) ----
     @staticmethod
     def run_flash_attn_split(q, k_layer, v_layer, kv_dtype, scratch_out, scratch_max, scratch_sum, n_heads,

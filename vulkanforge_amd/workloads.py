@@ -71,6 +71,31 @@ PREFILL = {
                                                      KvDtype.F8),
 }
 
+
+
+@dataclass(frozen=True)
+class RopeAppendWorkload:
+    """K RMS-norm * weight + RoPE + append of K and V, one launch per layer (the step in front of attention)."""
+    name: str
+    n_layers: int
+    n_kv_heads: int
+    head_dim: int
+    n_tokens: int           # rows appended per layer and step (1 = decode, chunk length = prefill)
+    base_pos: int
+    dtype: KvDtype
+
+    def bytes_step(self) -> int:
+        """Algorithmic bytes: K and V rows read as f32, written once in the cache dtype."""
+        return self.n_layers * 2 * self.n_tokens * self.n_kv_heads * self.head_dim * (4 + self.dtype.element_size())
+
+
+ROPE_APPEND = {
+    "k_rope_append_fp8_decode_32layers": RopeAppendWorkload("k_rope_append_fp8_decode_32layers", 32, 8, 128, 1, 8192,
+                                                            KvDtype.F8),
+    "k_rope_append_fp8_prefill_512_32layers": RopeAppendWorkload("k_rope_append_fp8_prefill_512_32layers", 32, 8, 128,
+                                                                 512, 4096, KvDtype.F8),
+}
+
 assert DECODE["decode_f16_2k_1layer"].kv_bytes_step() == 8_392_704
 assert DECODE["decode_fp8_8k_32layers"].kv_bytes_step() == 536_936_448
 assert DECODE["decode_fp8_32k_32layers"].kv_bytes_step() == 2_147_483_648

@@ -145,6 +145,18 @@ typedef struct {
     float eps;            /* rms_norm epsilon (cfg.rms_norm_eps); used only with a norm weight */
 } vfkv_rope_params;
 
+/* Forward::run_rms_norm_mul_rope (forward/runs.rs:2492-2600; rms_norm.comp:36-129 in its fused
+ * form) and, with `weight` NULL, Forward::run_rope_neox_with_pos_offset (runs.rs:647-720;
+ * rope_neox.comp / rope_norm.comp): `qk` is [m, heads_per_token, head_dim] f32; each (token, head)
+ * row is RMS-normalised, multiplied by weight[head_dim] and rotated with the token's position
+ * (positions[t], or pos0 + t when positions is NULL).  `qk_out` may alias `qk` (the production
+ * callers rotate in place).  This is the Q side (step_q_norm_rope / step_q_rope,
+ * executor/attention.rs:360-432,490-512); for K use vfkv_k_rope_kv_write, which also appends. */
+int vfkv_rms_norm_mul_rope(const float* qk, const float* weight, float* qk_out, uint32_t head_dim,
+                           uint32_t heads_per_token, uint32_t m, const int32_t* positions,
+                           uint32_t pos0, const float* freq_factors, const vfkv_rope_params* p,
+                           vfkv_stream stream);
+
 /* `KNormRope` or `KRope` followed by `KvWrite` (forward/layer_plan.rs:119-137) in one launch:
  * step_k_norm_rope / step_k_rope (executor/attention.rs:435-530; batch :2040-2075) =
  * run_rms_norm_mul_rope (forward/runs.rs:2492-2600, rms_norm.comp:36-129 fused with

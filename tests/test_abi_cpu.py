@@ -188,3 +188,17 @@ def test_k_rope_kv_write_rejects_bad_arguments():
     assert call(k=None) == -1 and call(v=None) == -1 and call(params=False) == -1
     assert call(fs=0.0) == -1
     cache.destroy()
+
+
+def test_rms_norm_mul_rope_rejects_bad_arguments():
+    L = _ffi.lib()
+    fake = 0x1000
+
+    def call(mode=_ffi.ROPE_NEOX, rot=128, hd=128, heads=32, m=1, fs=1.0, x=fake, out=fake, params=True):
+        p = _ffi.RopeParams(mode, rot, 0.9, fs, 1.0, 1e-6)
+        return L.vfkv_rms_norm_mul_rope(x, None, out, hd, heads, m, None, 0, None, C.byref(p) if params else None, None)
+
+    assert call(m=0) == 0 and call(heads=0) == 0
+    assert call(mode=24) == -4 and call(hd=1024, rot=64) == -4 and call(hd=130, rot=64) == -4
+    assert call(rot=129) == -1 and call(rot=256) == -1 and call(fs=-1.0) == -1
+    assert call(x=None) == -1 and call(out=None) == -1 and call(params=False) == -1

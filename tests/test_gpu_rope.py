@@ -188,3 +188,33 @@ def test_rotated_keys_feed_decode_attention():
     ref = oracle.attn_decode_ref(q, k16, v16, oracle.F16, h, hkv, d, seq, float(1 / np.sqrt(d)))
     assert np.abs(to_np(o) - ref).max() < 2e-3
     cache.destroy()
+
+
+@pytest.mark.parametrize("heads,d,m,rotary,mode,norm,in_place", (
+    (32, 128, 1, 128, _ffi.ROPE_NEOX, True, True),        # decode step_q_norm_rope
+    (32, 128, 512, 128, _ffi.ROPE_NEOX, True, False),     # prefill chunk
+    (16, 256, 7, 64, _ffi.ROPE_NEOX, False, True),        # plain RoPE, partial rotary (run_rope_neox_with_pos_offset)
+    (5, 96, 9, 96, _ffi.ROPE_NORM, True, False),
+))
+def test_rms_norm_mul_rope_matches_oracle(heads, d, m, rotary, mode, norm, in_place):
+    # the Q side of the fusion: forward/runs.rs:2492-2600 and :647-720
+    r = rng(heads * 1000 + d + m)
+    x = (r.standard_normal((m, heads, d)) * 1.5).astype(np.float32)
+    w = (1 + 0.2 * r.standard_normal(d)).astype(np.float32) if norm else None
+    pos = (4000 + np.arange(m) * 2).astype(np.int32)
+    ts = float(oracle.rope_theta_scale(1e6, rotary))
+    xd = to_dev(x)
+    out = xd if in_place else torch.full_like(xd, float("nan"))
+    vf.Forward.run_rms_norm_mul_rope(xd, to_dev(w) if norm else None, out, d, rotary, ts, heads, m, eps=1e-6,
+                                     positions=to_dev(pos), rope_mode=mode)
+    torch.cuda.synchronize()
+    ref = oracle.rms_norm_rope(x, pos, d, rotary, ts, mode=mode, weight=w, eps=1e-6)
+    got = to_np(out)
+    assert (np.abs(got - ref) <= k_tolerance(ref, pos)[:, None, None]).all(), float(np.abs(got - ref).max())
+    # implicit positions pos0 + t
+    out2 = torch.empty_like(out)
+    vf.Forward.run_rms_norm_mul_rope(to_dev(x), to_dev(w) if norm else None, out2, d, rotary, ts, heads, m, eps=1e-6,
+                                     pos0=77, rope_mode=mode)
+    torch.cuda.synchronize()
+    ref2 = oracle.rms_norm_rope(x, (77 + np.arange(m)).astype(np.int32), d, rotary, ts, mode=mode, weight=w, eps=1e-6)
+    assert (np.abs(to_np(out2) - ref2) <= k_tolerance(ref2, 77 + np.arange(m))[:, None, None]).all()

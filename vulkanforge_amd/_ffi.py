@@ -82,6 +82,7 @@ SIGNATURES = {
     "vfkv_copy_fp16": (C.c_int, [_vp, _vp, _u32, _u64, _vp]),
     "vfkv_fp8_to_f16": (C.c_int, [_vp, _vp, _u64, _vp]),
     "vfkv_kv_write": (C.c_int, [_vp, _u32, _u32, _u32, _vp, _vp, _vp]),
+    "vfkv_rms_norm_mul_rope": (C.c_int, [_vp, _vp, _vp, _u32, _u32, _u32, _vp, _u32, _vp, C.POINTER(RopeParams), _vp]),
     "vfkv_k_rope_kv_write": (C.c_int, [_vp, _u32, _u32, _u32, _vp, _vp, _vp, _vp, _vp, C.POINTER(RopeParams), _vp, _vp]),
     "vfkv_flash_attn_split": (C.c_int, [_vp, _vp, _vp, _u32, _vp, _vp, _vp, C.POINTER(SplitParams), _u32, _f, _vp]),
     "vfkv_flash_attn_split_interleaved": (C.c_int, [_vp, _vp, _vp, _u32, _vp, _vp, _vp, C.POINTER(SplitParams), _u32, _f, _vp]),

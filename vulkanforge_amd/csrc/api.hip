@@ -357,6 +357,29 @@ int vfkv_k_rope_kv_write(vfkv_cache* c, uint32_t layer, uint32_t pos, uint32_t n
     return VFKV_OK;
 }
 
+int vfkv_rms_norm_mul_rope(const float* qk, const float* weight, float* qk_out, uint32_t head_dim,
+                           uint32_t heads_per_token, uint32_t m, const int32_t* positions, uint32_t pos0,
+                           const float* freq_factors, const vfkv_rope_params* p, vfkv_stream stream) {
+    if (!p) return fail(VFKV_ERR_INVALID_ARG, "rms_norm_mul_rope: params is NULL");
+    if (m == 0 || heads_per_token == 0) return VFKV_OK;
+    if (!qk || !qk_out) return fail(VFKV_ERR_INVALID_ARG, "rms_norm_mul_rope: NULL buffer");
+    if (p->rope_mode != VFKV_ROPE_NORM && p->rope_mode != VFKV_ROPE_NEOX)
+        return fail(VFKV_ERR_UNSUPPORTED, "rms_norm_mul_rope: rope_mode %u (0 = NORM and 2 = NEOX are built)", p->rope_mode);
+    if (p->rotary_dim % 2u != 0u || p->rotary_dim > head_dim)
+        return fail(VFKV_ERR_INVALID_ARG, "rms_norm_mul_rope: rotary_dim %u must be even and <= head_dim %u", p->rotary_dim, head_dim);
+    if (head_dim == 0u || head_dim > 512u || head_dim % 4u != 0u)
+        return fail(VFKV_ERR_UNSUPPORTED, "rms_norm_mul_rope: head_dim %u (multiples of 4 up to 512 are built)", head_dim);
+    if (!(p->freq_scale > 0.f)) return fail(VFKV_ERR_INVALID_ARG, "rms_norm_mul_rope: freq_scale must be > 0");
+    if (heads_per_token > 65535u * 4u) return fail(VFKV_ERR_UNSUPPORTED, "rms_norm_mul_rope: %u heads per token", heads_per_token);
+    vfkv::RopeAppendLaunch L;
+    L.k_src = qk; L.weight = weight; L.positions = positions; L.freq_factors = freq_factors; L.k_out = qk_out;
+    L.dtype = vfkv::kF32; L.n_tokens = m; L.n_kv_heads = heads_per_token; L.head_dim = head_dim; L.rotary_dim = p->rotary_dim;
+    L.mode = p->rope_mode; L.pos0 = pos0;
+    L.theta_scale = p->theta_scale; L.freq_scale = p->freq_scale; L.attn_factor = p->attn_factor; L.eps = p->eps;
+    VFKV_HIP(vfkv::launch_rope_append(L, S(stream)));
+    return VFKV_OK;
+}
+
 // ---- decode attention ----------------------------------------------------------------------------------
 static int flash_attn_split_impl(const float* q, const void* k_layer, const void* v_layer, uint32_t kv_dtype,
                                  float* scratch_out, float* scratch_max, float* scratch_sum, const vfkv_split_params* p,

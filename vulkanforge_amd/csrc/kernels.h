@@ -18,7 +18,8 @@ struct RopeAppendLaunch {
     const int32_t* positions = nullptr;   // [n_tokens]; NULL = pos0 + token
     const float* freq_factors = nullptr;  // [rotary_dim / 2]; NULL = 1
     float* k_out = nullptr;               // rotated K as f32 (may alias k_src); NULL = not wanted
-    void* k_dst = nullptr;                // cache row of the first token (layer offset + pos0 * row_bytes applied)
+    void* k_dst = nullptr;                // cache row of the first token (layer offset + pos0 * row_bytes applied);
+                                          // NULL = no cache store: norm + RoPE into k_out only (v_src must be NULL too)
     void* v_dst = nullptr;
     uint32_t dtype = 0, n_tokens = 0, n_kv_heads = 0, head_dim = 0, rotary_dim = 0;
     uint32_t mode = 2;                    // 0 = NORM (adjacent pairs), 2 = NEOX (split halves)

@@ -24,7 +24,7 @@ struct RopeAppendArgs {
     const int32_t* positions; // [n_tokens] or NULL: pos0 + token
     const float* freq_factors;// [rotary_dim / 2] or NULL
     float* k_out;             // rotated K as f32 (may alias k_src) or NULL
-    uint8_t* k_dst;           // cache row of the first token, K
+    uint8_t* k_dst;           // cache row of the first token, K; NULL = no cache store (k_out only)
     uint8_t* v_dst;
     uint32_t n_kv_heads, head_dim, rotary_dim, mode, pos0, dtype;
     uint64_t row_bytes;       // distance between two tokens' rows in the cache
@@ -107,6 +107,7 @@ __global__ __launch_bounds__(kRopeWaves * kWave) void rope_append_kernel(RopeApp
         if (a.k_out != nullptr)
             for (uint32_t d = lane; d < D; d += kWave) a.k_out[src_off + d] = row[d];
     }
+    if (a.k_dst == nullptr) return;                        // norm + RoPE only (the Q side): no cache row to write
     // ---- the head's slice of the cache row as 32-bit words (kv_store_fp8.comp:42-67, kv_copy_fp16.comp:39-51)
     uint8_t* dst = (is_v ? a.v_dst : a.k_dst) + (uint64_t)tok * a.row_bytes;
     if (a.dtype == kF8) {

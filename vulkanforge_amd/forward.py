@@ -93,6 +93,18 @@ class Forward:
         _ffi.check(_ffi.lib().vfkv_kv_write(self.kv_cache.handle, layer, base_pos, seq_len, _ptr(batch_k),
                                             _ptr(batch_v), _stream(stream)))
 
+    @staticmethod
+    def run_rms_norm_mul_rope(qk, weight, qk_out, head_dim: int, rotary_dim: int, theta_scale: float,
+                              heads_per_token: int, m: int, eps: float = 1e-6, positions=None, pos0: int = 0,
+                              freq_factors=None, rope_mode: int = _ffi.ROPE_NEOX, freq_scale: float = 1.0,
+                              attn_factor: float = 1.0, stream=None) -> None:
+        """runs.rs:2492-2600 (``weight=None``: the plain run_rope_neox_with_pos_offset, runs.rs:647-720): per
+        (token, head) row RMS-norm * weight, then RoPE with the token's position.  ``qk_out`` may be ``qk``."""
+        p = _ffi.RopeParams(rope_mode, rotary_dim, theta_scale, freq_scale, attn_factor, eps)
+        _ffi.check(_ffi.lib().vfkv_rms_norm_mul_rope(_ptr(qk), _ptr(weight), _ptr(qk_out), head_dim, heads_per_token, m,
+                                                     _ptr(positions), pos0, _ptr(freq_factors), C.byref(p),
+                                                     _stream(stream)))
+
     def step_k_rope_kv_write(self, layer: int, position: int, n_tokens: int, k_src, v_src, rotary_dim: int,
                              theta_scale: float, k_norm_weight=None, positions=None, freq_factors=None,
                              rope_mode: int = _ffi.ROPE_NEOX, freq_scale: float = 1.0, attn_factor: float = 1.0,

@@ -85,6 +85,9 @@ def fill_cache(torch, vf, fwd, wl, n_tokens, seed, outliers):
 V_SKEW = int(os.environ.get("VFKV_BENCH_V_SKEW", "256"))
 
 
+STEP_SPREAD = {}   # filled by time_steps: percentiles of single event-timed steps, microseconds
+
+
 def time_steps(torch, step, args):
     """W untimed steps, then exactly K timed steps between two device synchronisations.  One step's
     launches are captured once into a HIP graph and replayed, so the host's per-launch cost (Python
@@ -108,7 +111,22 @@ def time_steps(torch, step, args):
     for _ in range(args.steps):
         run()
     torch.cuda.synchronize()
-    return (time.perf_counter() - t0) / args.steps
+    mean = (time.perf_counter() - t0) / args.steps
+    # spread of single steps: every replay bracketed by its own pair of events, after the timed region above
+    n = min(max(args.steps, 20), 200)
+    pairs = []
+    stream = torch.cuda.current_stream()
+    for _ in range(n):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record(stream)
+        run()
+        e1.record(stream)
+        pairs.append((e0, e1))
+    torch.cuda.synchronize()
+    us = sorted(e0.elapsed_time(e1) * 1e3 for e0, e1 in pairs)
+    STEP_SPREAD.clear()
+    STEP_SPREAD.update({"p10": us[n // 10], "p50": us[n // 2], "p90": us[(n * 9) // 10], "samples": n})
+    return mean
 
 
 def bench_decode(args, wl):
@@ -152,6 +170,7 @@ def bench_decode(args, wl):
                                     softcap=wl.softcap)
 
     sec_per_step = time_steps(torch, step, args)
+    step_spread = dict(STEP_SPREAD)
     bytes_step = wl.kv_bytes_step()
 
     # ---- duration of the split worker (the dominant kernel): its launches of one step, back to back on
@@ -209,6 +228,7 @@ def bench_decode(args, wl):
         "warmup": args.warmup,
         "ms_per_step": sec_per_step * 1e3,
         "us_per_decode_step": sec_per_step * 1e6,
+        "step_us_event_timed": step_spread,
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
@@ -289,6 +309,7 @@ def bench_prefill(args, wl):
             fwd.b_step_attention(layer, wl.base_pos, wl.m, q, o)
 
     sec_per_step = time_steps(torch, step, args)
+    step_spread = dict(STEP_SPREAD)
     flops_step = wl.flops_layer() * L
 
     stream = torch.cuda.current_stream()
@@ -308,6 +329,7 @@ def bench_prefill(args, wl):
         "value": flops_step / sec_per_step / 1e12,
         "unit": "TFLOP/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": sec_per_step * 1e3,
+        "step_us_event_timed": step_spread,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f16", "kv_dtype": wl.dtype.label(),
         "data": "synthetic, seeded N(0,1); queries " + ("general f32" if args.f32_queries else "cast to fp16 as the configuration states") + "; K/V rows cast to fp16 and written through the append kernels",
         "config": {"workload": wl.name, "n_layers": L, "n_heads": H, "n_kv_heads": Hkv, "head_dim": D,

@@ -1,7 +1,8 @@
 // Self-test of the C++ host layer: layout arithmetic without a device, then (with a GPU) one FP8
 // append + decode step checked against closed forms that need no reference implementation:
 //   * K = 0 makes every weight equal, so O = mean of the decoded V rows;
-//   * one key far larger than the rest makes O equal that key's decoded V row.
+//   * one key far larger than the rest makes O equal that key's decoded V row;
+//   * RoPE with theta_scale = 1 turns every (1, 0) pair into (cos pos, sin pos).
 #include <hip/hip_runtime.h>
 
 #include <cmath>
@@ -65,6 +66,28 @@ int main() {
     for (uint32_t h = 0; h < H; ++h) for (uint32_t d = 0; d < D; ++d) worst = std::fmax(worst, std::fabs(o[h * D + d] - v[123 * row + (h / 4) * D + d]));
     std::printf("dominant-key decode: max |O - V[123]| = %.3g\n", worst);
     REQUIRE(worst < 1e-6);
+    // K RoPE + append, closed forms: with theta_scale = 1 every pair turns by `position` radians.  A key whose pairs are
+    // (1, 0) scores sum(cos(pos)) * ... against q = 1 on the first halves only: use it through the F8 cache-free check of k_out.
+    {
+        std::vector<float> kr(row), kout(row);
+        for (size_t x = 0; x < row; ++x) kr[x] = (x % D) < D / 2 ? 1.0f : 0.0f;           // every NEOX pair = (1, 0)
+        float* dko; hipMalloc(&dko, row * 4);
+        hipMemcpy(dk, kr.data(), row * 4, hipMemcpyHostToDevice);
+        vfkv_rope_params rp{VFKV_ROPE_NEOX, D, 1.0f, 1.0f, 1.0f, 1e-6f};
+        for (uint32_t pos : {0u, 3u}) {
+            fwd.step_k_rope_kv_write(0, pos, 1, dk, dv, nullptr, rp, nullptr, nullptr, dko);
+            hipDeviceSynchronize();
+            hipMemcpy(kout.data(), dko, row * 4, hipMemcpyDeviceToHost);
+            double w2 = 0;
+            for (size_t x = 0; x < row; ++x) {
+                const double want = (x % D) < D / 2 ? std::cos((double)pos) : std::sin((double)pos);
+                w2 = std::fmax(w2, std::fabs(kout[x] - want));
+            }
+            std::printf("rope (1,0) pairs at position %u: max |k - (cos, sin)| = %.3g\n", pos, w2);
+            REQUIRE(w2 < 1e-6);
+        }
+        hipFree(dko);
+    }
     bool threw = false;
     try { fwd.step_attention(1, ctx + 1, dq, dout); } catch (const Error& e) { threw = e.status == VFKV_ERR_INVALID_ARG; }
     REQUIRE(threw);

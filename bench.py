@@ -35,8 +35,8 @@ MFMA_F16_PEAK_TFLOPS = 2500.0
 # (two runs) and scaled by what the same counters read for a plain 64 MiB device copy
 # (FETCH_SIZE x 1.9991, WRITE_SIZE x 1.0 to KiB).  Only the workloads that were profiled have an entry.
 MEASURED_TRAFFIC_BYTES = {
-    "decode_fp8_32k_32layers": (65635 + 520) * 1024,
-    "prefill_fp8_512x4608_32layers": (81365 + 8192) * 1024,
+    "decode_fp8_32k_32layers": (65634 + 520) * 1024,
+    "prefill_fp8_512x4608_32layers": (81369 + 8192) * 1024,
 }
 
 

@@ -1,7 +1,13 @@
 // Split-K decode attention for gfx950: worker (flash_attn_split.comp:82-162) and log-sum-exp
 // merge (flash_attn_reduce.comp:35-81), re-designed around the HBM stream.
 //
-// Worker.  One workgroup (NW wavefronts) owns one (tile of keys, KV head, group of GT query heads);
+//   split_mfma_kernel    (attn_decode_mfma.h) matrix-core worker: FP8 / F16 caches, head_dim 64 / 128 / 256 -- the
+//                        kernel every benchmark configuration runs on
+//   split_kernel         vector-ALU worker described below: F32 caches and head_dim 512
+//   split_generic_kernel one wavefront per (head, tile), any dtype, head_dim <= 512
+//   reduce_direct_kernel merge of up to 64 partials per head without LDS; reduce_kernel / reduce_generic_kernel beyond
+//
+// Vector-ALU worker.  One workgroup (NW wavefronts) owns one (tile of keys, KV head, group of GT query heads);
 // every K / V byte of the tile is requested from memory once and serves all GT heads of the GQA
 // group.  Each wavefront walks its share of the tile in runs of 64 rows:
 //

@@ -1,9 +1,11 @@
 // Matrix-core worker of the split-K decode attention (flash_attn_split.comp:82-162) for gfx950;
 // included by attn_decode.hip.
 //
-// One workgroup (NW wavefronts) owns one (tile of keys, KV head, slice of up to 8 query heads of the
-// GQA group); every K / V byte of the tile is requested from memory once and serves all heads of the
-// slice.  Each wavefront walks its share of the tile in runs of RUN rows and keeps both products on
+// One workgroup (NW wavefronts) owns one (share of the keys, KV head, slice of up to 8 query heads of the
+// GQA group); every K / V byte is requested from memory once and serves all heads of the slice.  The
+// share is either one tile of consecutive keys (partial j = tile j, the reference's meaning) or, in
+// interleaved mode, every n_tiles-th group of NW runs of the visible span.  Each wavefront walks its
+// runs of RUN rows and keeps both products on
 // v_mfma_f32_16x16x32_f16 (f32 accumulation), so the vector ALU only converts FP8, does the softmax
 // and packs the weights:
 //

@@ -64,6 +64,8 @@ CASES = [
     (vf.KvDtype.F8, 32, 2, 128, 700, 1024, 0, 0.0),   # G = 16: two slices of 8 heads, one ragged tile
     (vf.KvDtype.F8, 24, 2, 128, 1300, 448, 5, 0.0),   # G = 12: slices of 8 and 4 heads
     (vf.KvDtype.F8, 32, 8, 128, 3000, 1024, 1900, 0.0),  # window starting inside a tile, several runs per wavefront
+    (vf.KvDtype.F8, 32, 8, 128, 333, 16, 40, 0.0),       # tiles shorter than a run of the matrix-core worker
+    (vf.KvDtype.F16, 16, 8, 64, 1000, 48, 0, 0.0),       # tile not a multiple of the run length
     (vf.KvDtype.F16, 20, 4, 128, 1111, 320, 0, 20.0), # G = 5 with soft-cap
     (vf.KvDtype.F16, 32, 8, 128, 2049, 512, 0, 0.0),
     (vf.KvDtype.F16, 16, 8, 256, 1500, 256, 0, 50.0),

@@ -102,7 +102,10 @@ hipError_t launch_batch(const BatchLaunch& L, hipStream_t stream) {
     if (mfma_ok && v2_on && L.head_dim <= 128u) {
         // two heads per wavefront where the registers allow it
         static const int force_ncb = [] { const char* e = getenv("VFKV_PREFILL_NCB"); return e ? atoi(e) : 0; }();
-        uint32_t ncb = (g % 2u == 0u && (L.head_dim == 64u || (L.head_dim == 128u && L.dtype == kF8))) ? 2u : 1u;
+#ifndef VFKV_PREFILL_F16_128_NCB
+#define VFKV_PREFILL_F16_128_NCB 2     // heads per wavefront, F16 cache, head_dim 128 (even GQA groups)
+#endif
+        uint32_t ncb = (g % 2u == 0u && (L.head_dim == 64u || (L.head_dim == 128u && (L.dtype == kF8 || VFKV_PREFILL_F16_128_NCB == 2)))) ? 2u : 1u;
         if (force_ncb == 1) ncb = 1u;
         const uint32_t hp = g / ncb;
         if (hp <= 8u) {
@@ -122,7 +125,7 @@ hipError_t launch_batch(const BatchLaunch& L, hipStream_t stream) {
         else hipLaunchKernelGGL((batch_mfma2_kernel<DT, DD, NCBV, PFDV, false>), grid, block, lds, stream, a, (int)hp, (int)ns);      \
     } else
             VFKV_P2(kF8, 64, 2, 2) VFKV_P2(kF8, 64, 1, 2) VFKV_P2(kF8, 128, 2, 2) VFKV_P2(kF8, 128, 1, 2)
-            VFKV_P2(kF16, 64, 2, 2) VFKV_P2(kF16, 64, 1, 2) VFKV_P2(kF16, 128, 1, 1)
+            VFKV_P2(kF16, 64, 2, 2) VFKV_P2(kF16, 64, 1, 2) VFKV_P2(kF16, 128, 1, 1) VFKV_P2(kF16, 128, 2, 1)
             { launched = false; }
 #undef VFKV_P2
             if (launched) return hipGetLastError();

@@ -69,6 +69,9 @@ DECODE = {
 PREFILL = {
     "prefill_fp8_512x4608_32layers": PrefillWorkload("prefill_fp8_512x4608_32layers", 32, 32, 8, 128, 4096, 512,
                                                      KvDtype.F8),
+    # the same geometry over an F16 cache (not one of the reference configurations; used to tune the F16 variant)
+    "prefill_f16_512x4608_32layers": PrefillWorkload("prefill_f16_512x4608_32layers", 32, 32, 8, 128, 4096, 512,
+                                                     KvDtype.F16),
 }
 
 

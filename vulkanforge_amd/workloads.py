@@ -62,6 +62,8 @@ DECODE = {
     "decode_f16_2k_1layer": DecodeWorkload("decode_f16_2k_1layer", 1, 32, 8, 128, 2049, KvDtype.F16, True),
     "decode_fp8_8k_32layers": DecodeWorkload("decode_fp8_8k_32layers", 32, 32, 8, 128, 8193, KvDtype.F8, True),
     "decode_fp8_32k_32layers": DecodeWorkload("decode_fp8_32k_32layers", 32, 32, 8, 128, 32768, KvDtype.F8, False),
+    # the headline geometry over an F16 cache (not one of the reference configurations; used to tune the F16 variant)
+    "decode_f16_32k_32layers": DecodeWorkload("decode_f16_32k_32layers", 32, 32, 8, 128, 32768, KvDtype.F16, False),
     "decode_f16_hd256_sliding_12layers": DecodeWorkload("decode_f16_hd256_sliding_12layers", 12, 16, 8, 256, 16384,
                                                         KvDtype.F16, False, softcap=50.0, window=4096,
                                                         sliding_pattern=5),

@@ -158,7 +158,7 @@ int vfkv_rms_norm_mul_rope(const float* qk, const float* weight, float* qk_out, 
                            vfkv_stream stream);
 
 /* `KNormRope` or `KRope` followed by `KvWrite` (forward/layer_plan.rs:119-137) in one launch:
- * step_k_norm_rope / step_k_rope (executor/attention.rs:435-530; batch :2040-2075) =
+ * step_k_norm_rope / step_k_rope (executor/attention.rs:435-530; batch :2026-2133) =
  * run_rms_norm_mul_rope (forward/runs.rs:2492-2600, rms_norm.comp:36-129 fused with
  * rope_funcs.glsl:39-112) or run_rope_neox_with_pos_offset (runs.rs:647-720), then step_kv_write
  * (attention.rs:546-597).  K rows [n_tokens, kv_heads * head_dim] f32 are RMS-normalised per head

@@ -110,7 +110,7 @@ class Forward:
                              rope_mode: int = _ffi.ROPE_NEOX, freq_scale: float = 1.0, attn_factor: float = 1.0,
                              eps: float = 1e-6, k_out=None, stream=None) -> None:
         """step_k_norm_rope / step_k_rope followed by step_kv_write (executor/attention.rs:435-597; batch
-        :2040-2190) in one launch: K is RMS-normalised * ``k_norm_weight`` (None: plain RoPE), rotated and stored in
+        :2026-2190) in one launch: K is RMS-normalised * ``k_norm_weight`` (None: plain RoPE), rotated and stored in
         the cache dtype at ``position + t``; V is stored as ``step_kv_write`` stores it.  ``theta_scale`` =
         (1 / freq_base)^(2 / rotary_dim) (layer_plan.rs:532).  ``k_out`` (may be ``k_src``) receives the rotated K."""
         p = _ffi.RopeParams(rope_mode, rotary_dim, theta_scale, freq_scale, attn_factor, eps)

@@ -137,7 +137,7 @@ public:
         check(vfkv_kv_write(kv_cache.handle(), layer, base_pos, seq_len, batch_k, batch_v, stream));
     }
 
-    // step_k_norm_rope / step_k_rope + step_kv_write (attention.rs:435-597, batch :2040-2190) in one launch;
+    // step_k_norm_rope / step_k_rope + step_kv_write (attention.rs:435-597, batch :2026-2190) in one launch;
     // k_norm_weight == nullptr is the plain KRope
     void step_k_rope_kv_write(uint32_t layer, uint32_t position, uint32_t n_tokens, const float* k_src, const float* v_src,
                               const float* k_norm_weight, const vfkv_rope_params& rope, const int32_t* positions = nullptr,

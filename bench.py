@@ -394,8 +394,18 @@ def bench_rope_append(args, wl):
         for layer in range(L):
             fwd.b_step_kv_write(layer, wl.base_pos, T, k[layer], v[layer])
 
+    H = 4 * Hkv                                      # query heads of the same token rows (GQA group of 4)
+    qq = torch.randn((L, T, H * D), device=dev, generator=g)
+    fwd_q = vf.Forward(cache, H)
+
+    def qk():                                        # the Q rows in the same launch (QNormRope + KNormRope + KvWrite)
+        for layer in range(L):
+            fwd_q.step_qk_rope_kv_write(layer, wl.base_pos, T, qq[layer], k[layer], v[layer], D, theta_scale,
+                                        q_norm_weight=w, k_norm_weight=w)
+
     sec = time_steps(torch, step, args)
     sec_plain = time_steps(torch, plain, args)
+    sec_qk = time_steps(torch, qk, args)
     step()
     torch.cuda.synchronize()
     result = {
@@ -405,7 +415,8 @@ def bench_rope_append(args, wl):
         "data": "synthetic, seeded N(0,1)",
         "config": {"workload": wl.name, "n_layers": L, "n_kv_heads": Hkv, "head_dim": D, "tokens_per_layer": T,
                    "base_pos": wl.base_pos, "bytes_per_step": wl.bytes_step(),
-                   "plain_append_us_per_launch": sec_plain * 1e6 / L},
+                   "plain_append_us_per_launch": sec_plain * 1e6 / L,
+                   "with_32_query_heads_us_per_launch": sec_qk * 1e6 / L},
         "roofline": {"bound": "hbm", "kernel": "rope_append_kernel", "achieved": wl.bytes_step() / sec / 1e9,
                      "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": wl.bytes_step() / sec / 1e9 / HBM_PEAK_GBPS,
                      "traffic": None, "avg_launch_us": sec * 1e6 / L},

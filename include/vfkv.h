@@ -173,6 +173,17 @@ int vfkv_k_rope_kv_write(vfkv_cache* c, uint32_t layer, uint32_t pos, uint32_t n
                          const int32_t* positions, const float* freq_factors,
                          const vfkv_rope_params* p, float* k_out, vfkv_stream stream);
 
+/* The same launch with the query rows added: `QNormRope` / `QRope` + `KNormRope` / `KRope` + `KvWrite`
+ * of one layer (forward/layer_plan.rs:119-137; step_q_norm_rope, step_k_norm_rope, step_kv_write,
+ * executor/attention.rs:360-597) as ONE launch.  `q` is [n_tokens, n_heads, head_dim] f32 and is
+ * RMS-normalised * q_norm_weight (NULL: no norm) and rotated with the same angles into `q_out`
+ * (may alias `q`); K, V and the remaining arguments are those of vfkv_k_rope_kv_write. */
+int vfkv_qk_rope_kv_write(vfkv_cache* c, uint32_t layer, uint32_t pos, uint32_t n_tokens,
+                          uint32_t n_heads, const float* q, const float* q_norm_weight, float* q_out,
+                          const float* k_src, const float* v_src, const float* k_norm_weight,
+                          const int32_t* positions, const float* freq_factors,
+                          const vfkv_rope_params* p, float* k_out, vfkv_stream stream);
+
 /* ------------------------------------------------------------------------------------------ */
 /* Decode attention: split-K worker + log-sum-exp merge.                                      */
 /* ------------------------------------------------------------------------------------------ */

@@ -187,6 +187,11 @@ def test_k_rope_kv_write_rejects_bad_arguments():
     assert call(layer=2) == -1 and call(pos=64) == -1 and call(pos=60, n=5) == -1
     assert call(k=None) == -1 and call(v=None) == -1 and call(params=False) == -1
     assert call(fs=0.0) == -1
+    p = _ffi.RopeParams(_ffi.ROPE_NEOX, 128, 0.9, 1.0, 1.0, 1e-6)
+    assert L.vfkv_qk_rope_kv_write(cache.handle, 0, 0, 1, 32, None, None, fake, fake, fake, None, None, None, C.byref(p),
+                                   None, None) == -1          # NULL query
+    assert L.vfkv_qk_rope_kv_write(cache.handle, 0, 0, 1, 0, fake, None, fake, fake, fake, None, None, None, C.byref(p),
+                                   None, None) == -1          # no heads
     cache.destroy()
 
 

@@ -218,3 +218,36 @@ def test_rms_norm_mul_rope_matches_oracle(heads, d, m, rotary, mode, norm, in_pl
     torch.cuda.synchronize()
     ref2 = oracle.rms_norm_rope(x, (77 + np.arange(m)).astype(np.int32), d, rotary, ts, mode=mode, weight=w, eps=1e-6)
     assert (np.abs(to_np(out2) - ref2) <= k_tolerance(ref2, 77 + np.arange(m))[:, None, None]).all()
+
+
+@pytest.mark.parametrize("dtype,h,hkv,d,m,pos0", ((vf.KvDtype.F8, 32, 8, 128, 1, 8192), (vf.KvDtype.F16, 16, 8, 256, 40, 100),
+                                                  (vf.KvDtype.F8, 6, 3, 64, 9, 0)))
+def test_qk_rope_kv_write_is_the_two_calls_in_one(dtype, h, hkv, d, m, pos0):
+    # Q rows ride in the same launch: bit-identical to vfkv_rms_norm_mul_rope + vfkv_k_rope_kv_write
+    r = rng(h * 31 + d + m)
+    q = (r.standard_normal((m, h, d)) * 1.2).astype(np.float32)
+    k = (r.standard_normal((m, hkv, d)) * 1.2).astype(np.float32)
+    v = fp16_normal(r, (m, hkv, d))
+    wq = (1 + 0.1 * r.standard_normal(d)).astype(np.float32)
+    wk = (1 + 0.1 * r.standard_normal(d)).astype(np.float32)
+    ts = float(oracle.rope_theta_scale(1e6, d))
+    a = vf.KvCache(vf.KvCacheConfig(1, hkv, d, pos0 + m, dtype=dtype))
+    b = vf.KvCache(vf.KvCacheConfig(1, hkv, d, pos0 + m, dtype=dtype))
+    a.zero_fill(); b.zero_fill()
+    qa, qb = to_dev(q), to_dev(q)
+    ka = torch.empty((m, hkv, d), device=DEV)
+    kb = torch.empty((m, hkv, d), device=DEV)
+    vf.Forward(a, h).step_qk_rope_kv_write(0, pos0, m, qa, to_dev(k), to_dev(v), d, ts, q_norm_weight=to_dev(wq),
+                                           k_norm_weight=to_dev(wk), k_out=ka)
+    fb = vf.Forward(b, h)
+    fb.run_rms_norm_mul_rope(qb, to_dev(wq), qb, d, d, ts, h, m, pos0=pos0)
+    fb.step_k_rope_kv_write(0, pos0, m, to_dev(k), to_dev(v), d, ts, k_norm_weight=to_dev(wk), k_out=kb)
+    torch.cuda.synchronize()
+    n = a.bytes_per_buffer()
+    assert (read_device(a.k_ptr, n) == read_device(b.k_ptr, n)).all()
+    assert (read_device(a.v_ptr, n) == read_device(b.v_ptr, n)).all()
+    assert (to_np(qa) == to_np(qb)).all() and (to_np(ka) == to_np(kb)).all()
+    pos = (pos0 + np.arange(m)).astype(np.int32)
+    q_ref = oracle.rms_norm_rope(q, pos, d, d, ts, weight=wq, eps=1e-6)
+    assert (np.abs(to_np(qa) - q_ref) <= k_tolerance(q_ref, pos)[:, None, None]).all()
+    a.destroy(); b.destroy()

@@ -83,6 +83,8 @@ SIGNATURES = {
     "vfkv_fp8_to_f16": (C.c_int, [_vp, _vp, _u64, _vp]),
     "vfkv_kv_write": (C.c_int, [_vp, _u32, _u32, _u32, _vp, _vp, _vp]),
     "vfkv_rms_norm_mul_rope": (C.c_int, [_vp, _vp, _vp, _u32, _u32, _u32, _vp, _u32, _vp, C.POINTER(RopeParams), _vp]),
+    "vfkv_qk_rope_kv_write": (C.c_int, [_vp, _u32, _u32, _u32, _u32, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp,
+                                        C.POINTER(RopeParams), _vp, _vp]),
     "vfkv_k_rope_kv_write": (C.c_int, [_vp, _u32, _u32, _u32, _vp, _vp, _vp, _vp, _vp, C.POINTER(RopeParams), _vp, _vp]),
     "vfkv_flash_attn_split": (C.c_int, [_vp, _vp, _vp, _u32, _vp, _vp, _vp, C.POINTER(SplitParams), _u32, _f, _vp]),
     "vfkv_flash_attn_split_interleaved": (C.c_int, [_vp, _vp, _vp, _u32, _vp, _vp, _vp, C.POINTER(SplitParams), _u32, _f, _vp]),

@@ -327,9 +327,10 @@ int vfkv_kv_write(vfkv_cache* c, uint32_t layer, uint32_t pos, uint32_t n_tokens
     return VFKV_OK;
 }
 
-int vfkv_k_rope_kv_write(vfkv_cache* c, uint32_t layer, uint32_t pos, uint32_t n_tokens, const float* k_src,
-                         const float* v_src, const float* k_norm_weight, const int32_t* positions,
-                         const float* freq_factors, const vfkv_rope_params* p, float* k_out, vfkv_stream stream) {
+static int rope_kv_write_impl(vfkv_cache* c, uint32_t layer, uint32_t pos, uint32_t n_tokens, const float* q, uint32_t n_heads,
+                              const float* q_norm_weight, float* q_out, const float* k_src, const float* v_src,
+                              const float* k_norm_weight, const int32_t* positions, const float* freq_factors,
+                              const vfkv_rope_params* p, float* k_out, vfkv_stream stream) {
     if (!c || !c->k || !c->v) return fail(VFKV_ERR_INVALID_ARG, "k_rope_kv_write: cache has no buffers");
     if (!p) return fail(VFKV_ERR_INVALID_ARG, "k_rope_kv_write: params is NULL");
     if (layer >= c->n_layers) return fail(VFKV_ERR_INVALID_ARG, "k_rope_kv_write: layer %u out of range", layer);
@@ -349,12 +350,30 @@ int vfkv_k_rope_kv_write(vfkv_cache* c, uint32_t layer, uint32_t pos, uint32_t n
     const uint64_t off = layer_off(c, layer) + (uint64_t)pos * row_b(c, layer);
     vfkv::RopeAppendLaunch L;
     L.k_src = k_src; L.v_src = v_src; L.weight = k_norm_weight; L.positions = positions; L.freq_factors = freq_factors;
+    L.q_src = q; L.q_weight = q_norm_weight; L.q_out = q_out; L.n_q_heads = q ? n_heads : 0u;
     L.k_out = k_out; L.k_dst = (char*)c->k + off; L.v_dst = (char*)c->v + off;
     L.dtype = c->dtype; L.n_tokens = n_tokens; L.n_kv_heads = kvh; L.head_dim = hd; L.rotary_dim = p->rotary_dim;
     L.mode = p->rope_mode; L.pos0 = pos; L.row_bytes = row_b(c, layer);
     L.theta_scale = p->theta_scale; L.freq_scale = p->freq_scale; L.attn_factor = p->attn_factor; L.eps = p->eps;
     VFKV_HIP(vfkv::launch_rope_append(L, S(stream)));
     return VFKV_OK;
+}
+
+int vfkv_k_rope_kv_write(vfkv_cache* c, uint32_t layer, uint32_t pos, uint32_t n_tokens, const float* k_src,
+                         const float* v_src, const float* k_norm_weight, const int32_t* positions,
+                         const float* freq_factors, const vfkv_rope_params* p, float* k_out, vfkv_stream stream) {
+    return rope_kv_write_impl(c, layer, pos, n_tokens, nullptr, 0, nullptr, nullptr, k_src, v_src, k_norm_weight, positions,
+                              freq_factors, p, k_out, stream);
+}
+
+int vfkv_qk_rope_kv_write(vfkv_cache* c, uint32_t layer, uint32_t pos, uint32_t n_tokens, uint32_t n_heads, const float* q,
+                          const float* q_norm_weight, float* q_out, const float* k_src, const float* v_src,
+                          const float* k_norm_weight, const int32_t* positions, const float* freq_factors,
+                          const vfkv_rope_params* p, float* k_out, vfkv_stream stream) {
+    if (n_tokens != 0 && (!q || !q_out)) return fail(VFKV_ERR_INVALID_ARG, "qk_rope_kv_write: NULL query buffer");
+    if (n_heads == 0) return fail(VFKV_ERR_INVALID_ARG, "qk_rope_kv_write: n_heads must be > 0");
+    return rope_kv_write_impl(c, layer, pos, n_tokens, q, n_heads, q_norm_weight, q_out, k_src, v_src, k_norm_weight, positions,
+                              freq_factors, p, k_out, stream);
 }
 
 int vfkv_rms_norm_mul_rope(const float* qk, const float* weight, float* qk_out, uint32_t head_dim,

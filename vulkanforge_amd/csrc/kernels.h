@@ -12,6 +12,10 @@ hipError_t launch_fp8_to_f16(const void* src, void* dst, uint64_t n, hipStream_t
 
 // K RMS-norm * weight + RoPE + append of K and V rows in one launch (rope_append.hip).
 struct RopeAppendLaunch {
+    const float* q_src = nullptr;         // optional Q rows [n_tokens][n_q_heads][head_dim]: normed * q_weight, rotated -> q_out
+    const float* q_weight = nullptr;
+    float* q_out = nullptr;
+    uint32_t n_q_heads = 0;
     const float* k_src = nullptr;         // [n_tokens][n_kv_heads][head_dim]
     const float* v_src = nullptr;         // same shape; NULL = K only
     const float* weight = nullptr;        // [head_dim]; NULL = no RMS-norm

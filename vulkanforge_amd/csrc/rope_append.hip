@@ -18,6 +18,10 @@
 namespace vfkv {
 
 struct RopeAppendArgs {
+    const float* q_src;       // [n_tokens][n_q_heads][head_dim] or NULL: no Q rows in this launch
+    const float* q_weight;    // [head_dim] or NULL
+    float* q_out;             // rotated Q (may alias q_src)
+    uint32_t n_q_heads;
     const float* k_src;       // [n_tokens][n_kv_heads][head_dim]
     const float* v_src;       // same shape, or NULL: K only
     const float* weight;      // [head_dim] or NULL: no RMS-norm
@@ -42,28 +46,32 @@ __global__ __launch_bounds__(kRopeWaves * kWave) void rope_append_kernel(RopeApp
     const uint32_t tok = blockIdx.x;
     const uint32_t D = a.head_dim;
     const uint32_t half = a.rotary_dim / 2u;
-    const uint32_t n_units = a.v_src ? 2u * a.n_kv_heads : a.n_kv_heads;   // (tensor, head) rows of this token
+    // rows of this token: the Q heads (if any), then the K heads, then the V heads (if any)
+    const uint32_t nq = a.q_src ? a.n_q_heads : 0u;
+    const uint32_t n_units = nq + (a.v_src ? 2u * a.n_kv_heads : a.n_kv_heads);
     const uint32_t u = blockIdx.y * kRopeWaves + w;                         // this wavefront's row
     const bool active = u < n_units;
-    const bool is_v = u >= a.n_kv_heads;
-    const uint32_t kvh = is_v ? u - a.n_kv_heads : u;
-    const size_t src_off = ((size_t)tok * a.n_kv_heads + kvh) * D;
+    const bool is_q = u < nq;
+    const bool is_v = u >= nq + a.n_kv_heads;
+    const uint32_t head = is_q ? u : (is_v ? u - nq - a.n_kv_heads : u - nq);
+    const size_t src_off = ((size_t)tok * (is_q ? nq : a.n_kv_heads) + head) * D;
     float* const row = rows[w];
     // every global load of the wavefront (its row, the norm weight) is requested before the angles are computed, so the
     // latencies overlap
     float x[kRopeMaxPerLane], wt[kRopeMaxPerLane];
-    const bool normed = active && !is_v && a.weight != nullptr;
+    const float* const weight = is_q ? a.q_weight : a.weight;
+    const bool normed = active && !is_v && weight != nullptr;
     {
-        const float* src = (is_v ? a.v_src : a.k_src) + src_off;
+        const float* src = (is_q ? a.q_src : is_v ? a.v_src : a.k_src) + src_off;
 #pragma unroll
         for (int j = 0; j < kRopeMaxPerLane; ++j) {
             const uint32_t d = lane + j * kWave;
             x[j] = (active && d < D) ? src[d] : 0.f;
-            wt[j] = (normed && d < D) ? a.weight[d] : 1.f;
+            wt[j] = (normed && d < D) ? weight[d] : 1.f;
         }
     }
     // rope_funcs.glsl:63-67,97-101: theta = pos * theta_scale^p / freq_factor[p] * freq_scale, results scaled by attn_factor
-    if (blockIdx.y * kRopeWaves < a.n_kv_heads) {          // workgroup-uniform: workgroups that only hold V rows skip it
+    if (blockIdx.y * kRopeWaves < nq + a.n_kv_heads) {     // workgroup-uniform: workgroups that only hold V rows skip it
         const float pos = (float)(a.positions ? a.positions[tok] : (int32_t)(a.pos0 + tok));
         for (uint32_t p = tid; p < half; p += kRopeWaves * kWave) {
             const float theta_base = pos * powf(a.theta_scale, (float)p);
@@ -104,22 +112,23 @@ __global__ __launch_bounds__(kRopeWaves * kWave) void rope_append_kernel(RopeApp
             row[i1] = x0 * sn + x1 * cs;
         }
         __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
-        if (a.k_out != nullptr)
-            for (uint32_t d = lane; d < D; d += kWave) a.k_out[src_off + d] = row[d];
+        float* const out = is_q ? a.q_out : a.k_out;
+        if (out != nullptr)
+            for (uint32_t d = lane; d < D; d += kWave) out[src_off + d] = row[d];
     }
-    if (a.k_dst == nullptr) return;                        // norm + RoPE only (the Q side): no cache row to write
+    if (is_q || a.k_dst == nullptr) return;                // norm + RoPE only: no cache row to write
     // ---- the head's slice of the cache row as 32-bit words (kv_store_fp8.comp:42-67, kv_copy_fp16.comp:39-51)
     uint8_t* dst = (is_v ? a.v_dst : a.k_dst) + (uint64_t)tok * a.row_bytes;
     if (a.dtype == kF8) {
-        uint32_t* d32 = reinterpret_cast<uint32_t*>(dst + (size_t)kvh * D);
+        uint32_t* d32 = reinterpret_cast<uint32_t*>(dst + (size_t)head * D);
         for (uint32_t e = lane; e < D / 4u; e += kWave)
             d32[e] = pack4_e4m3(row[4 * e], row[4 * e + 1], row[4 * e + 2], row[4 * e + 3]);
     } else if (a.dtype == kF16) {
-        uint32_t* d32 = reinterpret_cast<uint32_t*>(dst + (size_t)kvh * D * 2u);
+        uint32_t* d32 = reinterpret_cast<uint32_t*>(dst + (size_t)head * D * 2u);
         for (uint32_t e = lane; e < D / 2u; e += kWave)
             d32[e] = f32_to_h16_bits(row[2 * e]) | (f32_to_h16_bits(row[2 * e + 1]) << 16);
     } else {
-        float* d32 = reinterpret_cast<float*>(dst + (size_t)kvh * D * 4u);
+        float* d32 = reinterpret_cast<float*>(dst + (size_t)head * D * 4u);
         for (uint32_t d = lane; d < D; d += kWave) d32[d] = row[d];
     }
 }
@@ -130,13 +139,15 @@ hipError_t launch_rope_append(const RopeAppendLaunch& L, hipStream_t stream) {
         L.rotary_dim % 2u != 0u || (L.mode != 0u && L.mode != 2u) || L.dtype > kF8 || L.n_kv_heads == 0u)
         return hipErrorInvalidValue;
     RopeAppendArgs a;
+    a.q_src = L.q_src; a.q_weight = L.q_weight; a.q_out = L.q_out; a.n_q_heads = L.n_q_heads;
     a.k_src = L.k_src; a.v_src = L.v_src; a.weight = L.weight; a.positions = L.positions;
     a.freq_factors = L.freq_factors; a.k_out = L.k_out;
     a.k_dst = (uint8_t*)L.k_dst; a.v_dst = (uint8_t*)L.v_dst;
     a.n_kv_heads = L.n_kv_heads; a.head_dim = L.head_dim; a.rotary_dim = L.rotary_dim; a.mode = L.mode;
     a.pos0 = L.pos0; a.dtype = L.dtype; a.row_bytes = L.row_bytes;
     a.theta_scale = L.theta_scale; a.freq_scale = L.freq_scale; a.attn_factor = L.attn_factor; a.eps = L.eps;
-    const uint32_t n_units = L.v_src ? 2u * L.n_kv_heads : L.n_kv_heads;
+    if (L.q_src != nullptr && (L.q_out == nullptr || L.n_q_heads == 0u)) return hipErrorInvalidValue;
+    const uint32_t n_units = (L.q_src ? L.n_q_heads : 0u) + (L.v_src ? 2u * L.n_kv_heads : L.n_kv_heads);
     if ((n_units + kRopeWaves - 1u) / kRopeWaves > 65535u) return hipErrorInvalidValue;
     hipLaunchKernelGGL(rope_append_kernel, dim3(L.n_tokens, (n_units + kRopeWaves - 1u) / kRopeWaves), dim3(kRopeWaves * kWave),
                        0, stream, a);

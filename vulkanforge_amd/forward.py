@@ -121,6 +121,19 @@ class Forward:
             _ptr(freq_factors) if freq_factors is not None else None, C.byref(p),
             _ptr(k_out) if k_out is not None else None, _stream(stream)))
 
+    def step_qk_rope_kv_write(self, layer: int, position: int, n_tokens: int, q, k_src, v_src, rotary_dim: int,
+                              theta_scale: float, q_norm_weight=None, k_norm_weight=None, q_out=None, positions=None,
+                              freq_factors=None, rope_mode: int = _ffi.ROPE_NEOX, freq_scale: float = 1.0,
+                              attn_factor: float = 1.0, eps: float = 1e-6, k_out=None, stream=None) -> None:
+        """step_q_norm_rope + step_k_norm_rope + step_kv_write (executor/attention.rs:360-597) as one launch: the
+        queries [n_tokens, n_heads, head_dim] are normed * ``q_norm_weight`` and rotated into ``q_out`` (default: in
+        place), K and V as in ``step_k_rope_kv_write``."""
+        p = _ffi.RopeParams(rope_mode, rotary_dim, theta_scale, freq_scale, attn_factor, eps)
+        _ffi.check(_ffi.lib().vfkv_qk_rope_kv_write(
+            self.kv_cache.handle, layer, position, n_tokens, self.n_heads, _ptr(q), _ptr(q_norm_weight),
+            _ptr(q_out if q_out is not None else q), _ptr(k_src), _ptr(v_src), _ptr(k_norm_weight), _ptr(positions),
+            _ptr(freq_factors), C.byref(p), _ptr(k_out), _stream(stream)))
+
     # ---- decode attention (runs.rs:722-822, 1463-1571) ----
     @staticmethod
     def run_flash_attn_split(q, k_layer, v_layer, kv_dtype, scratch_out, scratch_max, scratch_sum, n_heads,

@@ -146,6 +146,14 @@ public:
                                    freq_factors, &rope, k_out, stream));
     }
 
+    // step_q_norm_rope + step_k_norm_rope + step_kv_write (attention.rs:360-597) in one launch; q is rotated in place
+    void step_qk_rope_kv_write(uint32_t layer, uint32_t position, uint32_t n_tokens, float* q, const float* q_norm_weight,
+                               const float* k_src, const float* v_src, const float* k_norm_weight, const vfkv_rope_params& rope,
+                               const int32_t* positions = nullptr, const float* freq_factors = nullptr, float* k_out = nullptr) {
+        check(vfkv_qk_rope_kv_write(kv_cache.handle(), layer, position, n_tokens, n_heads, q, q_norm_weight, q, k_src, v_src,
+                                    k_norm_weight, positions, freq_factors, &rope, k_out, stream));
+    }
+
     // runs.rs:1463-1571
     void run_flash_attn_split_reduce(uint32_t layer, uint32_t position, uint32_t kv_layer, uint32_t kv_start, const float* q,
                                      float* attn_out, float softcap = 0.f) {

@@ -347,6 +347,25 @@ def test_heterogeneous_cache_and_kv_share():
         assert np.abs(to_np(o) - ref).max() < TIGHT
 
 
+def test_long_context_128k_fp8_and_window_edges():
+    # four times the benchmark's context in one layer (128 MiB slabs), plus windows that start on, just before and
+    # just after a run boundary and a window of a single key
+    heads, hkv, d, ctx = 32, 8, 128, 131072
+    cache, hist = _cache_with_history(vf.KvDtype.F8, 1, hkv, d, ctx, fp16_normal, 61)
+    fwd = vf.Forward(cache, heads)
+    q = fp16_normal(rng(62), (heads, d))
+    ke, ve = (encode_np(x, vf.KvDtype.F8).reshape(ctx, hkv, d) for x in hist[0])
+    scale = float(1.0 / np.sqrt(d))
+    for pos, kv_start in ((ctx - 1, 0), (ctx - 1, ctx - 4096), (100000, 99999 - 4097), (70001, 70001 - 31), (5000, 5000)):
+        o = torch.full((heads, d), float("nan"), device=DEV)
+        fwd.run_scalar_attn(0, pos, to_dev(q), o, kv_start=kv_start)
+        torch.cuda.synchronize()
+        ref = oracle.attn_decode_ref(q, ke, ve, oracle.F8, heads, hkv, d, pos + 1, scale, kv_start=kv_start)
+        err = np.abs(to_np(o) - ref).max()
+        assert err < TOL[vf.KvDtype.F8] and err < TIGHT, (pos, kv_start, err)
+    cache.destroy()
+
+
 def test_short_context_goes_through_the_same_path():
     # seq <= 64: the reference uses its single-workgroup shader (runs.rs:776-821); same attention
     heads, hkv, d = 32, 8, 128

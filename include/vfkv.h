@@ -70,10 +70,14 @@ typedef struct vfkv_cache_config {
 
 typedef struct vfkv_cache vfkv_cache;
 
-/* KvCache::new (kv_cache.rs:224-339): checked size arithmetic, then two device allocations. */
+/* KvCache::new (kv_cache.rs:224-339): checked size arithmetic, then two device allocations.  The V
+ * buffer starts 256 bytes into its allocation (vfkv_cache_v_ptr returns the shifted pointer): K and V
+ * of a row are requested together, and with equally aligned buffers one 128-byte column of every row
+ * is served measurably slower. */
 int vfkv_cache_create(const vfkv_cache_config* cfg, vfkv_cache** out);
 /* Same layout object over caller-owned buffers (either may be NULL for layout-only use, e.g. on a
- * host without a GPU).  No allocation happens and destroy() leaves the buffers alone. */
+ * host without a GPU).  No allocation happens and destroy() leaves the buffers alone.  For speed give
+ * the two buffers different alignment modulo 512 bytes (e.g. v_buffer = allocation + 256). */
 int vfkv_cache_create_external(const vfkv_cache_config* cfg, void* k_buffer, void* v_buffer,
                                vfkv_cache** out);
 /* KvCache::destroy (kv_cache.rs:496-499). */

@@ -351,7 +351,7 @@ def bench_prefill(args, wl):
         qh = q[wl.m - ms:].cpu().numpy()
         flops_sample = sum(qs + i + 1 for i in range(ms)) * H * 4 * D
         spent, reps, ref = 0.0, 0, None
-        while spent < args.cpu_seconds and reps < 64:
+        while spent < args.cpu_seconds and reps < 1024:
             c0 = time.perf_counter()
             ref = oracle.attn_batch_ref(qh, kh, vh, int(wl.dtype), ms, max_seq, H, Hkv, D, qs, 1.0 / D ** 0.5,
                                         threads=threads)

@@ -60,6 +60,10 @@ CASES = [
     (vf.KvDtype.F8, 12, 2, 128, 23, 2100, 1500, 0.0), # G = 6: three head pairs, two key splits, window
     (vf.KvDtype.F8, 16, 8, 64, 70, 600, 0, 30.0),     # G = 2: one head pair, eight key splits, soft-cap
     (vf.KvDtype.F16, 16, 2, 128, 33, 900, 0, 0.0),    # G = 8 on a 2-byte cache
+    (vf.KvDtype.F8, 16, 8, 256, 48, 700, 0, 50.0),    # head_dim 256, G = 2: three key splits, soft-cap
+    (vf.KvDtype.F16, 8, 2, 256, 35, 260, 100, 0.0),   # head_dim 256, G = 4 on a 2-byte cache, window
+    (vf.KvDtype.F8, 32, 4, 256, 18, 130, 0, 0.0),     # head_dim 256, G = 8: the Q planes leave no room for private tiles
+    (vf.KvDtype.F16, 16, 16, 256, 20, 90, 0, 20.0),   # head_dim 256, G = 1: seven key splits
 ]
 
 

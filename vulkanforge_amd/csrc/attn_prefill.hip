@@ -1,6 +1,8 @@
 // Chunked-prefill causal attention over the cache (flash_attn_batch.comp:105-208) for gfx950.
 //
-// batch_mfma_kernel    (attn_prefill_mfma.h) f16 matrix-core tiles for FP8 / F16 caches, head_dim 64/128/256.
+// batch_mfma2_kernel   (attn_prefill_mfma2.h) f16 matrix-core tiles, private K / V tiles per wavefront: FP8 / F16 caches,
+//                      head_dim 64 / 128 / 256, GQA groups that fit the workgroup.
+// batch_mfma_kernel    (attn_prefill_mfma.h) first generation (V tile shared behind a barrier): the remaining groups.
 // batch_generic_kernel one wavefront per (query, head); covers every dtype and head_dim <= 512.
 #include "device_utils.h"
 #include "kernels.h"
@@ -99,7 +101,7 @@ hipError_t launch_batch(const BatchLaunch& L, hipStream_t stream) {
                          (L.head_dim == 64u || L.head_dim == 128u || L.head_dim == 256u);
     // Second-generation kernel: NCB heads per wavefront, private tiles per wavefront, no barrier in the loop.
     static const bool v2_on = [] { const char* e = getenv("VFKV_PREFILL_KERNEL"); return !(e && e[0] == '1'); }();
-    if (mfma_ok && v2_on && L.head_dim <= 128u) {
+    if (mfma_ok && v2_on) {
         // two heads per wavefront where the registers allow it
         static const int force_ncb = [] { const char* e = getenv("VFKV_PREFILL_NCB"); return e ? atoi(e) : 0; }();
 #ifndef VFKV_PREFILL_F16_128_NCB
@@ -109,7 +111,14 @@ hipError_t launch_batch(const BatchLaunch& L, hipStream_t stream) {
         if (force_ncb == 1) ncb = 1u;
         const uint32_t hp = g / ncb;
         if (hp <= 8u) {
-            const uint32_t max_waves = ncb == 1u ? 12u : 8u;  // one head per wavefront needs fewer registers: three wavefronts per SIMD
+            uint32_t max_waves = (ncb == 1u && L.head_dim <= 128u) ? 12u : 8u;  // one head per wavefront needs fewer registers: three wavefronts per SIMD
+            {   // the private V tiles and the two Q planes have to fit in 160 KiB of LDS
+                const size_t qbytes = (size_t)2 * g * 16 * (L.head_dim + 8) * sizeof(_Float16);
+                const size_t per_wave = (size_t)32 * (L.head_dim + 16) * sizeof(_Float16);
+                const size_t fit = qbytes < 160u * 1024u ? (160u * 1024u - qbytes) / per_wave : 0u;
+                if (fit < max_waves) max_waves = (uint32_t)fit;
+            }
+            if (max_waves < hp) goto first_generation;
             const uint32_t ns = max_waves / hp;               // key splits: fill the workgroup
             const uint32_t nwaves = hp * ns;
             const dim3 grid((L.m + 15u) / 16u, L.n_kv_heads), block(nwaves * kWave);
@@ -126,11 +135,13 @@ hipError_t launch_batch(const BatchLaunch& L, hipStream_t stream) {
     } else
             VFKV_P2(kF8, 64, 2, 2) VFKV_P2(kF8, 64, 1, 2) VFKV_P2(kF8, 128, 2, 2) VFKV_P2(kF8, 128, 1, 2)
             VFKV_P2(kF16, 64, 2, 2) VFKV_P2(kF16, 64, 1, 2) VFKV_P2(kF16, 128, 1, 1) VFKV_P2(kF16, 128, 2, 1)
+            VFKV_P2(kF8, 256, 1, 1) VFKV_P2(kF16, 256, 1, 1)
             { launched = false; }
 #undef VFKV_P2
             if (launched) return hipGetLastError();
         }
     }
+first_generation:
     if (mfma_ok && g <= 16u) {
         // two key splits per workgroup while that still leaves two wavefronts per SIMD worth of registers
         const uint32_t nsplit = g <= 4u ? 2u : 1u;

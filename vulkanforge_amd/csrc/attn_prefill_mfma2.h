@@ -25,7 +25,7 @@
 namespace vfkv {
 
 template <int DT, int D, int NCB, int PFD, bool CAP>
-__global__ __launch_bounds__(NCB == 1 ? 768 : 512) void batch_mfma2_kernel(BatchArgs a, int HP, int NS) {
+__global__ __launch_bounds__((NCB == 1 && D <= 128) ? 768 : 512) void batch_mfma2_kernel(BatchArgs a, int HP, int NS) {
     constexpr int ES = DT == kF16 ? 2 : 1;
     constexpr int KT = 32;                       // keys per tile
     constexpr int KS = D / 32;                   // MFMA k-steps of the first product

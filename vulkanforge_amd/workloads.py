@@ -72,6 +72,11 @@ PREFILL = {
     "prefill_fp8_512x4608_32layers": PrefillWorkload("prefill_fp8_512x4608_32layers", 32, 32, 8, 128, 4096, 512,
                                                      KvDtype.F8),
     # the same geometry over an F16 cache (not one of the reference configurations; used to tune the F16 variant)
+    # Gemma-style geometry (16 query heads, 8 KV heads, head_dim 256): not a reference configuration either
+    "prefill_f16_hd256_512x4608_12layers": PrefillWorkload("prefill_f16_hd256_512x4608_12layers", 12, 16, 8, 256, 4096,
+                                                           512, KvDtype.F16),
+    "prefill_fp8_hd256_512x4608_12layers": PrefillWorkload("prefill_fp8_hd256_512x4608_12layers", 12, 16, 8, 256, 4096,
+                                                           512, KvDtype.F8),
     "prefill_f16_512x4608_32layers": PrefillWorkload("prefill_f16_512x4608_32layers", 32, 32, 8, 128, 4096, 512,
                                                      KvDtype.F16),
 }

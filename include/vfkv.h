@@ -111,6 +111,30 @@ int vfkv_guard_kv_precision(int is_gemma4_moe, uint32_t dtype, int force);
 uint32_t vfkv_kv_start_decode(uint32_t position, uint32_t sliding_window);
 /* b_step_attention (executor/attention.rs:2215-2219): window of the LAST query of the batch. */
 uint32_t vfkv_kv_start_batch(uint32_t base_pos, uint32_t seq_len, uint32_t window);
+/* Gemma4KvSource (gguf.rs:879-895): how a layer relates to the cross-layer KV share. */
+#define VFKV_KV_OWN 0u
+#define VFKV_KV_OWN_PUBLISHES_SLIDING 1u
+#define VFKV_KV_OWN_PUBLISHES_FULL 2u
+#define VFKV_KV_SUBSCRIBES_SLIDING 3u
+#define VFKV_KV_SUBSCRIBES_FULL 4u
+/* gemma4_kv_read_layer (forward/arch/gemma4.rs:27-49): the layer whose slab `layer` reads, i.e. the
+ * `kv_layer` argument of the attention entry points.  `kv_source` holds one VFKV_KV_* value per
+ * layer (NULL: no sharing).  Owners read themselves, subscribers the FIRST layer that publishes
+ * their kind, and themselves when nobody does.  `layer >= n_layers` returns `layer`. */
+uint32_t vfkv_kv_read_layer(const uint32_t* kv_source, uint32_t n_layers, uint32_t layer);
+/* build_kv_sources (gguf.rs:908-942): fills kv_source_out[n_layers] from the model's sliding /
+ * full pattern (is_sliding[i] != 0: sliding layer; layers beyond n_pattern count as sliding).
+ * Layers before `first_kv_shared` own their rows, the LAST sliding and the LAST full layer among
+ * them publish; every later layer subscribes to its kind. */
+void vfkv_build_kv_sources(const uint8_t* is_sliding, uint32_t n_pattern, uint32_t first_kv_shared,
+                           uint32_t n_layers, uint32_t* kv_source_out);
+/* The start position of a request that reuses the resident rows of the previous one
+ * (ServerSession::generate_reuse, server/state.rs:199-201, longest_common_prefix :49-51): the
+ * length of the common prefix of the two token sequences, capped at n_tokens - 1 so that at
+ * least one token is prefilled.  The caller then keeps rows [0, k) (k > 0:
+ * vfkv_cache_set_current_seq_len(c, k); k == 0: vfkv_cache_reset(c)) and prefills from base_pos k. */
+uint32_t vfkv_prefix_reuse_start(const uint32_t* cached_tokens, uint32_t n_cached,
+                                 const uint32_t* tokens, uint32_t n_tokens);
 
 /* ------------------------------------------------------------------------------------------ */
 /* KV append and expansion kernels.                                                           */

@@ -207,3 +207,56 @@ def test_rms_norm_mul_rope_rejects_bad_arguments():
     assert call(mode=24) == -4 and call(hd=1024, rot=64) == -4 and call(hd=130, rot=64) == -4
     assert call(rot=129) == -1 and call(rot=256) == -1 and call(fs=-1.0) == -1
     assert call(x=None) == -1 and call(out=None) == -1 and call(params=False) == -1
+
+
+def test_build_kv_sources_reference_patterns():
+    # gguf.rs:1531-1567 (E2B: 35 layers, every fifth is a full layer, the first 15 own their rows)
+    pattern = [(i % 5) != 4 for i in range(35)]
+    srcs = vf.build_kv_sources(pattern, 15, 35)
+    assert srcs[13] == vf.kv_cache.KV_OWN_PUBLISHES_SLIDING
+    assert srcs[14] == vf.kv_cache.KV_OWN_PUBLISHES_FULL
+    for i in (0, 1, 2, 3, 5, 6, 7, 8, 10, 11, 12, 4, 9):
+        assert srcs[i] == vf.kv_cache.KV_OWN, i
+    for i in range(15, 35):
+        want = vf.kv_cache.KV_SUBSCRIBES_FULL if i % 5 == 4 else vf.kv_cache.KV_SUBSCRIBES_SLIDING
+        assert srcs[i] == want, i
+    # gguf.rs:1569-1590: no full layer among the owners
+    p = [True] * 10
+    p[7] = False
+    srcs = vf.build_kv_sources(p, 5, 10)
+    assert srcs[4] == vf.kv_cache.KV_OWN_PUBLISHES_SLIDING
+    assert srcs[7] == vf.kv_cache.KV_SUBSCRIBES_FULL
+    assert [srcs[i] for i in (5, 6, 8, 9)] == [vf.kv_cache.KV_SUBSCRIBES_SLIDING] * 4
+    assert srcs[:4] == [vf.kv_cache.KV_OWN] * 4
+    # a pattern shorter than the stack: the missing layers count as sliding (gguf.rs:916-918)
+    assert vf.build_kv_sources([False], 2, 3) == [vf.kv_cache.KV_OWN_PUBLISHES_FULL, vf.kv_cache.KV_OWN_PUBLISHES_SLIDING,
+                                                   vf.kv_cache.KV_SUBSCRIBES_SLIDING]
+
+
+def test_kv_read_layer_follows_the_first_publisher():
+    # forward/arch/gemma4.rs:27-49 on the E2B stack: sliding subscribers read layer 13, full subscribers layer 14
+    srcs = vf.build_kv_sources([(i % 5) != 4 for i in range(35)], 15, 35)
+    for layer in range(35):
+        want = layer if layer < 15 else (14 if layer % 5 == 4 else 13)
+        assert vf.gemma4_kv_read_layer(srcs, layer) == want, layer
+    assert vf.gemma4_kv_read_layer(None, 7) == 7                    # not a Gemma-4 stack
+    assert vf.gemma4_kv_read_layer(srcs, 99) == 99
+    # a subscriber without publisher reads itself (`unwrap_or(layer)`)
+    srcs = vf.build_kv_sources([True] * 5 + [True, True, False, True, True], 5, 10)
+    assert vf.gemma4_kv_read_layer(srcs, 7) == 7
+    assert vf.gemma4_kv_read_layer(srcs, 8) == 4
+    # two publishers of one kind (hand-built): the first wins (`find`)
+    K = vf.kv_cache
+    assert vf.gemma4_kv_read_layer([K.KV_OWN_PUBLISHES_FULL, K.KV_OWN_PUBLISHES_FULL, K.KV_SUBSCRIBES_FULL], 2) == 0
+
+
+def test_prefix_reuse_start_reference_cases():
+    # server/state.rs:363-396
+    assert vf.prefix_reuse_start([], [1, 2, 3]) == 0
+    assert vf.prefix_reuse_start([9, 8, 7], [1, 2, 3]) == 0
+    assert vf.prefix_reuse_start([10, 11, 12, 13, 14], [10, 11, 12, 99]) == 3
+    assert vf.prefix_reuse_start([1, 2, 3, 4, 5], [1, 2, 3]) == 2        # lcp 3, capped at len - 1
+    assert vf.prefix_reuse_start([1, 2, 3], [1, 2, 3]) == 2
+    assert vf.prefix_reuse_start([1, 2, 3, 4], [1, 2, 3, 4]) == 3        # "k must be len-1, not the full length"
+    assert vf.prefix_reuse_start([1, 2, 3], []) == 0
+    assert vf.prefix_reuse_start([5], [5]) == 0

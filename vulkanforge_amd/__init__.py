@@ -8,8 +8,9 @@ everything through ctypes.  There is no CPU or eager fallback: importing works a
 compute entry point without the built library or without a GPU raises.
 """
 from ._ffi import VfkvError, lib, lib_path  # noqa: F401
-from .kv_cache import KvCache, KvCacheConfig, KvDtype, guard_kv_precision, kv_bytes_per_token  # noqa: F401
+from .kv_cache import (KvCache, KvCacheConfig, KvDtype, guard_kv_precision, kv_bytes_per_token,  # noqa: F401
+                       gemma4_kv_read_layer, build_kv_sources, prefix_reuse_start)
 from .forward import Forward, Workspace  # noqa: F401
 
 __all__ = ["KvCache", "KvCacheConfig", "KvDtype", "Forward", "Workspace", "VfkvError", "lib", "lib_path",
-           "guard_kv_precision", "kv_bytes_per_token"]
+           "guard_kv_precision", "kv_bytes_per_token", "gemma4_kv_read_layer", "build_kv_sources", "prefix_reuse_start"]

@@ -78,6 +78,9 @@ SIGNATURES = {
     "vfkv_guard_kv_precision": (C.c_int, [C.c_int, _u32, C.c_int]),
     "vfkv_kv_start_decode": (_u32, [_u32, _u32]),
     "vfkv_kv_start_batch": (_u32, [_u32, _u32, _u32]),
+    "vfkv_kv_read_layer": (_u32, [_u32p, _u32, _u32]),
+    "vfkv_build_kv_sources": (None, [C.POINTER(C.c_uint8), _u32, _u32, _u32, _u32p]),
+    "vfkv_prefix_reuse_start": (_u32, [_u32p, _u32, _u32p, _u32]),
     "vfkv_store_fp8": (C.c_int, [_vp, _vp, _u32, _u64, _vp]),
     "vfkv_copy_fp16": (C.c_int, [_vp, _vp, _u32, _u64, _vp]),
     "vfkv_fp8_to_f16": (C.c_int, [_vp, _vp, _u64, _vp]),

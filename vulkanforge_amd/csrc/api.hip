@@ -280,6 +280,41 @@ uint32_t vfkv_kv_start_batch(uint32_t base_pos, uint32_t seq_len, uint32_t windo
     return end > window ? (uint32_t)(end - window) : 0u;
 }
 
+uint32_t vfkv_kv_read_layer(const uint32_t* kv_source, uint32_t n_layers, uint32_t layer) {
+    if (!kv_source || layer >= n_layers) return layer;
+    uint32_t want;
+    switch (kv_source[layer]) {
+        case VFKV_KV_SUBSCRIBES_SLIDING: want = VFKV_KV_OWN_PUBLISHES_SLIDING; break;
+        case VFKV_KV_SUBSCRIBES_FULL: want = VFKV_KV_OWN_PUBLISHES_FULL; break;
+        default: return layer;
+    }
+    for (uint32_t i = 0; i < n_layers; ++i)
+        if (kv_source[i] == want) return i;
+    return layer;
+}
+
+void vfkv_build_kv_sources(const uint8_t* is_sliding, uint32_t n_pattern, uint32_t first_kv_shared, uint32_t n_layers,
+                           uint32_t* kv_source_out) {
+    if (!kv_source_out) return;
+    auto sliding = [&](uint32_t i) { return !is_sliding || i >= n_pattern || is_sliding[i] != 0; };
+    int64_t last_sliding = -1, last_full = -1;
+    for (uint32_t i = 0; i < first_kv_shared; ++i) (sliding(i) ? last_sliding : last_full) = i;
+    for (uint32_t i = 0; i < n_layers; ++i) {
+        if (i >= first_kv_shared) kv_source_out[i] = sliding(i) ? VFKV_KV_SUBSCRIBES_SLIDING : VFKV_KV_SUBSCRIBES_FULL;
+        else if ((int64_t)i == last_sliding) kv_source_out[i] = VFKV_KV_OWN_PUBLISHES_SLIDING;
+        else if ((int64_t)i == last_full) kv_source_out[i] = VFKV_KV_OWN_PUBLISHES_FULL;
+        else kv_source_out[i] = VFKV_KV_OWN;
+    }
+}
+
+uint32_t vfkv_prefix_reuse_start(const uint32_t* cached_tokens, uint32_t n_cached, const uint32_t* tokens,
+                                 uint32_t n_tokens) {
+    if (!cached_tokens || !tokens || n_tokens == 0u) return 0u;
+    uint32_t k = 0;
+    while (k < n_cached && k < n_tokens && cached_tokens[k] == tokens[k]) ++k;
+    return k < n_tokens - 1u ? k : n_tokens - 1u;
+}
+
 // ---- append / expansion ----------------------------------------------------------------------------
 static int append_one(uint32_t dtype, const float* src, void* dst, uint32_t n, uint64_t off, vfkv_stream stream,
                       const char* what) {

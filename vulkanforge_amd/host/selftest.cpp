@@ -30,6 +30,15 @@ int main() {
         try { KvCache c2(bad, true); } catch (const Error& e) { threw = e.status == VFKV_ERR_OVERFLOW; }
         REQUIRE(threw);
     }
+    {   // gguf.rs:1531-1567 (E2B share pattern), forward/arch/gemma4.rs:27-49, server/state.rs:363-396
+        std::vector<uint8_t> sliding(35);
+        for (int i = 0; i < 35; ++i) sliding[i] = (i % 5) != 4;
+        const std::vector<uint32_t> src = build_kv_sources(sliding, 15, 35);
+        REQUIRE(src[13] == VFKV_KV_OWN_PUBLISHES_SLIDING && src[14] == VFKV_KV_OWN_PUBLISHES_FULL && src[12] == VFKV_KV_OWN);
+        REQUIRE(gemma4_kv_read_layer(src, 20) == 13 && gemma4_kv_read_layer(src, 34) == 14 && gemma4_kv_read_layer(src, 9) == 9);
+        REQUIRE(prefix_reuse_start({10, 11, 12, 13, 14}, {10, 11, 12, 99}) == 3);
+        REQUIRE(prefix_reuse_start({1, 2, 3, 4}, {1, 2, 3, 4}) == 3 && prefix_reuse_start({}, {1, 2, 3}) == 0);
+    }
     if (vfkv_device_count() == 0) { std::printf("host selftest: layout checks passed (no GPU: compute checks skipped)\n"); return 0; }
 
     const uint32_t H = 32, Hkv = 8, D = 128, ctx = 1000;

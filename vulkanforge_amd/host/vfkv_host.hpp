@@ -53,6 +53,20 @@ inline void guard_kv_precision(bool is_gemma4_moe, KvDtype dtype, bool force = f
 }
 // gemma4_kv_start, forward/arch/gemma4.rs:59-73
 inline uint32_t gemma4_kv_start(uint32_t position, uint32_t sliding_window) { return vfkv_kv_start_decode(position, sliding_window); }
+// gemma4_kv_read_layer, forward/arch/gemma4.rs:27-49 (one VFKV_KV_* value per layer)
+inline uint32_t gemma4_kv_read_layer(const std::vector<uint32_t>& kv_source, uint32_t layer) {
+    return vfkv_kv_read_layer(kv_source.data(), (uint32_t)kv_source.size(), layer);
+}
+// build_kv_sources, gguf.rs:908-942
+inline std::vector<uint32_t> build_kv_sources(const std::vector<uint8_t>& is_sliding, uint32_t first_kv_shared, uint32_t n_layers) {
+    std::vector<uint32_t> out(n_layers);
+    vfkv_build_kv_sources(is_sliding.data(), (uint32_t)is_sliding.size(), first_kv_shared, n_layers, out.data());
+    return out;
+}
+// start position of a request that keeps the common prefix of the resident rows, server/state.rs:199-201
+inline uint32_t prefix_reuse_start(const std::vector<uint32_t>& cached, const std::vector<uint32_t>& tokens) {
+    return vfkv_prefix_reuse_start(cached.data(), (uint32_t)cached.size(), tokens.data(), (uint32_t)tokens.size());
+}
 
 class KvCache {
 public:

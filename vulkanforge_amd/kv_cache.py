@@ -53,6 +53,30 @@ def guard_kv_precision(is_gemma4_moe: bool, kv_dtype: KvDtype, force: bool = Fal
     _ffi.check(_ffi.lib().vfkv_guard_kv_precision(int(is_gemma4_moe), int(kv_dtype), int(force)))
 
 
+KV_OWN, KV_OWN_PUBLISHES_SLIDING, KV_OWN_PUBLISHES_FULL, KV_SUBSCRIBES_SLIDING, KV_SUBSCRIBES_FULL = range(5)
+
+
+def gemma4_kv_read_layer(kv_source: Optional[Sequence[int]], layer: int) -> int:
+    """forward/arch/gemma4.rs:27-49: the layer whose KV slab ``layer`` reads (one KV_* value per layer)."""
+    _a, pa = _u32_array(kv_source)
+    return int(_ffi.lib().vfkv_kv_read_layer(pa, 0 if kv_source is None else len(kv_source), layer))
+
+
+def build_kv_sources(is_sliding: Sequence[bool], first_kv_shared: int, n_layers: int) -> list:
+    """gguf.rs:908-942: one KV_* value per layer from the sliding / full pattern."""
+    pat = (C.c_uint8 * max(len(is_sliding), 1))(*[1 if b else 0 for b in is_sliding])
+    out = (C.c_uint32 * max(n_layers, 1))()
+    _ffi.lib().vfkv_build_kv_sources(pat, len(is_sliding), first_kv_shared, n_layers, out)
+    return list(out)[:n_layers]
+
+
+def prefix_reuse_start(cached_tokens: Sequence[int], tokens: Sequence[int]) -> int:
+    """server/state.rs:49-51,199-201: common prefix of the two sequences, capped at len(tokens) - 1."""
+    _a, pa = _u32_array(list(cached_tokens))
+    _b, pb = _u32_array(list(tokens))
+    return int(_ffi.lib().vfkv_prefix_reuse_start(pa, len(cached_tokens), pb, len(tokens)))
+
+
 class KvCache:
     """Two device buffers (K and V) in pos-major layout plus the offset arithmetic.
 

@@ -160,15 +160,27 @@ def bench_decode(args, wl):
     scale = 1.0 / (D ** 0.5)
     starts = [_ffi.lib().vfkv_kv_start_decode(pos, wl.layer_window(i)) if wl.layer_window(i) else 0 for i in range(L)]
 
+    gate = torch.randn((L, H * D), device=dev, generator=g) if wl.gated else None
+
+    def step_gate_separate():   # step_attention, then step_attn_gated_output as a launch of its own
+        for layer in range(L):
+            fwd.run_scalar_attn(layer, pos, q[layer], o[layer], kv_start=starts[layer], scale=scale, softcap=wl.softcap)
+            fwd.run_sigmoid_mul(gate[layer], o[layer], H * D, H * D, H * D, 0)
+
     def step():
         for layer in range(L):
-            if wl.append:       # step_kv_write + step_attention of the new token, issued as one call
+            if wl.gated:        # step_attention + step_attn_gated_output: the merge applies the gate
+                fwd.step_attention_gated(layer, pos, q[layer], o[layer], gate[layer], H * D, H * D, 0,
+                                         k_src=k_new[layer] if wl.append else None, v_src=v_new[layer] if wl.append else None,
+                                         kv_start=starts[layer], scale=scale, softcap=wl.softcap)
+            elif wl.append:     # step_kv_write + step_attention of the new token, issued as one call
                 fwd.step_kv_write_attention(layer, pos, q[layer], k_new[layer], v_new[layer], o[layer],
                                             kv_start=starts[layer], scale=scale, softcap=wl.softcap)
             else:
                 fwd.run_scalar_attn(layer, pos, q[layer], o[layer], kv_start=starts[layer], scale=scale,
                                     softcap=wl.softcap)
 
+    gate_separate_us = time_steps(torch, step_gate_separate, args) * 1e6 if wl.gated and not wl.append else None
     sec_per_step = time_steps(torch, step, args)
     step_spread = dict(STEP_SPREAD)
     bytes_step = wl.kv_bytes_step()
@@ -245,6 +257,9 @@ def bench_decode(args, wl):
                      "algorithmic_bytes_per_launch": bytes_launch},
     }
 
+    if gate_separate_us is not None:
+        result["config"]["us_per_step_with_separate_gate_launch"] = gate_separate_us
+
     if not args.no_cpu_baseline:
         import numpy as np
 
@@ -260,6 +275,8 @@ def bench_decode(args, wl):
             c0 = time.perf_counter()
             ref = oracle.attn_decode_ref(qh, kh, vh, int(wl.dtype), H, Hkv, D, wl.context, scale,
                                          kv_start=starts[layer], softcap=wl.softcap, threads=threads)
+            if wl.gated:
+                ref = oracle.sigmoid_mul(gate[layer].cpu().numpy(), ref.reshape(-1), H * D, H * D, 0).reshape(H, D)
             spent += time.perf_counter() - c0
             done_bytes += wl.kv_bytes_layer(layer)
             layers_done += 1

@@ -323,6 +323,42 @@ int vfkv_prefill_attention(vfkv_cache* c, uint32_t layer, uint32_t kv_layer, uin
                            const float* q, float* o, uint32_t m, uint32_t base_pos, uint32_t window,
                            float scale, float softcap, vfkv_stream stream);
 
+/* ------------------------------------------------------------------------------------------ */
+/* Gated attention output (Qwen3.6 full-attention layers).                                    */
+/* ------------------------------------------------------------------------------------------ */
+/* Where the gate of output element i lives (SigmoidMulPushConstants, forward/runs.rs:2667;
+ * vk_shaders/sigmoid_mul.comp:30-48): gate[(i / chunk) * stride + gate_offset + i % chunk],
+ * i = flat index into the output.  Decode passes (q_dim, q_dim, q_dim) with gate = q_buf
+ * (executor/attention.rs:655-664), the batch path (head_dim, 2 * head_dim, head_dim) with
+ * gate = batch_qgate (executor/attention.rs:2433-2441). */
+typedef struct vfkv_gate {
+    const float* gate;
+    uint32_t chunk;       /* > 0 */
+    uint32_t stride;
+    uint32_t gate_offset;
+} vfkv_gate;
+
+/* Forward::run_sigmoid_mul (forward/runs.rs:2649-2681) + sigmoid_mul.comp:40-53:
+ * data[i] *= 1 / (1 + exp(-gate[...])) for i < ne, in place. */
+int vfkv_sigmoid_mul(const vfkv_gate* gate, float* data, uint32_t ne, vfkv_stream stream);
+
+/* step_attention followed by step_attn_gated_output (executor/attention.rs:599-680), and with
+ * k_src / v_src != NULL also the step_kv_write before them (layer == kv_layer then, as in
+ * vfkv_kv_write_decode_attention): `o` leaves already multiplied by sigmoid(gate).  The merge
+ * kernel applies the gate in its own store, so no third launch runs (spans that fit one tile
+ * take a separate vfkv_sigmoid_mul launch).  Results are bit-identical to the separate calls.
+ * `gate->gate` must not overlap `o`. */
+int vfkv_decode_attention_gated(vfkv_cache* c, uint32_t layer, uint32_t kv_layer, uint32_t n_heads,
+                                const float* q, const float* k_src, const float* v_src, float* o,
+                                uint32_t position, uint32_t kv_start, float scale, float softcap,
+                                const vfkv_gate* gate, vfkv_workspace* ws, vfkv_stream stream);
+
+/* b_step_attention followed by b_step_attn_gated_output (executor/attention.rs:2192-2219,
+ * 2405-2444): vfkv_prefill_attention, then the gate on the m * n_heads * head_dim outputs. */
+int vfkv_prefill_attention_gated(vfkv_cache* c, uint32_t layer, uint32_t kv_layer, uint32_t n_heads,
+                                 const float* q, float* o, uint32_t m, uint32_t base_pos, uint32_t window,
+                                 float scale, float softcap, const vfkv_gate* gate, vfkv_stream stream);
+
 #ifdef __cplusplus
 }
 #endif

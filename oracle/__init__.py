@@ -81,6 +81,8 @@ def _declare(L: C.CDLL) -> None:
         getattr(L, name).restype = None
     L.vfo_rms_norm_rope.argtypes = [C.c_void_p] * 5 + [C.c_uint32] * 5 + [C.c_float] * 4
     L.vfo_rms_norm_rope.restype = None
+    L.vfo_sigmoid_mul.argtypes = [C.c_void_p, C.c_void_p, C.c_uint64, C.c_uint32, C.c_uint32, C.c_uint32]
+    L.vfo_sigmoid_mul.restype = None
     L.vfo_max_threads.argtypes = []
     L.vfo_max_threads.restype = C.c_int
 
@@ -261,4 +263,15 @@ def rms_norm_rope(x, pos, head_dim, n_dims, theta_scale, mode=ROPE_NEOX, weight=
     lib().vfo_rms_norm_rope(_p(x), _p(w) if w is not None else None, _p(pos), _p(f) if f is not None else None,
                             _p(out), m, heads, head_dim, mode, n_dims, float(theta_scale), float(freq_scale),
                             float(attn_factor), float(eps))
+    return out
+
+
+def sigmoid_mul(gate, data, chunk, stride, gate_offset) -> np.ndarray:
+    """data[i] * sigmoid(gate[(i // chunk) * stride + gate_offset + i % chunk]) as a new array (flat index i)."""
+    gate = np.ascontiguousarray(gate, dtype=np.float32)
+    out = np.array(data, dtype=np.float32, order="C", copy=True)
+    if out.size:
+        last = (out.size - 1) // chunk * stride + gate_offset + (out.size - 1) % chunk
+        assert last < gate.size, "gate buffer too small"
+    lib().vfo_sigmoid_mul(_p(gate), _p(out), out.size, chunk, stride, gate_offset)
     return out

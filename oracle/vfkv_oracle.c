@@ -37,6 +37,13 @@
  *                                                                                 NORM mode (adjacent pairs), partial rotary_dim and frequency
  *                                                                                 factors have no reference test: parity unpinned by the
  *                                                                                 reference, pinned by the formulations above only.
+ *   vfo_sigmoid_mul               vk_shaders/sigmoid_mul.comp:40-53                scipy.special.expit in f64 rounded once; g = 0 halves the value,
+ *                                                                                 g = +-100 keeps / zeroes it; the index map against a
+ *                                                                                 pure-Python loop for the decode form (chunk = stride = offset
+ *                                                                                 = q_dim, executor/attention.rs:655-664) and the interleaved
+ *                                                                                 per-head form (head_dim, 2 * head_dim, head_dim, :2433-2441).
+ *                                                                                 The reference holds no test of this shader: parity unpinned
+ *                                                                                 by the reference, pinned by the above only.
  *
  * Extensions that the reference does not implement (so no reference test can pin them):
  *   - `kv_start > 0` on every attention routine follows the shader text
@@ -598,4 +605,18 @@ int vfo_max_threads(void) {
 #else
     return 1;
 #endif
+}
+
+/* ------------------------------------------------------------------------------------------
+ * Gated attention output (vk_shaders/sigmoid_mul.comp:40-53):
+ *   data[i] *= sigmoid(gate[(i / chunk) * stride + gate_offset + i % chunk]),  sigmoid(g) = 1 / (1 + exp(-g)).
+ * The sigmoid is evaluated in f64 and rounded to f32 once; the product is an f32 multiply as in the shader.
+ * ---------------------------------------------------------------------------------------- */
+void vfo_sigmoid_mul(const float* gate, float* data, uint64_t ne, uint32_t chunk, uint32_t stride, uint32_t gate_offset) {
+    for (uint64_t i = 0; i < ne; ++i) {
+        const uint64_t token = i / chunk, within = i - token * chunk;
+        const double g = (double)gate[token * stride + gate_offset + within];
+        const float sg = (float)(1.0 / (1.0 + exp(-g)));
+        data[i] = data[i] * sg;
+    }
 }

@@ -260,3 +260,21 @@ def test_prefix_reuse_start_reference_cases():
     assert vf.prefix_reuse_start([1, 2, 3, 4], [1, 2, 3, 4]) == 3        # "k must be len-1, not the full length"
     assert vf.prefix_reuse_start([1, 2, 3], []) == 0
     assert vf.prefix_reuse_start([5], [5]) == 0
+
+
+def test_gated_entry_points_reject_bad_arguments_before_any_device_work():
+    L = _ffi.lib()
+    g = _ffi.Gate(0, 16, 16, 0)
+    assert L.vfkv_sigmoid_mul(C.byref(g), 64, 16, None) == -1                      # NULL gate buffer
+    assert L.vfkv_sigmoid_mul(None, 64, 16, None) == -1
+    g = _ffi.Gate(64, 0, 16, 0)
+    assert L.vfkv_sigmoid_mul(C.byref(g), 64, 16, None) == -1                      # chunk 0
+    assert b"chunk" in L.vfkv_last_error()
+    g = _ffi.Gate(66, 16, 16, 0)
+    assert L.vfkv_sigmoid_mul(C.byref(g), 64, 16, None) < 0                        # misaligned gate
+    g = _ffi.Gate(64, 16, 16, 0)
+    assert L.vfkv_sigmoid_mul(C.byref(g), 0, 16, None) == -1                       # NULL data
+    assert L.vfkv_sigmoid_mul(C.byref(g), 0, 0, None) == 0                         # nothing to do
+    assert L.vfkv_decode_attention_gated(None, 0, 0, 4, 64, None, None, 64, 0, 0, 1.0, 0.0, None, None, None) == -1
+    assert L.vfkv_prefill_attention_gated(None, 0, 0, 4, 64, 64, 1, 0, 0, 1.0, 0.0, None, None) == -1
+    assert L.vfkv_prefill_attention_gated(None, 0, 0, 4, 64, 64, 1, 0, 0, 1.0, 0.0, C.byref(g), None) == -1   # no cache

@@ -553,7 +553,8 @@ uint32_t vfkv_decode_tile_for(uint32_t span, uint32_t n_heads, uint32_t n_kv_hea
 
 static int decode_attention_impl(vfkv_cache* c, uint32_t layer, uint32_t kv_layer, uint32_t n_heads, const float* q, float* o,
                                  uint32_t position, uint32_t kv_start, float scale, float softcap, vfkv_workspace* ws,
-                                 const float* k_new, const float* v_new, vfkv_stream stream, const char* who) {
+                                 const float* k_new, const float* v_new, vfkv_stream stream, const char* who,
+                                 const vfkv::GateArgs* gate = nullptr) {
     if (!c || !c->k || !c->v) return fail(VFKV_ERR_INVALID_ARG, "%s: cache has no buffers", who);
     if (!ws) return fail(VFKV_ERR_INVALID_ARG, "%s: workspace is NULL", who);
     if (!q || !o) return fail(VFKV_ERR_INVALID_ARG, "%s: NULL buffer", who);
@@ -595,10 +596,14 @@ static int decode_attention_impl(vfkv_cache* c, uint32_t layer, uint32_t kv_laye
     if (vfkv::split_writes_output(L) && ((uintptr_t)o & 15u) == 0u) {   // one tile sees every key: the worker normalises and writes o itself
         L.o_direct = o;
         VFKV_HIP(vfkv::launch_split(L, S(stream)));
+        if (gate) VFKV_HIP(vfkv::launch_sigmoid_mul(o, n_heads * hd, *gate, S(stream)));
         return VFKV_OK;
     }
     VFKV_HIP(vfkv::launch_split(L, S(stream)));
-    VFKV_HIP(vfkv::launch_reduce(ws->scratch_out, ws->scratch_max, ws->scratch_sum, o, n_heads, hd, n_tiles, S(stream)));
+    bool gate_applied = false;
+    VFKV_HIP(vfkv::launch_reduce(ws->scratch_out, ws->scratch_max, ws->scratch_sum, o, n_heads, hd, n_tiles, S(stream), gate,
+                                 &gate_applied));
+    if (gate && !gate_applied) VFKV_HIP(vfkv::launch_sigmoid_mul(o, n_heads * hd, *gate, S(stream)));
     return VFKV_OK;
 }
 
@@ -663,6 +668,57 @@ int vfkv_prefill_attention(vfkv_cache* c, uint32_t layer, uint32_t kv_layer, uin
     p.kv_start = vfkv_kv_start_batch(base_pos, m, window);
     const uint64_t off = layer_off(c, kv_layer);
     return vfkv_flash_attn_batch(q, (char*)c->k + off, (char*)c->v + off, c->dtype, o, &p, softcap, stream);
+}
+
+// ---- gated output --------------------------------------------------------------------------------------
+static int check_gate(const vfkv_gate* gate, const char* who, vfkv::GateArgs* out) {
+    if (!gate || !gate->gate) return fail(VFKV_ERR_INVALID_ARG, "%s: gate is NULL", who);
+    if (gate->chunk == 0u) return fail(VFKV_ERR_INVALID_ARG, "%s: gate chunk must be > 0", who);
+    if ((((uintptr_t)gate->gate) & 3u) != 0u) return fail(VFKV_ERR_ALIGNMENT, "%s: gate must be 4-byte aligned", who);
+    out->gate = gate->gate; out->chunk = gate->chunk; out->stride = gate->stride; out->gate_offset = gate->gate_offset;
+    return VFKV_OK;
+}
+
+int vfkv_sigmoid_mul(const vfkv_gate* gate, float* data, uint32_t ne, vfkv_stream stream) {
+    if (ne == 0u) return VFKV_OK;
+    vfkv::GateArgs g;
+    const int rc = check_gate(gate, "sigmoid_mul", &g);
+    if (rc != VFKV_OK) return rc;
+    if (!data) return fail(VFKV_ERR_INVALID_ARG, "sigmoid_mul: NULL buffer");
+    if ((((uintptr_t)data) & 3u) != 0u) return fail(VFKV_ERR_ALIGNMENT, "sigmoid_mul: data must be 4-byte aligned");
+    VFKV_HIP(vfkv::launch_sigmoid_mul(data, ne, g, S(stream)));
+    return VFKV_OK;
+}
+
+int vfkv_decode_attention_gated(vfkv_cache* c, uint32_t layer, uint32_t kv_layer, uint32_t n_heads, const float* q,
+                                const float* k_src, const float* v_src, float* o, uint32_t position, uint32_t kv_start,
+                                float scale, float softcap, const vfkv_gate* gate, vfkv_workspace* ws, vfkv_stream stream) {
+    vfkv::GateArgs g;
+    const int rc = check_gate(gate, "decode_attention_gated", &g);
+    if (rc != VFKV_OK) return rc;
+    if ((k_src == nullptr) != (v_src == nullptr))
+        return fail(VFKV_ERR_INVALID_ARG, "decode_attention_gated: k_src and v_src must both be given or both be NULL");
+    if (k_src) {
+        if (layer != kv_layer) return fail(VFKV_ERR_INVALID_ARG, "decode_attention_gated: a layer that appends reads its own slab (layer %u, kv_layer %u)", layer, kv_layer);
+        if (c && layer < c->n_layers && (layer_off(c, layer) + (uint64_t)position * row_b(c, layer)) % 4u != 0u)
+            return fail(VFKV_ERR_ALIGNMENT, "decode_attention_gated: dst_byte_offset must be uint-aligned");
+    }
+    return decode_attention_impl(c, layer, kv_layer, n_heads, q, o, position, kv_start, scale, softcap, ws, k_src, v_src, stream,
+                                 "decode_attention_gated", &g);
+}
+
+int vfkv_prefill_attention_gated(vfkv_cache* c, uint32_t layer, uint32_t kv_layer, uint32_t n_heads, const float* q, float* o,
+                                 uint32_t m, uint32_t base_pos, uint32_t window, float scale, float softcap,
+                                 const vfkv_gate* gate, vfkv_stream stream) {
+    vfkv::GateArgs g;
+    int rc = check_gate(gate, "prefill_attention_gated", &g);
+    if (rc != VFKV_OK) return rc;
+    rc = vfkv_prefill_attention(c, layer, kv_layer, n_heads, q, o, m, base_pos, window, scale, softcap, stream);
+    if (rc != VFKV_OK || m == 0u) return rc;
+    const uint64_t ne = (uint64_t)m * n_heads * hd_for(c, layer);
+    if (ne > 0xFFFFFFFFull) return fail(VFKV_ERR_OVERFLOW, "prefill_attention_gated: %llu output elements", (unsigned long long)ne);
+    VFKV_HIP(vfkv::launch_sigmoid_mul(o, (uint32_t)ne, g, S(stream)));
+    return VFKV_OK;
 }
 
 }  // extern "C"

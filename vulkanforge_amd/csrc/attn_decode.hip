@@ -540,10 +540,12 @@ __global__ __launch_bounds__(kReduceThreads) void reduce_kernel(const float* __r
 // Few tiles (<= MAXT <= 64): one wavefront per (head, 64 output dimensions), no LDS and no barrier.  Lane j owns tile
 // j's max / sum and turns them into its merge weight; every lane also owns one output dimension and loads that
 // dimension of all partial outputs before the first reduction, so the kernel costs one memory round trip.
-template <int MAXT>
+// GATED: the output element is multiplied by sigmoid(gate) in the same store (the reference's separate sigmoid_mul dispatch,
+// executor/attention.rs:632-680); the gate value is requested with the partials.
+template <int MAXT, bool GATED>
 __global__ __launch_bounds__(kWave) void reduce_direct_kernel(const float* __restrict__ so, const float* __restrict__ sm,
                                                               const float* __restrict__ ss, float* __restrict__ o,
-                                                              uint32_t D, uint32_t n_tiles) {
+                                                              uint32_t D, uint32_t n_tiles, GateArgs gate) {
     const uint32_t h = blockIdx.y, lane = threadIdx.x;
     const uint32_t d = blockIdx.x * kWave + lane;
     const float* ho = so + (size_t)h * n_tiles * D + d;
@@ -552,6 +554,11 @@ __global__ __launch_bounds__(kWave) void reduce_direct_kernel(const float* __res
     for (int j = 0; j < MAXT; ++j) x[j] = ho[(size_t)((uint32_t)j < n_tiles ? j : 0) * D];
     const float mj = lane < n_tiles ? sm[(size_t)h * n_tiles + lane] : kMasked;
     const float sj = lane < n_tiles ? ss[(size_t)h * n_tiles + lane] : 0.f;
+    float gv = 0.f;
+    if (GATED) {   // the index arithmetic (one 32-bit division: n_heads * D < 2^32) runs while the partials are in flight
+        const uint32_t i = h * D + d, token = i / gate.chunk;
+        gv = gate.gate[(uint64_t)token * gate.stride + gate.gate_offset + (i - token * gate.chunk)];
+    }
     const float M = wave_max_uniform(mj);
     const float wj = lane < n_tiles ? __expf(mj - M) : 0.f;
     const float L = wave_sum_uniform(wj * sj);
@@ -559,7 +566,8 @@ __global__ __launch_bounds__(kWave) void reduce_direct_kernel(const float* __res
 #pragma unroll
     for (int j = 0; j < MAXT; ++j)
         acc = fmaf(__builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, wj), j)), x[j], acc);
-    o[(size_t)h * D + d] = acc * (1.0f / L);
+    const float r = acc * (1.0f / L);
+    o[(size_t)h * D + d] = GATED ? sigmoid_gate(r, gv) : r;
 }
 
 // scalar variant for head_dim not a multiple of 4 (or > 1024 threads' worth): one thread per d
@@ -722,14 +730,24 @@ hipError_t launch_split(const SplitLaunch& L, hipStream_t stream) {
 }
 
 hipError_t launch_reduce(const float* so, const float* sm, const float* ss, float* o, uint32_t n_heads,
-                         uint32_t D, uint32_t n_tiles, hipStream_t stream) {
+                         uint32_t D, uint32_t n_tiles, hipStream_t stream, const GateArgs* gate, bool* gate_applied) {
     if (n_heads == 0u || D == 0u || n_tiles == 0u) return hipErrorInvalidValue;
+    if (gate_applied) *gate_applied = false;
+    const bool gated = gate != nullptr && gate->gate != nullptr;
+    if (gated && gate->chunk == 0u) return hipErrorInvalidValue;
     const bool vec = (D % 4u == 0u) && (D / 4u <= (uint32_t)kReduceThreads) && n_tiles <= 8192u &&
                      ((((uintptr_t)so) & 15u) == 0u);
     if (n_tiles <= 64u && D % (uint32_t)kWave == 0u) {
         const dim3 grid(D / kWave, n_heads);
-        if (n_tiles <= 32u) hipLaunchKernelGGL(reduce_direct_kernel<32>, grid, dim3(kWave), 0, stream, so, sm, ss, o, D, n_tiles);
-        else hipLaunchKernelGGL(reduce_direct_kernel<64>, grid, dim3(kWave), 0, stream, so, sm, ss, o, D, n_tiles);
+        const GateArgs g = gated ? *gate : GateArgs();
+        if (gated) {
+            if (n_tiles <= 32u) hipLaunchKernelGGL((reduce_direct_kernel<32, true>), grid, dim3(kWave), 0, stream, so, sm, ss, o, D, n_tiles, g);
+            else hipLaunchKernelGGL((reduce_direct_kernel<64, true>), grid, dim3(kWave), 0, stream, so, sm, ss, o, D, n_tiles, g);
+            if (gate_applied) *gate_applied = true;
+        } else {
+            if (n_tiles <= 32u) hipLaunchKernelGGL((reduce_direct_kernel<32, false>), grid, dim3(kWave), 0, stream, so, sm, ss, o, D, n_tiles, g);
+            else hipLaunchKernelGGL((reduce_direct_kernel<64, false>), grid, dim3(kWave), 0, stream, so, sm, ss, o, D, n_tiles, g);
+        }
     } else if (vec) {
         const uint32_t d4n = D / 4u;
         const uint32_t parts = kReduceThreads / d4n;

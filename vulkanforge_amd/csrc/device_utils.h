@@ -165,4 +165,13 @@ __device__ __forceinline__ float wave_max_all(float v) {
     return v;
 }
 
+// vk_shaders/sigmoid_mul.comp:50-52: x * 1 / (1 + exp(-g)), f32 throughout
+__device__ __forceinline__ float sigmoid_gate(float x, float g) { return x * (1.0f / (1.0f + expf(-g))); }
+// vk_shaders/sigmoid_mul.comp:44-48
+template <typename G>
+__device__ __forceinline__ uint64_t gate_index(const G& g, uint64_t i) {
+    const uint64_t token = i / g.chunk;
+    return token * g.stride + g.gate_offset + (i - token * g.chunk);
+}
+
 }  // namespace vfkv

@@ -63,8 +63,19 @@ struct SplitLaunch {
 hipError_t launch_split(const SplitLaunch& a, hipStream_t stream);
 bool split_appends(const SplitLaunch& a);
 bool split_writes_output(const SplitLaunch& a);
+// Gate of the attention output (vk_shaders/sigmoid_mul.comp:30-53): element i of the output is multiplied by
+// sigmoid(gate[(i / chunk) * stride + gate_offset + i % chunk]).  gate == NULL: no gate.
+struct GateArgs {
+    const float* gate = nullptr;
+    uint32_t chunk = 1, stride = 1, gate_offset = 0;
+};
+// `gate` (optional) is applied in the merge's own store where the kernel chosen for the shape can do so; otherwise
+// (and only then) *gate_applied is false and the caller follows up with launch_sigmoid_mul.
 hipError_t launch_reduce(const float* scratch_out, const float* scratch_max, const float* scratch_sum, float* o,
-                         uint32_t n_heads, uint32_t head_dim, uint32_t n_tiles, hipStream_t stream);
+                         uint32_t n_heads, uint32_t head_dim, uint32_t n_tiles, hipStream_t stream,
+                         const GateArgs* gate = nullptr, bool* gate_applied = nullptr);
+// ---- gated_output.hip ----
+hipError_t launch_sigmoid_mul(float* data, uint32_t ne, const GateArgs& gate, hipStream_t stream);
 // Smallest tile granule (keys) the split kernel for this shape works in; 0 if unsupported.
 uint32_t split_tile_granule(uint32_t dtype, uint32_t head_dim);
 

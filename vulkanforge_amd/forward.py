@@ -197,5 +197,45 @@ class Forward:
                                                      _ptr(q), _ptr(o), seq_len, base_pos, kv_start_window, scale,
                                                      softcap, _stream(stream)))
 
+    # ---- gated attention output (runs.rs:2649-2681, executor/attention.rs:632-680, 2405-2444) ----
+    @staticmethod
+    def run_sigmoid_mul(gate, inout, ne: int, chunk: int, stride: int, gate_offset: int, stream=None) -> None:
+        """inout[i] *= sigmoid(gate[(i // chunk) * stride + gate_offset + i % chunk]) for i < ne."""
+        g = _ffi.Gate(_ptr(gate), chunk, stride, gate_offset)
+        _ffi.check(_ffi.lib().vfkv_sigmoid_mul(C.byref(g), _ptr(inout), ne, _stream(stream)))
+
+    def step_attn_gated_output(self, attn_out, q_buf, q_dim: int, stream=None) -> None:
+        """executor/attention.rs:632-680: one token, the gate sits behind Q in ``q_buf``."""
+        self.run_sigmoid_mul(q_buf, attn_out, q_dim, q_dim, q_dim, q_dim, stream)
+
+    def b_step_attn_gated_output(self, batch_attn_out, batch_qgate, seq_len: int, head_dim: int, stream=None) -> None:
+        """executor/attention.rs:2405-2444: per (token, head) the gate follows the head's Q in ``batch_qgate``."""
+        self.run_sigmoid_mul(batch_qgate, batch_attn_out, seq_len * self.n_heads * head_dim, head_dim, 2 * head_dim, head_dim,
+                             stream)
+
+    def step_attention_gated(self, layer: int, position: int, q, o, gate, chunk: int, stride: int, gate_offset: int,
+                             k_src=None, v_src=None, kv_layer: int | None = None, kv_start: int = 0,
+                             scale: float | None = None, softcap: float = 0.0, stream=None) -> None:
+        """(step_kv_write +) step_attention + step_attn_gated_output as one call: the merge applies the gate."""
+        if scale is None:
+            hd = self.kv_cache.head_dim_for(layer)
+            scale = self.attn_scale if hd == self.kv_cache.config.head_dim else 1.0 / math.sqrt(hd)
+        g = _ffi.Gate(_ptr(gate), chunk, stride, gate_offset)
+        _ffi.check(_ffi.lib().vfkv_decode_attention_gated(
+            self.kv_cache.handle, layer, layer if kv_layer is None else kv_layer, self.n_heads, _ptr(q), _ptr(k_src),
+            _ptr(v_src), _ptr(o), position, kv_start, scale, softcap, C.byref(g), self.workspace._h, _stream(stream)))
+
+    def b_step_attention_gated(self, layer: int, base_pos: int, seq_len: int, q, o, gate, chunk: int, stride: int,
+                               gate_offset: int, kv_layer: int | None = None, kv_start_window: int = 0,
+                               scale: float | None = None, softcap: float = 0.0, stream=None) -> None:
+        """b_step_attention + b_step_attn_gated_output."""
+        if scale is None:
+            hd = self.kv_cache.head_dim_for(layer)
+            scale = self.attn_scale if hd == self.kv_cache.config.head_dim else 1.0 / math.sqrt(hd)
+        g = _ffi.Gate(_ptr(gate), chunk, stride, gate_offset)
+        _ffi.check(_ffi.lib().vfkv_prefill_attention_gated(
+            self.kv_cache.handle, layer, layer if kv_layer is None else kv_layer, self.n_heads, _ptr(q), _ptr(o), seq_len,
+            base_pos, kv_start_window, scale, softcap, C.byref(g), _stream(stream)))
+
 
 __all__ = ["Forward", "Workspace", "KvDtype", "FA_TILE"]

@@ -204,6 +204,27 @@ public:
         check(vfkv_prefill_attention(kv_cache.handle(), layer, kv_layer, n_heads, q, o, seq_len, base_pos, kv_start_window,
                                      scale_for(layer), softcap, stream));
     }
+    // runs.rs:2649-2681
+    void run_sigmoid_mul(const float* gate, float* inout, uint32_t ne, uint32_t chunk, uint32_t stride, uint32_t gate_offset) {
+        const vfkv_gate g{gate, chunk, stride, gate_offset};
+        check(vfkv_sigmoid_mul(&g, inout, ne, stream));
+    }
+    // attention.rs:632-680 (one token: the gate sits behind Q in q_buf) and :2405-2444 (per (token, head) slices [Q | G])
+    void step_attn_gated_output(float* attn_out, const float* q_buf, uint32_t q_dim) { run_sigmoid_mul(q_buf, attn_out, q_dim, q_dim, q_dim, q_dim); }
+    void b_step_attn_gated_output(float* batch_attn_out, const float* batch_qgate, uint32_t seq_len, uint32_t head_dim) {
+        run_sigmoid_mul(batch_qgate, batch_attn_out, seq_len * n_heads * head_dim, head_dim, 2 * head_dim, head_dim);
+    }
+    // (step_kv_write +) step_attention + step_attn_gated_output as one call; k_src / v_src may be NULL
+    void step_attention_gated(uint32_t layer, uint32_t kv_layer, uint32_t position, const float* q, const float* k_src,
+                              const float* v_src, float* attn_out, const vfkv_gate& gate, uint32_t kv_start = 0, float softcap = 0.f) {
+        check(vfkv_decode_attention_gated(kv_cache.handle(), layer, kv_layer, n_heads, q, k_src, v_src, attn_out, position, kv_start,
+                                          scale_for(layer), softcap, &gate, ws_, stream));
+    }
+    void b_step_attention_gated(uint32_t layer, uint32_t base_pos, uint32_t seq_len, const float* q, float* o, uint32_t kv_layer,
+                                uint32_t kv_start_window, const vfkv_gate& gate, float softcap = 0.f) {
+        check(vfkv_prefill_attention_gated(kv_cache.handle(), layer, kv_layer, n_heads, q, o, seq_len, base_pos, kv_start_window,
+                                           scale_for(layer), softcap, &gate, stream));
+    }
 
     float scale_for(uint32_t layer) const {   // runs.rs:746-760 without the Gemma-4 special case (pass scale = 1 explicitly)
         const uint32_t hd = kv_cache.head_dim_for(layer);

@@ -20,6 +20,7 @@ class DecodeWorkload:
     softcap: float = 0.0
     window: int = 0         # sliding window of the sliding layers (0 = none)
     sliding_pattern: int = 0  # k sliding layers followed by one global layer, repeated
+    gated: bool = False     # the output is multiplied by sigmoid(gate), the gate sitting behind Q (Qwen3.6 full attention)
 
     def layer_window(self, layer: int) -> int:
         if not self.window or not self.sliding_pattern:
@@ -64,6 +65,9 @@ DECODE = {
     "decode_fp8_32k_32layers": DecodeWorkload("decode_fp8_32k_32layers", 32, 32, 8, 128, 32768, KvDtype.F8, False),
     # the headline geometry over an F16 cache (not one of the reference configurations; used to tune the F16 variant)
     "decode_f16_32k_32layers": DecodeWorkload("decode_f16_32k_32layers", 32, 32, 8, 128, 32768, KvDtype.F16, False),
+    # the headline geometry with the gated output of the Qwen3.6 full-attention layers (not a reference configuration)
+    "decode_fp8_32k_32layers_gated": DecodeWorkload("decode_fp8_32k_32layers_gated", 32, 32, 8, 128, 32768, KvDtype.F8, False,
+                                                    gated=True),
     "decode_f16_hd256_sliding_12layers": DecodeWorkload("decode_f16_hd256_sliding_12layers", 12, 16, 8, 256, 16384,
                                                         KvDtype.F16, False, softcap=50.0, window=4096,
                                                         sliding_pattern=5),
@@ -71,12 +75,12 @@ DECODE = {
 PREFILL = {
     "prefill_fp8_512x4608_32layers": PrefillWorkload("prefill_fp8_512x4608_32layers", 32, 32, 8, 128, 4096, 512,
                                                      KvDtype.F8),
-    # the same geometry over an F16 cache (not one of the reference configurations; used to tune the F16 variant)
-    # Gemma-style geometry (16 query heads, 8 KV heads, head_dim 256): not a reference configuration either
+    # Gemma-style geometry (16 query heads, 8 KV heads, head_dim 256): not a reference configuration
     "prefill_f16_hd256_512x4608_12layers": PrefillWorkload("prefill_f16_hd256_512x4608_12layers", 12, 16, 8, 256, 4096,
                                                            512, KvDtype.F16),
     "prefill_fp8_hd256_512x4608_12layers": PrefillWorkload("prefill_fp8_hd256_512x4608_12layers", 12, 16, 8, 256, 4096,
                                                            512, KvDtype.F8),
+    # the headline prefill geometry over an F16 cache (not a reference configuration; used to tune the F16 variant)
     "prefill_f16_512x4608_32layers": PrefillWorkload("prefill_f16_512x4608_32layers", 32, 32, 8, 128, 4096, 512,
                                                      KvDtype.F16),
 }

@@ -82,7 +82,8 @@ int vfkv_cache_create_external(const vfkv_cache_config* cfg, void* k_buffer, voi
                                vfkv_cache** out);
 /* KvCache::destroy (kv_cache.rs:496-499). */
 void vfkv_cache_destroy(vfkv_cache* c);
-/* KvCache::zero_fill (kv_cache.rs:357-380) / zero_layer (kv_cache.rs:389-407). */
+/* KvCache::zero_fill (kv_cache.rs:357-380) / zero_layer (kv_cache.rs:389-407).  Both enqueue fill
+ * kernels (no memset nodes), so they may be captured into a HIP graph like the compute calls. */
 int vfkv_cache_zero_fill(vfkv_cache* c, vfkv_stream stream);
 int vfkv_cache_zero_layer(vfkv_cache* c, uint32_t layer, vfkv_stream stream);
 /* current_seq_len field and KvCache::reset (kv_cache.rs:492-494). */

@@ -72,3 +72,38 @@ def test_captured_decode_step_replays_like_eager(dtype, ctx):
             (q * 2).sum().item()                 # unrelated eager work between replays
     for c in caches:
         c.destroy()
+
+
+def test_captured_zero_layer_clears_on_every_replay():
+    # zero_layer (kv_cache.rs:389-407: the MTP scratch layer is cleared per step) inside a graph: the rows written between
+    # the replays are gone after each one, the neighbouring layers keep theirs.  Odd sizes exercise the byte-wise ends.
+    hkv, d, n = 3, 20, 37                                  # F8 rows of 60 bytes: the layer slab is not a multiple of 16
+    cache = vf.KvCache(vf.KvCacheConfig(3, hkv, d, n, dtype=vf.KvDtype.F8))
+    fwd = vf.Forward(cache, 3)
+    cache.zero_fill()
+    r = rng(8)
+    rows = to_dev(fp16_normal(r, (n, hkv * d)) + 1.0)
+    for layer in range(3):
+        fwd.b_step_kv_write(layer, 0, n, rows, rows)
+    torch.cuda.synchronize()
+    full = read_device(cache.k_ptr, cache.bytes_per_buffer()).copy()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        cache.zero_layer(1, stream=side.cuda_stream)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        cache.zero_layer(1, stream=torch.cuda.current_stream().cuda_stream)
+    lo, hi = cache.layer_offset_bytes(1), cache.layer_offset_bytes(2)
+    for rep in range(3):
+        fwd.b_step_kv_write(1, 0, n, rows, rows)           # eager work between the replays
+        torch.cuda.synchronize()
+        assert (read_device(cache.k_ptr, cache.bytes_per_buffer()) == full).all()
+        graph.replay()
+        torch.cuda.synchronize()
+        for ptr in (cache.k_ptr, cache.v_ptr):
+            got = read_device(ptr, cache.bytes_per_buffer())
+            assert (got[lo:hi] == 0).all() and (got[:lo] == full[:lo]).all() and (got[hi:] == full[hi:]).all()
+    cache.destroy()

@@ -204,8 +204,8 @@ void vfkv_cache_destroy(vfkv_cache* c) {
 
 int vfkv_cache_zero_fill(vfkv_cache* c, vfkv_stream stream) {
     if (!c || !c->k || !c->v) return fail(VFKV_ERR_INVALID_ARG, "cache has no buffers");
-    VFKV_HIP(hipMemsetAsync(c->k, 0, c->bytes, S(stream)));
-    VFKV_HIP(hipMemsetAsync(c->v, 0, c->bytes, S(stream)));
+    VFKV_HIP(vfkv::launch_zero_bytes(c->k, c->bytes, S(stream)));
+    VFKV_HIP(vfkv::launch_zero_bytes(c->v, c->bytes, S(stream)));
     return VFKV_OK;
 }
 
@@ -215,8 +215,8 @@ int vfkv_cache_zero_layer(vfkv_cache* c, uint32_t layer, vfkv_stream stream) {
     const uint64_t off = layer_off(c, layer);
     const uint64_t size = (uint64_t)c->max_seq_len * row_b(c, layer);
     if (size == 0) return VFKV_OK;
-    VFKV_HIP(hipMemsetAsync((char*)c->k + off, 0, size, S(stream)));
-    VFKV_HIP(hipMemsetAsync((char*)c->v + off, 0, size, S(stream)));
+    VFKV_HIP(vfkv::launch_zero_bytes((char*)c->k + off, size, S(stream)));
+    VFKV_HIP(vfkv::launch_zero_bytes((char*)c->v + off, size, S(stream)));
     return VFKV_OK;
 }
 

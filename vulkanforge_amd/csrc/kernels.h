@@ -9,6 +9,7 @@ namespace vfkv {
 hipError_t launch_kv_append(uint32_t dtype, const float* k_src, const float* v_src, void* k_dst, void* v_dst,
                             uint32_t n_elements, int n_tensors, hipStream_t stream);
 hipError_t launch_fp8_to_f16(const void* src, void* dst, uint64_t n, hipStream_t stream);
+hipError_t launch_zero_bytes(void* dst, uint64_t n, hipStream_t stream);
 
 // K RMS-norm * weight + RoPE + append of K and V rows in one launch (rope_append.hip).
 struct RopeAppendLaunch {

@@ -112,4 +112,28 @@ hipError_t launch_fp8_to_f16(const void* src, void* dst, uint64_t n, hipStream_t
     return hipGetLastError();
 }
 
+// KvCache::zero_fill / zero_layer (kv_cache.rs:357-407) as a kernel, so that a caller may capture it into a HIP graph (memset
+// nodes are avoided on purpose): 16-byte stores over the aligned body, single bytes at the two ends.
+__global__ __launch_bounds__(256) void zero_bytes_kernel(uint8_t* __restrict__ p, uint64_t head, uint64_t n_vec, uint64_t n) {
+    const uint64_t tid = (uint64_t)blockIdx.x * 256u + threadIdx.x, stride = (uint64_t)gridDim.x * 256u;
+    uint4* body = reinterpret_cast<uint4*>(p + head);
+    for (uint64_t i = tid; i < n_vec; i += stride) body[i] = make_uint4(0u, 0u, 0u, 0u);
+    const uint64_t tail0 = head + n_vec * 16u;
+    for (uint64_t i = tid; i < head; i += stride) p[i] = 0;
+    for (uint64_t i = tail0 + tid; i < n; i += stride) p[i] = 0;
+}
+
+hipError_t launch_zero_bytes(void* dst, uint64_t n, hipStream_t stream) {
+    if (n == 0) return hipSuccess;
+    if (dst == nullptr) return hipErrorInvalidValue;
+    uint64_t head = (16u - (((uintptr_t)dst) & 15u)) & 15u;
+    if (head > n) head = n;
+    const uint64_t n_vec = (n - head) / 16u;
+    uint64_t blocks = (n_vec + 255u) / 256u;
+    if (blocks == 0u) blocks = 1u;
+    if (blocks > 4096u) blocks = 4096u;
+    hipLaunchKernelGGL(zero_bytes_kernel, dim3((uint32_t)blocks), dim3(256), 0, stream, (uint8_t*)dst, head, n_vec, n);
+    return hipGetLastError();
+}
+
 }  // namespace vfkv

@@ -147,3 +147,34 @@ def test_window_uses_the_last_querys_lower_bound():
                                 kv_start=kv_start)
     assert np.abs(to_np(o) - ref).max() < TIGHT
     cache.destroy()
+
+
+@pytest.mark.parametrize("dtype", (vf.KvDtype.F16, vf.KvDtype.F8))
+@pytest.mark.parametrize("shape", ("ascending", "descending", "steps"))
+def test_scores_that_drift_past_the_running_maximum(dtype, shape):
+    # the kernel keeps a reference maximum that is allowed to lag behind the true one; scores that climb slowly, fall, or
+    # jump by hundreds between tiles must come out as the oracle computes them
+    heads, hkv, d, m, q_start = 8, 2, 128, 40, 700
+    n_kv = q_start + m
+    r = rng({"ascending": 1, "descending": 2, "steps": 3}[shape] + int(dtype))
+    u = r.standard_normal(d).astype(np.float32)
+    u /= np.linalg.norm(u)
+    t = np.arange(n_kv, dtype=np.float32)
+    if shape == "ascending":
+        level = 70.0 * t / n_kv                               # +3 per tile of 32 keys: below the slack tile after tile
+    elif shape == "descending":
+        level = 70.0 * (1.0 - t / n_kv)
+    else:
+        level = 40.0 * ((t // 96) % 3)                        # plateaus 0 / 40 / 80, up and down
+    k = (level[:, None, None] * u[None, None, :] * np.ones((1, hkv, 1), np.float32)).astype(np.float32)
+    k += 0.05 * r.standard_normal(k.shape).astype(np.float32)
+    q = np.broadcast_to(u * np.float32(np.sqrt(d)), (m, heads, d)).astype(np.float32).copy()
+    q += 0.05 * r.standard_normal(q.shape).astype(np.float32)
+    v = fp16_normal(r, (n_kv, hkv, d))
+    ke, ve = encode_np(k, dtype), encode_np(v, dtype)
+    scale = float(1.0 / np.sqrt(d))
+    print(f"case dtype={dtype.label()} shape={shape}", flush=True)
+    o = gpu_batch(q, ke, ve, dtype, heads, hkv, d, m, q_start, n_kv, scale)
+    ref = oracle.attn_batch_ref(q, ke, ve, int(dtype), m, n_kv, heads, hkv, d, q_start, scale)
+    assert np.isfinite(o).all()
+    assert np.abs(o - ref).max() < 1e-4

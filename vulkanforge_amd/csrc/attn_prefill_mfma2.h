@@ -36,6 +36,7 @@ __global__ __launch_bounds__((NCB == 1 && D <= 128) ? 768 : 512) void batch_mfma
     constexpr int VCHUNK_ROW = D * ES / 16;      // 16-byte chunks per V row
     constexpr int VLD = KT * VCHUNK_ROW / 64;    // V loads per lane per tile
     constexpr int VROWS = 64 / VCHUNK_ROW;
+    constexpr float kMaxSlack = 8.0f;            // log2 units by which a score may exceed the running reference maximum
     constexpr uint32_t kNoTile = 0x80000000u;    // byte offset past any slab: the load returns zeros, no memory access
     static_assert(D % 32 == 0 && SEGB % 16 == 0 && VLD >= 1, "unsupported head_dim");
 
@@ -236,10 +237,15 @@ __global__ __launch_bounds__((NCB == 1 && D <= 128) ? 768 : 512) void batch_mfma
                             x[kt * 4 + i] = y;
                             tmax = fmaxf(tmax, y);
                         }
-                    { float y = tmax; swap16(tmax, y); tmax = fmaxf(tmax, y); y = tmax; swap32(tmax, y); tmax = fmaxf(tmax, y); }
                     if (FOLD) tmax *= scale_l2;
-                    const float m_new = fmaxf(m_run[cb], tmax);
-                    if (__builtin_amdgcn_ballot_w64(m_new > m_run[cb]) != 0ull) {
+                    // The reference maximum only moves when some query's tile maximum exceeds it by more than 2^kMaxSlack: until
+                    // then the weights are exp2(x - m) <= 2^kMaxSlack (exact in the f16 value + remainder pair, far from f32
+                    // overflow in the sums), the final division by l cancels the common factor, and the accumulators are
+                    // spared a multiplication per tile.  The four lanes of a query share m, so the test needs no reduction:
+                    // the ballot sees the lane that holds the query's largest score.
+                    if (__builtin_amdgcn_ballot_w64(tmax > m_run[cb] + kMaxSlack) != 0ull) {
+                        { float y = tmax; swap16(tmax, y); tmax = fmaxf(tmax, y); y = tmax; swap32(tmax, y); tmax = fmaxf(tmax, y); }
+                        const float m_new = fmaxf(m_run[cb], tmax);
                         const float alpha = __builtin_amdgcn_exp2f(m_run[cb] - m_new);
                         l_run[cb] *= alpha;
 #pragma unroll

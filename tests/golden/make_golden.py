@@ -43,7 +43,7 @@ def encode_vectors(table):
     # every power of two across the f32 range that matters, and its neighbours
     p2 = np.ldexp(np.float32(1.0), np.arange(-30, 12)).astype(np.float32)
     xs += [p2, -p2, np.nextafter(p2, np.float32(0)), np.nextafter(p2, np.float32(np.inf))]
-    # BASELINE-style data: N(0,1)*0.5 with a +-40 outlier tail, and N(0,1) cast to fp16
+    # benchmark-style data: N(0,1)*0.5 with a +-40 outlier tail, and N(0,1) cast to fp16
     xs.append((rng.standard_normal(1500) * 0.5).astype(np.float32))
     xs.append(rng.standard_normal(800).astype(np.float16).astype(np.float32))
     xs.append(np.array([40.0, -40.0, 447.9, 448.0, -448.0, 463.9, 464.0, 465.0, 1000.0, -1000.0,

@@ -9,7 +9,7 @@ import oracle
 import vulkanforge_amd as vf
 
 DEV = "cuda:0"
-# north-star tolerances (max-abs vs the CPU oracle): F16 KV 2e-3, FP8 KV 5e-3.  F32 KV follows the
+# tolerances of this path (max-abs vs the CPU oracle): F16 KV 2e-3, FP8 KV 5e-3.  F32 KV follows the
 # reference's own test bar of 1e-3 (tests/correctness.rs:2875-2894).
 TOL = {vf.KvDtype.F32: 1e-3, vf.KvDtype.F16: 2e-3, vf.KvDtype.F8: 5e-3}
 # what f32 arithmetic on identical decoded inputs is expected to reach; a regression guard

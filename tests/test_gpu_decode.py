@@ -201,7 +201,7 @@ def _cache_with_history(dtype, n_layers, hkv, d, max_seq, fill, seed, hd=None, k
 
 
 def test_config1_append_then_decode_f16():
-    # BASELINE config 1: one layer, F16 KV, 32/8/128, context 2048, append one token, attend
+    # benchmark configuration 1: one layer, F16 KV, 32/8/128, context 2048, append one token, attend
     heads, hkv, d, ctx = 32, 8, 128, 2048
     cache, hist = _cache_with_history(vf.KvDtype.F16, 1, hkv, d, ctx + 1, fp16_normal, 11)
     fwd = vf.Forward(cache, heads)
@@ -221,7 +221,7 @@ def test_config1_append_then_decode_f16():
 
 
 def test_config2_fp8_outliers_append_then_decode_two_layers():
-    # BASELINE config 2 geometry (FP8 KV, context 8192, +-40 outlier tail), two layers of the 32
+    # benchmark configuration 2 geometry (FP8 KV, context 8192, +-40 outlier tail), two layers of the 32
     heads, hkv, d, ctx = 32, 8, 128, 8192
     cache, hist = _cache_with_history(vf.KvDtype.F8, 2, hkv, d, ctx + 1, outlier_normal, 21)
     fwd = vf.Forward(cache, heads)
@@ -309,7 +309,7 @@ def test_spans_of_one_tile_skip_the_merge_launch(dtype, heads, hkv, d, seq):
 
 
 def test_config4_hd256_sliding_window_softcap_f16():
-    # BASELINE config 4 geometry: 16/8/256, F16 KV, window 4096 at context 16384, soft-cap 50;
+    # benchmark configuration 4 geometry: 16/8/256, F16 KV, window 4096 at context 16384, soft-cap 50;
     # layer 0 sliding, layer 1 global
     heads, hkv, d, ctx, window, cap = 16, 8, 256, 16384, 4096, 50.0
     cache, hist = _cache_with_history(vf.KvDtype.F16, 2, hkv, d, ctx, fp16_normal, 31)

@@ -101,7 +101,7 @@ def test_batch_with_f32_queries_keeps_f32_accuracy(dtype):
 
 
 def test_config5_chunk_append_then_prefill_fp8_one_layer():
-    # BASELINE config 5, one of its 32 layers: FP8 cache filled to 4096, append 512 tokens, then
+    # benchmark configuration 5, one of its 32 layers: FP8 cache filled to 4096, append 512 tokens, then
     # 512 causal queries over 4608 keys (32/8/128).  The oracle is run on a sample of query rows.
     heads, hkv, d, base, m = 32, 8, 128, 4096, 512
     cache = vf.KvCache(vf.KvCacheConfig(1, hkv, d, base + m, dtype=vf.KvDtype.F8))

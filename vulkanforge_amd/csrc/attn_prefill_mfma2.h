@@ -142,150 +142,198 @@ __global__ __launch_bounds__((NCB == 1 && D <= 128) ? 768 : 512) void batch_mfma
 #pragma unroll
     for (int cb = 0; cb < NCB; ++cb) { m_run[cb] = kMasked; l_run[cb] = 0.f; }
 
-    for (uint32_t tb = tb0; tb < kmax; tb += PFD * step) {
+    // ---- pieces of one tile ----
+    float4_t s[NCB][2];
+    float x[NCB][8], tmax[NCB];
+    // V tile -> f16 row-major in this wavefront's LDS area (first: the writes complete behind the first product and the
+    // softmax), the slot's next tile requested, then S^T = K Q^T for the NCB heads (Q operands re-read from LDS every tile)
+    auto stage_and_first_product = [&](int sl, uint32_t tcur) {
+        const uint32_t noff = tile_off(tcur + PFD * step);
+#pragma unroll
+        for (int c = 0; c < VLD; ++c) {
+            _Float16* dst = vb + (c * VROWS + vrow) * VPITCH + vcol * (16 / ES);
+            if (DT == kF8) {
+                uint32_t out[8];
+#pragma unroll
+                for (int q4 = 0; q4 < 4; ++q4) {
+                    const uint32_t wd = vraw[sl][c][q4];
+                    half2_t lo2, hi2;
+                    e4m3x4_to_h2(wd, lo2, hi2);
+                    out[2 * q4] = __builtin_bit_cast(uint32_t, lo2);
+                    out[2 * q4 + 1] = __builtin_bit_cast(uint32_t, hi2);
+                }
+                reinterpret_cast<u32x4*>(dst)[0] = u32x4{out[0], out[1], out[2], out[3]};
+                reinterpret_cast<u32x4*>(dst)[1] = u32x4{out[4], out[5], out[6], out[7]};
+            } else {
+                *reinterpret_cast<u32x4*>(dst) = vraw[sl][c];
+            }
+            vraw[sl][c] = __builtin_amdgcn_raw_buffer_load_b128(vrsrc, lane_voff, noff + (uint32_t)(c * VROWS) * row_stride, 0);
+        }
+        half8_t qhi[NCB][KS];
+#pragma unroll
+        for (int cb = 0; cb < NCB; ++cb)
+#pragma unroll
+            for (int c = 0; c < KS; ++c)
+                qhi[cb][c] = *reinterpret_cast<const half8_t*>(qhi_lds + ((size_t)(g0 + cb) * 16 + n16) * QPITCH + kg * SEG + c * 8);
+#pragma unroll
+        for (int kt = 0; kt < 2; ++kt) {
+            half8_t ka[KS];
+#pragma unroll
+            for (int c = 0; c < KS; ++c) {
+                if (DT == kF8) {
+                    const uint32_t w0 = kraw[sl][kt][c / 2][(c % 2) * 2], w1 = kraw[sl][kt][c / 2][(c % 2) * 2 + 1];
+                    half2_t p0, p1, p2, p3;
+                    e4m3x4_to_h2(w0, p0, p1);
+                    e4m3x4_to_h2(w1, p2, p3);
+                    ka[c][0] = p0[0]; ka[c][1] = p0[1]; ka[c][2] = p1[0]; ka[c][3] = p1[1];
+                    ka[c][4] = p2[0]; ka[c][5] = p2[1]; ka[c][6] = p3[0]; ka[c][7] = p3[1];
+                } else {
+                    const u32x4 wv = kraw[sl][kt][c % KLD];
+                    ka[c] = __builtin_bit_cast(half8_t, wv);
+                }
+            }
+#pragma unroll
+            for (int xx = 0; xx < KLD; ++xx)
+                kraw[sl][kt][xx] = __builtin_amdgcn_raw_buffer_load_b128(krsrc, lane_koff + xx * 16, noff + (uint32_t)(kt * 16) * row_stride, 0);
+#pragma unroll
+            for (int cb = 0; cb < NCB; ++cb) {
+                s[cb][kt] = float4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int c = 0; c < KS; ++c) s[cb][kt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ka[c], qhi[cb][c], s[cb][kt], 0, 0, 0);
+            }
+            if (has_lo) {
+#pragma unroll
+                for (int cb = 0; cb < NCB; ++cb) {
+                    const _Float16* lo_row = qlo_lds + ((size_t)(g0 + cb) * 16 + n16) * QPITCH + kg * SEG;
+#pragma unroll
+                    for (int c = 0; c < KS; ++c) {
+                        const half8_t ql = *reinterpret_cast<const half8_t*>(lo_row + c * 8);
+                        s[cb][kt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ka[c], ql, s[cb][kt], 0, 0, 0);
+                    }
+                }
+            }
+        }
+    };
+    // scores of the tile in log2 units (this lane owns keys tcur + kt*16 + kg*4 + i of query n16); returns whether one of
+    // them exceeds the lane's reference maximum by more than the slack
+    auto scores = [&](auto masked_tag, uint32_t tcur) -> bool {
+        constexpr bool MASKED = decltype(masked_tag)::value;
+        constexpr bool FOLD = !MASKED && !CAP;                   // scores stay unscaled until the exponent's FMA
+        bool moved = false;
+#pragma unroll
+        for (int cb = 0; cb < NCB; ++cb) {
+            tmax[cb] = kMasked;
+#pragma unroll
+            for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    float y = FOLD ? s[cb][kt][i] : s[cb][kt][i] * scale_l2;
+                    if (CAP) y = cap_l2 * tanhf(y / cap_l2);
+                    if (MASKED) {
+                        const uint32_t t = tcur + kt * 16 + kg * 4 + i;
+                        y = (t < my_len && t >= a.kv_start) ? y : kMasked;
+                    }
+                    x[cb][kt * 4 + i] = y;
+                    tmax[cb] = fmaxf(tmax[cb], y);
+                }
+            if (FOLD) tmax[cb] *= scale_l2;
+            moved |= tmax[cb] > m_run[cb] + kMaxSlack;
+        }
+        return moved;
+    };
+    auto move_maximum = [&]() {
+#pragma unroll
+        for (int cb = 0; cb < NCB; ++cb) {
+            float t = tmax[cb];
+            { float y = t; swap16(t, y); t = fmaxf(t, y); y = t; swap32(t, y); t = fmaxf(t, y); }
+            const float m_new = fmaxf(m_run[cb], t);
+            const float alpha = __builtin_amdgcn_exp2f(m_run[cb] - m_new);
+            l_run[cb] *= alpha;
+#pragma unroll
+            for (int dt = 0; dt < DTILES; ++dt) oacc[cb][dt] *= alpha;
+            m_run[cb] = m_new;
+        }
+    };
+    // weights as f16 value + f16 remainder, then O^T += V^T P^T for the NCB heads
+    auto weights_and_second_product = [&](auto masked_tag) {
+        constexpr bool MASKED = decltype(masked_tag)::value;
+        constexpr bool FOLD = !MASKED && !CAP;
+        u32x4 phi[NCB], plo[NCB];
+#pragma unroll
+        for (int cb = 0; cb < NCB; ++cb)
+#pragma unroll
+            for (int j2 = 0; j2 < 4; ++j2) {
+                float2_t pp;
+#pragma unroll
+                for (int e = 0; e < 2; ++e) {
+                    const float xe = x[cb][2 * j2 + e];
+                    float pv = __builtin_amdgcn_exp2f(FOLD ? __builtin_fmaf(xe, scale_l2, -m_run[cb]) : xe - m_run[cb]);
+                    if (MASKED) pv = xe > -1e29f ? pv : 0.f;
+                    pp[e] = pv;
+                }
+                l_run[cb] += pp[0] + pp[1];
+                phi[cb][j2] = __builtin_bit_cast(uint32_t, __builtin_convertvector(pp, half2_t));
+                plo[cb][j2] = pack_f16_remainder(pp[0], pp[1], phi[cb][j2]);
+            }
+#pragma unroll
+        for (int dt = 0; dt < DTILES; ++dt) {
+            // supplier lane s of a 16-lane group points at V[key = 4*kg + s/4 (+16)][d = dt*16 + 4*(s%4)]
+            const _Float16* p0 = vb + (kg * 4 + n16 / 4) * VPITCH + dt * 16 + 4 * (n16 % 4);
+            const half4_t v0 = lds_read_tr16(p0);
+            const half4_t v1 = lds_read_tr16(p0 + 16 * VPITCH);
+            half8_t va;
+            va[0] = v0[0]; va[1] = v0[1]; va[2] = v0[2]; va[3] = v0[3]; va[4] = v1[0]; va[5] = v1[1]; va[6] = v1[2]; va[7] = v1[3];
+#pragma unroll
+            for (int cb = 0; cb < NCB; ++cb)
+                oacc[cb][dt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(va, __builtin_bit_cast(half8_t, phi[cb]), oacc[cb][dt], 0, 0, 0);
+#pragma unroll
+            for (int cb = 0; cb < NCB; ++cb)
+                oacc[cb][dt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(va, __builtin_bit_cast(half8_t, plo[cb]), oacc[cb][dt], 0, 0, 0);
+        }
+    };
+
+    // ---- the wavefront's tiles.  The reference maximum m of a query only moves when some score of a tile exceeds it by more
+    // than 2^kMaxSlack: until then the weights are exp2(x - m) <= 2^kMaxSlack (exact in the f16 value + remainder pair, far
+    // from f32 overflow in the sums), the division by l at the end cancels the common factor, and the accumulators are
+    // spared a multiplication per tile.  The four lanes of a query share m, so the test needs no reduction: the ballot sees
+    // the lane that holds the query's largest score.  Tiles are processed in groups of PFD (one per prefetch slot) by
+    // two loops: the inner one only takes tiles that every query of the block sees completely and leaves as soon as a
+    // maximum has to move, so that its accumulators have a single definition per tile and stay in place; the outer one
+    // handles whatever the inner one left (first tiles, moved maxima, tiles on the causal diagonal or the window edge).
+    uint32_t tb = tb0;
+    int first_slot = 0;          // slots of the group at tb that the inner loop has already finished
+    bool s_ready = false;        // s[] of slot first_slot is already computed
+    while (tb < kmax) {
 #pragma unroll
         for (int sl = 0; sl < PFD; ++sl) {
             const uint32_t tcur = tb + sl * step;
             if (tcur >= kmax) break;                            // wavefront-uniform
-            const uint32_t noff = tile_off(tcur + PFD * step);
-            // ---------------- V tile -> f16 row-major in this wavefront's LDS area (first: the writes complete behind the first product and the softmax) ----------------
-#pragma unroll
-            for (int c = 0; c < VLD; ++c) {
-                _Float16* dst = vb + (c * VROWS + vrow) * VPITCH + vcol * (16 / ES);
-                if (DT == kF8) {
-                    uint32_t out[8];
-#pragma unroll
-                    for (int q4 = 0; q4 < 4; ++q4) {
-                        const uint32_t wd = vraw[sl][c][q4];
-                        half2_t lo2, hi2;
-                        e4m3x4_to_h2(wd, lo2, hi2);
-                        out[2 * q4] = __builtin_bit_cast(uint32_t, lo2);
-                        out[2 * q4 + 1] = __builtin_bit_cast(uint32_t, hi2);
-                    }
-                    reinterpret_cast<u32x4*>(dst)[0] = u32x4{out[0], out[1], out[2], out[3]};
-                    reinterpret_cast<u32x4*>(dst)[1] = u32x4{out[4], out[5], out[6], out[7]};
-                } else {
-                    *reinterpret_cast<u32x4*>(dst) = vraw[sl][c];
-                }
-                vraw[sl][c] = __builtin_amdgcn_raw_buffer_load_b128(vrsrc, lane_voff, noff + (uint32_t)(c * VROWS) * row_stride, 0);
+            if (sl < first_slot) continue;
+            if (!(s_ready && sl == first_slot)) stage_and_first_product(sl, tcur);
+            if (tcur >= a.kv_start && tcur + KT <= full_len) {  // every query of the block sees the whole tile
+                if (__builtin_amdgcn_ballot_w64(scores(std::false_type{}, tcur)) != 0ull) move_maximum();
+                weights_and_second_product(std::false_type{});
+            } else {
+                if (__builtin_amdgcn_ballot_w64(scores(std::true_type{}, tcur)) != 0ull) move_maximum();
+                weights_and_second_product(std::true_type{});
             }
-            // ---------------- S^T = K Q^T for the NCB heads (Q operands re-read from LDS every tile) ----------------
-            float4_t s[NCB][2];
-            half8_t qhi[NCB][KS];
+        }
+        tb += PFD * step;
+        first_slot = 0;
+        s_ready = false;
+        bool left = false;
+        while (!left && tb >= a.kv_start && tb + (PFD - 1) * step + KT <= full_len) {
 #pragma unroll
-            for (int cb = 0; cb < NCB; ++cb)
-#pragma unroll
-                for (int c = 0; c < KS; ++c)
-                    qhi[cb][c] = *reinterpret_cast<const half8_t*>(qhi_lds + ((size_t)(g0 + cb) * 16 + n16) * QPITCH + kg * SEG + c * 8);
-#pragma unroll
-            for (int kt = 0; kt < 2; ++kt) {
-                half8_t ka[KS];
-#pragma unroll
-                for (int c = 0; c < KS; ++c) {
-                    if (DT == kF8) {
-                        const uint32_t w0 = kraw[sl][kt][c / 2][(c % 2) * 2], w1 = kraw[sl][kt][c / 2][(c % 2) * 2 + 1];
-                        half2_t p0, p1, p2, p3;
-                        e4m3x4_to_h2(w0, p0, p1);
-                        e4m3x4_to_h2(w1, p2, p3);
-                        ka[c][0] = p0[0]; ka[c][1] = p0[1]; ka[c][2] = p1[0]; ka[c][3] = p1[1];
-                        ka[c][4] = p2[0]; ka[c][5] = p2[1]; ka[c][6] = p3[0]; ka[c][7] = p3[1];
-                    } else {
-                        const u32x4 wv = kraw[sl][kt][c % KLD];
-                        ka[c] = __builtin_bit_cast(half8_t, wv);
-                    }
+            for (int sl = 0; sl < PFD; ++sl) {
+                const uint32_t tcur = tb + sl * step;
+                stage_and_first_product(sl, tcur);
+                if (__builtin_amdgcn_ballot_w64(scores(std::false_type{}, tcur)) != 0ull) {
+                    first_slot = sl; s_ready = true; left = true;
+                    break;
                 }
-#pragma unroll
-                for (int x = 0; x < KLD; ++x)
-                    kraw[sl][kt][x] = __builtin_amdgcn_raw_buffer_load_b128(krsrc, lane_koff + x * 16, noff + (uint32_t)(kt * 16) * row_stride, 0);
-#pragma unroll
-                for (int cb = 0; cb < NCB; ++cb) {
-                    s[cb][kt] = float4_t{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-                    for (int c = 0; c < KS; ++c) s[cb][kt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ka[c], qhi[cb][c], s[cb][kt], 0, 0, 0);
-                }
-                if (has_lo) {
-#pragma unroll
-                    for (int cb = 0; cb < NCB; ++cb) {
-                        const _Float16* lo_row = qlo_lds + ((size_t)(g0 + cb) * 16 + n16) * QPITCH + kg * SEG;
-#pragma unroll
-                        for (int c = 0; c < KS; ++c) {
-                            const half8_t ql = *reinterpret_cast<const half8_t*>(lo_row + c * 8);
-                            s[cb][kt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ka[c], ql, s[cb][kt], 0, 0, 0);
-                        }
-                    }
-                }
+                weights_and_second_product(std::false_type{});
             }
-            // ---------------- online softmax: this lane owns keys tcur + kt*16 + kg*4 + i of query n16 ----------------
-            u32x4 phi[NCB], plo[NCB];
-            auto softmax = [&](auto masked_tag) {
-                constexpr bool MASKED = decltype(masked_tag)::value;
-                constexpr bool FOLD = !MASKED && !CAP;                   // scores stay unscaled until the exponent's FMA
-#pragma unroll
-                for (int cb = 0; cb < NCB; ++cb) {
-                    float x[8];
-                    float tmax = kMasked;
-#pragma unroll
-                    for (int kt = 0; kt < 2; ++kt)
-#pragma unroll
-                        for (int i = 0; i < 4; ++i) {
-                            float y = FOLD ? s[cb][kt][i] : s[cb][kt][i] * scale_l2;
-                            if (CAP) y = cap_l2 * tanhf(y / cap_l2);
-                            if (MASKED) {
-                                const uint32_t t = tcur + kt * 16 + kg * 4 + i;
-                                y = (t < my_len && t >= a.kv_start) ? y : kMasked;
-                            }
-                            x[kt * 4 + i] = y;
-                            tmax = fmaxf(tmax, y);
-                        }
-                    if (FOLD) tmax *= scale_l2;
-                    // The reference maximum only moves when some query's tile maximum exceeds it by more than 2^kMaxSlack: until
-                    // then the weights are exp2(x - m) <= 2^kMaxSlack (exact in the f16 value + remainder pair, far from f32
-                    // overflow in the sums), the final division by l cancels the common factor, and the accumulators are
-                    // spared a multiplication per tile.  The four lanes of a query share m, so the test needs no reduction:
-                    // the ballot sees the lane that holds the query's largest score.
-                    if (__builtin_amdgcn_ballot_w64(tmax > m_run[cb] + kMaxSlack) != 0ull) {
-                        { float y = tmax; swap16(tmax, y); tmax = fmaxf(tmax, y); y = tmax; swap32(tmax, y); tmax = fmaxf(tmax, y); }
-                        const float m_new = fmaxf(m_run[cb], tmax);
-                        const float alpha = __builtin_amdgcn_exp2f(m_run[cb] - m_new);
-                        l_run[cb] *= alpha;
-#pragma unroll
-                        for (int dt = 0; dt < DTILES; ++dt) oacc[cb][dt] *= alpha;
-                        m_run[cb] = m_new;
-                    }
-#pragma unroll
-                    for (int j2 = 0; j2 < 4; ++j2) {
-                        float2_t pp;
-#pragma unroll
-                        for (int e = 0; e < 2; ++e) {
-                            const float xe = x[2 * j2 + e];
-                            float pv = __builtin_amdgcn_exp2f(FOLD ? __builtin_fmaf(xe, scale_l2, -m_run[cb]) : xe - m_run[cb]);
-                            if (MASKED) pv = xe > -1e29f ? pv : 0.f;
-                            pp[e] = pv;
-                        }
-                        l_run[cb] += pp[0] + pp[1];
-                        phi[cb][j2] = __builtin_bit_cast(uint32_t, __builtin_convertvector(pp, half2_t));
-                        plo[cb][j2] = pack_f16_remainder(pp[0], pp[1], phi[cb][j2]);
-                    }
-                }
-            };
-            const bool interior = tcur >= a.kv_start && tcur + KT <= full_len;   // every query of the block sees the whole tile
-            if (interior) softmax(std::false_type{}); else softmax(std::true_type{});
-            // ---------------- O^T += V^T P^T for the NCB heads ----------------
-#pragma unroll
-            for (int dt = 0; dt < DTILES; ++dt) {
-                // supplier lane s of a 16-lane group points at V[key = 4*kg + s/4 (+16)][d = dt*16 + 4*(s%4)]
-                const _Float16* p0 = vb + (kg * 4 + n16 / 4) * VPITCH + dt * 16 + 4 * (n16 % 4);
-                const half4_t v0 = lds_read_tr16(p0);
-                const half4_t v1 = lds_read_tr16(p0 + 16 * VPITCH);
-                half8_t va;
-                va[0] = v0[0]; va[1] = v0[1]; va[2] = v0[2]; va[3] = v0[3]; va[4] = v1[0]; va[5] = v1[1]; va[6] = v1[2]; va[7] = v1[3];
-#pragma unroll
-                for (int cb = 0; cb < NCB; ++cb)
-                    oacc[cb][dt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(va, __builtin_bit_cast(half8_t, phi[cb]), oacc[cb][dt], 0, 0, 0);
-#pragma unroll
-                for (int cb = 0; cb < NCB; ++cb)
-                    oacc[cb][dt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(va, __builtin_bit_cast(half8_t, plo[cb]), oacc[cb][dt], 0, 0, 0);
-            }
+            if (!left) tb += PFD * step;
         }
     }
 #pragma unroll

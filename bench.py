@@ -29,6 +29,7 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBPS = 8000.0       # MI355X HBM3E, published
 MFMA_F16_PEAK_TFLOPS = 2500.0
+MFMA_F32_PEAK_TFLOPS = 157.3      # dense f32 matrix rate: what an F32 cache is multiplied at
 
 
 # HBM bytes per launch of the dominant kernel, measured with rocprofv3 --pmc FETCH_SIZE and --pmc WRITE_SIZE
@@ -341,18 +342,22 @@ def bench_prefill(args, wl):
     torch.cuda.synchronize()
     avg_ms = sum(a.elapsed_time(b) for a, b in pairs) / len(pairs)
     achieved = wl.flops_layer() / (avg_ms * 1e-3) / 1e12
+    f32_cache = wl.dtype.label() == "FP32"
+    peak = MFMA_F32_PEAK_TFLOPS if f32_cache else MFMA_F16_PEAK_TFLOPS
     result = {
         "metric": "prefill_attention_TFLOPs",
         "value": flops_step / sec_per_step / 1e12,
         "unit": "TFLOP/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": sec_per_step * 1e3,
         "step_us_event_timed": step_spread,
-        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f16", "kv_dtype": wl.dtype.label(),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32" if f32_cache else "f16",
+        "kv_dtype": wl.dtype.label(),
         "data": "synthetic, seeded N(0,1); queries " + ("general f32" if args.f32_queries else "cast to fp16 as the configuration states") + "; K/V rows cast to fp16 and written through the append kernels",
         "config": {"workload": wl.name, "n_layers": L, "n_heads": H, "n_kv_heads": Hkv, "head_dim": D,
                    "m": wl.m, "q_start": wl.base_pos, "n_kv": max_seq, "flop_per_step": flops_step},
-        "roofline": {"bound": "mfma", "kernel": "batch_mfma2_kernel", "achieved": achieved, "peak": MFMA_F16_PEAK_TFLOPS,
-                     "unit": "TFLOP/s", "frac": achieved / MFMA_F16_PEAK_TFLOPS, "traffic": MEASURED_TRAFFIC_BYTES.get(wl.name),
+        "roofline": {"bound": "mfma", "kernel": "batch_mfma_f32_kernel" if f32_cache else "batch_mfma2_kernel",
+                     "achieved": achieved, "peak": peak,
+                     "unit": "TFLOP/s", "frac": achieved / peak, "traffic": MEASURED_TRAFFIC_BYTES.get(wl.name),
                      "avg_launch_us": avg_ms * 1e3},
     }
     if not args.no_cpu_baseline:

@@ -60,6 +60,10 @@ CASES = [
     (vf.KvDtype.F8, 12, 2, 128, 23, 2100, 1500, 0.0), # G = 6: three head pairs, two key splits, window
     (vf.KvDtype.F8, 16, 8, 64, 70, 600, 0, 30.0),     # G = 2: one head pair, eight key splits, soft-cap
     (vf.KvDtype.F16, 16, 2, 128, 33, 900, 0, 0.0),    # G = 8 on a 2-byte cache
+    (vf.KvDtype.F32, 32, 8, 128, 37, 500, 0, 0.0),    # F32 cache on the f32 matrix-core kernel: G = 4
+    (vf.KvDtype.F32, 16, 2, 128, 20, 333, 120, 30.0), # G = 8 (two workgroups per KV head), window, soft-cap
+    (vf.KvDtype.F32, 3, 3, 256, 18, 70, 0, 0.0),      # G = 1, head_dim 256
+    (vf.KvDtype.F32, 10, 2, 64, 49, 0, 0, 0.0),       # G = 5: a workgroup with one live wavefront, from position 0
     (vf.KvDtype.F8, 16, 8, 256, 48, 700, 0, 50.0),    # head_dim 256, G = 2: three key splits, soft-cap
     (vf.KvDtype.F16, 8, 2, 256, 35, 260, 100, 0.0),   # head_dim 256, G = 4 on a 2-byte cache, window
     (vf.KvDtype.F8, 32, 4, 256, 18, 130, 0, 0.0),     # head_dim 256, G = 8: the Q planes leave no room for private tiles
@@ -149,7 +153,7 @@ def test_window_uses_the_last_querys_lower_bound():
     cache.destroy()
 
 
-@pytest.mark.parametrize("dtype", (vf.KvDtype.F16, vf.KvDtype.F8))
+@pytest.mark.parametrize("dtype", (vf.KvDtype.F16, vf.KvDtype.F8, vf.KvDtype.F32))
 @pytest.mark.parametrize("shape", ("ascending", "descending", "steps"))
 def test_scores_that_drift_past_the_running_maximum(dtype, shape):
     # the kernel keeps a reference maximum that is allowed to lag behind the true one; scores that climb slowly, fall, or

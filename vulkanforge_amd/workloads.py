@@ -80,6 +80,8 @@ PREFILL = {
                                                            512, KvDtype.F16),
     "prefill_fp8_hd256_512x4608_12layers": PrefillWorkload("prefill_fp8_hd256_512x4608_12layers", 12, 16, 8, 256, 4096,
                                                            512, KvDtype.F8),
+    # the headline prefill geometry over an F32 cache (the reference's VULKANFORGE_FP16_KV=0 mode), 4 layers
+    "prefill_f32_512x4608_4layers": PrefillWorkload("prefill_f32_512x4608_4layers", 4, 32, 8, 128, 4096, 512, KvDtype.F32),
     # the headline prefill geometry over an F16 cache (not a reference configuration; used to tune the F16 variant)
     "prefill_f16_512x4608_32layers": PrefillWorkload("prefill_f16_512x4608_32layers", 32, 32, 8, 128, 4096, 512,
                                                      KvDtype.F16),

@@ -64,6 +64,11 @@ CASES = [
     (vf.KvDtype.F32, 16, 2, 128, 20, 333, 120, 30.0), # G = 8 (two workgroups per KV head), window, soft-cap
     (vf.KvDtype.F32, 3, 3, 256, 18, 70, 0, 0.0),      # G = 1, head_dim 256
     (vf.KvDtype.F32, 10, 2, 64, 49, 0, 0, 0.0),       # G = 5: a workgroup with one live wavefront, from position 0
+    (vf.KvDtype.F8, 8, 2, 512, 40, 300, 0, 30.0),     # head_dim 512 (two wavefronts per head on the f32 matrix-core kernel), soft-cap
+    (vf.KvDtype.F16, 16, 2, 512, 20, 100, 64, 0.0),   # head_dim 512, G = 8, window
+    (vf.KvDtype.F8, 12, 4, 96, 33, 200, 0, 0.0),      # head_dim 96: 4-byte loads of the 24-byte row quarters
+    (vf.KvDtype.F16, 6, 6, 96, 17, 50, 10, 0.0),
+    (vf.KvDtype.F32, 8, 4, 96, 21, 80, 0, 0.0),
     (vf.KvDtype.F8, 16, 8, 256, 48, 700, 0, 50.0),    # head_dim 256, G = 2: three key splits, soft-cap
     (vf.KvDtype.F16, 8, 2, 256, 35, 260, 100, 0.0),   # head_dim 256, G = 4 on a 2-byte cache, window
     (vf.KvDtype.F8, 32, 4, 256, 18, 130, 0, 0.0),     # head_dim 256, G = 8: the Q planes leave no room for private tiles

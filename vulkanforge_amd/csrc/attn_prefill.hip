@@ -3,7 +3,8 @@
 // batch_mfma2_kernel   (attn_prefill_mfma2.h) f16 matrix-core tiles, private K / V tiles per wavefront: FP8 / F16 caches,
 //                      head_dim 64 / 128 / 256, GQA groups that fit the workgroup.
 // batch_mfma_kernel    (attn_prefill_mfma.h) first generation (V tile shared behind a barrier): the remaining groups.
-// batch_mfma_f32_kernel (attn_prefill_f32.h) f32 matrix-core tiles for F32 caches, head_dim 64 / 128 / 256.
+// batch_mfma_f32_kernel (attn_prefill_f32.h) f32 matrix-core tiles: F32 caches (head_dim 64 / 96 / 128 / 256), FP8 / F16 caches at
+//                      head_dim 96 and 512.
 // batch_generic_kernel one wavefront per (query, head); covers every dtype and head_dim <= 512.
 #include "device_utils.h"
 #include "kernels.h"
@@ -168,17 +169,18 @@ first_generation:
 #undef VFKV_PF2
 #undef VFKV_PF
     }
-    if (L.dtype == kF32 && aligned && slab_bytes < 0x7FFF0000ull && (L.head_dim == 64u || L.head_dim == 128u || L.head_dim == 256u) &&
-        L.n_kv_heads <= 65535u && (g + 3u) / 4u <= 65535u) {
-        const dim3 grid((L.m + 15u) / 16u, L.n_kv_heads, (g + 3u) / 4u), block(256);
+    // f32 matrix-core kernel: F32 caches, and the head sizes the f16 kernels above do not cover
+    if (aligned && slab_bytes < 0x7FFF0000ull && L.n_kv_heads <= 65535u && (g + 3u) / 4u * 2u <= 65535u) {
         const bool cap = L.softcap > 0.f;
-#define VFKV_PF32(DD)                                                                                          \
-    if (L.head_dim == DD) {                                                                                    \
-        if (cap) hipLaunchKernelGGL((batch_mfma_f32_kernel<DD, true>), grid, block, 0, stream, a);             \
-        else hipLaunchKernelGGL((batch_mfma_f32_kernel<DD, false>), grid, block, 0, stream, a);                \
-        return hipGetLastError();                                                                              \
+#define VFKV_PF32(DTV, DD, NHV)                                                                                        \
+    if (L.dtype == DTV && L.head_dim == DD) {                                                                          \
+        const dim3 grid((L.m + 15u) / 16u, L.n_kv_heads, (g + 3u) / 4u * NHV), block(256);                             \
+        if (cap) hipLaunchKernelGGL((batch_mfma_f32_kernel<DTV, DD, NHV, true>), grid, block, 0, stream, a);           \
+        else hipLaunchKernelGGL((batch_mfma_f32_kernel<DTV, DD, NHV, false>), grid, block, 0, stream, a);              \
+        return hipGetLastError();                                                                                      \
     }
-        VFKV_PF32(64) VFKV_PF32(128) VFKV_PF32(256)
+        VFKV_PF32(kF32, 64, 1) VFKV_PF32(kF32, 128, 1) VFKV_PF32(kF32, 256, 1) VFKV_PF32(kF32, 96, 1)
+        VFKV_PF32(kF16, 96, 1) VFKV_PF32(kF8, 96, 1) VFKV_PF32(kF16, 512, 2) VFKV_PF32(kF8, 512, 2)
 #undef VFKV_PF32
     }
     hipLaunchKernelGGL(batch_generic_kernel, dim3(L.n_heads, L.m), dim3(kWave), 0, stream, a);

@@ -64,6 +64,10 @@ CASES = [
     (vf.KvDtype.F32, 16, 2, 128, 20, 333, 120, 30.0), # G = 8 (two workgroups per KV head), window, soft-cap
     (vf.KvDtype.F32, 3, 3, 256, 18, 70, 0, 0.0),      # G = 1, head_dim 256
     (vf.KvDtype.F32, 10, 2, 64, 49, 0, 0, 0.0),       # G = 5: a workgroup with one live wavefront, from position 0
+    (vf.KvDtype.F8, 28, 4, 128, 45, 800, 0, 0.0),     # G = 7: four head pairs per KV head, the last one half empty
+    (vf.KvDtype.F16, 14, 2, 128, 19, 300, 100, 25.0), # G = 7 on a 2-byte cache, window, soft-cap
+    (vf.KvDtype.F8, 10, 2, 64, 50, 400, 0, 0.0),      # G = 5, head_dim 64
+    (vf.KvDtype.F16, 9, 3, 64, 31, 0, 0, 0.0),        # G = 3 from position 0
     (vf.KvDtype.F8, 8, 2, 512, 40, 300, 0, 30.0),     # head_dim 512 (two wavefronts per head on the f32 matrix-core kernel), soft-cap
     (vf.KvDtype.F16, 16, 2, 512, 20, 100, 64, 0.0),   # head_dim 512, G = 8, window
     (vf.KvDtype.F8, 12, 4, 96, 33, 200, 0, 0.0),      # head_dim 96: 4-byte loads of the 24-byte row quarters

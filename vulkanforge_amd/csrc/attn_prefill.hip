@@ -110,13 +110,27 @@ hipError_t launch_batch(const BatchLaunch& L, hipStream_t stream) {
 #ifndef VFKV_PREFILL_F16_128_NCB
 #define VFKV_PREFILL_F16_128_NCB 2     // heads per wavefront, F16 cache, head_dim 128 (even GQA groups)
 #endif
-        uint32_t ncb = (g % 2u == 0u && (L.head_dim == 64u || (L.head_dim == 128u && (L.dtype == kF8 || VFKV_PREFILL_F16_128_NCB == 2)))) ? 2u : 1u;
+        // (odd groups of three and more heads round up to whole pairs: the spare slot computes on zeros and stores nothing)
+        uint32_t ncb = (g >= 2u && (L.head_dim == 64u || (L.head_dim == 128u && (L.dtype == kF8 || VFKV_PREFILL_F16_128_NCB == 2)))) ? 2u : 1u;
         if (force_ncb == 1) ncb = 1u;
-        const uint32_t hp = g / ncb;
-        if (hp <= 8u) {
-            uint32_t max_waves = (ncb == 1u && L.head_dim <= 128u) ? 12u : 8u;  // one head per wavefront needs fewer registers: three wavefronts per SIMD
+        const uint32_t hp_group = (g + ncb - 1u) / ncb;          // head slices of a whole GQA group
+        // launches that would leave compute units without a workgroup spread the slices of a group over several workgroups
+        // (each then splits the keys further: same work per workgroup, more of them)
+        uint32_t hp = hp_group;
+        {
+            const uint64_t wgs = (uint64_t)((L.m + 15u) / 16u) * L.n_kv_heads;
+            if (wgs < 256u) {
+                uint32_t nz = (uint32_t)((256u + wgs - 1u) / wgs);
+                if (nz > hp_group) nz = hp_group;
+                hp = (hp_group + nz - 1u) / nz;
+            }
+            if (hp_group > 8u && hp > 8u) hp = 8u;               // more slices than a workgroup holds: several workgroups anyway
+        }
+        const uint32_t nz = (hp_group + hp - 1u) / hp;
+        if (hp <= 8u && nz <= 65535u) {
+            uint32_t max_waves = (ncb == 1u && L.head_dim <= 128u) ? (uint32_t)VFKV_PREFILL_NCB1_WAVES : 8u;  // one head per wavefront needs fewer registers: three wavefronts per SIMD
             {   // the private V tiles and the two Q planes have to fit in 160 KiB of LDS
-                const size_t qbytes = (size_t)2 * g * 16 * (L.head_dim + 8) * sizeof(_Float16);
+                const size_t qbytes = (size_t)2 * hp * ncb * 16 * (L.head_dim + 8) * sizeof(_Float16);
                 const size_t per_wave = (size_t)32 * (L.head_dim + 16) * sizeof(_Float16);
                 const size_t fit = qbytes < 160u * 1024u ? (160u * 1024u - qbytes) / per_wave : 0u;
                 if (fit < max_waves) max_waves = (uint32_t)fit;
@@ -124,9 +138,9 @@ hipError_t launch_batch(const BatchLaunch& L, hipStream_t stream) {
             if (max_waves < hp) goto first_generation;
             const uint32_t ns = max_waves / hp;               // key splits: fill the workgroup
             const uint32_t nwaves = hp * ns;
-            const dim3 grid((L.m + 15u) / 16u, L.n_kv_heads), block(nwaves * kWave);
+            const dim3 grid((L.m + 15u) / 16u, L.n_kv_heads, nz), block(nwaves * kWave);
             const size_t vbytes = (size_t)nwaves * 32 * (L.head_dim + 16) * sizeof(_Float16) +
-                                  (size_t)2 * g * 16 * (L.head_dim + 8) * sizeof(_Float16);
+                                  (size_t)2 * hp * ncb * 16 * (L.head_dim + 8) * sizeof(_Float16);
             const size_t mbytes = (size_t)(ns - 1) * hp * ncb * 64 * (L.head_dim / 4 + 2) * sizeof(float);
             const size_t lds = vbytes > mbytes ? vbytes : mbytes;
             const bool cap = L.softcap > 0.f;

@@ -24,8 +24,13 @@
 
 namespace vfkv {
 
+// wavefronts per workgroup when a wavefront serves one head at head_dim <= 128 (fewer registers: three per SIMD)
+#ifndef VFKV_PREFILL_NCB1_WAVES
+#define VFKV_PREFILL_NCB1_WAVES 12
+#endif
+
 template <int DT, int D, int NCB, int PFD, bool CAP>
-__global__ __launch_bounds__((NCB == 1 && D <= 128) ? 768 : 512) void batch_mfma2_kernel(BatchArgs a, int HP, int NS) {
+__global__ __launch_bounds__((NCB == 1 && D <= 128) ? VFKV_PREFILL_NCB1_WAVES * 64 : 512) void batch_mfma2_kernel(BatchArgs a, int HP, int NS) {
     constexpr int ES = DT == kF16 ? 2 : 1;
     constexpr int KT = 32;                       // keys per tile
     constexpr int KS = D / 32;                   // MFMA k-steps of the first product
@@ -40,7 +45,7 @@ __global__ __launch_bounds__((NCB == 1 && D <= 128) ? 768 : 512) void batch_mfma
     constexpr uint32_t kNoTile = 0x80000000u;    // byte offset past any slab: the load returns zeros, no memory access
     static_assert(D % 32 == 0 && SEGB % 16 == 0 && VLD >= 1, "unsupported head_dim");
 
-    extern __shared__ __attribute__((aligned(16))) _Float16 lds[];      // [waves][KT][VPITCH] V tiles | [G][16][D + 8] f16(q) | [G][16][D + 8] remainders
+    extern __shared__ __attribute__((aligned(16))) _Float16 lds[];      // [waves][KT][VPITCH] V tiles | [GP][16][D + 8] f16(q) | [GP][16][D + 8] remainders
     __shared__ int lds_haslo;
 
     const int tid = threadIdx.x, lane = tid & 63;
@@ -54,12 +59,14 @@ __global__ __launch_bounds__((NCB == 1 && D <= 128) ? 768 : 512) void batch_mfma
     const uint32_t qi = q0 + n16;                               // this lane's query (column of S^T)
     const bool q_ok = qi < a.m;
     const uint32_t row_stride = a.n_kv_heads * D * ES;
-    const int g0 = hp * NCB;                                    // first head (inside the group) of this wavefront
+    const int gz = blockIdx.z * HP * NCB;                       // first head (inside the group) of this workgroup
+    const int g0 = hp * NCB;                                    // first head slot (inside the workgroup) of this wavefront
 
     _Float16* const vb = lds + (size_t)w * KT * VPITCH;
     constexpr int QPITCH = D + 8;
-    _Float16* const qhi_lds = lds + (size_t)nwaves * KT * VPITCH;   // [G][16][D + 8] f16(q)
-    _Float16* const qlo_lds = qhi_lds + (size_t)G * 16 * QPITCH;    // [G][16][D + 8] f16(q - f16(q))
+    _Float16* const qhi_lds = lds + (size_t)nwaves * KT * VPITCH;   // [GP][16][D + 8] f16(q); the slots past G hold zeros
+    const int GP = HP * NCB;                                        // head slots of the workgroup: G rounded up to whole wavefronts
+    _Float16* const qlo_lds = qhi_lds + (size_t)GP * 16 * QPITCH;   // [GP][16][D + 8] f16(q - f16(q))
 
     // ---- key range ----
     uint32_t kmax = a.q_start + q0 + 16;                        // one past the last key any of the 16 queries sees
@@ -97,7 +104,7 @@ __global__ __launch_bounds__((NCB == 1 && D <= 128) ? 768 : 512) void batch_mfma
     // K / V requests, so waiting for it does not wait for them) and kept in LDS as an f16 value plane and a remainder plane
     constexpr int QLD = 4;                                      // query loads per thread and round
     const int nthreads = nwaves * 64;
-    const int q4_total = 16 * G * (D / 4);
+    const int q4_total = 16 * GP * (D / 4);
     if (tid == 0) lds_haslo = 0;
     bool any_lo = false;
     for (int base = 0; base < q4_total; base += QLD * nthreads) {
@@ -105,9 +112,9 @@ __global__ __launch_bounds__((NCB == 1 && D <= 128) ? 768 : 512) void batch_mfma
 #pragma unroll
         for (int i = 0; i < QLD; ++i) {
             const int idx = base + tid + i * nthreads;
-            const int qq = idx / (G * (D / 4)), rem = idx - qq * (G * (D / 4));
-            const bool ok = idx < q4_total && q0 + qq < a.m;
-            qf[i] = *reinterpret_cast<const float4*>(a.q + ((size_t)(ok ? q0 + qq : 0) * a.n_heads + kvh * G) * D + (ok ? rem * 4 : 0));
+            const int qq = idx / (GP * (D / 4)), rem = idx - qq * (GP * (D / 4));
+            const bool ok = idx < q4_total && q0 + qq < a.m && rem < (G - gz) * (D / 4);      // head slots past G read nothing
+            qf[i] = *reinterpret_cast<const float4*>(a.q + ((size_t)(ok ? q0 + qq : 0) * a.n_heads + kvh * G + gz) * D + (ok ? rem * 4 : 0));
             if (!ok) qf[i] = make_float4(0.f, 0.f, 0.f, 0.f);
         }
         if (base == 0) {
@@ -118,7 +125,7 @@ __global__ __launch_bounds__((NCB == 1 && D <= 128) ? 768 : 512) void batch_mfma
         for (int i = 0; i < QLD; ++i) {
             const int idx = base + tid + i * nthreads;
             if (idx >= q4_total) continue;
-            const int qq = idx / (G * (D / 4)), rem = idx - qq * (G * (D / 4));
+            const int qq = idx / (GP * (D / 4)), rem = idx - qq * (GP * (D / 4));
             const int g = rem / (D / 4), d = (rem - g * (D / 4)) * 4;
             const float v[4] = {qf[i].x, qf[i].y, qf[i].z, qf[i].w};
             _Float16 hv[4], lv[4];
@@ -378,7 +385,8 @@ __global__ __launch_bounds__((NCB == 1 && D <= 128) ? 768 : 512) void batch_mfma
     if (q_ok) {
 #pragma unroll
         for (int cb = 0; cb < NCB; ++cb) {
-            const uint32_t h = kvh * G + g0 + cb;
+            if (gz + g0 + cb >= G) continue;                                  // padding slot of an odd group
+            const uint32_t h = kvh * G + gz + g0 + cb;
             const float inv = 1.0f / l_run[cb];
             float* op = a.o + ((size_t)qi * a.n_heads + h) * D + kg * 4;      // lane (query n16) holds d = dt*16 + kg*4 + i
 #pragma unroll

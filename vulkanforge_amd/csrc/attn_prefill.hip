@@ -116,6 +116,7 @@ hipError_t launch_batch(const BatchLaunch& L, hipStream_t stream) {
         // F16 rows are twice the bytes: four heads per wavefront (one wavefront per SIMD, 512 registers) so that a K / V tile
         // is loaded by one wavefront of the workgroup only
         if (L.dtype == kF16 && g >= 3u && L.head_dim == 128u && force_ncb == 0) ncb = 4u;
+        if (L.head_dim == 256u && g >= 2u && force_ncb == 0) ncb = 2u;      // the same at head_dim 256 with two heads
         const uint32_t hp_group = (g + ncb - 1u) / ncb;          // head slices of a whole GQA group
         // launches that would leave compute units without a workgroup spread the slices of a group over several workgroups
         // (each then splits the keys further: same work per workgroup, more of them)
@@ -131,7 +132,7 @@ hipError_t launch_batch(const BatchLaunch& L, hipStream_t stream) {
         }
         const uint32_t nz = (hp_group + hp - 1u) / hp;
         if (hp <= 8u && nz <= 65535u) {
-            uint32_t max_waves = (ncb == 1u && L.head_dim <= 128u) ? (uint32_t)VFKV_PREFILL_NCB1_WAVES : (ncb == 4u || (L.dtype == kF16 && L.head_dim == 256u)) ? 4u : 8u;  // one head per wavefront needs fewer registers: three wavefronts per SIMD
+            uint32_t max_waves = (ncb == 1u && L.head_dim <= 128u) ? (uint32_t)VFKV_PREFILL_NCB1_WAVES : (ncb * L.head_dim >= 512u || (L.dtype == kF16 && L.head_dim == 256u)) ? 4u : 8u;  // one head per wavefront needs fewer registers: three wavefronts per SIMD
             {   // the private V tiles and the two Q planes have to fit in 160 KiB of LDS
                 const size_t qbytes = (size_t)2 * hp * ncb * 16 * (L.head_dim + 8) * sizeof(_Float16);
                 const size_t per_wave = (size_t)32 * (L.head_dim + 16) * sizeof(_Float16);
@@ -156,7 +157,7 @@ hipError_t launch_batch(const BatchLaunch& L, hipStream_t stream) {
             VFKV_P2(kF8, 64, 2, 2) VFKV_P2(kF8, 64, 1, 2) VFKV_P2(kF8, 128, 2, 2) VFKV_P2(kF8, 128, 1, 2)
             VFKV_P2(kF16, 64, 2, 2) VFKV_P2(kF16, 64, 1, 2) VFKV_P2(kF16, 128, 1, 1) VFKV_P2(kF16, 128, 2, 1)
             VFKV_P2(kF8, 256, 1, 1) VFKV_P2(kF16, 256, 1, 1)
-            VFKV_P2(kF16, 128, 4, 1)
+            VFKV_P2(kF16, 128, 4, 1) VFKV_P2(kF8, 256, 2, 1) VFKV_P2(kF16, 256, 2, 1)
             { launched = false; }
 #undef VFKV_P2
             if (launched) return hipGetLastError();

@@ -30,7 +30,7 @@ namespace vfkv {
 #endif
 
 template <int DT, int D, int NCB, int PFD, bool CAP>
-__global__ __launch_bounds__((NCB == 1 && D <= 128) ? VFKV_PREFILL_NCB1_WAVES * 64 : (NCB == 4 || (DT == kF16 && D == 256)) ? 256 : 512) void batch_mfma2_kernel(BatchArgs a, int HP, int NS) {
+__global__ __launch_bounds__((NCB == 1 && D <= 128) ? VFKV_PREFILL_NCB1_WAVES * 64 : (NCB * D >= 512 || (DT == kF16 && D == 256)) ? 256 : 512) void batch_mfma2_kernel(BatchArgs a, int HP, int NS) {
     constexpr int ES = DT == kF16 ? 2 : 1;
     constexpr int KT = 32;                       // keys per tile
     constexpr int KS = D / 32;                   // MFMA k-steps of the first product

@@ -75,7 +75,7 @@ CASES = [
     (vf.KvDtype.F32, 8, 4, 96, 21, 80, 0, 0.0),
     (vf.KvDtype.F8, 16, 8, 256, 48, 700, 0, 50.0),    # head_dim 256, G = 2: three key splits, soft-cap
     (vf.KvDtype.F16, 8, 2, 256, 35, 260, 100, 0.0),   # head_dim 256, G = 4 on a 2-byte cache, window
-    (vf.KvDtype.F8, 32, 4, 256, 18, 130, 0, 0.0),     # head_dim 256, G = 8: the Q planes leave no room for private tiles
+    (vf.KvDtype.F8, 32, 4, 256, 18, 130, 0, 0.0),     # head_dim 256, G = 8: the group is spread over workgroups so that the Q planes fit
     (vf.KvDtype.F16, 16, 16, 256, 20, 90, 0, 20.0),   # head_dim 256, G = 1: seven key splits
 ]
 

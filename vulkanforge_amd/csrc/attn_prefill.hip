@@ -1,8 +1,7 @@
 // Chunked-prefill causal attention over the cache (flash_attn_batch.comp:105-208) for gfx950.
 //
 // batch_mfma2_kernel   (attn_prefill_mfma2.h) f16 matrix-core tiles, private K / V tiles per wavefront: FP8 / F16 caches,
-//                      head_dim 64 / 128 / 256, GQA groups that fit the workgroup.
-// batch_mfma_kernel    (attn_prefill_mfma.h) first generation (V tile shared behind a barrier): the remaining groups.
+//                      head_dim 64 / 128 / 256, any GQA group.
 // batch_mfma_f32_kernel (attn_prefill_f32.h) f32 matrix-core tiles: F32 caches (head_dim 64 / 96 / 128 / 256), FP8 / F16 caches at
 //                      head_dim 96 and 512.
 // batch_generic_kernel one wavefront per (query, head); covers every dtype and head_dim <= 512.
@@ -23,7 +22,6 @@ struct BatchArgs {
 };
 
 }  // namespace vfkv
-#include "attn_prefill_mfma.h"
 #include "attn_prefill_mfma2.h"
 #include "attn_prefill_f32.h"
 namespace vfkv {
@@ -102,9 +100,8 @@ hipError_t launch_batch(const BatchLaunch& L, hipStream_t stream) {
     const bool aligned = ((((uintptr_t)L.k) | ((uintptr_t)L.v) | ((uintptr_t)L.q) | ((uintptr_t)L.o)) & 15u) == 0u;
     const bool mfma_ok = (L.dtype == kF8 || L.dtype == kF16) && aligned && slab_bytes < 0x7FFF0000ull &&
                          (L.head_dim == 64u || L.head_dim == 128u || L.head_dim == 256u);
-    // Second-generation kernel: NCB heads per wavefront, private tiles per wavefront, no barrier in the loop.
-    static const bool v2_on = [] { const char* e = getenv("VFKV_PREFILL_KERNEL"); return !(e && e[0] == '1'); }();
-    if (mfma_ok && v2_on) {
+    // f16 matrix-core kernel: NCB heads per wavefront, private tiles per wavefront, no barrier in the loop
+    if (mfma_ok) {
         // two heads per wavefront where the registers allow it
         static const int force_ncb = [] { const char* e = getenv("VFKV_PREFILL_NCB"); return e ? atoi(e) : 0; }();
 #ifndef VFKV_PREFILL_F16_128_NCB
@@ -118,28 +115,33 @@ hipError_t launch_batch(const BatchLaunch& L, hipStream_t stream) {
         if (L.dtype == kF16 && g >= 3u && L.head_dim == 128u && force_ncb == 0) ncb = 4u;
         if (L.head_dim == 256u && g >= 2u && force_ncb == 0) ncb = 2u;      // the same at head_dim 256 with two heads
         const uint32_t hp_group = (g + ncb - 1u) / ncb;          // head slices of a whole GQA group
-        // launches that would leave compute units without a workgroup spread the slices of a group over several workgroups
-        // (each then splits the keys further: same work per workgroup, more of them)
+        // wavefronts per workgroup the registers allow: one head per wavefront at head_dim <= 128 needs few (three wavefronts
+        // per SIMD), 512 accumulator columns per wavefront need the whole register file of a SIMD (one wavefront per SIMD)
+        const uint32_t reg_waves = (ncb == 1u && L.head_dim <= 128u) ? (uint32_t)VFKV_PREFILL_NCB1_WAVES
+                                 : (ncb * L.head_dim >= 512u || (L.dtype == kF16 && L.head_dim == 256u)) ? 4u : 8u;
+        // the private V tiles and the two Q planes have to fit in 160 KiB of LDS
+        auto waves_for = [&](uint32_t slices) -> uint32_t {
+            const size_t qbytes = (size_t)2 * slices * ncb * 16 * (L.head_dim + 8) * sizeof(_Float16);
+            const size_t per_wave = (size_t)32 * (L.head_dim + 16) * sizeof(_Float16);
+            const size_t fit = qbytes < 160u * 1024u ? (160u * 1024u - qbytes) / per_wave : 0u;
+            return fit < reg_waves ? (uint32_t)fit : reg_waves;
+        };
+        // Head slices per workgroup: the whole group where it fits; launches that would leave compute units without a
+        // workgroup, and groups whose Q planes or wavefronts do not fit one workgroup, spread the slices of a group over
+        // several workgroups (each then splits the keys further: same work per workgroup, more of them).
         uint32_t hp = hp_group;
         {
             const uint64_t wgs = (uint64_t)((L.m + 15u) / 16u) * L.n_kv_heads;
             if (wgs < 256u) {
-                uint32_t nz = (uint32_t)((256u + wgs - 1u) / wgs);
-                if (nz > hp_group) nz = hp_group;
-                hp = (hp_group + nz - 1u) / nz;
+                uint32_t want = (uint32_t)((256u + wgs - 1u) / wgs);
+                if (want > hp_group) want = hp_group;
+                hp = (hp_group + want - 1u) / want;
             }
-            if (hp_group > 8u && hp > 8u) hp = 8u;               // more slices than a workgroup holds: several workgroups anyway
+            while (hp > 1u && waves_for(hp) < hp) --hp;          // one slice always fits
         }
         const uint32_t nz = (hp_group + hp - 1u) / hp;
-        if (hp <= 8u && nz <= 65535u) {
-            uint32_t max_waves = (ncb == 1u && L.head_dim <= 128u) ? (uint32_t)VFKV_PREFILL_NCB1_WAVES : (ncb * L.head_dim >= 512u || (L.dtype == kF16 && L.head_dim == 256u)) ? 4u : 8u;  // one head per wavefront needs fewer registers: three wavefronts per SIMD
-            {   // the private V tiles and the two Q planes have to fit in 160 KiB of LDS
-                const size_t qbytes = (size_t)2 * hp * ncb * 16 * (L.head_dim + 8) * sizeof(_Float16);
-                const size_t per_wave = (size_t)32 * (L.head_dim + 16) * sizeof(_Float16);
-                const size_t fit = qbytes < 160u * 1024u ? (160u * 1024u - qbytes) / per_wave : 0u;
-                if (fit < max_waves) max_waves = (uint32_t)fit;
-            }
-            if (max_waves < hp) goto first_generation;
+        const uint32_t max_waves = waves_for(hp);
+        if (max_waves >= hp && nz <= 65535u) {
             const uint32_t ns = max_waves / hp;               // key splits: fill the workgroup
             const uint32_t nwaves = hp * ns;
             const dim3 grid((L.m + 15u) / 16u, L.n_kv_heads, nz), block(nwaves * kWave);
@@ -162,31 +164,6 @@ hipError_t launch_batch(const BatchLaunch& L, hipStream_t stream) {
 #undef VFKV_P2
             if (launched) return hipGetLastError();
         }
-    }
-first_generation:
-    if (mfma_ok && g <= 16u) {
-        // two key splits per workgroup while that still leaves two wavefronts per SIMD worth of registers
-        const uint32_t nsplit = g <= 4u ? 2u : 1u;
-        const dim3 grid((L.m + 15u) / 16u, L.n_kv_heads), block(g * nsplit * kWave);
-        const size_t vbytes = (size_t)nsplit * 2 * 32 * (L.head_dim + 16) * sizeof(_Float16);
-        const size_t mbytes = (size_t)(nsplit - 1) * g * 64 * (L.head_dim / 4 + 2) * sizeof(float);
-        const size_t lds = vbytes > mbytes ? vbytes : mbytes;
-// tiles in flight per key split: deeper for the shapes whose registers allow it
-#ifndef VFKV_PREFILL_PFD
-#define VFKV_PREFILL_PFD 3
-#endif
-#define VFKV_PF2(DT, DD, CAPV, MT, NS) hipLaunchKernelGGL((batch_mfma_kernel<DT, DD, CAPV, MT, NS, (DD <= 128 && MT <= 512 && DT == kF8) ? VFKV_PREFILL_PFD : 1>), grid, block, lds, stream, a)
-#define VFKV_PF(DT, DD)                                                                   \
-    if (L.dtype == DT && L.head_dim == DD) {                                              \
-        const bool cap = L.softcap > 0.f;                                                 \
-        if (g <= 4u) { if (cap) VFKV_PF2(DT, DD, true, 512, 2); else VFKV_PF2(DT, DD, false, 512, 2); }     \
-        else if (g <= 8u) { if (cap) VFKV_PF2(DT, DD, true, 512, 1); else VFKV_PF2(DT, DD, false, 512, 1); } \
-        else { if (cap) VFKV_PF2(DT, DD, true, 1024, 1); else VFKV_PF2(DT, DD, false, 1024, 1); }           \
-        return hipGetLastError();                                                         \
-    }
-        VFKV_PF(kF8, 64) VFKV_PF(kF8, 128) VFKV_PF(kF8, 256) VFKV_PF(kF16, 64) VFKV_PF(kF16, 128) VFKV_PF(kF16, 256)
-#undef VFKV_PF2
-#undef VFKV_PF
     }
     // f32 matrix-core kernel: F32 caches, and the head sizes the f16 kernels above do not cover
     if (aligned && slab_bytes < 0x7FFF0000ull && L.n_kv_heads <= 65535u && (g + 3u) / 4u * 2u <= 65535u) {

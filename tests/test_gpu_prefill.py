@@ -68,7 +68,9 @@ CASES = [
     (vf.KvDtype.F16, 14, 2, 128, 19, 300, 100, 25.0), # G = 7 on a 2-byte cache, window, soft-cap
     (vf.KvDtype.F8, 10, 2, 64, 50, 400, 0, 0.0),      # G = 5, head_dim 64
     (vf.KvDtype.F16, 9, 3, 64, 31, 0, 0, 0.0),        # G = 3 from position 0
-    (vf.KvDtype.F8, 8, 2, 512, 40, 300, 0, 30.0),     # head_dim 512 (two wavefronts per head on the f32 matrix-core kernel), soft-cap
+    (vf.KvDtype.F8, 8, 2, 512, 40, 300, 0, 30.0),     # head_dim 512 (two wavefronts per head, each half of the output columns), soft-cap
+    (vf.KvDtype.F32, 4, 2, 512, 23, 150, 0, 0.0),     # head_dim 512 over an F32 cache: the same split on the f32 matrix-core kernel
+    (vf.KvDtype.F8, 3, 1, 512, 70, 1000, 0, 0.0),     # head_dim 512, G = 3, several query blocks
     (vf.KvDtype.F16, 16, 2, 512, 20, 100, 64, 0.0),   # head_dim 512, G = 8, window
     (vf.KvDtype.F8, 12, 4, 96, 33, 200, 0, 0.0),      # head_dim 96: 4-byte loads of the 24-byte row quarters
     (vf.KvDtype.F16, 6, 6, 96, 17, 50, 10, 0.0),

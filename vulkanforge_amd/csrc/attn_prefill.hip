@@ -1,9 +1,9 @@
 // Chunked-prefill causal attention over the cache (flash_attn_batch.comp:105-208) for gfx950.
 //
 // batch_mfma2_kernel   (attn_prefill_mfma2.h) f16 matrix-core tiles, private K / V tiles per wavefront: FP8 / F16 caches,
-//                      head_dim 64 / 128 / 256, any GQA group.
-// batch_mfma_f32_kernel (attn_prefill_f32.h) f32 matrix-core tiles: F32 caches (head_dim 64 / 96 / 128 / 256), FP8 / F16 caches at
-//                      head_dim 96 and 512.
+//                      head_dim 64 / 128 / 256 / 512, any GQA group.
+// batch_mfma_f32_kernel (attn_prefill_f32.h) f32 matrix-core tiles: F32 caches (head_dim 64 / 96 / 128 / 256 / 512), FP8 / F16 caches at
+//                      head_dim 96.
 // batch_generic_kernel one wavefront per (query, head); covers every dtype and head_dim <= 512.
 #include "device_utils.h"
 #include "kernels.h"
@@ -99,7 +99,7 @@ hipError_t launch_batch(const BatchLaunch& L, hipStream_t stream) {
     const uint64_t slab_bytes = (uint64_t)L.n_kv * L.n_kv_heads * L.head_dim * elem_size(L.dtype);
     const bool aligned = ((((uintptr_t)L.k) | ((uintptr_t)L.v) | ((uintptr_t)L.q) | ((uintptr_t)L.o)) & 15u) == 0u;
     const bool mfma_ok = (L.dtype == kF8 || L.dtype == kF16) && aligned && slab_bytes < 0x7FFF0000ull &&
-                         (L.head_dim == 64u || L.head_dim == 128u || L.head_dim == 256u);
+                         (L.head_dim == 64u || L.head_dim == 128u || L.head_dim == 256u || L.head_dim == 512u);
     // f16 matrix-core kernel: NCB heads per wavefront, private tiles per wavefront, no barrier in the loop
     if (mfma_ok) {
         // two heads per wavefront where the registers allow it
@@ -114,15 +114,19 @@ hipError_t launch_batch(const BatchLaunch& L, hipStream_t stream) {
         // is loaded by one wavefront of the workgroup only
         if (L.dtype == kF16 && g >= 3u && L.head_dim == 128u && force_ncb == 0) ncb = 4u;
         if (L.head_dim == 256u && g >= 2u && force_ncb == 0) ncb = 2u;      // the same at head_dim 256 with two heads
-        const uint32_t hp_group = (g + ncb - 1u) / ncb;          // head slices of a whole GQA group
+        // head_dim 512: one head per wavefront, and two wavefronts share a head (each owns half of the output columns)
+        const uint32_t nh = L.head_dim == 512u ? 2u : 1u;
+        if (nh == 2u) ncb = 1u;
+        const uint32_t dv = L.head_dim / nh;
+        const uint32_t hp_group = (g + ncb - 1u) / ncb * nh;     // (head slice, output slice) units of a whole GQA group
         // wavefronts per workgroup the registers allow: one head per wavefront at head_dim <= 128 needs few (three wavefronts
         // per SIMD), 512 accumulator columns per wavefront need the whole register file of a SIMD (one wavefront per SIMD)
         const uint32_t reg_waves = (ncb == 1u && L.head_dim <= 128u) ? (uint32_t)VFKV_PREFILL_NCB1_WAVES
-                                 : (ncb * L.head_dim >= 512u || (L.dtype == kF16 && L.head_dim == 256u)) ? 4u : 8u;
+                                 : (ncb * L.head_dim >= 512u || (L.dtype == kF16 && L.head_dim == 256u)) ? 4u : 8u;   // (always 4 at head_dim 512)
         // the private V tiles and the two Q planes have to fit in 160 KiB of LDS
         auto waves_for = [&](uint32_t slices) -> uint32_t {
-            const size_t qbytes = (size_t)2 * slices * ncb * 16 * (L.head_dim + 8) * sizeof(_Float16);
-            const size_t per_wave = (size_t)32 * (L.head_dim + 16) * sizeof(_Float16);
+            const size_t qbytes = (size_t)2 * (slices / nh) * ncb * 16 * (L.head_dim + 8) * sizeof(_Float16);
+            const size_t per_wave = (size_t)32 * (dv + 16) * sizeof(_Float16);
             const size_t fit = qbytes < 160u * 1024u ? (160u * 1024u - qbytes) / per_wave : 0u;
             return fit < reg_waves ? (uint32_t)fit : reg_waves;
         };
@@ -134,10 +138,10 @@ hipError_t launch_batch(const BatchLaunch& L, hipStream_t stream) {
             const uint64_t wgs = (uint64_t)((L.m + 15u) / 16u) * L.n_kv_heads;
             if (wgs < 256u) {
                 uint32_t want = (uint32_t)((256u + wgs - 1u) / wgs);
-                if (want > hp_group) want = hp_group;
-                hp = (hp_group + want - 1u) / want;
+                if (want > hp_group / nh) want = hp_group / nh;
+                hp = (hp_group / nh + want - 1u) / want * nh;    // the output slices of a head stay in one workgroup
             }
-            while (hp > 1u && waves_for(hp) < hp) --hp;          // one slice always fits
+            while (hp > nh && waves_for(hp) < hp) hp -= nh;      // one head always fits
         }
         const uint32_t nz = (hp_group + hp - 1u) / hp;
         const uint32_t max_waves = waves_for(hp);
@@ -145,9 +149,9 @@ hipError_t launch_batch(const BatchLaunch& L, hipStream_t stream) {
             const uint32_t ns = max_waves / hp;               // key splits: fill the workgroup
             const uint32_t nwaves = hp * ns;
             const dim3 grid((L.m + 15u) / 16u, L.n_kv_heads, nz), block(nwaves * kWave);
-            const size_t vbytes = (size_t)nwaves * 32 * (L.head_dim + 16) * sizeof(_Float16) +
-                                  (size_t)2 * hp * ncb * 16 * (L.head_dim + 8) * sizeof(_Float16);
-            const size_t mbytes = (size_t)(ns - 1) * hp * ncb * 64 * (L.head_dim / 4 + 2) * sizeof(float);
+            const size_t vbytes = (size_t)nwaves * 32 * (dv + 16) * sizeof(_Float16) +
+                                  (size_t)2 * (hp / nh) * ncb * 16 * (L.head_dim + 8) * sizeof(_Float16);
+            const size_t mbytes = (size_t)(ns - 1) * hp * ncb * 64 * (dv / 4 + 2) * sizeof(float);
             const size_t lds = vbytes > mbytes ? vbytes : mbytes;
             const bool cap = L.softcap > 0.f;
             bool launched = true;
@@ -160,6 +164,13 @@ hipError_t launch_batch(const BatchLaunch& L, hipStream_t stream) {
             VFKV_P2(kF16, 64, 2, 2) VFKV_P2(kF16, 64, 1, 2) VFKV_P2(kF16, 128, 1, 1) VFKV_P2(kF16, 128, 2, 1)
             VFKV_P2(kF8, 256, 1, 1) VFKV_P2(kF16, 256, 1, 1)
             VFKV_P2(kF16, 128, 4, 1) VFKV_P2(kF8, 256, 2, 1) VFKV_P2(kF16, 256, 2, 1)
+            if (L.head_dim == 512u && L.dtype == kF8) {
+                if (cap) hipLaunchKernelGGL((batch_mfma2_kernel<kF8, 512, 1, 1, true, 2>), grid, block, lds, stream, a, (int)hp, (int)ns);
+                else hipLaunchKernelGGL((batch_mfma2_kernel<kF8, 512, 1, 1, false, 2>), grid, block, lds, stream, a, (int)hp, (int)ns);
+            } else if (L.head_dim == 512u && L.dtype == kF16) {
+                if (cap) hipLaunchKernelGGL((batch_mfma2_kernel<kF16, 512, 1, 1, true, 2>), grid, block, lds, stream, a, (int)hp, (int)ns);
+                else hipLaunchKernelGGL((batch_mfma2_kernel<kF16, 512, 1, 1, false, 2>), grid, block, lds, stream, a, (int)hp, (int)ns);
+            } else
             { launched = false; }
 #undef VFKV_P2
             if (launched) return hipGetLastError();
@@ -176,7 +187,7 @@ hipError_t launch_batch(const BatchLaunch& L, hipStream_t stream) {
         return hipGetLastError();                                                                                      \
     }
         VFKV_PF32(kF32, 64, 1) VFKV_PF32(kF32, 128, 1) VFKV_PF32(kF32, 256, 1) VFKV_PF32(kF32, 96, 1)
-        VFKV_PF32(kF16, 96, 1) VFKV_PF32(kF8, 96, 1) VFKV_PF32(kF16, 512, 2) VFKV_PF32(kF8, 512, 2)
+        VFKV_PF32(kF16, 96, 1) VFKV_PF32(kF8, 96, 1) VFKV_PF32(kF32, 512, 2)
 #undef VFKV_PF32
     }
     hipLaunchKernelGGL(batch_generic_kernel, dim3(L.n_heads, L.m), dim3(kWave), 0, stream, a);

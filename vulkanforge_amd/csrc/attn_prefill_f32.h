@@ -1,12 +1,11 @@
 // Chunked-prefill causal attention on the f32 matrix-core instruction (v_mfma_f32_16x16x4_f32).
 //
 // Replaces flash_attn_batch.comp:105-208 for the reference's FP32-KV mode (kv_cache.rs:76-102, VULKANFORGE_FP16_KV=0) and for
-// the head sizes the f16 matrix-core kernels do not cover (head_dim 512 of the Gemma-4 full-attention layers, which the
-// reference routes through run_flash_attn_cm_gemma_rs, runs.rs:1087-1180; head_dim 96): FP8 / F16 rows are widened to f32
-// in registers (exact), every product is an f32 x f32 product accumulated in f32, as in the shader.  One wavefront per
-// (16 queries, query head, slice of head_dim): four heads of a KV head per workgroup, no LDS, no barrier.  With NH = 2
-// two wavefronts share a head: both compute the scores over the whole head_dim, each accumulates and stores one half of
-// the output (the accumulators of a 512-wide head do not fit one wavefront).  Per tile of 16 keys:
+// head_dim 96, which the f16 matrix-core kernel does not cover: FP8 / F16 rows are widened to f32 in registers (exact),
+// every product is an f32 x f32 product accumulated in f32, as in the shader.  One wavefront per (16 queries, query head,
+// slice of head_dim): four heads of a KV head per workgroup, no LDS, no barrier.  With NH = 2 (head_dim 512) two
+// wavefronts share a head: both compute the scores over the whole head_dim, each accumulates and stores one half of the
+// output (the accumulators of a 512-wide head do not fit one wavefront).  Per tile of 16 keys:
 //   S^T = K Q^T     A = K: lane (key l % 16, group l / 16) holds the group's quarter of the key row (contiguous bytes, so the
 //                   loads are wide loads); B = Q: the same quarter of the lane's query row, loaded once.  The sum over
 //                   head_dim does not care in which order the MFMA steps take the elements, so step c multiplies element

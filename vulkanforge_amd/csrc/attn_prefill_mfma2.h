@@ -29,16 +29,21 @@ namespace vfkv {
 #define VFKV_PREFILL_NCB1_WAVES 12
 #endif
 
-template <int DT, int D, int NCB, int PFD, bool CAP>
+// NH > 1 (head_dim 512, NCB = 1): NH wavefronts share a head.  Each computes the scores over the whole head_dim and
+// accumulates, merges and stores its own slice of D / NH output elements: the accumulators of a 512-wide head do not fit
+// one wavefront.  HP then counts (head, slice) units.
+template <int DT, int D, int NCB, int PFD, bool CAP, int NH = 1>
 __global__ __launch_bounds__((NCB == 1 && D <= 128) ? VFKV_PREFILL_NCB1_WAVES * 64 : (NCB * D >= 512 || (DT == kF16 && D == 256)) ? 256 : 512) void batch_mfma2_kernel(BatchArgs a, int HP, int NS) {
+    static_assert(NH == 1 || NCB == 1, "output slices only with one head per wavefront");
+    constexpr int DV = D / NH;                   // output elements (V columns) of this wavefront
     constexpr int ES = DT == kF16 ? 2 : 1;
     constexpr int KT = 32;                       // keys per tile
     constexpr int KS = D / 32;                   // MFMA k-steps of the first product
-    constexpr int DTILES = D / 16;
+    constexpr int DTILES = DV / 16;
     constexpr int SEG = D / 4, SEGB = SEG * ES;  // a lane group's quarter of a key row
     constexpr int KLD = SEGB / 16;
-    constexpr int VPITCH = D + 16;               // halves per V row in LDS
-    constexpr int VCHUNK_ROW = D * ES / 16;      // 16-byte chunks per V row
+    constexpr int VPITCH = DV + 16;              // halves per V row (this wavefront's columns) in LDS
+    constexpr int VCHUNK_ROW = DV * ES / 16;     // 16-byte chunks per V row
     constexpr int VLD = KT * VCHUNK_ROW / 64;    // V loads per lane per tile
     constexpr int VROWS = 64 / VCHUNK_ROW;
     constexpr float kMaxSlack = 8.0f;            // log2 units by which a score may exceed the running reference maximum
@@ -59,13 +64,14 @@ __global__ __launch_bounds__((NCB == 1 && D <= 128) ? VFKV_PREFILL_NCB1_WAVES * 
     const uint32_t qi = q0 + n16;                               // this lane's query (column of S^T)
     const bool q_ok = qi < a.m;
     const uint32_t row_stride = a.n_kv_heads * D * ES;
-    const int gz = blockIdx.z * HP * NCB;                       // first head (inside the group) of this workgroup
-    const int g0 = hp * NCB;                                    // first head slot (inside the workgroup) of this wavefront
+    const int gz = blockIdx.z * (HP / NH) * NCB;                // first head (inside the group) of this workgroup
+    const int g0 = (hp / NH) * NCB;                             // first head slot (inside the workgroup) of this wavefront
+    const int dslice = hp % NH;                                 // which D / NH output elements this wavefront owns
 
     _Float16* const vb = lds + (size_t)w * KT * VPITCH;
     constexpr int QPITCH = D + 8;
     _Float16* const qhi_lds = lds + (size_t)nwaves * KT * VPITCH;   // [GP][16][D + 8] f16(q); the slots past G hold zeros
-    const int GP = HP * NCB;                                        // head slots of the workgroup: G rounded up to whole wavefronts
+    const int GP = (HP / NH) * NCB;                                 // head slots of the workgroup: G rounded up to whole wavefronts
     _Float16* const qlo_lds = qhi_lds + (size_t)GP * 16 * QPITCH;   // [GP][16][D + 8] f16(q - f16(q))
 
     // ---- key range ----
@@ -83,7 +89,7 @@ __global__ __launch_bounds__((NCB == 1 && D <= 128) ? VFKV_PREFILL_NCB1_WAVES * 
     const uint32_t head_b = kvh * D * ES;
     const uint32_t lane_koff = n16 * row_stride + head_b + kg * SEGB;
     const int vrow = lane / VCHUNK_ROW, vcol = lane % VCHUNK_ROW;
-    const uint32_t lane_voff = vrow * row_stride + head_b + vcol * 16;
+    const uint32_t lane_voff = vrow * row_stride + head_b + dslice * DV * ES + vcol * 16;
 
     u32x4 kraw[PFD][2][KLD];
     u32x4 vraw[PFD][VLD];
@@ -388,7 +394,7 @@ __global__ __launch_bounds__((NCB == 1 && D <= 128) ? VFKV_PREFILL_NCB1_WAVES * 
             if (gz + g0 + cb >= G) continue;                                  // padding slot of an odd group
             const uint32_t h = kvh * G + gz + g0 + cb;
             const float inv = 1.0f / l_run[cb];
-            float* op = a.o + ((size_t)qi * a.n_heads + h) * D + kg * 4;      // lane (query n16) holds d = dt*16 + kg*4 + i
+            float* op = a.o + ((size_t)qi * a.n_heads + h) * D + dslice * DV + kg * 4;   // lane (query n16) holds d = dslice*DV + dt*16 + kg*4 + i
 #pragma unroll
             for (int dt = 0; dt < DTILES; ++dt) {
                 const float4_t r = oacc[cb][dt] * inv;

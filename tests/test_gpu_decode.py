@@ -60,6 +60,8 @@ CASES = [
     (vf.KvDtype.F8, 64, 8, 128, 300, 64, 0, 0.0),     # G = 8 (two head groups)
     (vf.KvDtype.F8, 16, 2, 256, 600, 128, 0, 0.0),
     (vf.KvDtype.F8, 8, 2, 512, 300, 64, 100, 0.0),
+    (vf.KvDtype.F8, 16, 2, 512, 2100, 256, 0, 30.0),  # head_dim 512 on the matrix-core worker: G = 8, soft-cap, several runs per stream
+    (vf.KvDtype.F8, 4, 4, 512, 777, 96, 333, 0.0),    # head_dim 512, G = 1, tile not a multiple of the run, window inside a tile
     (vf.KvDtype.F8, 16, 4, 64, 900, 320, 0, 0.0),
     (vf.KvDtype.F8, 32, 2, 128, 700, 1024, 0, 0.0),   # G = 16: two slices of 8 heads, one ragged tile
     (vf.KvDtype.F8, 24, 2, 128, 1300, 448, 5, 0.0),   # G = 12: slices of 8 and 4 heads
@@ -71,6 +73,7 @@ CASES = [
     (vf.KvDtype.F16, 16, 8, 256, 1500, 256, 0, 50.0),
     (vf.KvDtype.F16, 16, 8, 256, 1500, 64, 1100, 50.0),
     (vf.KvDtype.F16, 8, 4, 512, 200, 64, 0, 0.0),
+    (vf.KvDtype.F16, 8, 2, 512, 1900, 192, 700, 40.0),   # head_dim 512 over a 2-byte cache: window, soft-cap
     (vf.KvDtype.F16, 12, 4, 64, 1000, 512, 0, 0.0),
     (vf.KvDtype.F32, 32, 8, 128, 700, 128, 0, 0.0),
     (vf.KvDtype.F32, 8, 2, 256, 300, 64, 50, 0.0),

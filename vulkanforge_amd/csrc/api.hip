@@ -540,7 +540,8 @@ uint32_t vfkv_decode_tile_for(uint32_t span, uint32_t n_heads, uint32_t n_kv_hea
     const uint32_t g = n_heads / n_kv_heads;
     // The matrix-core worker (1- and 2-byte caches, head_dim 64 / 128) runs best with one workgroup per CU and
     // serves up to 8 heads of a group per workgroup; the vector-ALU worker wants two and serves up to 4.
-    const bool mfma = (kv_dtype == VFKV_F8E4M3 || kv_dtype == VFKV_F16) && (head_dim == 64u || head_dim == 128u || head_dim == 256u);
+    const bool mfma = (kv_dtype == VFKV_F8E4M3 || kv_dtype == VFKV_F16) &&
+                      (head_dim == 64u || head_dim == 128u || head_dim == 256u || head_dim == 512u);
     if (mfma) {
         // short spans: one tile, so the worker writes the output itself and no merge launch follows
         static const bool forced = getenv("VFKV_DECODE_TILE") != nullptr;

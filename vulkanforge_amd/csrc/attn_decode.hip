@@ -1,9 +1,9 @@
 // Split-K decode attention for gfx950: worker (flash_attn_split.comp:82-162) and log-sum-exp
 // merge (flash_attn_reduce.comp:35-81), re-designed around the HBM stream.
 //
-//   split_mfma_kernel    (attn_decode_mfma.h) matrix-core worker: FP8 / F16 caches, head_dim 64 / 128 / 256 -- the
+//   split_mfma_kernel    (attn_decode_mfma.h) matrix-core worker: FP8 / F16 caches, head_dim 64 / 128 / 256 / 512 -- the
 //                        kernel every benchmark configuration runs on
-//   split_kernel         vector-ALU worker described below: F32 caches and head_dim 512
+//   split_kernel         vector-ALU worker described below: F32 caches (and every shape under VFKV_DECODE_WORKER=valu)
 //   split_generic_kernel one wavefront per (head, tile), any dtype, head_dim <= 512
 //   reduce_direct_kernel merge of up to 64 partials per head without LDS; reduce_kernel / reduce_generic_kernel beyond
 //
@@ -615,16 +615,21 @@ constexpr int kSplitWaves = 4;
 #define VFKV_MFMA_WAVES 4
 #endif
 
-template <int DT, int D, int RUN, int PF>
+template <int DT, int D, int RUN, int PF, int NH = 1>
 static hipError_t launch_split_mfma(const SplitArgs& a, uint32_t g, hipStream_t stream) {
     constexpr int NW = VFKV_MFMA_WAVES;
     const uint32_t gt = g < 8u ? g : 8u;
     dim3 grid(a.n_kv_heads, a.n_tiles, (g + gt - 1u) / gt);
     if (a.softcap > 0.f)
-        hipLaunchKernelGGL((split_mfma_kernel<DT, D, RUN, PF, NW, true>), grid, dim3(NW * kWave), 0, stream, a, gt);
+        hipLaunchKernelGGL((split_mfma_kernel<DT, D, RUN, PF, NW, true, NH>), grid, dim3(NW * kWave), 0, stream, a, gt);
     else
-        hipLaunchKernelGGL((split_mfma_kernel<DT, D, RUN, PF, NW, false>), grid, dim3(NW * kWave), 0, stream, a, gt);
+        hipLaunchKernelGGL((split_mfma_kernel<DT, D, RUN, PF, NW, false, NH>), grid, dim3(NW * kWave), 0, stream, a, gt);
     return hipGetLastError();
+}
+
+// Shapes the matrix-core worker is built for (head_dim 512: two wavefronts per run, each half of the output columns).
+static bool mfma_worker_shape(uint32_t dtype, uint32_t D) {
+    return (dtype == kF8 || dtype == kF16) && (D == 64u || D == 128u || D == 256u || D == 512u);
 }
 
 // VFKV_DECODE_WORKER=valu keeps the vector-ALU worker for every shape (for comparisons).
@@ -668,7 +673,7 @@ bool split_appends(const SplitLaunch& L) {
     const bool aligned = ((((uintptr_t)L.k) | ((uintptr_t)L.v) | ((uintptr_t)L.q) | ((uintptr_t)L.k_new) | ((uintptr_t)L.v_new) |
                            ((uintptr_t)L.scratch_out)) & 15u) == 0u;
     const uint64_t slab_bytes = (uint64_t)L.seq_len * L.n_kv_heads * L.head_dim * elem_size(L.dtype);
-    const bool mfma_shape = (L.dtype == kF8 || L.dtype == kF16) && (L.head_dim == 64u || L.head_dim == 128u || L.head_dim == 256u);
+    const bool mfma_shape = mfma_worker_shape(L.dtype, L.head_dim);
     return aligned && slab_bytes < 0x7FFF0000ull && mfma_worker_enabled() && mfma_shape && g <= 8u &&
            L.append_pos < L.seq_len && L.append_pos >= L.kv_start;
 }
@@ -678,7 +683,7 @@ bool split_writes_output(const SplitLaunch& L) {
     if (L.n_tiles != 1u || L.n_kv_heads == 0u) return false;
     const bool aligned = ((((uintptr_t)L.k) | ((uintptr_t)L.v) | ((uintptr_t)L.q) | ((uintptr_t)L.scratch_out)) & 15u) == 0u;
     const uint64_t slab_bytes = (uint64_t)L.seq_len * L.n_kv_heads * L.head_dim * elem_size(L.dtype);
-    const bool mfma_shape = (L.dtype == kF8 || L.dtype == kF16) && (L.head_dim == 64u || L.head_dim == 128u || L.head_dim == 256u);
+    const bool mfma_shape = mfma_worker_shape(L.dtype, L.head_dim);
     return aligned && slab_bytes < 0x7FFF0000ull && mfma_worker_enabled() && mfma_shape;
 }
 
@@ -715,6 +720,8 @@ hipError_t launch_split(const SplitLaunch& L, hipStream_t stream) {
         if (L.dtype == kF16 && L.head_dim == 128u) return launch_split_mfma<kF16, 128, VFKV_MFMA_RUN_F16, VFKV_MFMA_PF_F16>(a, g, stream);
         if (L.dtype == kF8 && L.head_dim == 256u) return launch_split_mfma<kF8, 256, 32, 1>(a, g, stream);
         if (L.dtype == kF16 && L.head_dim == 256u) return launch_split_mfma<kF16, 256, 32, 1>(a, g, stream);
+        if (L.dtype == kF8 && L.head_dim == 512u) return launch_split_mfma<kF8, 512, 32, 1, 2>(a, g, stream);
+        if (L.dtype == kF16 && L.head_dim == 512u) return launch_split_mfma<kF16, 512, 32, 1, 2>(a, g, stream);
     }
     if (fast_shape(L.dtype, L.head_dim) && aligned && slab_bytes < 0x7FFF0000ull) {
 #define VFKV_CASE(DT, DD) \

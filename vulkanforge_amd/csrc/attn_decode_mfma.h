@@ -31,21 +31,27 @@
 
 namespace vfkv {
 
-template <int DT, int D, int RUN, int PF, int NW, bool CAP>
+// NH > 1 (head_dim 512): NH wavefronts walk the same runs.  Each computes the scores over the whole head_dim and stages,
+// accumulates, merges and stores its own slice of D / NH output columns (the accumulators of a 512-wide head do not fit
+// one wavefront); the workgroup then walks NW / NH runs at a time.
+template <int DT, int D, int RUN, int PF, int NW, bool CAP, int NH = 1>
 __global__ __launch_bounds__(NW * 64) void split_mfma_kernel(SplitArgs a, uint32_t gt) {
     constexpr int ES = DT == kF16 ? 2 : 1;
+    constexpr int DV = D / NH;                   // output columns of a wavefront
+    constexpr int NP = NW / NH;                  // run streams of the workgroup
     constexpr int RT = RUN / 16;                 // 16-row tiles per run
     constexpr int PKS = RUN / 32;                // k-steps (32 rows) of the second product
     constexpr int KS = D / 32;                   // k-steps of the first product
-    constexpr int DTILES = D / 16;
+    constexpr int DTILES = DV / 16;
     constexpr int SEG = D / 4, SEGB = SEG * ES;  // a lane group's quarter of a K row
     constexpr int KLD = SEGB / 16;               // 16-byte loads per lane per K row
-    constexpr int VPITCH = D + 16;               // halves per V row in LDS (+32 B against bank conflicts)
-    constexpr int VCHUNK_ROW = D * ES / 16;      // 16-byte chunks per V row
+    constexpr int VPITCH = DV + 16;              // halves per V row in LDS (+32 B against bank conflicts)
+    constexpr int VCHUNK_ROW = DV * ES / 16;     // 16-byte chunks per V row (this wavefront's columns)
     constexpr int VLD = RUN * VCHUNK_ROW / 64;   // V loads per lane per run
     constexpr int VROWS = 64 / VCHUNK_ROW;       // rows covered by one V load of the wavefront
     static_assert(D % 32 == 0 && SEGB % 16 == 0 && RUN % 32 == 0 && VCHUNK_ROW <= 64 && VLD >= 1, "unsupported shape");
-    static_assert(NW * RUN * VPITCH * 2 >= NW * (D / 16) * 64 * 16, "merge buffer must fit in the V staging area");
+    static_assert(NW * RUN * VPITCH * 2 >= NW * (DV / 16) * 64 * 16, "merge buffer must fit in the V staging area");
+    static_assert(NW % NH == 0, "whole run streams");
 
     __shared__ __attribute__((aligned(16))) _Float16 vlds[NW][RUN * VPITCH];
     __shared__ float lds_m[NW][8], lds_l[NW][8];
@@ -53,6 +59,7 @@ __global__ __launch_bounds__(NW * 64) void split_mfma_kernel(SplitArgs a, uint32
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wp = w / NH, ds = w % NH;          // run stream of this wavefront, its slice of the output columns
     const int n16 = lane & 15, kg = lane >> 4;
     const int col = n16 & 7;
     const bool is_lo = n16 >= 8;
@@ -77,7 +84,7 @@ __global__ __launch_bounds__(NW * 64) void split_mfma_kernel(SplitArgs a, uint32
     const uint32_t head_b = kvh * D * ES;
     const uint32_t lane_koff = n16 * row_stride + head_b + kg * SEGB;
     const int vrow = lane / VCHUNK_ROW, vcol = lane % VCHUNK_ROW;
-    const uint32_t lane_voff = vrow * row_stride + head_b + vcol * 16;
+    const uint32_t lane_voff = vrow * row_stride + head_b + ds * DV * ES + vcol * 16;
     const float scale_l2 = a.scale * 1.44269504088896f;
     const float cap_l2 = a.softcap * 1.44269504088896f;
 
@@ -105,7 +112,7 @@ __global__ __launch_bounds__(NW * 64) void split_mfma_kernel(SplitArgs a, uint32
     // the lines were not touched by this workgroup before, so the loads fetch them from L2, where the stores went.
     bool owns_new_row = false;
     if (a.k_new != nullptr)
-        owns_new_row = il ? ((((a.append_pos - tile_base) / RUN - first_run) / NW) % a.n_tiles == jl)
+        owns_new_row = il ? ((((a.append_pos - tile_base) / RUN - first_run) / NP) % a.n_tiles == jl)
                           : (a.append_pos >= tile_base && a.append_pos < tile_end);
     if (owns_new_row) {
         constexpr int EPW = 4 / ES;                              // elements per 32-bit word of the cache
@@ -136,10 +143,10 @@ __global__ __launch_bounds__(NW * 64) void split_mfma_kernel(SplitArgs a, uint32
     // at the same time (with separate streams per tile that helps; the interleaved walk is better off without).
     // (No division by a run-time value on the way to the first load: the rotation is taken modulo the largest power
     // of two that fits, and the interleaved walk needs no count of its runs.)
-    const uint32_t rs = il ? NW * a.n_tiles : NW;                     // distance between two runs of a wavefront
-    const uint32_t r0 = first_run + (il ? jl * NW : 0u) + w;
+    const uint32_t rs = il ? NP * a.n_tiles : NP;                     // distance between two runs of a wavefront
+    const uint32_t r0 = first_run + (il ? jl * NP : 0u) + wp;
     const bool active = lo < tile_end && r0 < n_runs;
-    const uint32_t n_cyc = (active && !il) ? (n_runs - r0 + NW - 1) / NW : 0u;   // runs walked cyclically (contiguous tile)
+    const uint32_t n_cyc = (active && !il) ? (n_runs - r0 + NP - 1) / NP : 0u;   // runs walked cyclically (contiguous tile)
     const uint32_t rot = n_cyc != 0u ? (kvh * 3u) & ((1u << (31 - __builtin_clz(n_cyc))) - 1u) : 0u;
     auto nth_run = [&](uint32_t i) -> uint32_t {   // i-th run of this wavefront; n_runs (= none) past the last
         if (!active) return n_runs;
@@ -147,7 +154,7 @@ __global__ __launch_bounds__(NW * 64) void split_mfma_kernel(SplitArgs a, uint32
         if (i >= n_cyc) return n_runs;
         uint32_t ii = i + rot;
         if (ii >= n_cyc) ii -= n_cyc;
-        return r0 + ii * NW;
+        return r0 + ii * NP;
     };
     const uint32_t off0 = run_off(nth_run(0));
 #pragma unroll
@@ -334,7 +341,7 @@ __global__ __launch_bounds__(NW * 64) void split_mfma_kernel(SplitArgs a, uint32
 
     // ---------------- wavefront totals, then the workgroup merge through LDS ----------------
     // Every wavefront parks its accumulators in LDS in register order (lane-major: conflict-free 16-byte accesses),
-    // then wavefront w merges the d-tiles w, w + NW, ... of all wavefronts and stores them straight from registers.
+    // then wavefront w merges the d-tiles w, w + NW, ... of all wavefronts and stores them straight from registers
     l_run = xor32_sum(xor16_sum(l_run));
 #pragma unroll
     for (int dt = 0; dt < DTILES; ++dt)
@@ -347,25 +354,26 @@ __global__ __launch_bounds__(NW * 64) void split_mfma_kernel(SplitArgs a, uint32
     if (kg == 0 && !is_lo) { lds_m[w][col] = m_run; lds_l[w][col] = l_run; }
     __syncthreads();
     // all LDS reads of the merge are issued before the first use, so their latencies overlap
-    constexpr int MT = DTILES / NW;                    // d-tiles merged and stored by each wavefront
-    static_assert(DTILES % NW == 0, "d-tiles must divide evenly among the wavefronts");
-    float mw[NW], lw[NW];
-    float4_t part[MT][NW];
+    // (with output slices: among the NP wavefronts that own the same columns; their statistics are those of the streams)
+    constexpr int MT = DTILES / NP;                    // d-tiles merged and stored by each wavefront
+    static_assert(DTILES % NP == 0, "d-tiles must divide evenly among the wavefronts");
+    float mw[NP], lw[NP];
+    float4_t part[MT][NP];
 #pragma unroll
-    for (int ww = 0; ww < NW; ++ww) { mw[ww] = lds_m[ww][col]; lw[ww] = lds_l[ww][col]; }
+    for (int pp = 0; pp < NP; ++pp) { mw[pp] = lds_m[pp * NH + ds][col]; lw[pp] = lds_l[pp * NH + ds][col]; }
 #pragma unroll
     for (int t = 0; t < MT; ++t)
 #pragma unroll
-        for (int ww = 0; ww < NW; ++ww) part[t][ww] = slot[(ww * DTILES + t * NW + w) * 64 + lane];
+        for (int pp = 0; pp < NP; ++pp) part[t][pp] = slot[((pp * NH + ds) * DTILES + t * NP + wp) * 64 + lane];
     float M = mw[0];
 #pragma unroll
-    for (int ww = 1; ww < NW; ++ww) M = fmaxf(M, mw[ww]);
-    float fw[NW];
+    for (int pp = 1; pp < NP; ++pp) M = fmaxf(M, mw[pp]);
+    float fw[NP];
     float l = 0.f;
 #pragma unroll
-    for (int ww = 0; ww < NW; ++ww) {
-        fw[ww] = __builtin_amdgcn_exp2f(mw[ww] - M);
-        l = fmaf(fw[ww], lw[ww], l);
+    for (int pp = 0; pp < NP; ++pp) {
+        fw[pp] = __builtin_amdgcn_exp2f(mw[pp] - M);
+        l = fmaf(fw[pp], lw[pp], l);
     }
     const bool writer = !is_lo && (uint32_t)col < gcount;
     const size_t pidx = (size_t)(h0 + col) * a.n_tiles + jl;
@@ -373,17 +381,17 @@ __global__ __launch_bounds__(NW * 64) void split_mfma_kernel(SplitArgs a, uint32
     // forward/runs.rs:776-821): the merge is a plain normalisation, done here, and no merge launch follows
     const bool direct = a.o_direct != nullptr;
     const float inv_l = direct ? __builtin_amdgcn_rcpf(l) : 1.0f;
-    float* const obase = direct ? a.o_direct + (size_t)(h0 + col) * D : a.so + pidx * D;
+    float* const obase = (direct ? a.o_direct + (size_t)(h0 + col) * D : a.so + pidx * D) + ds * DV;
 #pragma unroll
     for (int t = 0; t < MT; ++t) {
         float4_t o = fw[0] * part[t][0];
 #pragma unroll
-        for (int ww = 1; ww < NW; ++ww) o += fw[ww] * part[t][ww];
+        for (int pp = 1; pp < NP; ++pp) o += fw[pp] * part[t][pp];
         if (direct) {                                  // one Newton step brings the reciprocal to f32 accuracy
             const float r = inv_l * (2.0f - l * inv_l);
             o *= r;
         }
-        if (writer) *reinterpret_cast<float4_t*>(obase + (t * NW + w) * 16 + kg * 4) = o;
+        if (writer) *reinterpret_cast<float4_t*>(obase + (t * NP + wp) * 16 + kg * 4) = o;
     }
     if (writer && w == 0 && kg == 0 && a.o_direct == nullptr) {
         a.sm[pidx] = M > -1e29f ? M * 0.693147180559945f : kMasked;

@@ -324,6 +324,16 @@ int vfkv_prefill_attention(vfkv_cache* c, uint32_t layer, uint32_t kv_layer, uin
                            const float* q, float* o, uint32_t m, uint32_t base_pos, uint32_t window,
                            float scale, float softcap, vfkv_stream stream);
 
+/* vfkv_prefill_attention with a workspace (the one of the decode path).  Short chunks over long
+ * histories -- the suffix of a request that keeps the resident rows of its prefix, server/state.rs:
+ * 199-224 -- leave most compute units without a workgroup; with a workspace the keys are also cut
+ * into chunks over workgroups and the decode merge (vfkv_flash_attn_reduce's kernel) combines the
+ * partials.  Same results within f32 rounding; falls back to the plain call whenever that is not
+ * worth it or the workspace is too small (it needs m * n_heads * chunks * head_dim floats). */
+int vfkv_prefill_attention_ws(vfkv_cache* c, uint32_t layer, uint32_t kv_layer, uint32_t n_heads,
+                              const float* q, float* o, uint32_t m, uint32_t base_pos, uint32_t window,
+                              float scale, float softcap, vfkv_workspace* ws, vfkv_stream stream);
+
 /* ------------------------------------------------------------------------------------------ */
 /* Gated attention output (Qwen3.6 full-attention layers).                                    */
 /* ------------------------------------------------------------------------------------------ */

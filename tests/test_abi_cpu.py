@@ -278,3 +278,10 @@ def test_gated_entry_points_reject_bad_arguments_before_any_device_work():
     assert L.vfkv_decode_attention_gated(None, 0, 0, 4, 64, None, None, 64, 0, 0, 1.0, 0.0, None, None, None) == -1
     assert L.vfkv_prefill_attention_gated(None, 0, 0, 4, 64, 64, 1, 0, 0, 1.0, 0.0, None, None) == -1
     assert L.vfkv_prefill_attention_gated(None, 0, 0, 4, 64, 64, 1, 0, 0, 1.0, 0.0, C.byref(g), None) == -1   # no cache
+
+
+def test_prefill_attention_ws_rejects_bad_arguments_before_any_device_work():
+    L = _ffi.lib()
+    assert L.vfkv_prefill_attention_ws(None, 0, 0, 4, 64, 64, 1, 0, 0, 1.0, 0.0, None, None) == -1      # no workspace
+    assert b"workspace" in L.vfkv_last_error()
+    assert L.vfkv_prefill_attention_ws(None, 0, 0, 4, 64, 64, 1, 0, 0, 1.0, 0.0, 64, None) == -1        # no cache

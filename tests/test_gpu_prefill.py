@@ -193,3 +193,56 @@ def test_scores_that_drift_past_the_running_maximum(dtype, shape):
     ref = oracle.attn_batch_ref(q, ke, ve, int(dtype), m, n_kv, heads, hkv, d, q_start, scale)
     assert np.isfinite(o).all()
     assert np.abs(o - ref).max() < 1e-4
+
+
+@pytest.mark.parametrize("dtype,heads,hkv,d,m,base,window,cap", (
+    (vf.KvDtype.F8, 32, 8, 128, 64, 4096, 0, 0.0),       # the suffix of a request over its reused prefix
+    (vf.KvDtype.F16, 32, 8, 128, 20, 9000, 0, 0.0),      # one partly filled query block, four-heads-per-wavefront form
+    (vf.KvDtype.F8, 16, 8, 256, 37, 3000, 2048, 30.0),   # window and soft-cap: chunks start at the window
+    (vf.KvDtype.F8, 8, 2, 512, 16, 2500, 0, 0.0),        # head_dim 512: output slices and key chunks together
+    (vf.KvDtype.F16, 28, 4, 128, 50, 1500, 0, 0.0),      # G = 7
+    (vf.KvDtype.F8, 32, 8, 128, 512, 4096, 0, 0.0),      # a full chunk: plenty of workgroups, the plain path is taken
+    (vf.KvDtype.F32, 8, 2, 128, 16, 2000, 0, 0.0),       # F32 cache: no key chunks, same result
+))
+def test_prefill_with_workspace_matches_plain_call_and_oracle(dtype, heads, hkv, d, m, base, window, cap):
+    # vfkv_prefill_attention_ws cuts the keys into chunks over workgroups and merges the partials
+    r = rng(base + m + d)
+    n = base + m
+    cache = vf.KvCache(vf.KvCacheConfig(1, hkv, d, n, dtype=dtype))
+    fwd = vf.Forward(cache, heads)
+    fwd.workspace = vf.Workspace(heads, d, 32768)            # sized for a serving context, as the decode path has it
+    fill = outlier_normal if dtype == vf.KvDtype.F8 else fp16_normal
+    k, v = fill(r, (n, hkv, d)), fill(r, (n, hkv, d))
+    fwd.b_step_kv_write(0, 0, n, to_dev(k), to_dev(v))
+    q = to_dev(r.standard_normal((m, heads, d)).astype(np.float32))
+    a = torch.full((m, heads, d), float("nan"), device=DEV)
+    b = torch.full((m, heads, d), float("nan"), device=DEV)
+    print(f"case dtype={dtype.label()} H={heads} Hkv={hkv} D={d} m={m} base={base} window={window} cap={cap}", flush=True)
+    for rep in range(2):                                     # twice: the workspace is reused
+        fwd.b_step_attention(0, base, m, q, a, kv_start_window=window, softcap=cap, use_workspace=True)
+    fwd.b_step_attention(0, base, m, q, b, kv_start_window=window, softcap=cap)
+    torch.cuda.synchronize()
+    assert np.isfinite(to_np(a)).all()
+    assert np.abs(to_np(a) - to_np(b)).max() < 2e-6 * max(1.0, float(np.abs(to_np(b)).max())) + 2e-5   # f32 rounding of another summation order
+    kv_start = oracle.kv_start_batch(base, m, window)
+    ref = oracle.attn_batch_ref(to_np(q), encode_np(k, dtype), encode_np(v, dtype), int(dtype), m, n, heads, hkv, d, base,
+                                float(1.0 / np.sqrt(d)), kv_start=kv_start, softcap=cap)
+    assert np.abs(to_np(a) - ref).max() < TOL[dtype]
+    cache.destroy()
+
+
+def test_prefill_with_a_small_workspace_falls_back():
+    heads, hkv, d, m, base = 32, 8, 128, 64, 4096
+    r = rng(5)
+    cache = vf.KvCache(vf.KvCacheConfig(1, hkv, d, base + m, dtype=vf.KvDtype.F8))
+    fwd = vf.Forward(cache, heads)
+    fwd.workspace = vf.Workspace(heads, d, 64)               # one tile per head: no room for partials of 64 x 32 rows
+    k = fp16_normal(r, (base + m, hkv, d))
+    fwd.b_step_kv_write(0, 0, base + m, to_dev(k), to_dev(k))
+    q = to_dev(fp16_normal(r, (m, heads, d)))
+    a, b = torch.empty((m, heads, d), device=DEV), torch.empty((m, heads, d), device=DEV)
+    fwd.b_step_attention(0, base, m, q, a, use_workspace=True)
+    fwd.b_step_attention(0, base, m, q, b)
+    torch.cuda.synchronize()
+    assert (to_np(a) == to_np(b)).all()
+    cache.destroy()

@@ -104,6 +104,7 @@ SIGNATURES = {
     "vfkv_decode_attention": (C.c_int, [_vp, _u32, _u32, _u32, _vp, _vp, _u32, _u32, _f, _f, _vp, _vp]),
     "vfkv_flash_attn_batch": (C.c_int, [_vp, _vp, _vp, _u32, _vp, C.POINTER(BatchParams), _f, _vp]),
     "vfkv_prefill_attention": (C.c_int, [_vp, _u32, _u32, _u32, _vp, _vp, _u32, _u32, _u32, _f, _f, _vp]),
+    "vfkv_prefill_attention_ws": (C.c_int, [_vp, _u32, _u32, _u32, _vp, _vp, _u32, _u32, _u32, _f, _f, _vp, _vp]),
     "vfkv_sigmoid_mul": (C.c_int, [C.POINTER(Gate), _vp, _u32, _vp]),
     "vfkv_decode_attention_gated": (C.c_int, [_vp, _u32, _u32, _u32, _vp, _vp, _vp, _vp, _u32, _u32, _f, _f, C.POINTER(Gate),
                                               _vp, _vp]),

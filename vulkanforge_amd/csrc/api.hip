@@ -626,8 +626,8 @@ int vfkv_kv_write_decode_attention(vfkv_cache* c, uint32_t layer, uint32_t n_hea
 }
 
 // ---- prefill attention -------------------------------------------------------------------------------
-int vfkv_flash_attn_batch(const float* q, const void* k_layer, const void* v_layer, uint32_t kv_dtype, float* o,
-                          const vfkv_batch_params* p, float softcap, vfkv_stream stream) {
+static int flash_attn_batch_impl(const float* q, const void* k_layer, const void* v_layer, uint32_t kv_dtype, float* o,
+                                 const vfkv_batch_params* p, float softcap, vfkv_workspace* ws, vfkv_stream stream) {
     if (!p) return fail(VFKV_ERR_INVALID_ARG, "flash_attn_batch: params is NULL");
     if (!q || !k_layer || !v_layer || !o) return fail(VFKV_ERR_INVALID_ARG, "flash_attn_batch: NULL buffer");
     if (kv_dtype > VFKV_F8E4M3) return fail(VFKV_ERR_INVALID_ARG, "flash_attn_batch: unknown kv dtype %u", kv_dtype);
@@ -645,13 +645,23 @@ int vfkv_flash_attn_batch(const float* q, const void* k_layer, const void* v_lay
     L.dtype = kv_dtype; L.n_heads = p->n_heads; L.n_kv_heads = p->n_kv_heads; L.head_dim = p->head_dim;
     L.m = p->m; L.n_kv = p->n_kv; L.q_start = p->q_start; L.kv_start = p->kv_start;
     L.scale = p->scale; L.softcap = softcap;
+    if (ws) {
+        L.scratch_out = ws->scratch_out; L.scratch_max = ws->scratch_max; L.scratch_sum = ws->scratch_sum;
+        L.scratch_ml_floats = (uint64_t)ws->n_heads * ws->max_tiles;
+        L.scratch_out_floats = L.scratch_ml_floats * ws->head_dim;
+    }
     VFKV_HIP(vfkv::launch_batch(L, S(stream)));
     return VFKV_OK;
 }
 
-int vfkv_prefill_attention(vfkv_cache* c, uint32_t layer, uint32_t kv_layer, uint32_t n_heads, const float* q, float* o,
-                           uint32_t m, uint32_t base_pos, uint32_t window, float scale, float softcap,
-                           vfkv_stream stream) {
+int vfkv_flash_attn_batch(const float* q, const void* k_layer, const void* v_layer, uint32_t kv_dtype, float* o,
+                          const vfkv_batch_params* p, float softcap, vfkv_stream stream) {
+    return flash_attn_batch_impl(q, k_layer, v_layer, kv_dtype, o, p, softcap, nullptr, stream);
+}
+
+static int prefill_attention_impl(vfkv_cache* c, uint32_t layer, uint32_t kv_layer, uint32_t n_heads, const float* q, float* o,
+                                  uint32_t m, uint32_t base_pos, uint32_t window, float scale, float softcap,
+                                  vfkv_workspace* ws, vfkv_stream stream) {
     if (!c || !c->k || !c->v) return fail(VFKV_ERR_INVALID_ARG, "prefill_attention: cache has no buffers");
     if (layer >= c->n_layers || kv_layer >= c->n_layers)
         return fail(VFKV_ERR_INVALID_ARG, "prefill_attention: layer %u / kv_layer %u out of range", layer, kv_layer);
@@ -668,7 +678,20 @@ int vfkv_prefill_attention(vfkv_cache* c, uint32_t layer, uint32_t kv_layer, uin
     p.scale = scale;
     p.kv_start = vfkv_kv_start_batch(base_pos, m, window);
     const uint64_t off = layer_off(c, kv_layer);
-    return vfkv_flash_attn_batch(q, (char*)c->k + off, (char*)c->v + off, c->dtype, o, &p, softcap, stream);
+    return flash_attn_batch_impl(q, (char*)c->k + off, (char*)c->v + off, c->dtype, o, &p, softcap, ws, stream);
+}
+
+int vfkv_prefill_attention(vfkv_cache* c, uint32_t layer, uint32_t kv_layer, uint32_t n_heads, const float* q, float* o,
+                           uint32_t m, uint32_t base_pos, uint32_t window, float scale, float softcap,
+                           vfkv_stream stream) {
+    return prefill_attention_impl(c, layer, kv_layer, n_heads, q, o, m, base_pos, window, scale, softcap, nullptr, stream);
+}
+
+int vfkv_prefill_attention_ws(vfkv_cache* c, uint32_t layer, uint32_t kv_layer, uint32_t n_heads, const float* q, float* o,
+                              uint32_t m, uint32_t base_pos, uint32_t window, float scale, float softcap,
+                              vfkv_workspace* ws, vfkv_stream stream) {
+    if (!ws) return fail(VFKV_ERR_INVALID_ARG, "prefill_attention_ws: workspace is NULL");
+    return prefill_attention_impl(c, layer, kv_layer, n_heads, q, o, m, base_pos, window, scale, softcap, ws, stream);
 }
 
 // ---- gated output --------------------------------------------------------------------------------------

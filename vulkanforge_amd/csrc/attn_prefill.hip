@@ -19,6 +19,12 @@ struct BatchArgs {
     uint32_t m, n_kv, q_start, kv_start;
     float scale, softcap;
     uint32_t dtype;
+    // key chunks over workgroups (f16 matrix-core kernel only): workgroup z handles keys [kc * chunk, (kc + 1) * chunk) and
+    // stores an unnormalised partial (o, m, l) per (query, head, chunk) for the decode merge kernel; so == NULL: off
+    float* so;
+    float* sm;
+    float* ss;
+    uint32_t nk, chunk;
 };
 
 }  // namespace vfkv
@@ -95,6 +101,7 @@ hipError_t launch_batch(const BatchLaunch& L, hipStream_t stream) {
     a.n_heads = L.n_heads; a.n_kv_heads = L.n_kv_heads; a.head_dim = L.head_dim;
     a.m = L.m; a.n_kv = L.n_kv; a.q_start = L.q_start; a.kv_start = L.kv_start;
     a.scale = L.scale; a.softcap = L.softcap; a.dtype = L.dtype;
+    a.so = nullptr; a.sm = nullptr; a.ss = nullptr; a.nk = 1u; a.chunk = 0u;
     const uint32_t g = L.n_heads / L.n_kv_heads;
     const uint64_t slab_bytes = (uint64_t)L.n_kv * L.n_kv_heads * L.head_dim * elem_size(L.dtype);
     const bool aligned = ((((uintptr_t)L.k) | ((uintptr_t)L.v) | ((uintptr_t)L.q) | ((uintptr_t)L.o)) & 15u) == 0u;
@@ -148,7 +155,29 @@ hipError_t launch_batch(const BatchLaunch& L, hipStream_t stream) {
         if (max_waves >= hp && nz <= 65535u) {
             const uint32_t ns = max_waves / hp;               // key splits: fill the workgroup
             const uint32_t nwaves = hp * ns;
-            const dim3 grid((L.m + 15u) / 16u, L.n_kv_heads, nz), block(nwaves * kWave);
+            // Short chunks over long histories (the suffix of a request that reuses its prefix) still leave most compute
+            // units idle: with a workspace the keys are also cut into chunks over workgroups, every workgroup stores a
+            // partial per (query, head, chunk), and the decode merge kernel combines them.
+            uint32_t nk = 1u;
+            if (L.scratch_out != nullptr && L.n_heads != 0u) {
+                const uint64_t wgs = (uint64_t)((L.m + 15u) / 16u) * L.n_kv_heads * nz;
+                const uint32_t t0 = (L.kv_start / 32u) * 32u;
+                const uint32_t kend = L.q_start + L.m < L.n_kv ? L.q_start + L.m : L.n_kv;
+                const uint32_t span = kend > t0 ? kend - t0 : 0u;
+                if (wgs < 192u && span >= 1024u) {
+                    nk = (uint32_t)((256u + wgs - 1u) / wgs);
+                    if (nk > span / 512u) nk = span / 512u;   // at least 512 keys per chunk
+                    if (nk > 32u) nk = 32u;
+                    const uint64_t rows = (uint64_t)L.m * L.n_heads;
+                    while (nk > 1u && (rows * nk * L.head_dim > L.scratch_out_floats || rows * nk > L.scratch_ml_floats)) --nk;
+                    if (rows > 0xFFFFFFFFull / 64u) nk = 1u;
+                }
+                if (nk > 1u) {
+                    a.so = L.scratch_out; a.sm = L.scratch_max; a.ss = L.scratch_sum; a.nk = nk;
+                    a.chunk = ((span + nk - 1u) / nk + 31u) / 32u * 32u;
+                }
+            }
+            const dim3 grid((L.m + 15u) / 16u, L.n_kv_heads, nz * nk), block(nwaves * kWave);
             const size_t vbytes = (size_t)nwaves * 32 * (dv + 16) * sizeof(_Float16) +
                                   (size_t)2 * (hp / nh) * ncb * 16 * (L.head_dim + 8) * sizeof(_Float16);
             const size_t mbytes = (size_t)(ns - 1) * hp * ncb * 64 * (dv / 4 + 2) * sizeof(float);
@@ -173,7 +202,13 @@ hipError_t launch_batch(const BatchLaunch& L, hipStream_t stream) {
             } else
             { launched = false; }
 #undef VFKV_P2
-            if (launched) return hipGetLastError();
+            if (launched) {
+                hipError_t e = hipGetLastError();
+                if (e == hipSuccess && nk > 1u)
+                    e = launch_reduce(a.so, a.sm, a.ss, L.o, L.m * L.n_heads, L.head_dim, nk, stream);
+                return e;
+            }
+            a.so = nullptr; a.nk = 1u;
         }
     }
     // f32 matrix-core kernel: F32 caches, and the head sizes the f16 kernels above do not cover

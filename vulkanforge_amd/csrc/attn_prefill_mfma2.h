@@ -64,7 +64,8 @@ __global__ __launch_bounds__((NCB == 1 && D <= 128) ? VFKV_PREFILL_NCB1_WAVES * 
     const uint32_t qi = q0 + n16;                               // this lane's query (column of S^T)
     const bool q_ok = qi < a.m;
     const uint32_t row_stride = a.n_kv_heads * D * ES;
-    const int gz = blockIdx.z * (HP / NH) * NCB;                // first head (inside the group) of this workgroup
+    const uint32_t kc = blockIdx.z % a.nk;                      // key chunk of this workgroup (a.nk == 1: all keys)
+    const int gz = (blockIdx.z / a.nk) * (HP / NH) * NCB;       // first head (inside the group) of this workgroup
     const int g0 = (hp / NH) * NCB;                             // first head slot (inside the workgroup) of this wavefront
     const int dslice = hp % NH;                                 // which D / NH output elements this wavefront owns
 
@@ -80,7 +81,13 @@ __global__ __launch_bounds__((NCB == 1 && D <= 128) ? VFKV_PREFILL_NCB1_WAVES * 
     const uint32_t my_len = q_ok ? (a.q_start + qi + 1 < a.n_kv ? a.q_start + qi + 1 : a.n_kv) : 0;   // causal_len of this lane's query
     uint32_t full_len = a.q_start + q0 + 1;                     // keys every query of the block sees
     if (full_len > a.n_kv) full_len = a.n_kv;
-    const uint32_t t_first = (a.kv_start / KT) * KT;
+    uint32_t t_first = (a.kv_start / KT) * KT;
+    if (a.nk > 1u) {                                            // this workgroup's chunk of the keys (multiples of KT)
+        t_first += kc * a.chunk;
+        const uint32_t hi = t_first + a.chunk;
+        if (kmax > hi) kmax = hi;
+    }
+    const uint32_t fast_end = full_len < kmax ? full_len : kmax;   // tiles below it are seen completely by every query (and are this workgroup's)
     const float scale_l2 = a.scale * 1.44269504088896f;
     const float cap_l2 = a.softcap * 1.44269504088896f;
 
@@ -335,7 +342,7 @@ __global__ __launch_bounds__((NCB == 1 && D <= 128) ? VFKV_PREFILL_NCB1_WAVES * 
         first_slot = 0;
         s_ready = false;
         bool left = false;
-        while (!left && tb >= a.kv_start && tb + (PFD - 1) * step + KT <= full_len) {
+        while (!left && tb >= a.kv_start && tb + (PFD - 1) * step + KT <= fast_end) {
 #pragma unroll
             for (int sl = 0; sl < PFD; ++sl) {
                 const uint32_t tcur = tb + sl * step;
@@ -393,6 +400,22 @@ __global__ __launch_bounds__((NCB == 1 && D <= 128) ? VFKV_PREFILL_NCB1_WAVES * 
         for (int cb = 0; cb < NCB; ++cb) {
             if (gz + g0 + cb >= G) continue;                                  // padding slot of an odd group
             const uint32_t h = kvh * G + gz + g0 + cb;
+            if (a.so != nullptr) {
+                // key chunks: the unnormalised partial of this chunk in the layout of the decode merge ([row][chunk][D], the
+                // maximum in natural-log units); a query that sees no key of the chunk leaves (0, "minus infinity", 0)
+                const size_t pidx = ((size_t)qi * a.n_heads + h) * a.nk + kc;
+                float* op = a.so + pidx * D + dslice * DV + kg * 4;
+#pragma unroll
+                for (int dt = 0; dt < DTILES; ++dt) {
+                    const float4_t r = oacc[cb][dt];
+                    *reinterpret_cast<float4*>(op + dt * 16) = make_float4(r[0], r[1], r[2], r[3]);
+                }
+                if (kg == 0 && dslice == 0) {
+                    a.sm[pidx] = m_run[cb] > -1e29f ? m_run[cb] * 0.693147180559945f : kMasked;
+                    a.ss[pidx] = l_run[cb];
+                }
+                continue;
+            }
             const float inv = 1.0f / l_run[cb];
             float* op = a.o + ((size_t)qi * a.n_heads + h) * D + dslice * DV + kg * 4;   // lane (query n16) holds d = dslice*DV + dt*16 + kg*4 + i
 #pragma unroll

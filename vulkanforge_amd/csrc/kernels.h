@@ -89,6 +89,12 @@ struct BatchLaunch {
     uint32_t dtype, n_heads, n_kv_heads, head_dim;
     uint32_t m, n_kv, q_start, kv_start;
     float scale, softcap;
+    // optional scratch for partials of key chunks (short query chunks over long histories): [rows][chunks][head_dim] floats and
+    // two [rows][chunks] arrays, rows = m * n_heads; NULL: every workgroup walks all keys of its queries
+    float* scratch_out = nullptr;
+    float* scratch_max = nullptr;
+    float* scratch_sum = nullptr;
+    uint64_t scratch_out_floats = 0, scratch_ml_floats = 0;
 };
 hipError_t launch_batch(const BatchLaunch& a, hipStream_t stream);
 

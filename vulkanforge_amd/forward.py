@@ -188,10 +188,18 @@ class Forward:
 
     def b_step_attention(self, layer: int, base_pos: int, seq_len: int, q, o, kv_layer: int | None = None,
                          kv_start_window: int = 0, scale: float | None = None, softcap: float = 0.0,
-                         stream=None) -> None:
+                         stream=None, use_workspace: bool = False) -> None:
+        """``use_workspace=True``: vfkv_prefill_attention_ws (key chunks over workgroups for short chunks over long
+        histories, merged through the decode workspace)."""
         if scale is None:
             hd = self.kv_cache.head_dim_for(layer)
             scale = self.attn_scale if hd == self.kv_cache.config.head_dim else 1.0 / math.sqrt(hd)
+        if use_workspace:
+            _ffi.check(_ffi.lib().vfkv_prefill_attention_ws(self.kv_cache.handle, layer,
+                                                            layer if kv_layer is None else kv_layer, self.n_heads,
+                                                            _ptr(q), _ptr(o), seq_len, base_pos, kv_start_window, scale,
+                                                            softcap, self.workspace._h, _stream(stream)))
+            return
         _ffi.check(_ffi.lib().vfkv_prefill_attention(self.kv_cache.handle, layer,
                                                      layer if kv_layer is None else kv_layer, self.n_heads,
                                                      _ptr(q), _ptr(o), seq_len, base_pos, kv_start_window, scale,

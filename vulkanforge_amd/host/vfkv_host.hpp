@@ -204,6 +204,12 @@ public:
         check(vfkv_prefill_attention(kv_cache.handle(), layer, kv_layer, n_heads, q, o, seq_len, base_pos, kv_start_window,
                                      scale_for(layer), softcap, stream));
     }
+    // the same with the decode workspace: short chunks over long histories cut the keys into chunks over workgroups
+    void b_step_attention_ws(uint32_t layer, uint32_t base_pos, uint32_t seq_len, const float* q, float* o, uint32_t kv_layer,
+                             uint32_t kv_start_window, float softcap = 0.f) {
+        check(vfkv_prefill_attention_ws(kv_cache.handle(), layer, kv_layer, n_heads, q, o, seq_len, base_pos, kv_start_window,
+                                        scale_for(layer), softcap, ws_, stream));
+    }
     // runs.rs:2649-2681
     void run_sigmoid_mul(const float* gate, float* inout, uint32_t ne, uint32_t chunk, uint32_t stride, uint32_t gate_offset) {
         const vfkv_gate g{gate, chunk, stride, gate_offset};

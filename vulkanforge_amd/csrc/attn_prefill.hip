@@ -170,7 +170,7 @@ hipError_t launch_batch(const BatchLaunch& L, hipStream_t stream) {
                     if (nk > 32u) nk = 32u;
                     const uint64_t rows = (uint64_t)L.m * L.n_heads;
                     while (nk > 1u && (rows * nk * L.head_dim > L.scratch_out_floats || rows * nk > L.scratch_ml_floats)) --nk;
-                    if (rows > 0xFFFFFFFFull / 64u) nk = 1u;
+                    if (rows > 65535u) nk = 1u;               // rows are a grid dimension of the merge launch
                 }
                 if (nk > 1u) {
                     a.so = L.scratch_out; a.sm = L.scratch_max; a.ss = L.scratch_sum; a.nk = nk;

@@ -34,7 +34,7 @@ class Stack:
         self.fwd = vf.Forward(self.cache, H)
         self.cached_tokens = []
 
-    def prefill(self, tokens, base_pos):
+    def prefill(self, tokens, base_pos, use_workspace=False):
         """Rows [base_pos, len(tokens)) of every layer; returns the attention outputs of those rows."""
         ids = np.asarray(tokens[base_pos:], dtype=np.int64)
         m = len(ids)
@@ -44,7 +44,7 @@ class Stack:
             o = torch.empty((m, H, D), device=DEV)
             self.fwd.step_qk_rope_kv_write(layer, base_pos, m, q, to_dev(self.k[layer][ids]), to_dev(self.v[layer][ids]),
                                            D, self.ts, q_norm_weight=to_dev(self.wq), k_norm_weight=to_dev(self.wk))
-            self.fwd.b_step_attention(layer, base_pos, m, q, o)
+            self.fwd.b_step_attention(layer, base_pos, m, q, o, use_workspace=use_workspace)
             outs.append(o)
         torch.cuda.synchronize()
         self.cache.current_seq_len = len(tokens)
@@ -98,6 +98,31 @@ def test_clean_and_divergent_reuse_match_a_fresh_prefill(dtype):
         assert np.abs(full[:, k:] - out).max() < 2e-5
         fresh.cache.destroy(); single.cache.destroy()
     served.cache.destroy()
+
+
+def test_short_suffix_over_a_long_reused_prefix_with_the_workspace():
+    # the serving pattern of prefix reuse: a few new tokens over thousands of resident rows.  With the decode workspace the
+    # keys are cut into chunks over workgroups; the result is that of a fresh prefill of the whole sequence.
+    global MAX_SEQ
+    old_max, MAX_SEQ = MAX_SEQ, 3000
+    try:
+        r = rng(9)
+        first = list(r.integers(0, VOCAB, 2900))
+        second = first[:2870] + list(r.integers(0, VOCAB, 40))
+        served = Stack(vf.KvDtype.F8)
+        served.fwd.workspace = vf.Workspace(H, D, 32768)
+        served.request(first)
+        k = vf.prefix_reuse_start(served.cached_tokens, second)
+        assert k >= 2870
+        served.cache.current_seq_len = k
+        out = served.prefill(second, k, use_workspace=True)
+        single = Stack(vf.KvDtype.F8)
+        full = single.prefill(second, 0)
+        assert (served.rows(len(second)) == single.rows(len(second))).all()
+        assert np.abs(full[:, k:] - out).max() < 2e-5
+        served.cache.destroy(); single.cache.destroy()
+    finally:
+        MAX_SEQ = old_max
 
 
 def test_reuse_past_the_common_prefix_is_detectably_wrong():

@@ -309,6 +309,8 @@ def bench_prefill(args, wl):
     cache = vf.KvCache(vf.KvCacheConfig(L, Hkv, D, max_seq, dtype=wl.dtype), k_buffer=kbuf.data_ptr(),
                        v_buffer=vbuf.data_ptr())
     fwd = vf.Forward(cache, H)
+    if wl.workspace:                  # sized for a serving context, as the decode path has it
+        fwd.workspace = vf.Workspace(H, D, max(max_seq, 32768))
 
     class _W:  # fill_cache only needs n_layers
         n_layers = L
@@ -324,7 +326,7 @@ def bench_prefill(args, wl):
     def step():
         for layer in range(L):
             fwd.b_step_kv_write(layer, wl.base_pos, wl.m, kn, vn)
-            fwd.b_step_attention(layer, wl.base_pos, wl.m, q, o)
+            fwd.b_step_attention(layer, wl.base_pos, wl.m, q, o, use_workspace=wl.workspace)
 
     sec_per_step = time_steps(torch, step, args)
     step_spread = dict(STEP_SPREAD)
@@ -336,7 +338,7 @@ def bench_prefill(args, wl):
         for layer in range(L):
             e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
             e0.record(stream)
-            fwd.b_step_attention(layer, wl.base_pos, wl.m, q, o)
+            fwd.b_step_attention(layer, wl.base_pos, wl.m, q, o, use_workspace=wl.workspace)
             e1.record(stream)
             pairs.append((e0, e1))
     torch.cuda.synchronize()

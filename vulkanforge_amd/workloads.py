@@ -47,6 +47,7 @@ class PrefillWorkload:
     base_pos: int
     m: int
     dtype: KvDtype
+    workspace: bool = False   # attention through vfkv_prefill_attention_ws (key chunks over workgroups)
 
     def pairs_per_head(self) -> int:
         return sum(self.base_pos + i + 1 for i in range(self.m))
@@ -80,6 +81,11 @@ PREFILL = {
                                                            512, KvDtype.F16),
     "prefill_fp8_hd256_512x4608_12layers": PrefillWorkload("prefill_fp8_hd256_512x4608_12layers", 12, 16, 8, 256, 4096,
                                                            512, KvDtype.F8),
+    # the suffix of a request that reuses its prefix: 64 new tokens over 16 k resident rows, with and without the workspace
+    "prefill_fp8_suffix64_over_16k_32layers": PrefillWorkload("prefill_fp8_suffix64_over_16k_32layers", 32, 32, 8, 128,
+                                                              16384, 64, KvDtype.F8, workspace=True),
+    "prefill_fp8_suffix64_over_16k_32layers_plain": PrefillWorkload("prefill_fp8_suffix64_over_16k_32layers_plain", 32, 32,
+                                                                    8, 128, 16384, 64, KvDtype.F8),
     # the headline prefill geometry over an F32 cache (the reference's VULKANFORGE_FP16_KV=0 mode), 4 layers
     "prefill_f32_512x4608_4layers": PrefillWorkload("prefill_f32_512x4608_4layers", 4, 32, 8, 128, 4096, 512, KvDtype.F32),
     # the headline prefill geometry over an F16 cache (not a reference configuration; used to tune the F16 variant)

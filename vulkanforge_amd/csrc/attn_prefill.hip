@@ -109,21 +109,19 @@ hipError_t launch_batch(const BatchLaunch& L, hipStream_t stream) {
                          (L.head_dim == 64u || L.head_dim == 128u || L.head_dim == 256u || L.head_dim == 512u);
     // f16 matrix-core kernel: NCB heads per wavefront, private tiles per wavefront, no barrier in the loop
     if (mfma_ok) {
-        // two heads per wavefront where the registers allow it
-        static const int force_ncb = [] { const char* e = getenv("VFKV_PREFILL_NCB"); return e ? atoi(e) : 0; }();
-#ifndef VFKV_PREFILL_F16_128_NCB
-#define VFKV_PREFILL_F16_128_NCB 2     // heads per wavefront, F16 cache, head_dim 128 (even GQA groups)
-#endif
-        // (odd groups of three and more heads round up to whole pairs: the spare slot computes on zeros and stores nothing)
-        uint32_t ncb = (g >= 2u && (L.head_dim == 64u || (L.head_dim == 128u && (L.dtype == kF8 || VFKV_PREFILL_F16_128_NCB == 2)))) ? 2u : 1u;
-        if (force_ncb == 1) ncb = 1u;
-        // F16 rows are twice the bytes: four heads per wavefront (one wavefront per SIMD, 512 registers) so that a K / V tile
-        // is loaded by one wavefront of the workgroup only
-        if (L.dtype == kF16 && g >= 3u && L.head_dim == 128u && force_ncb == 0) ncb = 4u;
-        if (L.head_dim == 256u && g >= 2u && force_ncb == 0) ncb = 2u;      // the same at head_dim 256 with two heads
         // head_dim 512: one head per wavefront, and two wavefronts share a head (each owns half of the output columns)
         const uint32_t nh = L.head_dim == 512u ? 2u : 1u;
-        if (nh == 2u) ncb = 1u;
+        // Heads per wavefront.  Two where the registers allow it (a K / V tile is then converted once for both); odd groups
+        // of three and more heads round up, the spare slot computes on zeros and stores nothing.  Where the rows are wide
+        // (F16 at head_dim 128, everything at head_dim 256) the traffic between L2 and the CUs is what binds: four / two heads
+        // per wavefront in workgroups of four wavefronts (one per SIMD, up to 512 registers), so that a K / V tile is loaded
+        // by one wavefront of the workgroup only.  VFKV_PREFILL_NCB=1 forces one head per wavefront (for comparisons).
+        static const int force_ncb = [] { const char* e = getenv("VFKV_PREFILL_NCB"); return e ? atoi(e) : 0; }();
+        uint32_t ncb = 1u;
+        if (force_ncb != 1 && nh == 1u && g >= 2u) {
+            if (L.head_dim == 128u && L.dtype == kF16 && g >= 3u) ncb = 4u;
+            else ncb = 2u;
+        }
         const uint32_t dv = L.head_dim / nh;
         const uint32_t hp_group = (g + ncb - 1u) / ncb * nh;     // (head slice, output slice) units of a whole GQA group
         // wavefronts per workgroup the registers allow: one head per wavefront at head_dim <= 128 needs few (three wavefronts

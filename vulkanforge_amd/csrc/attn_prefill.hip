@@ -118,8 +118,11 @@ hipError_t launch_batch(const BatchLaunch& L, hipStream_t stream) {
         // by one wavefront of the workgroup only.  VFKV_PREFILL_NCB=1 forces one head per wavefront (for comparisons).
         static const int force_ncb = [] { const char* e = getenv("VFKV_PREFILL_NCB"); return e ? atoi(e) : 0; }();
         uint32_t ncb = 1u;
-        if (force_ncb != 1 && nh == 1u && g >= 2u) {
-            if (L.head_dim == 128u && L.dtype == kF16 && g >= 3u) ncb = 4u;
+        if (force_ncb != 1 && g >= 2u) {
+            // head_dim 512: a second head per wavefront only for FP8 rows (F16 rows leave no registers for it) and only while
+            // head pairs still give every compute unit a workgroup
+            if (nh == 2u) ncb = (L.dtype == kF8 && (uint64_t)((L.m + 15u) / 16u) * L.n_kv_heads * ((g + 1u) / 2u) >= 256u) ? 2u : 1u;
+            else if (L.head_dim == 128u && L.dtype == kF16 && g >= 3u) ncb = 4u;
             else ncb = 2u;
         }
         const uint32_t dv = L.head_dim / nh;
@@ -191,7 +194,10 @@ hipError_t launch_batch(const BatchLaunch& L, hipStream_t stream) {
             VFKV_P2(kF16, 64, 2, 2) VFKV_P2(kF16, 64, 1, 2) VFKV_P2(kF16, 128, 1, 1) VFKV_P2(kF16, 128, 2, 1)
             VFKV_P2(kF8, 256, 1, 1) VFKV_P2(kF16, 256, 1, 1)
             VFKV_P2(kF16, 128, 4, 1) VFKV_P2(kF8, 256, 2, 1) VFKV_P2(kF16, 256, 2, 1)
-            if (L.head_dim == 512u && L.dtype == kF8) {
+            if (L.head_dim == 512u && L.dtype == kF8 && ncb == 2u) {
+                if (cap) hipLaunchKernelGGL((batch_mfma2_kernel<kF8, 512, 2, 1, true, 2>), grid, block, lds, stream, a, (int)hp, (int)ns);
+                else hipLaunchKernelGGL((batch_mfma2_kernel<kF8, 512, 2, 1, false, 2>), grid, block, lds, stream, a, (int)hp, (int)ns);
+            } else if (L.head_dim == 512u && L.dtype == kF8) {
                 if (cap) hipLaunchKernelGGL((batch_mfma2_kernel<kF8, 512, 1, 1, true, 2>), grid, block, lds, stream, a, (int)hp, (int)ns);
                 else hipLaunchKernelGGL((batch_mfma2_kernel<kF8, 512, 1, 1, false, 2>), grid, block, lds, stream, a, (int)hp, (int)ns);
             } else if (L.head_dim == 512u && L.dtype == kF16) {

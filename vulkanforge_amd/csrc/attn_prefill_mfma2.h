@@ -34,7 +34,6 @@ namespace vfkv {
 // one wavefront.  HP then counts (head, slice) units.
 template <int DT, int D, int NCB, int PFD, bool CAP, int NH = 1>
 __global__ __launch_bounds__((NCB == 1 && D <= 128) ? VFKV_PREFILL_NCB1_WAVES * 64 : (NCB * D >= 512 || (DT == kF16 && D == 256)) ? 256 : 512) void batch_mfma2_kernel(BatchArgs a, int HP, int NS) {
-    static_assert(NH == 1 || NCB == 1, "output slices only with one head per wavefront");
     constexpr int DV = D / NH;                   // output elements (V columns) of this wavefront
     constexpr int ES = DT == kF16 ? 2 : 1;
     constexpr int KT = 32;                       // keys per tile

@@ -259,7 +259,8 @@ int vfkv_flash_attn_reduce(const float* scratch_out, const float* scratch_max,
                            uint32_t n_tiles, vfkv_stream stream);
 
 /* Scratch for vfkv_decode_attention -- replaces fa_scratch_out/max/sum (forward/setup.rs:203-230),
- * sized for ceil(max_seq_len / 64) tiles of n_heads * head_dim floats. */
+ * sized for ceil(max_seq_len / 64) tiles of n_heads * head_dim floats.  vfkv_prefill_attention_ws
+ * borrows the same buffers.  Calls that share a workspace must be ordered on one stream. */
 typedef struct vfkv_workspace vfkv_workspace;
 int vfkv_workspace_create(uint32_t n_heads, uint32_t head_dim, uint32_t max_seq_len,
                           vfkv_workspace** out);

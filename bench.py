@@ -322,12 +322,26 @@ def bench_prefill(args, wl):
     kn = torch.randn((wl.m, Hkv * D), device=dev, generator=g).half().float()
     vn = torch.randn((wl.m, Hkv * D), device=dev, generator=g).half().float()
     o = torch.zeros((wl.m, H, D), device=dev)
+    qgate = torch.randn((wl.m, H, 2, D), device=dev, generator=g) if wl.gated else None   # per (token, head): [Q | G]
+
+    def attention(layer):
+        if wl.gated:   # b_step_attention + b_step_attn_gated_output: the attention kernel's store applies the gate
+            fwd.b_step_attention_gated(layer, wl.base_pos, wl.m, q, o, qgate, D, 2 * D, D)
+        else:
+            fwd.b_step_attention(layer, wl.base_pos, wl.m, q, o, use_workspace=wl.workspace)
 
     def step():
         for layer in range(L):
             fwd.b_step_kv_write(layer, wl.base_pos, wl.m, kn, vn)
-            fwd.b_step_attention(layer, wl.base_pos, wl.m, q, o, use_workspace=wl.workspace)
+            attention(layer)
 
+    def step_gate_separate():   # the gate as a launch of its own after the attention
+        for layer in range(L):
+            fwd.b_step_kv_write(layer, wl.base_pos, wl.m, kn, vn)
+            fwd.b_step_attention(layer, wl.base_pos, wl.m, q, o)
+            fwd.b_step_attn_gated_output(o, qgate, wl.m, D)
+
+    gate_separate_ms = time_steps(torch, step_gate_separate, args) * 1e3 if wl.gated else None
     sec_per_step = time_steps(torch, step, args)
     step_spread = dict(STEP_SPREAD)
     flops_step = wl.flops_layer() * L
@@ -338,7 +352,7 @@ def bench_prefill(args, wl):
         for layer in range(L):
             e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
             e0.record(stream)
-            fwd.b_step_attention(layer, wl.base_pos, wl.m, q, o, use_workspace=wl.workspace)
+            attention(layer)
             e1.record(stream)
             pairs.append((e0, e1))
     torch.cuda.synchronize()
@@ -362,6 +376,8 @@ def bench_prefill(args, wl):
                      "unit": "TFLOP/s", "frac": achieved / peak, "traffic": MEASURED_TRAFFIC_BYTES.get(wl.name),
                      "avg_launch_us": avg_ms * 1e3},
     }
+    if gate_separate_ms is not None:
+        result["config"]["ms_per_step_gate_as_separate_launch"] = gate_separate_ms
     if not args.no_cpu_baseline:
         import numpy as np
 
@@ -379,6 +395,8 @@ def bench_prefill(args, wl):
             c0 = time.perf_counter()
             ref = oracle.attn_batch_ref(qh, kh, vh, int(wl.dtype), ms, max_seq, H, Hkv, D, qs, 1.0 / D ** 0.5,
                                         threads=threads)
+            if wl.gated:
+                ref = oracle.sigmoid_mul(qgate[wl.m - ms:].cpu().numpy().reshape(-1), ref.reshape(-1), D, 2 * D, D).reshape(ms, H, D)
             spent += time.perf_counter() - c0
             reps += 1
         err = float(np.abs(o[wl.m - ms:].cpu().numpy() - ref).max())

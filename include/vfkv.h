@@ -366,7 +366,12 @@ int vfkv_decode_attention_gated(vfkv_cache* c, uint32_t layer, uint32_t kv_layer
                                 const vfkv_gate* gate, vfkv_workspace* ws, vfkv_stream stream);
 
 /* b_step_attention followed by b_step_attn_gated_output (executor/attention.rs:2192-2219,
- * 2405-2444): vfkv_prefill_attention, then the gate on the m * n_heads * head_dim outputs. */
+ * 2405-2444): vfkv_prefill_attention with the gate on the m * n_heads * head_dim outputs.  The
+ * FP8 / F16 matrix-core kernel applies the gate in its own store when gate->chunk is a multiple of
+ * head_dim, chunk / stride / gate_offset are multiples of 4 and gate->gate is 16-byte aligned (the
+ * reference's [Q | G] per (token, head) layout qualifies); otherwise a vfkv_sigmoid_mul launch
+ * follows on the same stream.  Results are bit-identical to the separate calls either way.
+ * `gate->gate` must not overlap `o`. */
 int vfkv_prefill_attention_gated(vfkv_cache* c, uint32_t layer, uint32_t kv_layer, uint32_t n_heads,
                                  const float* q, float* o, uint32_t m, uint32_t base_pos, uint32_t window,
                                  float scale, float softcap, const vfkv_gate* gate, vfkv_stream stream);

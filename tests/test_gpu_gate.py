@@ -113,7 +113,14 @@ def test_decode_attention_gated_is_attention_then_gate(dtype, heads, hkv, d, n, 
         c.destroy()
 
 
-@pytest.mark.parametrize("dtype,heads,hkv,d,m,base", ((vf.KvDtype.F8, 16, 4, 128, 70, 300), (vf.KvDtype.F16, 8, 2, 256, 33, 0)))
+@pytest.mark.parametrize("dtype,heads,hkv,d,m,base", (
+    (vf.KvDtype.F8, 16, 4, 128, 70, 300), (vf.KvDtype.F16, 8, 2, 256, 33, 0),
+    (vf.KvDtype.F8, 12, 4, 128, 17, 40),        # odd group: a padded head slot stores nothing
+    (vf.KvDtype.F8, 8, 2, 512, 21, 100),        # two wavefronts share a head, each gates its own output columns
+    (vf.KvDtype.F16, 4, 4, 64, 1, 0),
+    (vf.KvDtype.F32, 4, 2, 128, 20, 10),        # kernels without a gated store: the gate follows as its own launch
+    (vf.KvDtype.F8, 6, 2, 96, 20, 10),
+))
 def test_prefill_attention_gated_is_attention_then_gate(dtype, heads, hkv, d, m, base):
     r = rng(m + d)
     n = base + m
@@ -135,6 +142,34 @@ def test_prefill_attention_gated_is_attention_then_gate(dtype, heads, hkv, d, m,
                                 hkv, d, base, float(1.0 / np.sqrt(d)))
     ref = oracle.sigmoid_mul(qg.reshape(-1), ref.reshape(-1), d, 2 * d, d).reshape(m, heads, d)
     assert np.abs(to_np(a) - ref).max() < TOL[dtype]
+    cache.destroy()
+
+
+@pytest.mark.parametrize("layout", ("token_chunks", "token_chunks_interleaved", "half_head_chunks", "unaligned_gate"))
+def test_prefill_attention_gated_gate_layouts(layout):
+    # gate geometries that do and do not qualify for the attention kernel's own gated store give the same bits
+    dtype, heads, hkv, d, m, base = vf.KvDtype.F8, 8, 2, 128, 40, 200
+    r = rng(len(layout))
+    n = base + m
+    cache = vf.KvCache(vf.KvCacheConfig(1, hkv, d, n, dtype=dtype))
+    fwd = vf.Forward(cache, heads)
+    fwd.b_step_kv_write(0, 0, n, to_dev(fp16_normal(r, (n, hkv, d))), to_dev(fp16_normal(r, (n, hkv, d))))
+    q = to_dev(r.standard_normal((m, heads, d)).astype(np.float32))
+    row = heads * d
+    chunk, stride, off = {"token_chunks": (row, row, 0), "token_chunks_interleaved": (row, 2 * row, row),
+                          "half_head_chunks": (d // 2, d, d // 2), "unaligned_gate": (row, row, 0)}[layout]
+    n_gate = (m * row // chunk) * stride + off + chunk
+    gbuf = to_dev(r.standard_normal(n_gate + 1).astype(np.float32) * 3)
+    gate = gbuf[1:] if layout == "unaligned_gate" else gbuf[:-1]
+    a, b = torch.empty((m, heads, d), device=DEV), torch.empty((m, heads, d), device=DEV)
+    fwd.b_step_attention_gated(0, base, m, q, a, gate, chunk, stride, off)
+    fwd.b_step_attention(0, base, m, q, b)
+    torch.cuda.synchronize()
+    plain = to_np(b).reshape(-1)
+    fwd.run_sigmoid_mul(gate, b, m * row, chunk, stride, off)
+    torch.cuda.synchronize()
+    assert (to_np(a) == to_np(b)).all()
+    assert close_to_oracle(to_np(a).reshape(-1), oracle.sigmoid_mul(to_np(gate), plain, chunk, stride, off))
     cache.destroy()
 
 

@@ -627,7 +627,8 @@ int vfkv_kv_write_decode_attention(vfkv_cache* c, uint32_t layer, uint32_t n_hea
 
 // ---- prefill attention -------------------------------------------------------------------------------
 static int flash_attn_batch_impl(const float* q, const void* k_layer, const void* v_layer, uint32_t kv_dtype, float* o,
-                                 const vfkv_batch_params* p, float softcap, vfkv_workspace* ws, vfkv_stream stream) {
+                                 const vfkv_batch_params* p, float softcap, vfkv_workspace* ws, vfkv_stream stream,
+                                 const vfkv::GateArgs* gate = nullptr) {
     if (!p) return fail(VFKV_ERR_INVALID_ARG, "flash_attn_batch: params is NULL");
     if (!q || !k_layer || !v_layer || !o) return fail(VFKV_ERR_INVALID_ARG, "flash_attn_batch: NULL buffer");
     if (kv_dtype > VFKV_F8E4M3) return fail(VFKV_ERR_INVALID_ARG, "flash_attn_batch: unknown kv dtype %u", kv_dtype);
@@ -640,7 +641,11 @@ static int flash_attn_batch_impl(const float* q, const void* k_layer, const void
     const uint64_t vis0 = first_len < p->n_kv ? first_len : p->n_kv;
     if (p->kv_start >= vis0)
         return fail(VFKV_ERR_INVALID_ARG, "flash_attn_batch: kv_start %u leaves query 0 without a visible key", p->kv_start);
+    if (gate && (uint64_t)p->m * p->n_heads * p->head_dim > 0xFFFFFFFFull)
+        return fail(VFKV_ERR_OVERFLOW, "prefill_attention_gated: %llu output elements",
+                    (unsigned long long)p->m * p->n_heads * p->head_dim);
     vfkv::BatchLaunch L;
+    L.gate = gate;
     L.q = q; L.k = k_layer; L.v = v_layer; L.o = o;
     L.dtype = kv_dtype; L.n_heads = p->n_heads; L.n_kv_heads = p->n_kv_heads; L.head_dim = p->head_dim;
     L.m = p->m; L.n_kv = p->n_kv; L.q_start = p->q_start; L.kv_start = p->kv_start;
@@ -661,7 +666,7 @@ int vfkv_flash_attn_batch(const float* q, const void* k_layer, const void* v_lay
 
 static int prefill_attention_impl(vfkv_cache* c, uint32_t layer, uint32_t kv_layer, uint32_t n_heads, const float* q, float* o,
                                   uint32_t m, uint32_t base_pos, uint32_t window, float scale, float softcap,
-                                  vfkv_workspace* ws, vfkv_stream stream) {
+                                  vfkv_workspace* ws, vfkv_stream stream, const vfkv::GateArgs* gate = nullptr) {
     if (!c || !c->k || !c->v) return fail(VFKV_ERR_INVALID_ARG, "prefill_attention: cache has no buffers");
     if (layer >= c->n_layers || kv_layer >= c->n_layers)
         return fail(VFKV_ERR_INVALID_ARG, "prefill_attention: layer %u / kv_layer %u out of range", layer, kv_layer);
@@ -678,7 +683,7 @@ static int prefill_attention_impl(vfkv_cache* c, uint32_t layer, uint32_t kv_lay
     p.scale = scale;
     p.kv_start = vfkv_kv_start_batch(base_pos, m, window);
     const uint64_t off = layer_off(c, kv_layer);
-    return flash_attn_batch_impl(q, (char*)c->k + off, (char*)c->v + off, c->dtype, o, &p, softcap, ws, stream);
+    return flash_attn_batch_impl(q, (char*)c->k + off, (char*)c->v + off, c->dtype, o, &p, softcap, ws, stream, gate);
 }
 
 int vfkv_prefill_attention(vfkv_cache* c, uint32_t layer, uint32_t kv_layer, uint32_t n_heads, const float* q, float* o,
@@ -737,12 +742,7 @@ int vfkv_prefill_attention_gated(vfkv_cache* c, uint32_t layer, uint32_t kv_laye
     vfkv::GateArgs g;
     int rc = check_gate(gate, "prefill_attention_gated", &g);
     if (rc != VFKV_OK) return rc;
-    rc = vfkv_prefill_attention(c, layer, kv_layer, n_heads, q, o, m, base_pos, window, scale, softcap, stream);
-    if (rc != VFKV_OK || m == 0u) return rc;
-    const uint64_t ne = (uint64_t)m * n_heads * hd_for(c, layer);
-    if (ne > 0xFFFFFFFFull) return fail(VFKV_ERR_OVERFLOW, "prefill_attention_gated: %llu output elements", (unsigned long long)ne);
-    VFKV_HIP(vfkv::launch_sigmoid_mul(o, (uint32_t)ne, g, S(stream)));
-    return VFKV_OK;
+    return prefill_attention_impl(c, layer, kv_layer, n_heads, q, o, m, base_pos, window, scale, softcap, nullptr, stream, &g);
 }
 
 }  // extern "C"

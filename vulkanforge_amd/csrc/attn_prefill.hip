@@ -25,6 +25,11 @@ struct BatchArgs {
     float* sm;
     float* ss;
     uint32_t nk, chunk;
+    // gated output (f16 matrix-core kernel only, and only when it stores final values): o *= sigmoid(gate[...]) in the
+    // kernel's own store; gate == NULL: off.  The launcher guarantees gchunk % head_dim == 0, gchunk, gstride and goff
+    // multiples of 4, a 16-byte aligned gate and fewer than 2^32 output elements.
+    const float* gate;
+    uint32_t gchunk, gstride, goff;
 };
 
 }  // namespace vfkv
@@ -93,15 +98,16 @@ __global__ __launch_bounds__(kWave) void batch_generic_kernel(BatchArgs a) {
     }
 }
 
-hipError_t launch_batch(const BatchLaunch& L, hipStream_t stream) {
-    if (L.dtype > kF8 || L.head_dim == 0u || L.head_dim > 512u) return hipErrorInvalidValue;
-    if (L.m == 0u) return hipSuccess;
+// Launches the attention kernel(s) for L.  *gate_applied tells whether L.gate went into their stores.
+static hipError_t launch_batch_kernels(const BatchLaunch& L, hipStream_t stream, bool* gate_applied) {
+    *gate_applied = false;
     BatchArgs a;
     a.q = L.q; a.k = (const uint8_t*)L.k; a.v = (const uint8_t*)L.v; a.o = L.o;
     a.n_heads = L.n_heads; a.n_kv_heads = L.n_kv_heads; a.head_dim = L.head_dim;
     a.m = L.m; a.n_kv = L.n_kv; a.q_start = L.q_start; a.kv_start = L.kv_start;
     a.scale = L.scale; a.softcap = L.softcap; a.dtype = L.dtype;
     a.so = nullptr; a.sm = nullptr; a.ss = nullptr; a.nk = 1u; a.chunk = 0u;
+    a.gate = nullptr; a.gchunk = 1u; a.gstride = 0u; a.goff = 0u;
     const uint32_t g = L.n_heads / L.n_kv_heads;
     const uint64_t slab_bytes = (uint64_t)L.n_kv * L.n_kv_heads * L.head_dim * elem_size(L.dtype);
     const bool aligned = ((((uintptr_t)L.k) | ((uintptr_t)L.v) | ((uintptr_t)L.q) | ((uintptr_t)L.o)) & 15u) == 0u;
@@ -178,6 +184,12 @@ hipError_t launch_batch(const BatchLaunch& L, hipStream_t stream) {
                     a.chunk = ((span + nk - 1u) / nk + 31u) / 32u * 32u;
                 }
             }
+            // the gate goes into the kernel's store when a lane's four output elements share a chunk and a 16-byte gate
+            // load, and a head's elements share a chunk; with key chunks the merge applies it instead
+            const bool gate_in_store = L.gate != nullptr && nk == 1u && L.gate->chunk % L.head_dim == 0u &&
+                                       ((L.gate->chunk | L.gate->stride | L.gate->gate_offset) % 4u) == 0u &&
+                                       (((uintptr_t)L.gate->gate) & 15u) == 0u;
+            if (gate_in_store) { a.gate = L.gate->gate; a.gchunk = L.gate->chunk; a.gstride = L.gate->stride; a.goff = L.gate->gate_offset; }
             const dim3 grid((L.m + 15u) / 16u, L.n_kv_heads, nz * nk), block(nwaves * kWave);
             const size_t vbytes = (size_t)nwaves * 32 * (dv + 16) * sizeof(_Float16) +
                                   (size_t)2 * (hp / nh) * ncb * 16 * (L.head_dim + 8) * sizeof(_Float16);
@@ -209,10 +221,12 @@ hipError_t launch_batch(const BatchLaunch& L, hipStream_t stream) {
             if (launched) {
                 hipError_t e = hipGetLastError();
                 if (e == hipSuccess && nk > 1u)
-                    e = launch_reduce(a.so, a.sm, a.ss, L.o, L.m * L.n_heads, L.head_dim, nk, stream);
+                    e = launch_reduce(a.so, a.sm, a.ss, L.o, L.m * L.n_heads, L.head_dim, nk, stream, L.gate, gate_applied);
+                else
+                    *gate_applied = gate_in_store;
                 return e;
             }
-            a.so = nullptr; a.nk = 1u;
+            a.so = nullptr; a.nk = 1u; a.gate = nullptr;
         }
     }
     // f32 matrix-core kernel: F32 caches, and the head sizes the f16 kernels above do not cover
@@ -231,6 +245,17 @@ hipError_t launch_batch(const BatchLaunch& L, hipStream_t stream) {
     }
     hipLaunchKernelGGL(batch_generic_kernel, dim3(L.n_heads, L.m), dim3(kWave), 0, stream, a);
     return hipGetLastError();
+}
+
+hipError_t launch_batch(const BatchLaunch& L, hipStream_t stream) {
+    if (L.dtype > kF8 || L.head_dim == 0u || L.head_dim > 512u) return hipErrorInvalidValue;
+    if (L.m == 0u) return hipSuccess;
+    const uint64_t ne = (uint64_t)L.m * L.n_heads * L.head_dim;
+    if (L.gate != nullptr && (L.gate->gate == nullptr || L.gate->chunk == 0u || ne > 0xFFFFFFFFull)) return hipErrorInvalidValue;
+    bool gate_applied = false;
+    hipError_t e = launch_batch_kernels(L, stream, &gate_applied);
+    if (e == hipSuccess && L.gate != nullptr && !gate_applied) e = launch_sigmoid_mul(L.o, (uint32_t)ne, *L.gate, stream);
+    return e;
 }
 
 }  // namespace vfkv

@@ -358,6 +358,25 @@ __global__ __launch_bounds__((NCB == 1 && D <= 128) ? VFKV_PREFILL_NCB1_WAVES * 
 #pragma unroll
     for (int cb = 0; cb < NCB; ++cb) l_run[cb] = xor32_sum(xor16_sum(l_run[cb]));   // every lane of a query column has its wavefront's sum
 
+    // ---- gated output (vk_shaders/sigmoid_mul.comp:44-52 in this kernel's store): the wavefronts that will store request
+    // their gate values and turn them into factors before the merge, so that the round trip overlaps it.  A head's D
+    // elements lie in one gate chunk.
+    float4_t gfac[NCB][DTILES];
+    if (a.gate != nullptr && sp == 0 && q_ok) {
+#pragma unroll
+        for (int cb = 0; cb < NCB; ++cb) {
+            if (gz + g0 + cb >= G) continue;
+            const uint32_t i0 = (qi * a.n_heads + kvh * G + gz + g0 + cb) * D;
+            const uint32_t token = i0 / a.gchunk;
+            const float* gp = a.gate + (size_t)token * a.gstride + a.goff + (i0 - token * a.gchunk) + dslice * DV + kg * 4;
+#pragma unroll
+            for (int dt = 0; dt < DTILES; ++dt) {
+                const float4 gv = *reinterpret_cast<const float4*>(gp + dt * 16);
+                gfac[cb][dt] = float4_t{sigmoid_gate(1.0f, gv.x), sigmoid_gate(1.0f, gv.y), sigmoid_gate(1.0f, gv.z), sigmoid_gate(1.0f, gv.w)};
+            }
+        }
+    }
+
     // ---- merge the key splits through LDS (split 0 collects), normalise and store ----
     constexpr int REC = DTILES * 4 + 2;
     if (NS > 1) {
@@ -417,6 +436,14 @@ __global__ __launch_bounds__((NCB == 1 && D <= 128) ? VFKV_PREFILL_NCB1_WAVES * 
             }
             const float inv = 1.0f / l_run[cb];
             float* op = a.o + ((size_t)qi * a.n_heads + h) * D + dslice * DV + kg * 4;   // lane (query n16) holds d = dslice*DV + dt*16 + kg*4 + i
+            if (a.gate != nullptr) {
+#pragma unroll
+                for (int dt = 0; dt < DTILES; ++dt) {
+                    const float4_t r = oacc[cb][dt] * inv * gfac[cb][dt];
+                    *reinterpret_cast<float4*>(op + dt * 16) = make_float4(r[0], r[1], r[2], r[3]);
+                }
+                continue;
+            }
 #pragma unroll
             for (int dt = 0; dt < DTILES; ++dt) {
                 const float4_t r = oacc[cb][dt] * inv;

@@ -95,6 +95,9 @@ struct BatchLaunch {
     float* scratch_max = nullptr;
     float* scratch_sum = nullptr;
     uint64_t scratch_out_floats = 0, scratch_ml_floats = 0;
+    // optional gated output: o *= sigmoid(gate[...]), in the attention kernel's or the merge's own store where the shape
+    // allows it and as a follow-up launch otherwise
+    const GateArgs* gate = nullptr;
 };
 hipError_t launch_batch(const BatchLaunch& a, hipStream_t stream);
 

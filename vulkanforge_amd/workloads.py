@@ -48,6 +48,7 @@ class PrefillWorkload:
     m: int
     dtype: KvDtype
     workspace: bool = False   # attention through vfkv_prefill_attention_ws (key chunks over workgroups)
+    gated: bool = False       # the output is multiplied by sigmoid(gate), per (token, head) the gate follows Q (Qwen3.6)
 
     def pairs_per_head(self) -> int:
         return sum(self.base_pos + i + 1 for i in range(self.m))
@@ -76,6 +77,9 @@ DECODE = {
 PREFILL = {
     "prefill_fp8_512x4608_32layers": PrefillWorkload("prefill_fp8_512x4608_32layers", 32, 32, 8, 128, 4096, 512,
                                                      KvDtype.F8),
+    # the same with the gated output of the Qwen3.6 full-attention layers (not a reference configuration)
+    "prefill_fp8_512x4608_32layers_gated": PrefillWorkload("prefill_fp8_512x4608_32layers_gated", 32, 32, 8, 128, 4096,
+                                                           512, KvDtype.F8, gated=True),
     # Gemma-style geometry (16 query heads, 8 KV heads, head_dim 256): not a reference configuration
     "prefill_f16_hd256_512x4608_12layers": PrefillWorkload("prefill_f16_hd256_512x4608_12layers", 12, 16, 8, 256, 4096,
                                                            512, KvDtype.F16),

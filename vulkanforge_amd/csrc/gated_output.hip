@@ -3,8 +3,9 @@
 // Replaces the reference's `run_sigmoid_mul` dispatch (forward/runs.rs:2649-2681, vk_shaders/sigmoid_mul.comp:40-53) as
 // `step_attn_gated_output` / `b_step_attn_gated_output` issue it (executor/attention.rs:632-680, 2405-2444).  HBM bound:
 // 8 bytes read and 4 written per element.  Four consecutive elements per lane as 16-byte accesses when the chunk
-// geometry and the pointers allow it, one element per lane otherwise.  The decode merge applies the same gate in its
-// own store (attn_decode.hip), so a decode step only comes here when its span fits one tile.
+// geometry and the pointers allow it, one element per lane otherwise.  The decode merge (attn_decode.hip) and the f16
+// matrix-core prefill kernel (attn_prefill_mfma2.h) apply the same gate in their own stores, so a decode step only comes
+// here when its span fits one tile and a prefill chunk only for gate geometries or kernels without that store.
 #include "device_utils.h"
 #include "kernels.h"
 

@@ -200,10 +200,13 @@ def bench_decode(args, wl):
         for layer in range(L):
             span = wl.context - starts[layer]
             tile = lib.vfkv_decode_tile_for(span, H, Hkv, D, int(wl.dtype))
-            klay = cache.k_ptr + cache.layer_offset_bytes(layer)
-            vlay = cache.v_ptr + cache.layer_offset_bytes(layer)
-            fwd.run_flash_attn_split(q[layer], klay, vlay, wl.dtype, so, sm, ss, H, Hkv, D, wl.context, scale,
-                                     kv_start=starts[layer], tile=tile, softcap=wl.softcap, interleaved=True)
+            # the step's own launch starts at the tile that holds kv_start; the standalone split call numbers its tiles
+            # from row 0 (flash_attn_split.comp), so a windowed layer is handed the slab from that tile on
+            skip = starts[layer] // tile * tile
+            klay = cache.k_ptr + cache.layer_offset_bytes(layer) + skip * cache.row_bytes(layer)
+            vlay = cache.v_ptr + cache.layer_offset_bytes(layer) + skip * cache.row_bytes(layer)
+            fwd.run_flash_attn_split(q[layer], klay, vlay, wl.dtype, so, sm, ss, H, Hkv, D, wl.context - skip, scale,
+                                     kv_start=starts[layer] - skip, tile=tile, softcap=wl.softcap, interleaved=True)
 
     run_split = split_only
     if not args.no_graph:

@@ -45,6 +45,11 @@ __global__ __launch_bounds__(NW * 64) void split_mfma_kernel(SplitArgs a, uint32
     constexpr int DTILES = DV / 16;
     constexpr int SEG = D / 4, SEGB = SEG * ES;  // a lane group's quarter of a K row
     constexpr int KLD = SEGB / 16;               // 16-byte loads per lane per K row
+    // Wide rows (a lane's quarter row would be a whole 128-byte line, read by 8 loads that other traffic can evict the line
+    // between): the four lane groups read consecutive 16-byte pieces instead, piece x of group kg at byte (x * 4 + kg) * 16,
+    // so a load instruction covers 64 contiguous bytes of each row and a line is done after two.  The query operand is
+    // permuted the same way.
+    constexpr bool KIL = SEGB >= 128;
     constexpr int VPITCH = DV + 16;              // halves per V row in LDS (+32 B against bank conflicts)
     constexpr int VCHUNK_ROW = DV * ES / 16;     // 16-byte chunks per V row (this wavefront's columns)
     constexpr int VLD = RUN * VCHUNK_ROW / 64;   // V loads per lane per run
@@ -82,7 +87,7 @@ __global__ __launch_bounds__(NW * 64) void split_mfma_kernel(SplitArgs a, uint32
     const __amdgpu_buffer_rsrc_t krsrc = __builtin_amdgcn_make_buffer_rsrc((void*)a.k, 0, a.seq_len * row_stride, 0x00020000);
     const __amdgpu_buffer_rsrc_t vrsrc = __builtin_amdgcn_make_buffer_rsrc((void*)a.v, 0, a.seq_len * row_stride, 0x00020000);
     const uint32_t head_b = kvh * D * ES;
-    const uint32_t lane_koff = n16 * row_stride + head_b + kg * SEGB;
+    const uint32_t lane_koff = n16 * row_stride + head_b + kg * (KIL ? 16 : SEGB);
     const int vrow = lane / VCHUNK_ROW, vcol = lane % VCHUNK_ROW;
     const uint32_t lane_voff = vrow * row_stride + head_b + ds * DV * ES + vcol * 16;
     const float scale_l2 = a.scale * 1.44269504088896f;
@@ -100,7 +105,7 @@ __global__ __launch_bounds__(NW * 64) void split_mfma_kernel(SplitArgs a, uint32
     auto issue_k = [&](int b, int t, uint32_t off) {
 #pragma unroll
         for (int x = 0; x < KLD; ++x)
-            kraw[b][t][x] = __builtin_amdgcn_raw_buffer_load_b128(krsrc, lane_koff + x * 16, off + (uint32_t)(t * 16) * row_stride, 0);
+            kraw[b][t][x] = __builtin_amdgcn_raw_buffer_load_b128(krsrc, lane_koff + x * (KIL ? 64 : 16), off + (uint32_t)(t * 16) * row_stride, 0);
     };
     auto issue_v = [&](int b, int c, uint32_t off) {
         vraw[b][c] = __builtin_amdgcn_raw_buffer_load_b128(vrsrc, lane_voff, off + (uint32_t)(c * VROWS) * row_stride, 0);
@@ -202,7 +207,9 @@ __global__ __launch_bounds__(NW * 64) void split_mfma_kernel(SplitArgs a, uint32
         const bool col_ok = (uint32_t)col < gcount;
 #pragma unroll
         for (int c = 0; c < KS; ++c) {
-            const u32x4 raw = *reinterpret_cast<const u32x4*>(&qlds[col_ok ? n16 : 0][kg * SEG + c * 8]);
+            // first query element of k-step c in this lane group (16-byte pieces hold 8 halves or 16 FP8 values = two k-steps)
+            const int qe = !KIL ? kg * SEG + c * 8 : ES == 2 ? (c * 4 + kg) * 8 : ((c / 2) * 4 + kg) * 16 + (c % 2) * 8;
+            const u32x4 raw = *reinterpret_cast<const u32x4*>(&qlds[col_ok ? n16 : 0][qe]);
             qb[c] = __builtin_bit_cast(half8_t, col_ok ? raw : u32x4{0u, 0u, 0u, 0u});
         }
     }

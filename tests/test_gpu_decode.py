@@ -187,6 +187,29 @@ def test_tile_invariance_and_linearity_full_size_fp8():
     assert np.abs(to_np(o512) - ref).max() < TIGHT
 
 
+@pytest.mark.parametrize("n_tiles", (1, 2, 33, 64, 65, 127, 128, 129, 200, 256, 257, 700))
+@pytest.mark.parametrize("heads,d", ((6, 64), (8, 256), (3, 512), (5, 80)))
+def test_reduce_alone_matches_oracle_for_every_tile_count(n_tiles, heads, d):
+    # flash_attn_reduce.comp on synthetic partials: every merge kernel (one wavefront up to 64 tiles, four up to 256,
+    # the looping ones beyond and for head sizes that are no multiple of 64), with empty tiles mixed in
+    r = rng(n_tiles * 1000 + d)
+    so = r.standard_normal((heads, n_tiles, d)).astype(np.float32)
+    sm = (r.standard_normal((heads, n_tiles)) * 6).astype(np.float32)
+    ss = (r.random((heads, n_tiles)) * 50 + 0.5).astype(np.float32)
+    empty = r.random((heads, n_tiles)) < 0.2
+    empty[:, r.integers(0, n_tiles)] = False                 # every head keeps a live tile
+    if n_tiles > 130:
+        empty[0, 64:128] = True                              # a whole wavefront's share of tiles without keys
+    so[empty] = 0.0
+    sm[empty] = -1e30
+    ss[empty] = 0.0
+    o = torch.full((heads, d), float("nan"), device=DEV)
+    vf.Forward.run_flash_attn_reduce(to_dev(so), to_dev(sm), to_dev(ss), o, heads, d, n_tiles)
+    torch.cuda.synchronize()
+    ref = oracle.attn_reduce(so, sm, ss)
+    assert np.abs(to_np(o) - ref).max() < 2e-6 * max(1.0, np.abs(ref).max())
+
+
 def _cache_with_history(dtype, n_layers, hkv, d, max_seq, fill, seed, hd=None, kvh=None):
     cfg = vf.KvCacheConfig(n_layers, hkv, d, max_seq, hd, kvh, dtype)
     cache = vf.KvCache(cfg)
@@ -257,6 +280,8 @@ def test_config2_fp8_outliers_append_then_decode_two_layers():
     (vf.KvDtype.F16, 8, 8, 64, 64, 0),          # the new row opens a tile of its own
     (vf.KvDtype.F8, 24, 2, 128, 500, 0),        # GQA group of 12: two head slices, separate append launch
     (vf.KvDtype.F32, 8, 2, 128, 300, 0),        # 4-byte cache: separate append launch
+    (vf.KvDtype.F16, 8, 1, 256, 16000, 0),      # one KV head: 250 tiles, merged by four wavefronts per 64 outputs
+    (vf.KvDtype.F8, 16, 2, 512, 9000, 0),       # Gemma-4 full-attention geometry: 2 KV heads, 128 tiles
 ])
 def test_kv_write_attention_in_one_call_matches_the_two_calls(dtype, heads, hkv, d, ctx, window):
     # step_kv_write + step_attention (executor/attention.rs:546-625) through the single entry point: cache bytes and

@@ -71,6 +71,7 @@ DECODE_CASES = (
     (vf.KvDtype.F8, 16, 4, 128, 100, 0, True),         # one tile: the worker writes o, the gate runs as its own launch
     (vf.KvDtype.F32, 8, 2, 64, 700, 0, True),          # vector-ALU worker, separate append
     (vf.KvDtype.F8, 6, 2, 80, 300, 0, False),          # generic kernels: the merge cannot take the gate
+    (vf.KvDtype.F16, 8, 1, 256, 12000, 0, True),       # one KV head, 188 tiles: the four-wavefront merge applies the gate
 )
 
 

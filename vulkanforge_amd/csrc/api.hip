@@ -543,9 +543,12 @@ uint32_t vfkv_decode_tile_for(uint32_t span, uint32_t n_heads, uint32_t n_kv_hea
     const bool mfma = (kv_dtype == VFKV_F8E4M3 || kv_dtype == VFKV_F16) &&
                       (head_dim == 64u || head_dim == 128u || head_dim == 256u || head_dim == 512u);
     if (mfma) {
-        // short spans: one tile, so the worker writes the output itself and no merge launch follows
+        // short spans: one tile, so the worker writes the output itself and no merge launch follows.  The tile's runs of 32
+        // keys are walked by the workgroup's four run streams (two at head_dim 512) one after the other, and a further round
+        // costs more than the merge launch saves: up to two rounds (one at head_dim 512: 8 / 1 / 512 F16 over 256 keys took
+        // 22.7 us in one tile against 13.6 us in four).
         static const bool forced = getenv("VFKV_DECODE_TILE") != nullptr;
-        if (span <= 256u && !forced) return 256u;
+        if (span <= (head_dim == 512u ? 64u : 256u) && !forced) return 256u;
         return choose_tile(span, n_kv_heads, (g + 7u) / 8u, 256u);
     }
     const uint32_t groups = (g % 4u == 0u) ? g / 4u : (g % 2u == 0u) ? g / 2u : g;

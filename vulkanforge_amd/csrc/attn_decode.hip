@@ -570,10 +570,11 @@ __global__ __launch_bounds__(kWave) void reduce_direct_kernel(const float* __res
     o[(size_t)h * D + d] = GATED ? sigmoid_gate(r, gv) : r;
 }
 
-// 65 to 256 tiles (few KV heads over long contexts: one tile per compute unit then means many per head): the same scheme
-// with four wavefronts per (head, 64 output dimensions).  Wavefront w merges tiles [64 w, 64 w + 64) into a partial (maximum,
-// sum, 64 outputs) exactly as above, the four partials are combined through LDS.  One memory round trip like the kernel
-// above, where the generic kernel below walks the tiles of a head in a loop of one workgroup.
+// 65 to 2 048 tiles (few KV heads over long contexts: one tile per compute unit then means many per head; the reference's
+// 64-key tiles at long contexts): the same scheme with four wavefronts per (head, 64 output dimensions).  Wavefront w
+// merges tiles [64 w, 64 w + 64) into a partial (maximum, sum, 64 outputs) exactly as above, then the tiles 256 further
+// on into another that it folds into the first, and so on; the four partials are combined through LDS.  One memory
+// round trip per 256 tiles, where the generic kernel below walks the tiles of a head in a loop of one workgroup.
 template <bool GATED>
 __global__ __launch_bounds__(4 * kWave) void reduce_direct4_kernel(const float* __restrict__ so, const float* __restrict__ sm,
                                                                   const float* __restrict__ ss, float* __restrict__ o,
@@ -582,28 +583,35 @@ __global__ __launch_bounds__(4 * kWave) void reduce_direct4_kernel(const float* 
     __shared__ float pm[4], pl[4];
     const uint32_t h = blockIdx.y, lane = threadIdx.x & (kWave - 1), w = threadIdx.x >> 6;
     const uint32_t d = blockIdx.x * kWave + lane;
-    const uint32_t base = w * kWave;
-    const uint32_t cnt = n_tiles > base ? (n_tiles - base < (uint32_t)kWave ? n_tiles - base : (uint32_t)kWave) : 0u;   // wavefront-uniform
-    const float* ho = so + ((size_t)h * n_tiles + (cnt ? base : 0u)) * D + d;
-    float x[kWave];
-#pragma unroll
-    for (int j = 0; j < kWave; ++j) x[j] = ho[(size_t)((uint32_t)j < cnt ? j : 0) * D];
-    const float mj = lane < cnt ? sm[(size_t)h * n_tiles + base + lane] : kMasked;
-    const float sj = lane < cnt ? ss[(size_t)h * n_tiles + base + lane] : 0.f;
     float gv = 0.f;
     if (GATED && w == 0u) {
         const uint32_t i = h * D + d, token = i / gate.chunk;
         gv = gate.gate[(uint64_t)token * gate.stride + gate.gate_offset + (i - token * gate.chunk)];
     }
-    const float M = wave_max_uniform(mj);
-    const float wj = lane < cnt ? __expf(mj - M) : 0.f;
-    const float L = wave_sum_uniform(wj * sj);
-    float acc = 0.f;
+    float Mr = kMasked, Lr = 0.f, ar = 0.f;                       // this wavefront's partial so far
+    for (uint32_t base = w * kWave; base < n_tiles; base += 4u * kWave) {   // wavefront-uniform
+        const uint32_t cnt = n_tiles - base < (uint32_t)kWave ? n_tiles - base : (uint32_t)kWave;
+        const float* ho = so + ((size_t)h * n_tiles + base) * D + d;
+        float x[kWave];
 #pragma unroll
-    for (int j = 0; j < kWave; ++j)
-        acc = fmaf(__builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, wj), j)), x[j], acc);
-    pacc[w][lane] = acc;
-    if (lane == 0u) { pm[w] = M; pl[w] = L; }
+        for (int j = 0; j < kWave; ++j) x[j] = ho[(size_t)((uint32_t)j < cnt ? j : 0) * D];
+        const float mj = lane < cnt ? sm[(size_t)h * n_tiles + base + lane] : kMasked;
+        const float sj = lane < cnt ? ss[(size_t)h * n_tiles + base + lane] : 0.f;
+        const float M = wave_max_uniform(mj);
+        const float wj = lane < cnt ? __expf(mj - M) : 0.f;
+        const float L = wave_sum_uniform(wj * sj);
+        float acc = 0.f;
+#pragma unroll
+        for (int j = 0; j < kWave; ++j)
+            acc = fmaf(__builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, wj), j)), x[j], acc);
+        const float Mn = fmaxf(Mr, M);
+        const float fr = __expf(Mr - Mn), fc = __expf(M - Mn);   // first round: fr scales zeros
+        ar = ar * fr + acc * fc;
+        Lr = Lr * fr + L * fc;
+        Mr = Mn;
+    }
+    pacc[w][lane] = ar;
+    if (lane == 0u) { pm[w] = Mr; pl[w] = Lr; }
     __syncthreads();
     if (w != 0u) return;
     const float Mt = fmaxf(fmaxf(pm[0], pm[1]), fmaxf(pm[2], pm[3]));
@@ -803,7 +811,7 @@ hipError_t launch_reduce(const float* so, const float* sm, const float* ss, floa
             if (n_tiles <= 32u) hipLaunchKernelGGL((reduce_direct_kernel<32, false>), grid, dim3(kWave), 0, stream, so, sm, ss, o, D, n_tiles, g);
             else hipLaunchKernelGGL((reduce_direct_kernel<64, false>), grid, dim3(kWave), 0, stream, so, sm, ss, o, D, n_tiles, g);
         }
-    } else if (n_tiles <= 256u && D % (uint32_t)kWave == 0u) {
+    } else if (n_tiles <= 2048u && D % (uint32_t)kWave == 0u) {
         const dim3 grid(D / kWave, n_heads);
         const GateArgs g = gated ? *gate : GateArgs();
         if (gated) {

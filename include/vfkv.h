@@ -285,6 +285,23 @@ int vfkv_decode_attention(vfkv_cache* c, uint32_t layer, uint32_t kv_layer, uint
                           const float* q, float* o, uint32_t position, uint32_t kv_start, float scale,
                           float softcap, vfkv_workspace* ws, vfkv_stream stream);
 
+/* vfkv_decode_attention for callers that cannot allocate device memory or carry a workspace object:
+ * code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  It has no
+ * counterpart in the reference (whose scratch buffers are allocated once in forward/setup.rs:203-230).
+ * The partials live in a device array that is part of the loaded library (VFKV_STATIC_SCRATCH_BYTES
+ * per GPU, held until the process ends); the call makes no hipMalloc / hipFree and returns
+ * VFKV_ERR_WORKSPACE when n_heads * partials * (head_dim + 2) floats exceed that size (32 / 8 / 128 at
+ * any context needs 0.5 MiB; few KV heads at head_dim 512 need the most).  Same kernels, same tile
+ * choice and bit-identical output as vfkv_decode_attention.  Every call on one GPU shares that GPU's
+ * array: calls that overlap in time on one GPU (two streams, two threads) race; order them on one
+ * stream.  Nothing in the array needs clearing between calls (every partial a merge reads is written
+ * by the launch before it).  The array's address is looked up on the first call on each device,
+ * which should therefore happen outside stream capture. */
+#define VFKV_STATIC_SCRATCH_BYTES (5u << 20)
+int vfkv_decode_attention_static(vfkv_cache* c, uint32_t layer, uint32_t kv_layer, uint32_t n_heads,
+                                 const float* q, float* o, uint32_t position, uint32_t kv_start,
+                                 float scale, float softcap, vfkv_stream stream);
+
 /* step_kv_write followed by step_attention for the same layer and token, as the executor issues them
  * back to back (executor/attention.rs:546-625): appends the token's K and V rows (f32,
  * kv_heads_for(layer) * head_dim_for(layer) elements each) at `position`, then attends over keys

@@ -32,6 +32,13 @@ def test_library_exports_every_declared_symbol():
     assert L.vfkv_status_string(0) == b"ok" and L.vfkv_status_string(-3) == b"misaligned offset"
 
 
+def test_rust_binding_text_declares_every_exported_symbol():
+    # the extern "C" block a Rust host would paste must not drift from the header
+    text = open(os.path.join(ROOT, "INTEGRATION.md")).read()
+    rust = sorted(set(re.findall(r"pub fn (vfkv_[a-z0-9_]+)\s*\(", text)))
+    assert rust == _declared_symbols()
+
+
 def test_param_structs_are_32_bytes():
     # pipeline.rs:569 and :611
     assert C.sizeof(_ffi.SplitParams) == 32 and C.sizeof(_ffi.BatchParams) == 32
@@ -285,3 +292,28 @@ def test_prefill_attention_ws_rejects_bad_arguments_before_any_device_work():
     assert L.vfkv_prefill_attention_ws(None, 0, 0, 4, 64, 64, 1, 0, 0, 1.0, 0.0, None, None) == -1      # no workspace
     assert b"workspace" in L.vfkv_last_error()
     assert L.vfkv_prefill_attention_ws(None, 0, 0, 4, 64, 64, 1, 0, 0, 1.0, 0.0, 64, None) == -1        # no cache
+
+
+def test_static_decode_call_rejects_partials_beyond_its_array():
+    # vfkv_decode_attention_static holds its partials in a fixed device array; a launch whose partials exceed it must
+    # fail with VFKV_ERR_WORKSPACE before any device work.  The library's own tile choice never needs more than the
+    # array holds, so the case is forced with 64-key tiles (VFKV_DECODE_TILE is read once per process: child process).
+    import subprocess
+    import sys
+    code = (
+        "import ctypes as C\n"
+        "from vulkanforge_amd import _ffi\n"
+        "L = _ffi.lib()\n"
+        "cfg = _ffi.CacheConfig(1, 8, 128, 65536, None, None, 2)\n"
+        "h = C.c_void_p()\n"
+        "assert L.vfkv_cache_create_external(C.byref(cfg), 0x1000, 0x2000, C.byref(h)) == 0\n"
+        "rc = L.vfkv_decode_attention_static(h, 0, 0, 32, 0x1000, 0x1000, 65535, 0, 1.0, 0.0, None)\n"
+        "msg = L.vfkv_last_error().decode()\n"
+        "assert rc == -7, (rc, msg)\n"
+        "assert 'static buffer holds 5242880' in msg, msg\n"
+        "rc = L.vfkv_decode_attention_static(h, 0, 0, 32, None, 0x1000, 10, 0, 1.0, 0.0, None)\n"
+        "assert rc == -1\n"
+        "print('ok')\n")
+    env = dict(os.environ, VFKV_DECODE_TILE="64", PYTHONPATH=ROOT)
+    out = subprocess.run([sys.executable, "-c", code], env=env, capture_output=True, text=True, timeout=300)
+    assert out.returncode == 0 and out.stdout.strip() == "ok", out.stderr

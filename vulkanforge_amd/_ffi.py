@@ -102,6 +102,7 @@ SIGNATURES = {
     "vfkv_kv_write_decode_attention": (C.c_int, [_vp, _u32, _u32, _vp, _vp, _vp, _vp, _u32, _u32, _f, _f, _vp, _vp]),
     "vfkv_decode_tile_for": (_u32, [_u32, _u32, _u32, _u32, _u32]),
     "vfkv_decode_attention": (C.c_int, [_vp, _u32, _u32, _u32, _vp, _vp, _u32, _u32, _f, _f, _vp, _vp]),
+    "vfkv_decode_attention_static": (C.c_int, [_vp, _u32, _u32, _u32, _vp, _vp, _u32, _u32, _f, _f, _vp]),
     "vfkv_flash_attn_batch": (C.c_int, [_vp, _vp, _vp, _u32, _vp, C.POINTER(BatchParams), _f, _vp]),
     "vfkv_prefill_attention": (C.c_int, [_vp, _u32, _u32, _u32, _vp, _vp, _u32, _u32, _u32, _f, _f, _vp]),
     "vfkv_prefill_attention_ws": (C.c_int, [_vp, _u32, _u32, _u32, _vp, _vp, _u32, _u32, _u32, _f, _f, _vp, _vp]),

@@ -7,6 +7,7 @@
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <mutex>
 #include <new>
 #include <vector>
 
@@ -62,6 +63,11 @@ struct vfkv_workspace {
     float* scratch_max;
     float* scratch_sum;
 };
+
+// Decode partials of vfkv_decode_attention_static: device memory that exists from the moment the library is loaded, so
+// the call needs no allocation.  Every GPU holds its own copy at its own address; host code never uses the array's
+// name as an address, only what hipGetSymbolAddress returned for the current device (static_scratch() below).
+static __device__ __align__(256) unsigned char scratch[VFKV_STATIC_SCRATCH_BYTES];
 
 namespace {
 
@@ -513,6 +519,25 @@ int vfkv_workspace_create(uint32_t n_heads, uint32_t head_dim, uint32_t max_seq_
     return VFKV_OK;
 }
 
+// Device address of `scratch` on the current device, looked up once per device.
+static int static_scratch(void** out) {
+    constexpr int kMaxDevices = 64;
+    static std::mutex mu;
+    static void* ptr[kMaxDevices] = {};
+    int dev = -1;
+    VFKV_HIP(hipGetDevice(&dev));
+    if (dev < 0 || dev >= kMaxDevices) return fail(VFKV_ERR_UNSUPPORTED, "decode_attention_static: device index %d", dev);
+    std::lock_guard<std::mutex> lock(mu);
+    if (!ptr[dev]) {
+        void* p = nullptr;
+        VFKV_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+        if (!p) return fail(VFKV_ERR_HIP, "decode_attention_static: hipGetSymbolAddress returned NULL");
+        ptr[dev] = p;
+    }
+    *out = ptr[dev];
+    return VFKV_OK;
+}
+
 void vfkv_workspace_destroy(vfkv_workspace* w) {
     if (!w) return;
     if (w->scratch_out) (void)hipFree(w->scratch_out);
@@ -558,9 +583,9 @@ uint32_t vfkv_decode_tile_for(uint32_t span, uint32_t n_heads, uint32_t n_kv_hea
 static int decode_attention_impl(vfkv_cache* c, uint32_t layer, uint32_t kv_layer, uint32_t n_heads, const float* q, float* o,
                                  uint32_t position, uint32_t kv_start, float scale, float softcap, vfkv_workspace* ws,
                                  const float* k_new, const float* v_new, vfkv_stream stream, const char* who,
-                                 const vfkv::GateArgs* gate = nullptr) {
+                                 const vfkv::GateArgs* gate = nullptr, bool static_ws = false) {
     if (!c || !c->k || !c->v) return fail(VFKV_ERR_INVALID_ARG, "%s: cache has no buffers", who);
-    if (!ws) return fail(VFKV_ERR_INVALID_ARG, "%s: workspace is NULL", who);
+    if (!ws && !static_ws) return fail(VFKV_ERR_INVALID_ARG, "%s: workspace is NULL", who);
     if (!q || !o) return fail(VFKV_ERR_INVALID_ARG, "%s: NULL buffer", who);
     if (layer >= c->n_layers || kv_layer >= c->n_layers)
         return fail(VFKV_ERR_INVALID_ARG, "%s: layer %u / kv_layer %u out of range", who, layer, kv_layer);
@@ -572,12 +597,30 @@ static int decode_attention_impl(vfkv_cache* c, uint32_t layer, uint32_t kv_laye
     if (rc != VFKV_OK) return rc;
     const uint32_t seq_len = position + 1u;
     if (kv_start >= seq_len) return fail(VFKV_ERR_INVALID_ARG, "%s: kv_start %u leaves no visible key (seq_len %u)", who, kv_start, seq_len);
-    if (n_heads > ws->n_heads || hd > ws->head_dim)
+    if (ws && (n_heads > ws->n_heads || hd > ws->head_dim))
         return fail(VFKV_ERR_WORKSPACE, "%s: workspace built for %u heads x %u dims, need %u x %u", who,
                     ws->n_heads, ws->head_dim, n_heads, hd);
     const uint32_t tile = vfkv_decode_tile_for(seq_len - kv_start, n_heads, kvh, hd, c->dtype);
     const uint32_t first = kv_start / tile;
     const uint32_t n_tiles = (seq_len + tile - 1u) / tile - first;
+    vfkv_workspace fixed;
+    if (static_ws) {
+        // the partials of this launch laid out in the static array: [out | max | sum], each part 256-byte aligned
+        const uint64_t n_ml = (uint64_t)n_heads * n_tiles;
+        const uint64_t out_b = (n_ml * hd * 4u + 255u) & ~255ull, ml_b = (n_ml * 4u + 255u) & ~255ull;
+        if (out_b + 2u * ml_b > (uint64_t)VFKV_STATIC_SCRATCH_BYTES)
+            return fail(VFKV_ERR_WORKSPACE, "%s: %u heads x %u partials x %u dims need %llu bytes of scratch, the static buffer holds %llu "
+                        "(use vfkv_decode_attention with a workspace)", who, n_heads, n_tiles, hd,
+                        (unsigned long long)(out_b + 2u * ml_b), (unsigned long long)VFKV_STATIC_SCRATCH_BYTES);
+        void* base = nullptr;
+        rc = static_scratch(&base);
+        if (rc != VFKV_OK) return rc;
+        fixed.n_heads = n_heads; fixed.head_dim = hd; fixed.max_tiles = n_tiles;
+        fixed.scratch_out = (float*)base;
+        fixed.scratch_max = (float*)((char*)base + out_b);
+        fixed.scratch_sum = (float*)((char*)base + out_b + ml_b);
+        ws = &fixed;
+    }
     if (n_tiles > ws->max_tiles) return fail(VFKV_ERR_WORKSPACE, "%s: %u tiles > workspace capacity %u", who, n_tiles, ws->max_tiles);
     const uint64_t off = layer_off(c, kv_layer);
     vfkv::SplitLaunch L;
@@ -616,6 +659,12 @@ int vfkv_decode_attention(vfkv_cache* c, uint32_t layer, uint32_t kv_layer, uint
                           vfkv_stream stream) {
     return decode_attention_impl(c, layer, kv_layer, n_heads, q, o, position, kv_start, scale, softcap, ws, nullptr, nullptr,
                                  stream, "decode_attention");
+}
+
+int vfkv_decode_attention_static(vfkv_cache* c, uint32_t layer, uint32_t kv_layer, uint32_t n_heads, const float* q, float* o,
+                                 uint32_t position, uint32_t kv_start, float scale, float softcap, vfkv_stream stream) {
+    return decode_attention_impl(c, layer, kv_layer, n_heads, q, o, position, kv_start, scale, softcap, nullptr, nullptr, nullptr,
+                                 stream, "decode_attention_static", nullptr, true);
 }
 
 int vfkv_kv_write_decode_attention(vfkv_cache* c, uint32_t layer, uint32_t n_heads, const float* q, const float* k_src,

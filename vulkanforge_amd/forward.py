@@ -167,6 +167,19 @@ class Forward:
 
     step_attention = run_scalar_attn  # executor/attention.rs:599-625
 
+    def run_scalar_attn_static(self, layer: int, position: int, q, o, kv_layer: int | None = None, kv_start: int = 0,
+                               scale: float | None = None, softcap: float = 0.0, stream=None) -> None:
+        """``run_scalar_attn`` without the workspace: vfkv_decode_attention_static keeps the partials in the library's
+        static device array and allocates nothing (for callers under graph capture or in loops that must not allocate).
+        Calls that overlap in time on one GPU race."""
+        if scale is None:
+            hd = self.kv_cache.head_dim_for(layer)
+            scale = self.attn_scale if hd == self.kv_cache.config.head_dim else 1.0 / math.sqrt(hd)
+        _ffi.check(_ffi.lib().vfkv_decode_attention_static(self.kv_cache.handle, layer,
+                                                           layer if kv_layer is None else kv_layer, self.n_heads,
+                                                           _ptr(q), _ptr(o), position, kv_start, scale, softcap,
+                                                           _stream(stream)))
+
     def step_kv_write_attention(self, layer: int, position: int, q, k_src, v_src, o, kv_start: int = 0,
                                 scale: float | None = None, softcap: float = 0.0, stream=None) -> None:
         """step_kv_write + step_attention of one token (executor/attention.rs:546-625) as one call: where the

@@ -182,6 +182,13 @@ public:
     void step_attention(uint32_t layer, uint32_t position, const float* q, float* attn_out) {   // attention.rs:599-625
         run_scalar_attn(layer, position, q, attn_out, layer, 0);
     }
+    // run_scalar_attn for callers that must not allocate or pass a workspace: the partials live in the library's own
+    // static device array (one per GPU; calls that overlap in time on one GPU race)
+    void run_scalar_attn_static(uint32_t layer, uint32_t position, const float* q, float* attn_out, uint32_t kv_layer,
+                                uint32_t kv_start, float softcap = 0.f) {
+        check(vfkv_decode_attention_static(kv_cache.handle(), layer, kv_layer, n_heads, q, attn_out, position, kv_start,
+                                           scale_for(layer), softcap, stream));
+    }
     // step_kv_write + step_attention of one token (attention.rs:546-625) in one call; the decode worker writes the
     // new rows itself where it can
     void step_kv_write_attention(uint32_t layer, uint32_t position, const float* q, const float* k_src, const float* v_src,

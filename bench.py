@@ -34,11 +34,58 @@ MFMA_F32_PEAK_TFLOPS = 157.3      # dense f32 matrix rate: what an F32 cache is 
 
 # HBM bytes per launch of the dominant kernel, measured with rocprofv3 --pmc FETCH_SIZE and --pmc WRITE_SIZE
 # (two runs) and scaled by what the same counters read for a plain 64 MiB device copy
-# (FETCH_SIZE x 1.9991, WRITE_SIZE x 1.0 to KiB).  Only the workloads that were profiled have an entry.
-MEASURED_TRAFFIC_BYTES = {
-    "decode_fp8_32k_32layers": (65634 + 520) * 1024,
-    "prefill_fp8_512x4608_32layers": (81369 + 8192) * 1024,
+# (FETCH_SIZE x 1.9991, WRITE_SIZE x 1.0 to KiB).  Only the workloads that were profiled have an entry.  Counters cannot
+# be read from inside this process, so an entry names the summary it comes from and the digest of the kernel sources
+# it was taken with: when the sources have changed since, the line reports null instead of a stale figure.
+PROFILED_TRAFFIC = {
+    "decode_fp8_32k_32layers": {
+        "bytes": (65634 + 520) * 1024, "profile": "profiles/decode_fp8_32k_split_mfma_kernel.md",
+        "sources": ("attn_decode.hip", "attn_decode_mfma.h", "device_utils.h"), "sha256_16": "2f2ec6d675d73d3a"},
+    "prefill_fp8_512x4608_32layers": {
+        "bytes": (81369 + 8192) * 1024, "profile": "profiles/prefill_fp8_512x4608_batch_mfma2_kernel.md",
+        "sources": ("attn_prefill.hip", "attn_prefill_mfma2.h", "device_utils.h"), "sha256_16": "4a01f15e97324471"},
 }
+
+
+def kernel_sources_digest(names):
+    import hashlib
+    h = hashlib.sha256()
+    for n in names:
+        with open(os.path.join(ROOT, "vulkanforge_amd", "csrc", n), "rb") as f:
+            h.update(f.read())
+    return h.hexdigest()[:16]
+
+
+def profiled_traffic(workload):
+    """(bytes or None, where the figure comes from) for the roofline entry of `workload`."""
+    e = PROFILED_TRAFFIC.get(workload)
+    if e is None:
+        return None, None
+    if kernel_sources_digest(e["sources"]) != e["sha256_16"]:
+        return None, e["profile"] + " (kernel sources changed since that profile: not reported)"
+    return e["bytes"], e["profile"]
+
+
+def host_cpu():
+    model = "unknown"
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.startswith("model name"):
+                    model = line.split(":", 1)[1].strip()
+                    break
+    except OSError:
+        pass
+    return {"cpu_model": model, "hardware_concurrency": os.cpu_count()}
+
+
+MFMA_DTYPE = "f16 mfma on value + remainder operand pairs, f32 accumulate"   # what the matrix-core kernels compute in
+
+
+def mfma_decode_worker(dtype_label, head_dim):
+    """Mirrors the library's choice: FP8 / F16 caches at head_dim 64 / 128 / 256 / 512 run on the matrix-core worker."""
+    return (os.environ.get("VFKV_DECODE_WORKER", "m")[:1] != "v" and dtype_label in ("FP8", "FP16")
+            and head_dim in (64, 128, 256, 512))
 
 
 def parse_args():
@@ -54,6 +101,8 @@ def parse_args():
                     help="leave the queries as general f32 values instead of casting them to fp16 first")
     ap.add_argument("--no-graph", action="store_true",
                     help="launch every kernel from Python instead of replaying one captured HIP graph per step")
+    ap.add_argument("--no-other-workloads", action="store_true",
+                    help="headline run only: skip the short runs of the other benchmark configurations ('workloads' array)")
     return ap.parse_args()
 
 
@@ -208,33 +257,71 @@ def bench_decode(args, wl):
             fwd.run_flash_attn_split(q[layer], klay, vlay, wl.dtype, so, sm, ss, H, Hkv, D, wl.context - skip, scale,
                                      kv_start=starts[layer] - skip, tile=tile, softcap=wl.softcap, interleaved=True)
 
-    run_split = split_only
-    if not args.no_graph:
-        split_only()
+    def event_timed(fn, reps):
+        """Total milliseconds of `reps` replays of fn's launches (captured once into a graph) between two events."""
+        run = fn
+        if not args.no_graph:
+            fn()
+            torch.cuda.synchronize()
+            gr = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(gr):
+                fn()
+            run = gr.replay
+        run()
         torch.cuda.synchronize()
-        g2 = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(g2):
-            split_only()
-        run_split = g2.replay
-    run_split()
-    torch.cuda.synchronize()
+        evs = []
+        for _ in range(reps):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record(stream)
+            run()
+            e1.record(stream)
+            evs.append((e0, e1))
+        torch.cuda.synchronize()
+        return sum(e0.elapsed_time(e1) for e0, e1 in evs)
+
     n_ev = min(max(args.steps, 5), 20)
-    pairs = []
-    for _ in range(n_ev):
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        e0.record(stream)
-        run_split()
-        e1.record(stream)
-        pairs.append((e0, e1))
-    torch.cuda.synchronize()
-    split_ms = sum(e0.elapsed_time(e1) for e0, e1 in pairs)
+    split_ms = event_timed(split_only, n_ev)
     launches = n_ev * L
     bytes_launch = bytes_step / L          # mean over the layers of the step
     avg_ms = split_ms / launches
     achieved = bytes_launch / (avg_ms * 1e-3) / 1e9
 
-    mfma_worker = os.environ.get("VFKV_DECODE_WORKER", "m")[:1] != "v" and D <= 256 and wl.dtype.label() != "FP32"
+    # ---- what the same bytes cost without any arithmetic, timed the same way over the same slabs (compute-free kernels
+    # of libvfkv_calib.so): a plain contiguous read, the worker's own walk and request pattern, and an empty launch of
+    # the worker's grid.  Only for the geometry the pattern kernel is written for (FP8 rows, head_dim 128, no window).
+    floors = None
+    if wl.dtype.label() == "FP8" and D == 128 and not wl.window:
+        import ctypes as C
+        calib_path = os.path.join(ROOT, "vulkanforge_amd", "libvfkv_calib.so")
+        if not os.path.exists(calib_path):
+            raise ImportError(f"{calib_path} is missing: build it with `make -C vulkanforge_amd/csrc`")
+        calib = C.CDLL(calib_path)
+        calib.vfkv_calib_stream_read.argtypes = [C.c_void_p, C.c_void_p, C.c_uint64, C.c_void_p, C.c_void_p]
+        calib.vfkv_calib_pattern_read.argtypes = [C.c_void_p, C.c_void_p, C.c_uint32, C.c_uint32, C.c_uint32, C.c_void_p, C.c_void_p]
+        calib.vfkv_calib_empty.argtypes = [C.c_uint32, C.c_uint32, C.c_void_p, C.c_void_p]
+        sink = torch.zeros(1024, dtype=torch.int32, device=dev)
+        tile = lib.vfkv_decode_tile_for(wl.context, H, Hkv, D, int(wl.dtype))
+        n_tiles = (wl.context + tile - 1) // tile
+        layer_bytes = wl.context * Hkv * D * es
+
+        def per_layer(call):
+            def run():
+                st = torch.cuda.current_stream().cuda_stream
+                for layer in range(L):
+                    kp = cache.k_ptr + cache.layer_offset_bytes(layer)
+                    vp = cache.v_ptr + cache.layer_offset_bytes(layer)
+                    rc = call(kp, vp, st)
+                    assert rc == 0, rc
+            return run
+
+        stream_us = event_timed(per_layer(lambda kp, vp, st: calib.vfkv_calib_stream_read(kp, vp, layer_bytes // 16 * 16, sink.data_ptr(), st)), n_ev) * 1e3 / launches
+        pattern_us = event_timed(per_layer(lambda kp, vp, st: calib.vfkv_calib_pattern_read(kp, vp, wl.context, Hkv, n_tiles, sink.data_ptr(), st)), n_ev) * 1e3 / launches
+        empty_us = event_timed(per_layer(lambda kp, vp, st: calib.vfkv_calib_empty(Hkv, n_tiles, sink.data_ptr(), st)), n_ev) * 1e3 / launches
+        floors = {"stream_floor_us": stream_us, "pattern_floor_us": pattern_us, "empty_launch_us": empty_us}
+
+    mfma_worker = mfma_decode_worker(wl.dtype.label(), D)
     worker_name = "split_mfma_kernel" if mfma_worker else "split_kernel"
+    traffic, traffic_source = profiled_traffic(wl.name)
     result = {
         "metric": "kv_read_GBps_decode_step",
         "value": bytes_step / sec_per_step / 1e9,
@@ -248,7 +335,7 @@ def bench_decode(args, wl):
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "f32",
+        "dtype": MFMA_DTYPE if mfma_worker else "f32",
         "kv_dtype": wl.dtype.label(),
         "launch": "eager" if args.no_graph else "hip_graph",
         "data": "synthetic, seeded N(0,1); queries " + ("general f32" if args.f32_queries else "cast to fp16 as the configuration states") + "; K/V rows cast to fp16 and written through the append kernels",
@@ -256,10 +343,13 @@ def bench_decode(args, wl):
                    "context": wl.context, "append_per_step": wl.append, "kv_bytes_per_step": bytes_step,
                    "pct_of_hbm_peak": 100.0 * bytes_step / sec_per_step / 1e9 / HBM_PEAK_GBPS},
         "roofline": {"bound": "hbm", "kernel": worker_name, "achieved": achieved, "peak": HBM_PEAK_GBPS,
-                     "unit": "GB/s", "frac": achieved / HBM_PEAK_GBPS, "traffic": MEASURED_TRAFFIC_BYTES.get(wl.name),
+                     "unit": "GB/s", "frac": achieved / HBM_PEAK_GBPS, "traffic": traffic, "traffic_source": traffic_source,
                      "avg_launch_us": avg_ms * 1e3, "launches_timed": launches,
                      "algorithmic_bytes_per_launch": bytes_launch},
     }
+    if floors is not None:   # same bytes, same slabs, same timing method, no arithmetic
+        result["roofline"].update(floors)
+        result["roofline"]["frac_of_pattern_floor"] = floors["pattern_floor_us"] / (avg_ms * 1e3)
 
     if gate_separate_us is not None:
         result["config"]["us_per_step_with_separate_gate_launch"] = gate_separate_us
@@ -291,7 +381,7 @@ def bench_decode(args, wl):
                 break
         result["cpu_baseline"] = {"value": done_bytes / spent / 1e9, "unit": "GB/s", "cores": threads, "kind": "port",
                                   "sample": f"{layers_done} of {L} layers of the same step, CPU oracle "
-                                            f"(attn_decode_ref, f64 accumulation), {spent:.1f} s"}
+                                            f"(attn_decode_ref, f64 accumulation), {spent:.1f} s", **host_cpu()}
     cache.destroy()
     return result
 
@@ -363,20 +453,21 @@ def bench_prefill(args, wl):
     achieved = wl.flops_layer() / (avg_ms * 1e-3) / 1e12
     f32_cache = wl.dtype.label() == "FP32"
     peak = MFMA_F32_PEAK_TFLOPS if f32_cache else MFMA_F16_PEAK_TFLOPS
+    traffic, traffic_source = profiled_traffic(wl.name)
     result = {
         "metric": "prefill_attention_TFLOPs",
         "value": flops_step / sec_per_step / 1e12,
         "unit": "TFLOP/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": sec_per_step * 1e3,
         "step_us_event_timed": step_spread,
-        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32" if f32_cache else "f16",
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32 mfma" if f32_cache else MFMA_DTYPE,
         "kv_dtype": wl.dtype.label(),
         "data": "synthetic, seeded N(0,1); queries " + ("general f32" if args.f32_queries else "cast to fp16 as the configuration states") + "; K/V rows cast to fp16 and written through the append kernels",
         "config": {"workload": wl.name, "n_layers": L, "n_heads": H, "n_kv_heads": Hkv, "head_dim": D,
                    "m": wl.m, "q_start": wl.base_pos, "n_kv": max_seq, "flop_per_step": flops_step},
         "roofline": {"bound": "mfma", "kernel": "batch_mfma_f32_kernel" if f32_cache else "batch_mfma2_kernel",
                      "achieved": achieved, "peak": peak,
-                     "unit": "TFLOP/s", "frac": achieved / peak, "traffic": MEASURED_TRAFFIC_BYTES.get(wl.name),
+                     "unit": "TFLOP/s", "frac": achieved / peak, "traffic": traffic, "traffic_source": traffic_source,
                      "avg_launch_us": avg_ms * 1e3},
     }
     if gate_separate_ms is not None:
@@ -407,7 +498,7 @@ def bench_prefill(args, wl):
         result["cpu_baseline"] = {"value": flops_sample * reps / spent / 1e12, "unit": "TFLOP/s", "cores": threads,
                                   "kind": "port",
                                   "sample": f"last {ms} of {wl.m} query rows of one layer, {reps} repetitions, CPU "
-                                            f"oracle (attn_batch_ref, f64), {spent:.1f} s"}
+                                            f"oracle (attn_batch_ref, f64), {spent:.1f} s", **host_cpu()}
     cache.destroy()
     return result
 
@@ -502,6 +593,41 @@ def copy_calibration(args):
             "launches": args.steps, "value": 2 * n * args.steps / dt / 1e9, "unit": "GB/s", "n_gpus": 1}
 
 
+HEADLINE = "decode_fp8_32k_32layers"
+# the other benchmark configurations, run briefly after the headline workload so that one invocation witnesses all five
+OTHER_CONFIGS = ("decode_f16_2k_1layer", "decode_fp8_8k_32layers", "decode_f16_hd256_sliding_12layers",
+                 "prefill_fp8_512x4608_32layers")
+
+
+def run_workload(args, name):
+    from vulkanforge_amd import workloads
+    if name in workloads.DECODE:
+        return bench_decode(args, workloads.DECODE[name])
+    if name in workloads.PREFILL:
+        return bench_prefill(args, workloads.PREFILL[name])
+    if name in workloads.ROPE_APPEND:
+        return bench_rope_append(args, workloads.ROPE_APPEND[name])
+    if name == "copy_calibration":
+        return copy_calibration(args)
+    return None
+
+
+def summary(res):
+    """The fields of a workload's own JSON line that the headline line carries along in its 'workloads' array."""
+    cfg, roof = res["config"], res["roofline"]
+    err = cfg.get("max_abs_err_vs_oracle_layer0", cfg.get("max_abs_err_vs_oracle_last_rows"))
+    out = {"workload": cfg["workload"], "ms_per_step": res["ms_per_step"], "steps": res["steps"], "value": res["value"],
+           "unit": res["unit"], "kv_dtype": res["kv_dtype"],
+           "roofline": {k: roof[k] for k in ("kernel", "bound", "frac", "avg_launch_us", "achieved", "peak", "unit") if k in roof},
+           "max_abs_err_vs_oracle": err}
+    for k in ("stream_floor_us", "pattern_floor_us", "empty_launch_us"):
+        if k in roof:
+            out["roofline"][k] = roof[k]
+    if "cpu_baseline" in res:
+        out["cpu_baseline"] = {k: res["cpu_baseline"][k] for k in ("value", "unit", "cores")}
+    return out
+
+
 def main():
     args = parse_args()
     if args.gpus != 1:
@@ -509,18 +635,20 @@ def main():
               file=sys.stderr)
         sys.exit(2)
     from vulkanforge_amd import workloads
-    if args.workload in workloads.DECODE:
-        res = bench_decode(args, workloads.DECODE[args.workload])
-    elif args.workload in workloads.PREFILL:
-        res = bench_prefill(args, workloads.PREFILL[args.workload])
-    elif args.workload in workloads.ROPE_APPEND:
-        res = bench_rope_append(args, workloads.ROPE_APPEND[args.workload])
-    elif args.workload == "copy_calibration":
-        res = copy_calibration(args)
-    else:
+    res = run_workload(args, args.workload)
+    if res is None:
         print("unknown workload; choose from: " + ", ".join(list(workloads.DECODE) + list(workloads.PREFILL) + list(workloads.ROPE_APPEND) + ["copy_calibration"]),
               file=sys.stderr)
         sys.exit(2)
+    if args.workload == HEADLINE and not args.no_other_workloads:
+        import copy
+        brief = copy.copy(args)
+        brief.cpu_seconds = min(args.cpu_seconds, 1.0)
+        res["workloads"] = []
+        for name in OTHER_CONFIGS:
+            brief.steps = min(args.steps, 5 if name in workloads.PREFILL else 30)
+            brief.warmup = min(args.warmup, 2 if name in workloads.PREFILL else 10)
+            res["workloads"].append(summary(run_workload(brief, name)))
     print(json.dumps(res))
 
 

@@ -132,7 +132,7 @@ def fill_cache(torch, vf, fwd, wl, n_tokens, seed, outliers):
 
 # The V buffer starts 256 bytes into its allocation, as in the caches vfkv_cache_create allocates itself: K and V
 # of one row then differ in address bits 7-8 (see the comment there).
-V_SKEW = int(os.environ.get("VFKV_BENCH_V_SKEW", "256"))
+V_SKEW = 256
 
 
 STEP_SPREAD = {}   # filled by time_steps: percentiles of single event-timed steps, microseconds

@@ -16,6 +16,11 @@
  *     threads; one workspace must not be used by two in-flight calls at once.
  *   - There is no CPU fallback: without a HIP device every compute entry point fails with
  *     VFKV_ERR_HIP / VFKV_ERR_NO_DEVICE.  Layout arithmetic works without a device.
+ *   - Two environment variables are read, once per process, and nothing else is tunable at run time:
+ *       VFKV_DECODE_TILE=<multiple of 64>   keys per workgroup in vfkv_decode_attention, instead of the library's own
+ *                                            choice (the reference's split-chunk size, runs.rs:766);
+ *       VFKV_DECODE_WORKER=valu              serve every decode shape with the vector-ALU worker instead of the
+ *                                            matrix-core worker (for comparisons).
  */
 #ifndef VFKV_H
 #define VFKV_H
@@ -77,7 +82,9 @@ typedef struct vfkv_cache vfkv_cache;
 int vfkv_cache_create(const vfkv_cache_config* cfg, vfkv_cache** out);
 /* Same layout object over caller-owned buffers (either may be NULL for layout-only use, e.g. on a
  * host without a GPU).  No allocation happens and destroy() leaves the buffers alone.  For speed give
- * the two buffers different alignment modulo 512 bytes (e.g. v_buffer = allocation + 256). */
+ * the two buffers different alignment modulo 512 bytes (e.g. v_buffer = allocation + 256): results are
+ * identical either way, but equally aligned buffers cost the attention kernels up to 8 %.  The call
+ * still returns VFKV_OK then and leaves a one-line note in vfkv_last_error() (empty otherwise). */
 int vfkv_cache_create_external(const vfkv_cache_config* cfg, void* k_buffer, void* v_buffer,
                                vfkv_cache** out);
 /* KvCache::destroy (kv_cache.rs:496-499). */

@@ -317,3 +317,43 @@ def test_static_decode_call_rejects_partials_beyond_its_array():
     env = dict(os.environ, VFKV_DECODE_TILE="64", PYTHONPATH=ROOT)
     out = subprocess.run([sys.executable, "-c", code], env=env, capture_output=True, text=True, timeout=300)
     assert out.returncode == 0 and out.stdout.strip() == "ok", out.stderr
+
+
+def test_validation_of_out_pointer_kv_layer_geometry_and_scale():
+    L = _ffi.lib()
+    fake = 0x1000
+    cfg = _ffi.CacheConfig(2, 8, 128, 64, None, None, 2)
+    assert L.vfkv_cache_create(C.byref(cfg), None) == -1                       # NULL out: an error, not a crash
+    # a layer may only read the slab of a layer with the same row geometry (heterogeneous cache, gemma4.rs:27-49)
+    hd = (C.c_uint32 * 3)(256, 512, 256)
+    kvh = (C.c_uint32 * 3)(8, 2, 8)
+    cfg = _ffi.CacheConfig(3, 8, 256, 128, hd, kvh, 2)
+    h = C.c_void_p()
+    assert L.vfkv_cache_create_external(C.byref(cfg), fake, fake + 256, C.byref(h)) == 0
+    ws = C.c_void_p(fake)                                                      # never dereferenced: validation fails first
+    assert L.vfkv_decode_attention(h, 0, 1, 16, fake, fake, 10, 0, 0.1, 0.0, ws, None) == -1
+    assert b"cannot read the slab" in L.vfkv_last_error()
+    assert L.vfkv_prefill_attention(h, 0, 1, 16, fake, fake, 4, 0, 0, 0.1, 0.0, None) == -1
+    assert L.vfkv_decode_attention_static(h, 2, 1, 16, fake, fake, 10, 0, 0.1, 0.0, None) == -1
+    # the softmax scale must be positive and finite
+    for bad in (0.0, -0.5, float("inf"), float("nan")):
+        assert L.vfkv_decode_attention(h, 0, 2, 16, fake, fake, 10, 0, bad, 0.0, ws, None) == -1
+        assert b"scale" in L.vfkv_last_error()
+        p = _ffi.SplitParams(32, 8, 128, 100, 0, bad, 2, 0)
+        assert L.vfkv_flash_attn_split(fake, fake, fake, 2, fake, fake, fake, C.byref(p), 64, 0.0, None) == -1
+        b = _ffi.BatchParams(32, 8, 128, 4, 64, 60, bad, 0)
+        assert L.vfkv_flash_attn_batch(fake, fake, fake, 0, fake, C.byref(b), 0.0, None) == -1
+        assert L.vfkv_prefill_attention(h, 0, 2, 16, fake, fake, 4, 0, 0, bad, 0.0, None) == -1
+    L.vfkv_cache_destroy(h)
+
+
+def test_external_buffers_of_equal_alignment_leave_a_note_not_an_error():
+    L = _ffi.lib()
+    cfg = _ffi.CacheConfig(1, 8, 128, 64, None, None, 2)
+    h = C.c_void_p()
+    assert L.vfkv_cache_create_external(C.byref(cfg), 0x10000, 0x20000, C.byref(h)) == 0
+    assert b"256 bytes" in L.vfkv_last_error()
+    L.vfkv_cache_destroy(h)
+    assert L.vfkv_cache_create_external(C.byref(cfg), 0x10000, 0x20100, C.byref(h)) == 0
+    assert L.vfkv_last_error() == b""
+    L.vfkv_cache_destroy(h)

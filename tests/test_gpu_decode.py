@@ -282,6 +282,11 @@ def test_config2_fp8_outliers_append_then_decode_two_layers():
     (vf.KvDtype.F32, 8, 2, 128, 300, 0),        # 4-byte cache: separate append launch
     (vf.KvDtype.F16, 8, 1, 256, 16000, 0),      # one KV head: 250 tiles, merged by four wavefronts per 64 outputs
     (vf.KvDtype.F8, 16, 2, 512, 9000, 0),       # Gemma-4 full-attention geometry: 2 KV heads, 128 tiles
+    # FP8 rows of head_dim 64 are half a 128-byte line: two workgroups (neighbouring KV heads) store into and read from the
+    # same line of the new row
+    (vf.KvDtype.F8, 16, 8, 64, 1000, 0),
+    (vf.KvDtype.F8, 16, 8, 64, 8192, 0),        # interleaved walk: the owner of the new row is not the last workgroup
+    (vf.KvDtype.F8, 16, 8, 64, 5000, 700),      # the same under a sliding window
 ])
 def test_kv_write_attention_in_one_call_matches_the_two_calls(dtype, heads, hkv, d, ctx, window):
     # step_kv_write + step_attention (executor/attention.rs:546-625) through the single entry point: cache bytes and
@@ -411,3 +416,40 @@ def test_short_context_goes_through_the_same_path():
         fwd.run_scalar_attn(0, 64, to_dev(q), torch.empty((heads, d), device=DEV))      # beyond max_seq
     with pytest.raises(vf.VfkvError):
         fwd.run_scalar_attn(0, 10, to_dev(q), torch.empty((heads, d), device=DEV), kv_start=11)
+
+
+@pytest.mark.parametrize("dtype,heads,hkv,d,ctx", [(vf.KvDtype.F8, 32, 8, 128, 4097), (vf.KvDtype.F16, 16, 8, 256, 1500)])
+def test_caller_owned_buffers_give_the_same_output_at_any_relative_alignment(dtype, heads, hkv, d, ctx):
+    # KvCache over buffers the caller allocated (kv_cache.rs:224-339 with the host's own allocator): equal alignment of K
+    # and V modulo 512 bytes only costs speed (vfkv_cache_create_external leaves a note), the bytes and the output of decode
+    # and prefill attention are the same as with V offset by 256 bytes
+    from gpu_util import read_device
+    fill = outlier_normal if dtype == vf.KvDtype.F8 else fp16_normal
+    es = dtype.element_size()
+    nbytes = ctx * hkv * d * es
+    r = rng(404)
+    k, v = fill(r, (ctx, hkv * d)), fill(r, (ctx, hkv * d))
+    q, qb = fp16_normal(r, (heads, d)), fp16_normal(r, (16, heads, d))
+    outs = []
+    for skew in (0, 256, 128):
+        kbuf = torch.zeros(nbytes + 512, dtype=torch.uint8, device=DEV)
+        vbuf = torch.zeros(nbytes + 1024, dtype=torch.uint8, device=DEV)
+        kp = (kbuf.data_ptr() + 511) // 512 * 512
+        vp = (vbuf.data_ptr() + 511) // 512 * 512 + skew
+        cache = vf.KvCache(vf.KvCacheConfig(1, hkv, d, ctx, dtype=dtype), k_buffer=kp, v_buffer=vp)
+        note = vf._ffi.lib().vfkv_last_error()
+        assert (b"256 bytes" in note) == (skew == 0)
+        fwd = vf.Forward(cache, heads)
+        fwd.b_step_kv_write(0, 0, ctx, to_dev(k), to_dev(v))
+        o = torch.full((heads, d), float("nan"), device=DEV)
+        fwd.run_scalar_attn(0, ctx - 1, to_dev(q), o)
+        ob = torch.full((16, heads, d), float("nan"), device=DEV)
+        fwd.b_step_attention(0, ctx - 16, 16, to_dev(qb), ob)
+        torch.cuda.synchronize()
+        outs.append((to_np(o).copy(), to_np(ob).copy(), read_device(vp, nbytes).copy()))
+        cache.destroy()
+    for o, ob, vbytes in outs[1:]:
+        assert np.array_equal(o, outs[0][0]) and np.array_equal(ob, outs[0][1]) and np.array_equal(vbytes, outs[0][2])
+    ke, ve = encode_np(k, dtype).reshape(-1, hkv, d), encode_np(v, dtype).reshape(-1, hkv, d)
+    ref = oracle.attn_decode_ref(q, ke, ve, int(dtype), heads, hkv, d, ctx, 1.0 / np.sqrt(d))
+    assert np.abs(outs[0][0] - ref).max() < TOL[dtype]

@@ -5,8 +5,7 @@ import ctypes as C
 import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-# VFKV_LIBRARY selects another build of the library (e.g. one compiled with different tuning macros)
-_SO = os.environ.get("VFKV_LIBRARY") or os.path.join(_HERE, "libvfkv.so")
+_SO = os.path.join(_HERE, "libvfkv.so")
 
 OK = 0
 STATUS_NAMES = {0: "VFKV_OK", -1: "VFKV_ERR_INVALID_ARG", -2: "VFKV_ERR_OVERFLOW", -3: "VFKV_ERR_ALIGNMENT",

@@ -124,6 +124,22 @@ inline uint64_t row_b(const vfkv_cache* c, uint32_t layer) {
     return (uint64_t)kvh_for(c, layer) * hd_for(c, layer) * esize(c->dtype);
 }
 
+// The kernels fold the softmax scale into the exponent (max(x) * scale), which needs a positive finite scale.
+int check_scale(float scale, const char* who) {
+    if (!(scale > 0.f) || !(scale < __builtin_inff()))
+        return fail(VFKV_ERR_INVALID_ARG, "%s: scale must be positive and finite (got %g)", who, (double)scale);
+    return VFKV_OK;
+}
+
+// A layer that reads another layer's slab (cross-layer KV share) must agree with it on the row geometry: the slab is
+// addressed with the reading layer's head_dim and n_kv_heads.
+int check_kv_layer(const vfkv_cache* c, uint32_t layer, uint32_t kv_layer, const char* who) {
+    if (kv_layer != layer && (hd_for(c, layer) != hd_for(c, kv_layer) || kvh_for(c, layer) != kvh_for(c, kv_layer)))
+        return fail(VFKV_ERR_INVALID_ARG, "%s: layer %u (%u kv heads x %u) cannot read the slab of kv_layer %u (%u kv heads x %u)", who,
+                    layer, kvh_for(c, layer), hd_for(c, layer), kv_layer, kvh_for(c, kv_layer), hd_for(c, kv_layer));
+    return VFKV_OK;
+}
+
 int check_attn_dims(uint32_t n_heads, uint32_t n_kv_heads, uint32_t head_dim) {
     if (n_heads == 0 || n_kv_heads == 0 || head_dim == 0)
         return fail(VFKV_ERR_INVALID_ARG, "n_heads, n_kv_heads and head_dim must be > 0");
@@ -173,10 +189,17 @@ int vfkv_cache_create_external(const vfkv_cache_config* cfg, void* k_buffer, voi
     c->v_alloc = nullptr;
     c->owns = false;
     *out = c;
+    g_err[0] = '\0';
+    // Not an error, but worth telling the caller once: K and V buffers whose addresses agree in bits 7-8 cost the
+    // attention kernels up to 8 % (see vfkv_cache_create).  The note is readable through vfkv_last_error().
+    if (k_buffer && v_buffer && ((((uintptr_t)k_buffer) ^ ((uintptr_t)v_buffer)) & 0x180u) == 0u)
+        snprintf(g_err, sizeof(g_err), "note: k_buffer and v_buffer have the same alignment modulo 512 bytes; "
+                 "offsetting v_buffer by 256 bytes inside its allocation makes decode attention up to 8 %% faster");
     return VFKV_OK;
 }
 
 int vfkv_cache_create(const vfkv_cache_config* cfg, vfkv_cache** out) {
+    if (!out) return fail(VFKV_ERR_INVALID_ARG, "out is NULL");
     vfkv_cache* c = nullptr;
     const int rc = vfkv_cache_create_external(cfg, nullptr, nullptr, &c);
     if (rc != VFKV_OK) return rc;
@@ -186,7 +209,7 @@ int vfkv_cache_create(const vfkv_cache_config* cfg, vfkv_cache** out) {
     // agree in bits 7-8 (two allocations of the same alignment, same offset inside the row) the requests of one
     // 128-byte column of the row collide in the memory system and that column's reads run ~17 % slower; V
     // therefore starts 256 bytes into its allocation.
-    static const size_t v_skew = [] { const char* e = getenv("VFKV_CACHE_V_SKEW"); return e ? (size_t)atoi(e) & ~(size_t)15 : (size_t)256; }();
+    constexpr size_t v_skew = 256;
     hipError_t e = hipMalloc(&c->k, c->bytes);
     if (e == hipSuccess) {
         e = hipMalloc(&c->v_alloc, c->bytes + v_skew);
@@ -457,6 +480,8 @@ static int flash_attn_split_impl(const float* q, const void* k_layer, const void
     if (p->n_tiles != need)
         return fail(VFKV_ERR_INVALID_ARG, "flash_attn_split: n_tiles (%u) != ceil(seq_len / tile) (%u)", p->n_tiles, need);
     if (!(softcap >= 0.f)) return fail(VFKV_ERR_INVALID_ARG, "flash_attn_split: softcap must be >= 0");
+    rc = check_scale(p->scale, "flash_attn_split");
+    if (rc != VFKV_OK) return rc;
     vfkv::SplitLaunch L;
     L.q = q; L.k = k_layer; L.v = v_layer;
     L.scratch_out = scratch_out; L.scratch_max = scratch_max; L.scratch_sum = scratch_sum;
@@ -595,6 +620,8 @@ static int decode_attention_impl(vfkv_cache* c, uint32_t layer, uint32_t kv_laye
     const uint32_t hd = hd_for(c, layer), kvh = kvh_for(c, layer);
     int rc = check_attn_dims(n_heads, kvh, hd);
     if (rc != VFKV_OK) return rc;
+    if ((rc = check_scale(scale, who)) != VFKV_OK) return rc;
+    if ((rc = check_kv_layer(c, layer, kv_layer, who)) != VFKV_OK) return rc;
     const uint32_t seq_len = position + 1u;
     if (kv_start >= seq_len) return fail(VFKV_ERR_INVALID_ARG, "%s: kv_start %u leaves no visible key (seq_len %u)", who, kv_start, seq_len);
     if (ws && (n_heads > ws->n_heads || hd > ws->head_dim))
@@ -629,9 +656,8 @@ static int decode_attention_impl(vfkv_cache* c, uint32_t layer, uint32_t kv_laye
     L.dtype = c->dtype; L.n_heads = n_heads; L.n_kv_heads = kvh; L.head_dim = hd;
     L.seq_len = seq_len; L.kv_start = kv_start; L.tile = tile; L.tile_first = first; L.n_tiles = n_tiles;
     L.scale = scale; L.softcap = softcap;
-    // the partials stay inside the workspace, so they need not correspond to tiles (VFKV_DECODE_INTERLEAVE=0: they do)
-    static const bool interleave = [] { const char* e = getenv("VFKV_DECODE_INTERLEAVE"); return !(e && e[0] == '0'); }();
-    L.interleave = interleave;
+    // the partials stay inside the workspace, so they need not correspond to tiles
+    L.interleave = true;
     if (k_new) {
         L.k_new = k_new; L.v_new = v_new; L.append_pos = position;
         if (!vfkv::split_appends(L)) {          // this shape's worker cannot write the row itself: append in its own launch
@@ -689,6 +715,7 @@ static int flash_attn_batch_impl(const float* q, const void* k_layer, const void
     if (p->m == 0) return VFKV_OK;
     if (p->n_kv == 0) return fail(VFKV_ERR_INVALID_ARG, "flash_attn_batch: n_kv must be > 0");
     if (!(softcap >= 0.f)) return fail(VFKV_ERR_INVALID_ARG, "flash_attn_batch: softcap must be >= 0");
+    if ((rc = check_scale(p->scale, "flash_attn_batch")) != VFKV_OK) return rc;
     const uint64_t first_len = (uint64_t)p->q_start + 1u;
     const uint64_t vis0 = first_len < p->n_kv ? first_len : p->n_kv;
     if (p->kv_start >= vis0)
@@ -725,6 +752,8 @@ static int prefill_attention_impl(vfkv_cache* c, uint32_t layer, uint32_t kv_lay
     if ((uint64_t)base_pos + m > c->max_seq_len)
         return fail(VFKV_ERR_INVALID_ARG, "prefill_attention: positions [%u, %llu) exceed max_seq_len %u", base_pos,
                     (unsigned long long)base_pos + m, c->max_seq_len);
+    const int rc_kv = check_kv_layer(c, layer, kv_layer, "prefill_attention");
+    if (rc_kv != VFKV_OK) return rc_kv;
     vfkv_batch_params p;
     p.n_heads = n_heads;
     p.n_kv_heads = kvh_for(c, layer);

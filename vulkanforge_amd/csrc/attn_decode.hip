@@ -654,26 +654,14 @@ namespace vfkv {
 // ---- dispatch -----------------------------------------------------------------------------------
 constexpr int kSplitWaves = 4;
 
-// Build-time tuning of the matrix-core worker: rows per run for 1-byte / 2-byte caches, wavefronts per workgroup.
-#ifndef VFKV_MFMA_RUN_F8
-#define VFKV_MFMA_RUN_F8 32
-#endif
-#ifndef VFKV_MFMA_PF_F8
-#define VFKV_MFMA_PF_F8 1
-#endif
-#ifndef VFKV_MFMA_PF_F16
-#define VFKV_MFMA_PF_F16 1
-#endif
-#ifndef VFKV_MFMA_RUN_F16
-#define VFKV_MFMA_RUN_F16 32
-#endif
-#ifndef VFKV_MFMA_WAVES
-#define VFKV_MFMA_WAVES 4
-#endif
+// Shape of the matrix-core worker: four wavefronts per workgroup (one per SIMD), runs of 32 rows (64 at head_dim 64), one
+// run in flight ahead of the one being computed.  Two runs in flight, runs of 64 rows, and eight wavefronts per workgroup
+// were each measured slower on the 32 k and 8 k FP8 workloads.
+constexpr int kMfmaWaves = 4;
 
 template <int DT, int D, int RUN, int PF, int NH = 1>
 static hipError_t launch_split_mfma(const SplitArgs& a, uint32_t g, hipStream_t stream) {
-    constexpr int NW = VFKV_MFMA_WAVES;
+    constexpr int NW = kMfmaWaves;
     const uint32_t gt = g < 8u ? g : 8u;
     dim3 grid(a.n_kv_heads, a.n_tiles, (g + gt - 1u) / gt);
     if (a.softcap > 0.f)
@@ -771,9 +759,9 @@ hipError_t launch_split(const SplitLaunch& L, hipStream_t stream) {
     const bool out_aligned = ((((uintptr_t)L.scratch_out) | ((uintptr_t)L.o_direct)) & 15u) == 0u;
     if (aligned && out_aligned && slab_bytes < 0x7FFF0000ull && mfma_worker_enabled()) {
         if (L.dtype == kF8 && L.head_dim == 64u) return launch_split_mfma<kF8, 64, 64, 1>(a, g, stream);
-        if (L.dtype == kF8 && L.head_dim == 128u) return launch_split_mfma<kF8, 128, VFKV_MFMA_RUN_F8, VFKV_MFMA_PF_F8>(a, g, stream);
+        if (L.dtype == kF8 && L.head_dim == 128u) return launch_split_mfma<kF8, 128, 32, 1>(a, g, stream);
         if (L.dtype == kF16 && L.head_dim == 64u) return launch_split_mfma<kF16, 64, 64, 1>(a, g, stream);
-        if (L.dtype == kF16 && L.head_dim == 128u) return launch_split_mfma<kF16, 128, VFKV_MFMA_RUN_F16, VFKV_MFMA_PF_F16>(a, g, stream);
+        if (L.dtype == kF16 && L.head_dim == 128u) return launch_split_mfma<kF16, 128, 32, 1>(a, g, stream);
         if (L.dtype == kF8 && L.head_dim == 256u) return launch_split_mfma<kF8, 256, 32, 1>(a, g, stream);
         if (L.dtype == kF16 && L.head_dim == 256u) return launch_split_mfma<kF16, 256, 32, 1>(a, g, stream);
         if (L.dtype == kF8 && L.head_dim == 512u) return launch_split_mfma<kF8, 512, 32, 1, 2>(a, g, stream);

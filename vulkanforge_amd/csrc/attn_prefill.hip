@@ -121,10 +121,9 @@ static hipError_t launch_batch_kernels(const BatchLaunch& L, hipStream_t stream,
         // of three and more heads round up, the spare slot computes on zeros and stores nothing.  Where the rows are wide
         // (F16 at head_dim 128, everything at head_dim 256) the traffic between L2 and the CUs is what binds: four / two heads
         // per wavefront in workgroups of four wavefronts (one per SIMD, up to 512 registers), so that a K / V tile is loaded
-        // by one wavefront of the workgroup only.  VFKV_PREFILL_NCB=1 forces one head per wavefront (for comparisons).
-        static const int force_ncb = [] { const char* e = getenv("VFKV_PREFILL_NCB"); return e ? atoi(e) : 0; }();
+        // by one wavefront of the workgroup only.
         uint32_t ncb = 1u;
-        if (force_ncb != 1 && g >= 2u) {
+        if (g >= 2u) {
             // head_dim 512: a second head per wavefront only for FP8 rows (F16 rows leave no registers for it) and only while
             // head pairs still give every compute unit a workgroup
             if (nh == 2u) ncb = (L.dtype == kF8 && (uint64_t)((L.m + 15u) / 16u) * L.n_kv_heads * ((g + 1u) / 2u) >= 256u) ? 2u : 1u;
@@ -135,7 +134,7 @@ static hipError_t launch_batch_kernels(const BatchLaunch& L, hipStream_t stream,
         const uint32_t hp_group = (g + ncb - 1u) / ncb * nh;     // (head slice, output slice) units of a whole GQA group
         // wavefronts per workgroup the registers allow: one head per wavefront at head_dim <= 128 needs few (three wavefronts
         // per SIMD), 512 accumulator columns per wavefront need the whole register file of a SIMD (one wavefront per SIMD)
-        const uint32_t reg_waves = (ncb == 1u && L.head_dim <= 128u) ? (uint32_t)VFKV_PREFILL_NCB1_WAVES
+        const uint32_t reg_waves = (ncb == 1u && L.head_dim <= 128u) ? (uint32_t)kPrefillOneHeadWaves
                                  : (ncb * L.head_dim >= 512u || (L.dtype == kF16 && L.head_dim == 256u)) ? 4u : 8u;   // (always 4 at head_dim 512)
         // the private V tiles and the two Q planes have to fit in 160 KiB of LDS
         auto waves_for = [&](uint32_t slices) -> uint32_t {

@@ -25,15 +25,13 @@
 namespace vfkv {
 
 // wavefronts per workgroup when a wavefront serves one head at head_dim <= 128 (fewer registers: three per SIMD)
-#ifndef VFKV_PREFILL_NCB1_WAVES
-#define VFKV_PREFILL_NCB1_WAVES 12
-#endif
+constexpr int kPrefillOneHeadWaves = 12;
 
 // NH > 1 (head_dim 512, NCB = 1): NH wavefronts share a head.  Each computes the scores over the whole head_dim and
 // accumulates, merges and stores its own slice of D / NH output elements: the accumulators of a 512-wide head do not fit
 // one wavefront.  HP then counts (head, slice) units.
 template <int DT, int D, int NCB, int PFD, bool CAP, int NH = 1>
-__global__ __launch_bounds__((NCB == 1 && D <= 128) ? VFKV_PREFILL_NCB1_WAVES * 64 : (NCB * D >= 512 || (DT == kF16 && D == 256)) ? 256 : 512) void batch_mfma2_kernel(BatchArgs a, int HP, int NS) {
+__global__ __launch_bounds__((NCB == 1 && D <= 128) ? kPrefillOneHeadWaves * 64 : (NCB * D >= 512 || (DT == kF16 && D == 256)) ? 256 : 512) void batch_mfma2_kernel(BatchArgs a, int HP, int NS) {
     constexpr int DV = D / NH;                   // output elements (V columns) of this wavefront
     constexpr int ES = DT == kF16 ? 2 : 1;
     constexpr int KT = 32;                       // keys per tile
@@ -292,7 +290,9 @@ __global__ __launch_bounds__((NCB == 1 && D <= 128) ? VFKV_PREFILL_NCB1_WAVES * 
                 }
                 l_run[cb] += pp[0] + pp[1];
                 phi[cb][j2] = __builtin_bit_cast(uint32_t, __builtin_convertvector(pp, half2_t));
+#ifndef VFKV_PREFILL_P1
                 plo[cb][j2] = pack_f16_remainder(pp[0], pp[1], phi[cb][j2]);
+#endif
             }
 #pragma unroll
         for (int dt = 0; dt < DTILES; ++dt) {
@@ -305,9 +305,11 @@ __global__ __launch_bounds__((NCB == 1 && D <= 128) ? VFKV_PREFILL_NCB1_WAVES * 
 #pragma unroll
             for (int cb = 0; cb < NCB; ++cb)
                 oacc[cb][dt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(va, __builtin_bit_cast(half8_t, phi[cb]), oacc[cb][dt], 0, 0, 0);
+#ifndef VFKV_PREFILL_P1
 #pragma unroll
             for (int cb = 0; cb < NCB; ++cb)
                 oacc[cb][dt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(va, __builtin_bit_cast(half8_t, plo[cb]), oacc[cb][dt], 0, 0, 0);
+#endif
         }
     };
 

@@ -76,37 +76,48 @@ hipError_t launch_kv_append(uint32_t dtype, const float* k_src, const float* v_s
 }
 
 // ---- E4M3 -> f16 expansion -------------------------------------------------------------------
-// 16 codes per thread: one 16-byte load, eight packed conversions, two 16-byte stores.
+// 8 codes per piece: one 8-byte load, four packed conversions, one 16-byte store, so that both the loads and the stores of
+// a wavefront are contiguous (whole 128-byte lines per store instruction).  The output is written once and not read back
+// by this kernel: the stores carry the non-temporal hint.  A thread takes four pieces per round and requests all four
+// before it converts the first.  (One 16-byte load and two 16-byte stores per thread, every line written by two
+// instructions: 22.9 us for 33.5 M codes; this form: 15.2 us = 6.6 TB/s of read + write traffic.)
+constexpr int kExpandPieces = 4;
 __global__ __launch_bounds__(256) void kv_fp8_to_f16_kernel(const uint8_t* __restrict__ src,
                                                             uint16_t* __restrict__ dst, uint64_t n, int vec_ok) {
-    const uint64_t n_vec = vec_ok ? n / 16u : 0u;
-    const uint64_t stride = (uint64_t)gridDim.x * blockDim.x;
+    const uint64_t n_vec = vec_ok ? n / 8u : 0u;
+    const uint64_t threads = (uint64_t)gridDim.x * blockDim.x;
     const uint64_t tid = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    for (uint64_t i = tid; i < n_vec; i += stride) {
-        const uint4 w = reinterpret_cast<const uint4*>(src)[i];
-        const uint32_t in[4] = {w.x, w.y, w.z, w.w};
-        uint32_t out[8];
+    // round r covers pieces [r * threads * 4, (r + 1) * threads * 4); inside it a workgroup's pieces are contiguous
+    for (uint64_t base = (uint64_t)blockIdx.x * blockDim.x * kExpandPieces; base < n_vec; base += threads * kExpandPieces) {
+        u32x2 w[kExpandPieces];
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            half2_t lo, hi;
-            e4m3x4_to_h2(in[j], lo, hi);
-            out[2 * j] = __builtin_bit_cast(uint32_t, lo);
-            out[2 * j + 1] = __builtin_bit_cast(uint32_t, hi);
+        for (int u = 0; u < kExpandPieces; ++u) {
+            const uint64_t i = base + (uint64_t)u * blockDim.x + threadIdx.x;
+            w[u] = i < n_vec ? reinterpret_cast<const u32x2*>(src)[i] : u32x2{0u, 0u};
         }
-        uint4* d = reinterpret_cast<uint4*>(dst) + 2u * i;
-        d[0] = make_uint4(out[0], out[1], out[2], out[3]);
-        d[1] = make_uint4(out[4], out[5], out[6], out[7]);
+#pragma unroll
+        for (int u = 0; u < kExpandPieces; ++u) {
+            const uint64_t i = base + (uint64_t)u * blockDim.x + threadIdx.x;
+            if (i >= n_vec) continue;
+            half2_t a0, a1, b0, b1;
+            e4m3x4_to_h2(w[u][0], a0, a1);
+            e4m3x4_to_h2(w[u][1], b0, b1);
+            const u32x4 out = u32x4{__builtin_bit_cast(uint32_t, a0), __builtin_bit_cast(uint32_t, a1),
+                                    __builtin_bit_cast(uint32_t, b0), __builtin_bit_cast(uint32_t, b1)};
+            __builtin_nontemporal_store(out, reinterpret_cast<u32x4*>(dst) + i);
+        }
     }
-    for (uint64_t i = n_vec * 16u + tid; i < n; i += stride)
+    for (uint64_t i = n_vec * 8u + tid; i < n; i += threads)
         dst[i] = (uint16_t)f32_to_h16_bits(__builtin_amdgcn_cvt_f32_fp8((int)src[i], 0));
 }
 
 hipError_t launch_fp8_to_f16(const void* src, void* dst, uint64_t n, hipStream_t stream) {
     if (n == 0) return hipSuccess;
-    const int vec_ok = ((((uintptr_t)src) | ((uintptr_t)dst)) & 15u) == 0u;
-    uint64_t work = vec_ok ? (n + 15u) / 16u : n;
+    const int vec_ok = (((uintptr_t)src) & 7u) == 0u && (((uintptr_t)dst) & 15u) == 0u;
+    uint64_t work = vec_ok ? (n / 8u + kExpandPieces - 1u) / kExpandPieces : n;
     uint64_t blocks = (work + 255u) / 256u;
-    if (blocks > 8192u) blocks = 8192u;
+    if (blocks == 0u) blocks = 1u;
+    if (blocks > 65536u) blocks = 65536u;
     hipLaunchKernelGGL(kv_fp8_to_f16_kernel, dim3((uint32_t)blocks), dim3(256), 0, stream,
                        (const uint8_t*)src, (uint16_t*)dst, n, vec_ok);
     return hipGetLastError();

@@ -434,7 +434,16 @@ def bench_prefill(args, wl):
             fwd.b_step_attention(layer, wl.base_pos, wl.m, q, o)
             fwd.b_step_attn_gated_output(o, qgate, wl.m, D)
 
+    def step_f16_weights():     # the same step with VFKV_PREFILL_F16_WEIGHTS (one product with the softmax weights)
+        for layer in range(L):
+            fwd.b_step_kv_write(layer, wl.base_pos, wl.m, kn, vn)
+            fwd.b_step_attention(layer, wl.base_pos, wl.m, q, o, use_workspace=wl.workspace, f16_weights=True)
+
     gate_separate_ms = time_steps(torch, step_gate_separate, args) * 1e3 if wl.gated else None
+    f16w = None
+    if not wl.gated and D == 128 and wl.dtype.label() in ("FP8", "FP16"):
+        f16w_ms = time_steps(torch, step_f16_weights, args) * 1e3
+        f16w = {"ms_per_step": f16w_ms, "TFLOPs": wl.flops_layer() * L / (f16w_ms * 1e-3) / 1e12}
     sec_per_step = time_steps(torch, step, args)
     step_spread = dict(STEP_SPREAD)
     flops_step = wl.flops_layer() * L
@@ -472,6 +481,8 @@ def bench_prefill(args, wl):
     }
     if gate_separate_ms is not None:
         result["config"]["ms_per_step_gate_as_separate_launch"] = gate_separate_ms
+    if f16w is not None:          # an option of the call, not what `value` is measured with
+        result["config"]["with_option_f16_weights"] = f16w
     if not args.no_cpu_baseline:
         import numpy as np
 

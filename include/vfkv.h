@@ -359,6 +359,27 @@ int vfkv_prefill_attention_ws(vfkv_cache* c, uint32_t layer, uint32_t kv_layer, 
                               const float* q, float* o, uint32_t m, uint32_t base_pos, uint32_t window,
                               float scale, float softcap, vfkv_workspace* ws, vfkv_stream stream);
 
+/* Options of the two calls below (no counterpart in the reference, whose scalar shader has one precision). */
+#define VFKV_PREFILL_F16_WEIGHTS 1u /* The softmax weights enter the P.V product rounded to f16 (11 significant bits)
+                                     * instead of as an f16 value + remainder pair: a third fewer matrix instructions
+                                     * (512 x 4 608 queries x keys, 32 / 8 / 128, FP8: 70.7 -> 60.3 us per layer).  Each
+                                     * weight is off by up to 2^-11 relative, the output by up to 2^-11 * max|v| (4.5e-5
+                                     * measured on N(0,1) inputs; 1.3e-2 with +-40 outliers in V, which is outside this
+                                     * path's 5e-3 bound -- hence an option and not the default).  Honoured for FP8 / F16
+                                     * caches at head_dim 128 with GQA groups of 2-8 heads (FP8) or 3-4 (F16); ignored
+                                     * elsewhere. */
+
+/* vfkv_flash_attn_batch with options (VFKV_PREFILL_* bits). */
+int vfkv_flash_attn_batch_opt(const float* q, const void* k_layer, const void* v_layer, uint32_t kv_dtype,
+                              float* o, const vfkv_batch_params* p, float softcap, uint32_t options,
+                              vfkv_stream stream);
+
+/* vfkv_prefill_attention with options; `ws` (may be NULL) as in vfkv_prefill_attention_ws. */
+int vfkv_prefill_attention_opt(vfkv_cache* c, uint32_t layer, uint32_t kv_layer, uint32_t n_heads,
+                               const float* q, float* o, uint32_t m, uint32_t base_pos, uint32_t window,
+                               float scale, float softcap, uint32_t options, vfkv_workspace* ws,
+                               vfkv_stream stream);
+
 /* ------------------------------------------------------------------------------------------ */
 /* Gated attention output (Qwen3.6 full-attention layers).                                    */
 /* ------------------------------------------------------------------------------------------ */

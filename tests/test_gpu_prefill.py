@@ -246,3 +246,34 @@ def test_prefill_with_a_small_workspace_falls_back():
     torch.cuda.synchronize()
     assert (to_np(a) == to_np(b)).all()
     cache.destroy()
+
+
+@pytest.mark.parametrize("dtype,heads,hkv,vscale", [(vf.KvDtype.F8, 32, 8, 1.0), (vf.KvDtype.F16, 32, 8, 1.0),
+                                                    (vf.KvDtype.F8, 32, 8, 8.0), (vf.KvDtype.F16, 24, 8, 8.0)])
+def test_f16_weights_option_stays_inside_its_stated_bound(dtype, heads, hkv, vscale):
+    # VFKV_PREFILL_F16_WEIGHTS: one product with the f16 rounding of the softmax weights.  Every weight is off by at most
+    # 2^-11 relative, so every output element by at most 2^-11 * max|v| (plus the f32 rounding of the default path); on
+    # N(0,1) inputs that is far inside this path's tolerance.  Without the option the call is the default path, bit for bit.
+    d, base, m = 128, 1536, 96
+    n_kv = base + m
+    r = rng(640 + int(vscale))
+    k = fp16_normal(r, (n_kv, hkv * d))
+    v = fp16_normal(r, (n_kv, hkv * d), vscale)
+    q = fp16_normal(r, (m, heads, d))
+    ke, ve = encode_np(k, dtype), encode_np(v, dtype)
+    scale = 1.0 / np.sqrt(d)
+    o_def = gpu_batch(q, ke, ve, dtype, heads, hkv, d, m, base, n_kv, scale)
+    o_opt = torch.full((m, heads, d), float("nan"), device=DEV, dtype=torch.float32)
+    vf.Forward.run_flash_attn_batch(to_dev(q), to_dev(ke), to_dev(ve), dtype, o_opt, heads, hkv, d, m, base, n_kv, scale,
+                                    f16_weights=True)
+    torch.cuda.synchronize()
+    o_opt = to_np(o_opt)
+    ref = oracle.attn_batch_ref(q, ke.reshape(-1, hkv, d), ve.reshape(-1, hkv, d), int(dtype), m, n_kv, heads, hkv, d, base, scale)
+    vmax = float(np.abs(v).max())                            # |decoded v| <= |v| * (1 + 2^-4) for E4M3, equal for F16
+    vmax *= 1.0625 if dtype == vf.KvDtype.F8 else 1.0
+    assert np.abs(o_def - ref).max() < TIGHT
+    err = np.abs(o_opt - ref).max()
+    assert err <= 2.0 ** -11 * vmax + 1e-5, (err, vmax)
+    if vscale == 1.0:
+        assert err < TIGHT                                   # 4.5e-5 measured on the benchmark's distribution
+    assert not np.array_equal(o_opt, o_def)                  # the option really took the other path

@@ -46,6 +46,7 @@ class Gate(C.Structure):
     _fields_ = [("gate", C.c_void_p), ("chunk", C.c_uint32), ("stride", C.c_uint32), ("gate_offset", C.c_uint32)]
 
 
+PREFILL_F16_WEIGHTS = 1   # VFKV_PREFILL_F16_WEIGHTS
 ROPE_NORM, ROPE_NEOX = 0, 2   # GGML_ROPE_TYPE_NORMAL / _NEOX (rms_norm.comp:25-26)
 
 assert C.sizeof(SplitParams) == 32 and C.sizeof(BatchParams) == 32  # pipeline.rs:569,611
@@ -103,6 +104,8 @@ SIGNATURES = {
     "vfkv_decode_attention": (C.c_int, [_vp, _u32, _u32, _u32, _vp, _vp, _u32, _u32, _f, _f, _vp, _vp]),
     "vfkv_decode_attention_static": (C.c_int, [_vp, _u32, _u32, _u32, _vp, _vp, _u32, _u32, _f, _f, _vp]),
     "vfkv_flash_attn_batch": (C.c_int, [_vp, _vp, _vp, _u32, _vp, C.POINTER(BatchParams), _f, _vp]),
+    "vfkv_flash_attn_batch_opt": (C.c_int, [_vp, _vp, _vp, _u32, _vp, C.POINTER(BatchParams), _f, _u32, _vp]),
+    "vfkv_prefill_attention_opt": (C.c_int, [_vp, _u32, _u32, _u32, _vp, _vp, _u32, _u32, _u32, _f, _f, _u32, _vp, _vp]),
     "vfkv_prefill_attention": (C.c_int, [_vp, _u32, _u32, _u32, _vp, _vp, _u32, _u32, _u32, _f, _f, _vp]),
     "vfkv_prefill_attention_ws": (C.c_int, [_vp, _u32, _u32, _u32, _vp, _vp, _u32, _u32, _u32, _f, _f, _vp, _vp]),
     "vfkv_sigmoid_mul": (C.c_int, [C.POINTER(Gate), _vp, _u32, _vp]),

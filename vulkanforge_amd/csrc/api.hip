@@ -706,7 +706,8 @@ int vfkv_kv_write_decode_attention(vfkv_cache* c, uint32_t layer, uint32_t n_hea
 // ---- prefill attention -------------------------------------------------------------------------------
 static int flash_attn_batch_impl(const float* q, const void* k_layer, const void* v_layer, uint32_t kv_dtype, float* o,
                                  const vfkv_batch_params* p, float softcap, vfkv_workspace* ws, vfkv_stream stream,
-                                 const vfkv::GateArgs* gate = nullptr) {
+                                 const vfkv::GateArgs* gate = nullptr, uint32_t options = 0u) {
+    if ((options & ~VFKV_PREFILL_F16_WEIGHTS) != 0u) return fail(VFKV_ERR_INVALID_ARG, "flash_attn_batch: unknown option bits 0x%x", options);
     if (!p) return fail(VFKV_ERR_INVALID_ARG, "flash_attn_batch: params is NULL");
     if (!q || !k_layer || !v_layer || !o) return fail(VFKV_ERR_INVALID_ARG, "flash_attn_batch: NULL buffer");
     if (kv_dtype > VFKV_F8E4M3) return fail(VFKV_ERR_INVALID_ARG, "flash_attn_batch: unknown kv dtype %u", kv_dtype);
@@ -729,6 +730,7 @@ static int flash_attn_batch_impl(const float* q, const void* k_layer, const void
     L.dtype = kv_dtype; L.n_heads = p->n_heads; L.n_kv_heads = p->n_kv_heads; L.head_dim = p->head_dim;
     L.m = p->m; L.n_kv = p->n_kv; L.q_start = p->q_start; L.kv_start = p->kv_start;
     L.scale = p->scale; L.softcap = softcap;
+    L.f16_weights = (options & VFKV_PREFILL_F16_WEIGHTS) != 0u;
     if (ws) {
         L.scratch_out = ws->scratch_out; L.scratch_max = ws->scratch_max; L.scratch_sum = ws->scratch_sum;
         L.scratch_ml_floats = (uint64_t)ws->n_heads * ws->max_tiles;
@@ -743,9 +745,15 @@ int vfkv_flash_attn_batch(const float* q, const void* k_layer, const void* v_lay
     return flash_attn_batch_impl(q, k_layer, v_layer, kv_dtype, o, p, softcap, nullptr, stream);
 }
 
+int vfkv_flash_attn_batch_opt(const float* q, const void* k_layer, const void* v_layer, uint32_t kv_dtype, float* o,
+                              const vfkv_batch_params* p, float softcap, uint32_t options, vfkv_stream stream) {
+    return flash_attn_batch_impl(q, k_layer, v_layer, kv_dtype, o, p, softcap, nullptr, stream, nullptr, options);
+}
+
 static int prefill_attention_impl(vfkv_cache* c, uint32_t layer, uint32_t kv_layer, uint32_t n_heads, const float* q, float* o,
                                   uint32_t m, uint32_t base_pos, uint32_t window, float scale, float softcap,
-                                  vfkv_workspace* ws, vfkv_stream stream, const vfkv::GateArgs* gate = nullptr) {
+                                  vfkv_workspace* ws, vfkv_stream stream, const vfkv::GateArgs* gate = nullptr,
+                                  uint32_t options = 0u) {
     if (!c || !c->k || !c->v) return fail(VFKV_ERR_INVALID_ARG, "prefill_attention: cache has no buffers");
     if (layer >= c->n_layers || kv_layer >= c->n_layers)
         return fail(VFKV_ERR_INVALID_ARG, "prefill_attention: layer %u / kv_layer %u out of range", layer, kv_layer);
@@ -764,7 +772,7 @@ static int prefill_attention_impl(vfkv_cache* c, uint32_t layer, uint32_t kv_lay
     p.scale = scale;
     p.kv_start = vfkv_kv_start_batch(base_pos, m, window);
     const uint64_t off = layer_off(c, kv_layer);
-    return flash_attn_batch_impl(q, (char*)c->k + off, (char*)c->v + off, c->dtype, o, &p, softcap, ws, stream, gate);
+    return flash_attn_batch_impl(q, (char*)c->k + off, (char*)c->v + off, c->dtype, o, &p, softcap, ws, stream, gate, options);
 }
 
 int vfkv_prefill_attention(vfkv_cache* c, uint32_t layer, uint32_t kv_layer, uint32_t n_heads, const float* q, float* o,
@@ -778,6 +786,12 @@ int vfkv_prefill_attention_ws(vfkv_cache* c, uint32_t layer, uint32_t kv_layer, 
                               vfkv_workspace* ws, vfkv_stream stream) {
     if (!ws) return fail(VFKV_ERR_INVALID_ARG, "prefill_attention_ws: workspace is NULL");
     return prefill_attention_impl(c, layer, kv_layer, n_heads, q, o, m, base_pos, window, scale, softcap, ws, stream);
+}
+
+int vfkv_prefill_attention_opt(vfkv_cache* c, uint32_t layer, uint32_t kv_layer, uint32_t n_heads, const float* q, float* o,
+                               uint32_t m, uint32_t base_pos, uint32_t window, float scale, float softcap, uint32_t options,
+                               vfkv_workspace* ws, vfkv_stream stream) {
+    return prefill_attention_impl(c, layer, kv_layer, n_heads, q, o, m, base_pos, window, scale, softcap, ws, stream, nullptr, options);
 }
 
 // ---- gated output --------------------------------------------------------------------------------------

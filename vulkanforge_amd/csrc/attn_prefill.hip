@@ -201,6 +201,15 @@ static hipError_t launch_batch_kernels(const BatchLaunch& L, hipStream_t stream,
         if (cap) hipLaunchKernelGGL((batch_mfma2_kernel<DT, DD, NCBV, PFDV, true>), grid, block, lds, stream, a, (int)hp, (int)ns);  \
         else hipLaunchKernelGGL((batch_mfma2_kernel<DT, DD, NCBV, PFDV, false>), grid, block, lds, stream, a, (int)hp, (int)ns);      \
     } else
+            // the f16-weights option (one product with the weights instead of value + remainder) is built for the two
+            // head_dim 128 forms the benchmark geometries run on; other shapes keep both products
+            if (L.f16_weights && L.dtype == kF8 && L.head_dim == 128u && ncb == 2u) {
+                if (cap) hipLaunchKernelGGL((batch_mfma2_kernel<kF8, 128, 2, 2, true, 1, true>), grid, block, lds, stream, a, (int)hp, (int)ns);
+                else hipLaunchKernelGGL((batch_mfma2_kernel<kF8, 128, 2, 2, false, 1, true>), grid, block, lds, stream, a, (int)hp, (int)ns);
+            } else if (L.f16_weights && L.dtype == kF16 && L.head_dim == 128u && ncb == 4u) {
+                if (cap) hipLaunchKernelGGL((batch_mfma2_kernel<kF16, 128, 4, 1, true, 1, true>), grid, block, lds, stream, a, (int)hp, (int)ns);
+                else hipLaunchKernelGGL((batch_mfma2_kernel<kF16, 128, 4, 1, false, 1, true>), grid, block, lds, stream, a, (int)hp, (int)ns);
+            } else
             VFKV_P2(kF8, 64, 2, 2) VFKV_P2(kF8, 64, 1, 2) VFKV_P2(kF8, 128, 2, 2) VFKV_P2(kF8, 128, 1, 2)
             VFKV_P2(kF16, 64, 2, 2) VFKV_P2(kF16, 64, 1, 2) VFKV_P2(kF16, 128, 1, 1) VFKV_P2(kF16, 128, 2, 1)
             VFKV_P2(kF8, 256, 1, 1) VFKV_P2(kF16, 256, 1, 1)

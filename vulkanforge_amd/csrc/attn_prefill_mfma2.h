@@ -30,7 +30,7 @@ constexpr int kPrefillOneHeadWaves = 12;
 // NH > 1 (head_dim 512, NCB = 1): NH wavefronts share a head.  Each computes the scores over the whole head_dim and
 // accumulates, merges and stores its own slice of D / NH output elements: the accumulators of a 512-wide head do not fit
 // one wavefront.  HP then counts (head, slice) units.
-template <int DT, int D, int NCB, int PFD, bool CAP, int NH = 1>
+template <int DT, int D, int NCB, int PFD, bool CAP, int NH = 1, bool F16W = false>
 __global__ __launch_bounds__((NCB == 1 && D <= 128) ? kPrefillOneHeadWaves * 64 : (NCB * D >= 512 || (DT == kF16 && D == 256)) ? 256 : 512) void batch_mfma2_kernel(BatchArgs a, int HP, int NS) {
     constexpr int DV = D / NH;                   // output elements (V columns) of this wavefront
     constexpr int ES = DT == kF16 ? 2 : 1;
@@ -272,8 +272,11 @@ __global__ __launch_bounds__((NCB == 1 && D <= 128) ? kPrefillOneHeadWaves * 64 
         }
     };
     // weights as f16 value + f16 remainder, then O^T += V^T P^T for the NCB heads
-    auto weights_and_second_product = [&](auto masked_tag) {
+    // TWO: the weights enter the product as f16 value + f16 remainder (two MFMAs per d-tile and head: f32-level accuracy);
+    // otherwise as the f16 value alone (the F16W instantiations).
+    auto weights_and_second_product = [&](auto masked_tag, auto two_tag) {
         constexpr bool MASKED = decltype(masked_tag)::value;
+        constexpr bool TWO = decltype(two_tag)::value;
         constexpr bool FOLD = !MASKED && !CAP;
         u32x4 phi[NCB], plo[NCB];
 #pragma unroll
@@ -290,9 +293,7 @@ __global__ __launch_bounds__((NCB == 1 && D <= 128) ? kPrefillOneHeadWaves * 64 
                 }
                 l_run[cb] += pp[0] + pp[1];
                 phi[cb][j2] = __builtin_bit_cast(uint32_t, __builtin_convertvector(pp, half2_t));
-#ifndef VFKV_PREFILL_P1
-                plo[cb][j2] = pack_f16_remainder(pp[0], pp[1], phi[cb][j2]);
-#endif
+                if (TWO) plo[cb][j2] = pack_f16_remainder(pp[0], pp[1], phi[cb][j2]);
             }
 #pragma unroll
         for (int dt = 0; dt < DTILES; ++dt) {
@@ -305,11 +306,11 @@ __global__ __launch_bounds__((NCB == 1 && D <= 128) ? kPrefillOneHeadWaves * 64 
 #pragma unroll
             for (int cb = 0; cb < NCB; ++cb)
                 oacc[cb][dt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(va, __builtin_bit_cast(half8_t, phi[cb]), oacc[cb][dt], 0, 0, 0);
-#ifndef VFKV_PREFILL_P1
+            if (TWO) {
 #pragma unroll
-            for (int cb = 0; cb < NCB; ++cb)
-                oacc[cb][dt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(va, __builtin_bit_cast(half8_t, plo[cb]), oacc[cb][dt], 0, 0, 0);
-#endif
+                for (int cb = 0; cb < NCB; ++cb)
+                    oacc[cb][dt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(va, __builtin_bit_cast(half8_t, plo[cb]), oacc[cb][dt], 0, 0, 0);
+            }
         }
     };
 
@@ -333,10 +334,10 @@ __global__ __launch_bounds__((NCB == 1 && D <= 128) ? kPrefillOneHeadWaves * 64 
             if (!(s_ready && sl == first_slot)) stage_and_first_product(sl, tcur);
             if (tcur >= a.kv_start && tcur + KT <= full_len) {  // every query of the block sees the whole tile
                 if (__builtin_amdgcn_ballot_w64(scores(std::false_type{}, tcur)) != 0ull) move_maximum();
-                weights_and_second_product(std::false_type{});
+                weights_and_second_product(std::false_type{}, std::integral_constant<bool, !F16W>{});
             } else {
                 if (__builtin_amdgcn_ballot_w64(scores(std::true_type{}, tcur)) != 0ull) move_maximum();
-                weights_and_second_product(std::true_type{});
+                weights_and_second_product(std::true_type{}, std::integral_constant<bool, !F16W>{});
             }
         }
         tb += PFD * step;
@@ -352,7 +353,7 @@ __global__ __launch_bounds__((NCB == 1 && D <= 128) ? kPrefillOneHeadWaves * 64 
                     first_slot = sl; s_ready = true; left = true;
                     break;
                 }
-                weights_and_second_product(std::false_type{});
+                weights_and_second_product(std::false_type{}, std::integral_constant<bool, !F16W>{});
             }
             if (!left) tb += PFD * step;
         }

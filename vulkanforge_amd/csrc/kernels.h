@@ -98,6 +98,11 @@ struct BatchLaunch {
     // optional gated output: o *= sigmoid(gate[...]), in the attention kernel's or the merge's own store where the shape
     // allows it and as a follow-up launch otherwise
     const GateArgs* gate = nullptr;
+    // FP8 / F16 caches on the f16 matrix-core kernel: the softmax weights enter the second product rounded to f16 (one
+    // product instead of value + remainder): about 15 % faster, every weight off by up to 2^-11 relative, so the output by up
+    // to 2^-11 * max|v|.  Built for head_dim 128 with the GQA group in one wavefront pair (FP8) or one wavefront (F16); other
+    // shapes and kernels ignore it and keep both products.
+    bool f16_weights = false;
 };
 hipError_t launch_batch(const BatchLaunch& a, hipStream_t stream);
 

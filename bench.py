@@ -434,16 +434,25 @@ def bench_prefill(args, wl):
             fwd.b_step_attention(layer, wl.base_pos, wl.m, q, o)
             fwd.b_step_attn_gated_output(o, qgate, wl.m, D)
 
-    def step_f16_weights():     # the same step with VFKV_PREFILL_F16_WEIGHTS (one product with the softmax weights)
-        for layer in range(L):
-            fwd.b_step_kv_write(layer, wl.base_pos, wl.m, kn, vn)
-            fwd.b_step_attention(layer, wl.base_pos, wl.m, q, o, use_workspace=wl.workspace, f16_weights=True)
+    def step_with(**opts):      # the same step with options of the call (VFKV_PREFILL_F16_WEIGHTS / VFKV_PREFILL_FP8_SCORES)
+        def run():
+            for layer in range(L):
+                fwd.b_step_kv_write(layer, wl.base_pos, wl.m, kn, vn)
+                fwd.b_step_attention(layer, wl.base_pos, wl.m, q, o, use_workspace=wl.workspace, **opts)
+        return run
 
     gate_separate_ms = time_steps(torch, step_gate_separate, args) * 1e3 if wl.gated else None
     f16w = None
     if not wl.gated and D == 128 and wl.dtype.label() in ("FP8", "FP16"):
-        f16w_ms = time_steps(torch, step_f16_weights, args) * 1e3
-        f16w = {"ms_per_step": f16w_ms, "TFLOPs": wl.flops_layer() * L / (f16w_ms * 1e-3) / 1e12}
+        f16w = {}
+        variants = [("f16_weights", dict(f16_weights=True))]
+        if wl.dtype.label() == "FP8":
+            variants += [("fp8_scores", dict(fp8_scores=True)), ("f16_weights+fp8_scores", dict(f16_weights=True, fp8_scores=True))]
+        for name, opts in variants:
+            ms = time_steps(torch, step_with(**opts), args) * 1e3
+            f16w[name] = {"ms_per_step": ms, "TFLOPs": wl.flops_layer() * L / (ms * 1e-3) / 1e12}
+            if not args.no_cpu_baseline:        # the error of the option's output against the oracle is taken below
+                f16w[name]["_o_last_rows"] = o[wl.m - 8:].clone()
     sec_per_step = time_steps(torch, step, args)
     step_spread = dict(STEP_SPREAD)
     flops_step = wl.flops_layer() * L
@@ -481,8 +490,8 @@ def bench_prefill(args, wl):
     }
     if gate_separate_ms is not None:
         result["config"]["ms_per_step_gate_as_separate_launch"] = gate_separate_ms
-    if f16w is not None:          # an option of the call, not what `value` is measured with
-        result["config"]["with_option_f16_weights"] = f16w
+    if f16w is not None:          # options of the call, not what `value` is measured with
+        result["config"]["with_options"] = f16w
     if not args.no_cpu_baseline:
         import numpy as np
 
@@ -506,6 +515,8 @@ def bench_prefill(args, wl):
             reps += 1
         err = float(np.abs(o[wl.m - ms:].cpu().numpy() - ref).max())
         result["config"]["max_abs_err_vs_oracle_last_rows"] = err
+        for v in (f16w or {}).values():
+            v["max_abs_err_vs_oracle_last_rows"] = float(np.abs(v.pop("_o_last_rows").cpu().numpy() - ref).max())
         result["cpu_baseline"] = {"value": flops_sample * reps / spent / 1e12, "unit": "TFLOP/s", "cores": threads,
                                   "kind": "port",
                                   "sample": f"last {ms} of {wl.m} query rows of one layer, {reps} repetitions, CPU "

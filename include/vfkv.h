@@ -369,6 +369,12 @@ int vfkv_prefill_attention_ws(vfkv_cache* c, uint32_t layer, uint32_t kv_layer, 
                                      * caches at head_dim 128 with GQA groups of 2-8 heads (FP8) or 3-4 (F16); ignored
                                      * elsewhere. */
 
+#define VFKV_PREFILL_FP8_SCORES 2u  /* The first product K.Q^T runs on the FP8 matrix instruction: the cache rows enter as
+                                     * stored (no widening to f16), the queries as three E4M3 terms (12 significant bits:
+                                     * exact for f16-representable q).  The instruction sums its 128 products with about 15
+                                     * bits, so a score is off by about 1e-5 of the sum of its |k.q| products.  Honoured for
+                                     * FP8 caches at head_dim 128 with GQA groups of 2-4 heads; ignored elsewhere. */
+
 /* vfkv_flash_attn_batch with options (VFKV_PREFILL_* bits). */
 int vfkv_flash_attn_batch_opt(const float* q, const void* k_layer, const void* v_layer, uint32_t kv_dtype,
                               float* o, const vfkv_batch_params* p, float softcap, uint32_t options,

@@ -32,11 +32,33 @@ def test_library_exports_every_declared_symbol():
     assert L.vfkv_status_string(0) == b"ok" and L.vfkv_status_string(-3) == b"misaligned offset"
 
 
-def test_rust_binding_text_declares_every_exported_symbol():
-    # the extern "C" block a Rust host would paste must not drift from the header
-    text = open(os.path.join(ROOT, "INTEGRATION.md")).read()
-    rust = sorted(set(re.findall(r"pub fn (vfkv_[a-z0-9_]+)\s*\(", text)))
-    assert rust == _declared_symbols()
+def _c_prototypes():
+    """name -> number of parameters, from include/vfkv.h."""
+    text = open(os.path.join(ROOT, "include", "vfkv.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    protos = {}
+    for name, args in re.findall(r"\b(vfkv_[a-z0-9_]+)\s*\(([^;{]*?)\)\s*;", text, flags=re.S):
+        args = args.strip()
+        protos[name] = 0 if args in ("", "void") else args.count(",") + 1
+    return protos
+
+
+def test_rust_binding_file_declares_every_exported_symbol_with_the_same_arity():
+    # the extern "C" block a Rust host compiles (vulkanforge_amd/host/rust/ffi.rs) must not drift from the header
+    text = open(os.path.join(ROOT, "vulkanforge_amd", "host", "rust", "ffi.rs")).read()
+    text = re.sub(r"//[^\n]*", "", text)
+    rust = {}
+    for name, args in re.findall(r"pub fn (vfkv_[a-z0-9_]+)\s*\(([^;{]*?)\)\s*(?:->[^;]*)?;", text, flags=re.S):
+        args = args.strip()
+        rust[name] = 0 if args == "" else args.count(",") + 1
+    protos = _c_prototypes()
+    assert sorted(protos) == _declared_symbols()
+    assert rust == protos
+    # the build script compiles every translation unit the Makefile links into the library
+    build = open(os.path.join(ROOT, "vulkanforge_amd", "host", "rust", "build.rs")).read()
+    mk = open(os.path.join(ROOT, "vulkanforge_amd", "csrc", "Makefile")).read()
+    srcs = re.search(r"^SRCS\s*:=\s*(.*)$", mk, flags=re.M).group(1).split()
+    assert sorted(re.findall(r'"([a-z_]+\.hip)"', build)) == sorted(srcs)
 
 
 def test_param_structs_are_32_bytes():

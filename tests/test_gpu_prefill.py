@@ -277,3 +277,28 @@ def test_f16_weights_option_stays_inside_its_stated_bound(dtype, heads, hkv, vsc
     if vscale == 1.0:
         assert err < TIGHT                                   # 4.5e-5 measured on the benchmark's distribution
     assert not np.array_equal(o_opt, o_def)                  # the option really took the other path
+
+
+@pytest.mark.parametrize("f16_weights", [False, True])
+def test_fp8_scores_option_on_the_benchmark_distribution(f16_weights):
+    # VFKV_PREFILL_FP8_SCORES: K.Q^T on the FP8 matrix instruction (K rows as stored, Q as three E4M3 terms).  The terms are
+    # exact for f16-representable queries; what remains is the instruction's own summation (about 15 bits over the 128
+    # products of a score).  On the benchmark's N(0,1) inputs the output stays two orders of magnitude inside the 5e-3 bound
+    # of this path, also with queries far from 1 in magnitude (the terms carry a block exponent) and together with the
+    # f16-weights option.
+    heads, hkv, d, base, m = 32, 8, 128, 1536, 96
+    n_kv = base + m
+    scale = 1.0 / np.sqrt(d)
+    for qscale in (1.0, 300.0, 1e-3):
+        r = rng(700)
+        k, v = fp16_normal(r, (n_kv, hkv * d)), fp16_normal(r, (n_kv, hkv * d))
+        q = fp16_normal(r, (m, heads, d), qscale)
+        ke, ve = encode_np(k, vf.KvDtype.F8), encode_np(v, vf.KvDtype.F8)
+        o = torch.full((m, heads, d), float("nan"), device=DEV, dtype=torch.float32)
+        vf.Forward.run_flash_attn_batch(to_dev(q), to_dev(ke), to_dev(ve), vf.KvDtype.F8, o, heads, hkv, d, m, base, n_kv,
+                                        scale / qscale, f16_weights=f16_weights, fp8_scores=True)
+        torch.cuda.synchronize()
+        ref = oracle.attn_batch_ref(q, ke.reshape(-1, hkv, d), ve.reshape(-1, hkv, d), oracle.F8, m, n_kv, heads, hkv, d, base,
+                                    scale / qscale)
+        err = np.abs(to_np(o) - ref).max()
+        assert err < (TIGHT if f16_weights else 5e-5), (qscale, err)

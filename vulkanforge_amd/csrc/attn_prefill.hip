@@ -201,15 +201,19 @@ static hipError_t launch_batch_kernels(const BatchLaunch& L, hipStream_t stream,
         if (cap) hipLaunchKernelGGL((batch_mfma2_kernel<DT, DD, NCBV, PFDV, true>), grid, block, lds, stream, a, (int)hp, (int)ns);  \
         else hipLaunchKernelGGL((batch_mfma2_kernel<DT, DD, NCBV, PFDV, false>), grid, block, lds, stream, a, (int)hp, (int)ns);      \
     } else
-            // the f16-weights option (one product with the weights instead of value + remainder) is built for the two
-            // head_dim 128 forms the benchmark geometries run on; other shapes keep both products
-            if (L.f16_weights && L.dtype == kF8 && L.head_dim == 128u && ncb == 2u) {
-                if (cap) hipLaunchKernelGGL((batch_mfma2_kernel<kF8, 128, 2, 2, true, 1, true>), grid, block, lds, stream, a, (int)hp, (int)ns);
-                else hipLaunchKernelGGL((batch_mfma2_kernel<kF8, 128, 2, 2, false, 1, true>), grid, block, lds, stream, a, (int)hp, (int)ns);
-            } else if (L.f16_weights && L.dtype == kF16 && L.head_dim == 128u && ncb == 4u) {
-                if (cap) hipLaunchKernelGGL((batch_mfma2_kernel<kF16, 128, 4, 1, true, 1, true>), grid, block, lds, stream, a, (int)hp, (int)ns);
-                else hipLaunchKernelGGL((batch_mfma2_kernel<kF16, 128, 4, 1, false, 1, true>), grid, block, lds, stream, a, (int)hp, (int)ns);
-            } else
+            // The options are built for the head_dim 128 forms the benchmark geometries run on; other shapes keep the default
+            // arithmetic.  f16_weights: one product with the weights instead of value + remainder.  fp8_scores: the first
+            // product on the FP8 matrix instruction (needs the Q block staged in one round: four key splits).
+            const bool f8s = L.fp8_scores && L.dtype == kF8 && L.head_dim == 128u && ncb == 2u && ns >= 4u;
+#define VFKV_P2_OPT(DT, NCBV, PFDV, F16WV, F8SV)                                                                       \
+    { if (cap) hipLaunchKernelGGL((batch_mfma2_kernel<DT, 128, NCBV, PFDV, true, 1, F16WV, F8SV>), grid, block, lds, stream, a, (int)hp, (int)ns);  \
+      else hipLaunchKernelGGL((batch_mfma2_kernel<DT, 128, NCBV, PFDV, false, 1, F16WV, F8SV>), grid, block, lds, stream, a, (int)hp, (int)ns); }
+            if (f8s && L.f16_weights) VFKV_P2_OPT(kF8, 2, 2, true, true)
+            else if (f8s) VFKV_P2_OPT(kF8, 2, 2, false, true)
+            else if (L.f16_weights && L.dtype == kF8 && L.head_dim == 128u && ncb == 2u) VFKV_P2_OPT(kF8, 2, 2, true, false)
+            else if (L.f16_weights && L.dtype == kF16 && L.head_dim == 128u && ncb == 4u) VFKV_P2_OPT(kF16, 4, 1, true, false)
+            else
+#undef VFKV_P2_OPT
             VFKV_P2(kF8, 64, 2, 2) VFKV_P2(kF8, 64, 1, 2) VFKV_P2(kF8, 128, 2, 2) VFKV_P2(kF8, 128, 1, 2)
             VFKV_P2(kF16, 64, 2, 2) VFKV_P2(kF16, 64, 1, 2) VFKV_P2(kF16, 128, 1, 1) VFKV_P2(kF16, 128, 2, 1)
             VFKV_P2(kF8, 256, 1, 1) VFKV_P2(kF16, 256, 1, 1)

@@ -30,7 +30,7 @@ constexpr int kPrefillOneHeadWaves = 12;
 // NH > 1 (head_dim 512, NCB = 1): NH wavefronts share a head.  Each computes the scores over the whole head_dim and
 // accumulates, merges and stores its own slice of D / NH output elements: the accumulators of a 512-wide head do not fit
 // one wavefront.  HP then counts (head, slice) units.
-template <int DT, int D, int NCB, int PFD, bool CAP, int NH = 1, bool F16W = false>
+template <int DT, int D, int NCB, int PFD, bool CAP, int NH = 1, bool F16W = false, bool F8S = false>
 __global__ __launch_bounds__((NCB == 1 && D <= 128) ? kPrefillOneHeadWaves * 64 : (NCB * D >= 512 || (DT == kF16 && D == 256)) ? 256 : 512) void batch_mfma2_kernel(BatchArgs a, int HP, int NS) {
     constexpr int DV = D / NH;                   // output elements (V columns) of this wavefront
     constexpr int ES = DT == kF16 ? 2 : 1;
@@ -46,9 +46,11 @@ __global__ __launch_bounds__((NCB == 1 && D <= 128) ? kPrefillOneHeadWaves * 64 
     constexpr float kMaxSlack = 8.0f;            // log2 units by which a score may exceed the running reference maximum
     constexpr uint32_t kNoTile = 0x80000000u;    // byte offset past any slab: the load returns zeros, no memory access
     static_assert(D % 32 == 0 && SEGB % 16 == 0 && VLD >= 1, "unsupported head_dim");
+    static_assert(!F8S || (DT == kF8 && D == 128 && NH == 1), "the fp8 first product is built for FP8 rows of 128 elements");
 
     extern __shared__ __attribute__((aligned(16))) _Float16 lds[];      // [waves][KT][VPITCH] V tiles | [GP][16][D + 8] f16(q) | [GP][16][D + 8] remainders
     __shared__ int lds_haslo;
+    __shared__ uint32_t lds_qmax;                                // F8S: bits of the largest |q| of the workgroup's Q block
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -115,6 +117,55 @@ __global__ __launch_bounds__((NCB == 1 && D <= 128) ? kPrefillOneHeadWaves * 64 
     constexpr int QLD = 4;                                      // query loads per thread and round
     const int nthreads = nwaves * 64;
     const int q4_total = 16 * GP * (D / 4);
+    // F8S: Q as three E4M3 planes q ~ 2^e (t1 + t2 / 16 + t3 / 256), every term the E4M3 rounding of what the terms before it
+    // left (12 significant bits: exact for f16-representable q; e keeps the largest |q| of the block below 256).  The first
+    // product then runs on the FP8 matrix instruction with the cache rows as they are.
+    constexpr int Q8PITCH = D + 16;                             // bytes per (head slot, query) row of a term plane
+    uint8_t* const q8_lds = reinterpret_cast<uint8_t*>(qhi_lds);    // [3][GP][16][Q8PITCH]
+    int q_exp = 0;
+    bool has_lo = false;
+    if constexpr (F8S) {
+        if (tid == 0) lds_qmax = 0u;
+        float4 qf[QLD];                                         // the launcher guarantees q4_total <= QLD * nthreads
+        float amax = 0.f;
+#pragma unroll
+        for (int i = 0; i < QLD; ++i) {
+            const int idx = tid + i * nthreads;
+            const int qq = idx / (GP * (D / 4)), rem = idx - qq * (GP * (D / 4));
+            const bool ok = idx < q4_total && q0 + qq < a.m && rem < (G - gz) * (D / 4);
+            qf[i] = *reinterpret_cast<const float4*>(a.q + ((size_t)(ok ? q0 + qq : 0) * a.n_heads + kvh * G + gz) * D + (ok ? rem * 4 : 0));
+            if (!ok) qf[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+            amax = fmaxf(fmaxf(amax, fmaxf(fabsf(qf[i].x), fabsf(qf[i].y))), fmaxf(fabsf(qf[i].z), fabsf(qf[i].w)));
+        }
+#pragma unroll
+        for (int sl = 0; sl < PFD; ++sl) issue(sl, tile_off(tb0 + sl * step));
+        __syncthreads();                                        // lds_qmax cleared
+        amax = wave_max_uniform(amax);
+        if (lane == 0) atomicMax(&lds_qmax, __builtin_bit_cast(uint32_t, amax));   // non-negative floats order like their bits
+        __syncthreads();
+        const uint32_t mb = lds_qmax;
+        q_exp = (int)((mb >> 23) & 0xFFu) - 127 - 7;            // floor(log2(max|q|)) - 7: max|q| * 2^-e < 256
+        q_exp = q_exp < -100 ? -100 : q_exp > 100 ? 100 : q_exp;
+        const float down = __builtin_bit_cast(float, (uint32_t)(127 - q_exp) << 23);
+#pragma unroll
+        for (int i = 0; i < QLD; ++i) {
+            const int idx = tid + i * nthreads;
+            if (idx >= q4_total) continue;
+            const int qq = idx / (GP * (D / 4)), rem = idx - qq * (GP * (D / 4));
+            const int g = rem / (D / 4), d = (rem - g * (D / 4)) * 4;
+            float r[4] = {qf[i].x * down, qf[i].y * down, qf[i].z * down, qf[i].w * down};
+#pragma unroll
+            for (int t = 0; t < 3; ++t) {
+                int w8 = __builtin_amdgcn_cvt_pk_fp8_f32(r[0], r[1], 0, false);
+                w8 = __builtin_amdgcn_cvt_pk_fp8_f32(r[2], r[3], w8, true);
+                *reinterpret_cast<uint32_t*>(q8_lds + ((size_t)(t * GP + g) * 16 + qq) * Q8PITCH + d) = (uint32_t)w8;
+                const float2_t d01 = __builtin_amdgcn_cvt_pk_f32_fp8(w8, false), d23 = __builtin_amdgcn_cvt_pk_f32_fp8(w8, true);
+                r[0] = (r[0] - d01[0]) * 16.f; r[1] = (r[1] - d01[1]) * 16.f;
+                r[2] = (r[2] - d23[0]) * 16.f; r[3] = (r[3] - d23[1]) * 16.f;
+            }
+        }
+        __syncthreads();                                        // planes written
+    } else {
     if (tid == 0) lds_haslo = 0;
     bool any_lo = false;
     for (int base = 0; base < q4_total; base += QLD * nthreads) {
@@ -148,7 +199,8 @@ __global__ __launch_bounds__((NCB == 1 && D <= 128) ? kPrefillOneHeadWaves * 64 
     __syncthreads();                                            // lds_haslo cleared, planes written
     if (any_lo) lds_haslo = 1;
     __syncthreads();
-    const bool has_lo = __builtin_amdgcn_readfirstlane(lds_haslo) != 0;   // workgroup-uniform
+    has_lo = __builtin_amdgcn_readfirstlane(lds_haslo) != 0;   // workgroup-uniform
+    }
 
     float4_t oacc[NCB][DTILES];
 #pragma unroll
@@ -185,6 +237,41 @@ __global__ __launch_bounds__((NCB == 1 && D <= 128) ? kPrefillOneHeadWaves * 64 
                 *reinterpret_cast<u32x4*>(dst) = vraw[sl][c];
             }
             vraw[sl][c] = __builtin_amdgcn_raw_buffer_load_b128(vrsrc, lane_voff, noff + (uint32_t)(c * VROWS) * row_stride, 0);
+        }
+        if constexpr (F8S) {
+            // S^T = K Q^T on the FP8 matrix instruction: A = the lane's quarter row of K as loaded (32 codes), B = the same
+            // quarter of the query's three term planes, each with its power-of-two weight as the instruction's block scale
+#pragma unroll
+            for (int cb = 0; cb < NCB; ++cb)
+#pragma unroll
+                for (int kt = 0; kt < 2; ++kt) s[cb][kt] = float4_t{0.f, 0.f, 0.f, 0.f};
+            typedef int v8i_t __attribute__((ext_vector_type(8)));
+            v8i_t ka8[2];
+#pragma unroll
+            for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+                for (int j = 0; j < 8; ++j) ka8[kt][j] = (int)kraw[sl][kt][j / 4][j % 4];
+#pragma unroll
+            for (int t = 0; t < 3; ++t) {
+                const int sb = 127 + q_exp - 4 * t;             // E8M0 code of 2^(e - 4t)
+#pragma unroll
+                for (int cb = 0; cb < NCB; ++cb) {
+                    const uint8_t* qrow = q8_lds + ((size_t)(t * GP + g0 + cb) * 16 + n16) * Q8PITCH + kg * 32;
+                    const u32x4 b0 = *reinterpret_cast<const u32x4*>(qrow), b1 = *reinterpret_cast<const u32x4*>(qrow + 16);
+                    v8i_t qb8;
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) { qb8[j] = (int)b0[j]; qb8[4 + j] = (int)b1[j]; }
+#pragma unroll
+                    for (int kt = 0; kt < 2; ++kt)
+                        s[cb][kt] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(ka8[kt], qb8, s[cb][kt], 0, 0, 0, 127, 0, sb);
+                }
+            }
+#pragma unroll
+            for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+                for (int xx = 0; xx < KLD; ++xx)
+                    kraw[sl][kt][xx] = __builtin_amdgcn_raw_buffer_load_b128(krsrc, lane_koff + xx * 16, noff + (uint32_t)(kt * 16) * row_stride, 0);
+            return;
         }
         half8_t qhi[NCB][KS];
 #pragma unroll

@@ -103,6 +103,9 @@ struct BatchLaunch {
     // to 2^-11 * max|v|.  Built for head_dim 128 with the GQA group in one wavefront pair (FP8) or one wavefront (F16); other
     // shapes and kernels ignore it and keep both products.
     bool f16_weights = false;
+    // FP8 caches at head_dim 128, GQA groups of 2-4 heads: the first product K Q^T runs on the FP8 matrix instruction, K rows as
+    // stored and Q as three E4M3 terms (12 significant bits); no widening of K.  Other shapes ignore it.
+    bool fp8_scores = false;
 };
 hipError_t launch_batch(const BatchLaunch& a, hipStream_t stream);
 

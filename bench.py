@@ -39,11 +39,11 @@ MFMA_F32_PEAK_TFLOPS = 157.3      # dense f32 matrix rate: what an F32 cache is 
 # it was taken with: when the sources have changed since, the line reports null instead of a stale figure.
 PROFILED_TRAFFIC = {
     "decode_fp8_32k_32layers": {
-        "bytes": (65634 + 520) * 1024, "profile": "profiles/decode_fp8_32k_split_mfma_kernel.md",
-        "sources": ("attn_decode.hip", "attn_decode_mfma.h", "device_utils.h"), "sha256_16": "2f2ec6d675d73d3a"},
+        "bytes": (65635 + 520) * 1024, "profile": "profiles/decode_floor_calibration.md",
+        "sources": ("attn_decode.hip", "attn_decode_mfma.h", "device_utils.h"), "sha256_16": "0145bfacb7bdfd49"},
     "prefill_fp8_512x4608_32layers": {
-        "bytes": (81369 + 8192) * 1024, "profile": "profiles/prefill_fp8_512x4608_batch_mfma2_kernel.md",
-        "sources": ("attn_prefill.hip", "attn_prefill_mfma2.h", "device_utils.h"), "sha256_16": "4a01f15e97324471"},
+        "bytes": (83020 + 9728) * 1024, "profile": "profiles/prefill_fp8_512x4608_batch_mfma2_kernel.md",
+        "sources": ("attn_prefill.hip", "attn_prefill_mfma2.h", "device_utils.h"), "sha256_16": "0d78085a41cacb85"},
 }
 
 

@@ -64,3 +64,48 @@ def test_static_scratch_matches_workspace_call_twice_in_a_row(dtype, heads, hkv,
         ref = oracle.attn_decode_ref(q, ke, ve, int(dtype), heads, hkv, d, position + 1, 1.0 / np.sqrt(d), kv_start=kv_start)
         assert np.abs(o_static - ref).max() < TOL[dtype]
     cache.destroy()
+
+
+def test_static_scratch_call_captured_into_a_graph_replays_like_eager():
+    # the callers this entry point is for: a decode step under HIP graph capture.  The array's address is looked up on the
+    # first (eager) call; the captured calls then only enqueue kernels.  Every replay, with new queries and eager work in
+    # between, must reproduce the eager call bit for bit.
+    dtype, heads, hkv, d, ctx, layers = vf.KvDtype.F8, 32, 8, 128, 5000, 2
+    L = _ffi.lib()
+    cache = vf.KvCache(vf.KvCacheConfig(layers, hkv, d, ctx, dtype=dtype))
+    cache.zero_fill()
+    r = rng(910)
+    fwd = vf.Forward(cache, heads)
+    for layer in range(layers):
+        fwd.b_step_kv_write(layer, 0, ctx, to_dev(outlier_normal(r, (ctx, hkv * d))), to_dev(outlier_normal(r, (ctx, hkv * d))))
+    q = torch.zeros((layers, heads, d), device=DEV)
+    o = torch.zeros((layers, heads, d), device=DEV)
+    scale = 1.0 / np.sqrt(d)
+
+    def step(out):
+        stream = torch.cuda.current_stream().cuda_stream
+        for layer in range(layers):
+            _ffi.check(L.vfkv_decode_attention_static(cache.handle, layer, layer, heads, q[layer].data_ptr(), out[layer].data_ptr(),
+                                                      ctx - 1, 0, scale, 0.0, stream))
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        step(o)                                  # first use outside the capture
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        step(o)
+    for rep in range(3):
+        print(f"case graph replay {rep}", flush=True)
+        q.copy_(to_dev(fp16_normal(r, (layers, heads, d))))
+        graph.replay()
+        torch.cuda.synchronize()
+        got = to_np(o).copy()
+        o_eager = torch.full_like(o, float("nan"))
+        step(o_eager)
+        torch.cuda.synchronize()
+        assert np.isfinite(got).all() and np.array_equal(got, to_np(o_eager)), rep
+        (q * 2).sum().item()                     # unrelated eager work between replays
+    cache.destroy()

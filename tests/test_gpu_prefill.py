@@ -200,6 +200,10 @@ def test_scores_that_drift_past_the_running_maximum(dtype, shape):
     (vf.KvDtype.F16, 32, 8, 128, 20, 9000, 0, 0.0),      # one partly filled query block, four-heads-per-wavefront form
     (vf.KvDtype.F8, 16, 8, 256, 37, 3000, 2048, 30.0),   # window and soft-cap: chunks start at the window
     (vf.KvDtype.F8, 8, 2, 512, 16, 2500, 0, 0.0),        # head_dim 512: output slices and key chunks together
+    (vf.KvDtype.F16, 8, 1, 512, 21, 3624, 3000, 0.0),    # head_dim 512: the two wavefronts of a head swap score halves behind a
+                                                         # barrier per tile, so every wavefront also walks (masked) padding tiles
+                                                         # past the end of its key chunk
+    (vf.KvDtype.F16, 8, 8, 512, 20, 2001, 0, 0.0),       # head_dim 512, one head per KV head: two key splits of unequal length
     (vf.KvDtype.F16, 28, 4, 128, 50, 1500, 0, 0.0),      # G = 7
     (vf.KvDtype.F8, 32, 8, 128, 512, 4096, 0, 0.0),      # a full chunk: plenty of workgroups, the plain path is taken
     (vf.KvDtype.F32, 8, 2, 128, 16, 2000, 0, 0.0),       # F32 cache: no key chunks, same result

@@ -139,7 +139,8 @@ static hipError_t launch_batch_kernels(const BatchLaunch& L, hipStream_t stream,
         // the private V tiles and the two Q planes have to fit in 160 KiB of LDS
         auto waves_for = [&](uint32_t slices) -> uint32_t {
             const size_t qbytes = (size_t)2 * (slices / nh) * ncb * 16 * (L.head_dim + 8) * sizeof(_Float16);
-            const size_t per_wave = (size_t)32 * (dv + 16) * sizeof(_Float16);
+            // private V tile, and with two wavefronts per head the two buffers through which they swap score halves
+            const size_t per_wave = (size_t)32 * (dv + 16) * sizeof(_Float16) + (nh == 2u ? (size_t)2 * ncb * 64 * 16 : 0u);   // (unused by the two-heads FP8 form)
             const size_t fit = qbytes < 160u * 1024u ? (160u * 1024u - qbytes) / per_wave : 0u;
             return fit < reg_waves ? (uint32_t)fit : reg_waves;
         };
@@ -191,7 +192,8 @@ static hipError_t launch_batch_kernels(const BatchLaunch& L, hipStream_t stream,
             if (gate_in_store) { a.gate = L.gate->gate; a.gchunk = L.gate->chunk; a.gstride = L.gate->stride; a.goff = L.gate->gate_offset; }
             const dim3 grid((L.m + 15u) / 16u, L.n_kv_heads, nz * nk), block(nwaves * kWave);
             const size_t vbytes = (size_t)nwaves * 32 * (dv + 16) * sizeof(_Float16) +
-                                  (size_t)2 * (hp / nh) * ncb * 16 * (L.head_dim + 8) * sizeof(_Float16);
+                                  (size_t)2 * (hp / nh) * ncb * 16 * (L.head_dim + 8) * sizeof(_Float16) +
+                                  (nh == 2u ? (size_t)2 * nwaves * ncb * 64 * 16 : 0u);
             const size_t mbytes = (size_t)(ns - 1) * hp * ncb * 64 * (dv / 4 + 2) * sizeof(float);
             const size_t lds = vbytes > mbytes ? vbytes : mbytes;
             const bool cap = L.softcap > 0.f;

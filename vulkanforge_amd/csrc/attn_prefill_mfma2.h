@@ -27,7 +27,9 @@ namespace vfkv {
 // wavefronts per workgroup when a wavefront serves one head at head_dim <= 128 (fewer registers: three per SIMD)
 constexpr int kPrefillOneHeadWaves = 12;
 
-// NH > 1 (head_dim 512, NCB = 1): NH wavefronts share a head.  Each computes the scores over the whole head_dim and
+// NH > 1 (head_dim 512): NH = 2 wavefronts share a head.  Each computes the scores of one of the tile's two 16-key halves
+// over the whole head_dim (so each loads and widens half of the K tile), the two swap their halves through LDS behind one
+// workgroup barrier per tile, and each then
 // accumulates, merges and stores its own slice of D / NH output elements: the accumulators of a 512-wide head do not fit
 // one wavefront.  HP then counts (head, slice) units.
 template <int DT, int D, int NCB, int PFD, bool CAP, int NH = 1, bool F16W = false, bool F8S = false>
@@ -45,6 +47,12 @@ __global__ __launch_bounds__((NCB == 1 && D <= 128) ? kPrefillOneHeadWaves * 64 
     constexpr int VROWS = 64 / VCHUNK_ROW;
     constexpr float kMaxSlack = 8.0f;            // log2 units by which a score may exceed the running reference maximum
     constexpr uint32_t kNoTile = 0x80000000u;    // byte offset past any slab: the load returns zeros, no memory access
+    // the two wavefronts of a head score one 16-key half of a tile each and swap (not with two heads per wavefront over
+    // FP8 rows, where a K tile is already widened once for both heads and the barrier per tile costs more than it saves:
+    // 16 / 2 / 512, 512 x 4 608: 218 us without, 245 us with)
+    constexpr bool XCH = NH == 2 && !(DT == kF8 && NCB == 2);
+    constexpr int NKT = XCH ? 1 : 2;             // 16-key halves of a tile this wavefront loads and scores
+    static_assert(NH == 1 || NH == 2, "one or two wavefronts per head");
     static_assert(D % 32 == 0 && SEGB % 16 == 0 && VLD >= 1, "unsupported head_dim");
     static_assert(!F8S || (DT == kF8 && D == 128 && NH == 1), "the fp8 first product is built for FP8 rows of 128 elements");
 
@@ -73,6 +81,7 @@ __global__ __launch_bounds__((NCB == 1 && D <= 128) ? kPrefillOneHeadWaves * 64 
     _Float16* const qhi_lds = lds + (size_t)nwaves * KT * VPITCH;   // [GP][16][D + 8] f16(q); the slots past G hold zeros
     const int GP = (HP / NH) * NCB;                                 // head slots of the workgroup: G rounded up to whole wavefronts
     _Float16* const qlo_lds = qhi_lds + (size_t)GP * 16 * QPITCH;   // [GP][16][D + 8] f16(q - f16(q))
+    float4_t* const xbuf = reinterpret_cast<float4_t*>(qlo_lds + (size_t)GP * 16 * QPITCH);   // XCH: [2][waves][NCB][64] score halves
 
     // ---- key range ----
     uint32_t kmax = a.q_start + q0 + 16;                        // one past the last key any of the 16 queries sees
@@ -97,20 +106,26 @@ __global__ __launch_bounds__((NCB == 1 && D <= 128) ? kPrefillOneHeadWaves * 64 
     const int vrow = lane / VCHUNK_ROW, vcol = lane % VCHUNK_ROW;
     const uint32_t lane_voff = vrow * row_stride + head_b + dslice * DV * ES + vcol * 16;
 
-    u32x4 kraw[PFD][2][KLD];
+    const uint32_t kt_own = XCH ? (uint32_t)dslice : 0u;         // XCH: the half this wavefront scores
+    u32x4 kraw[PFD][NKT][KLD];
     u32x4 vraw[PFD][VLD];
     auto issue = [&](int slot, uint32_t toff) {
 #pragma unroll
-        for (int kt = 0; kt < 2; ++kt)
+        for (int kt = 0; kt < NKT; ++kt)
 #pragma unroll
             for (int x = 0; x < KLD; ++x)
-                kraw[slot][kt][x] = __builtin_amdgcn_raw_buffer_load_b128(krsrc, lane_koff + x * 16, toff + (uint32_t)(kt * 16) * row_stride, 0);
+                kraw[slot][kt][x] = __builtin_amdgcn_raw_buffer_load_b128(krsrc, lane_koff + x * 16, toff + ((uint32_t)kt + kt_own) * 16u * row_stride, 0);
 #pragma unroll
         for (int c = 0; c < VLD; ++c)
             vraw[slot][c] = __builtin_amdgcn_raw_buffer_load_b128(vrsrc, lane_voff, toff + (uint32_t)(c * VROWS) * row_stride, 0);
     };
     const uint32_t step = KT * NS;
     const uint32_t tb0 = t_first + sp * KT;                     // this wavefront's first tile (may already be past the end)
+    // XCH: every tile has a workgroup barrier, so every wavefront walks the same number of tiles; the ones past the last key
+    // load nothing (zero-returning offsets) and are masked out entirely
+    const uint32_t n_my = kmax > t_first ? ((kmax - t_first + KT - 1) / KT + NS - 1) / NS : 0u;
+    const uint32_t kloop = XCH ? tb0 + n_my * step : kmax;      // where this wavefront's walk ends
+    int xpar = 0;                                               // XCH: which of the two exchange buffers the next tile uses
     auto tile_off = [&](uint32_t t) -> uint32_t { return t < kmax ? t * row_stride : kNoTile; };
     // ---- Q block of the workgroup: 16 queries x G heads x D floats, loaded once with coalesced 16-byte loads (before the
     // K / V requests, so waiting for it does not wait for them) and kept in LDS as an f16 value plane and a remainder plane
@@ -279,8 +294,9 @@ __global__ __launch_bounds__((NCB == 1 && D <= 128) ? kPrefillOneHeadWaves * 64 
 #pragma unroll
             for (int c = 0; c < KS; ++c)
                 qhi[cb][c] = *reinterpret_cast<const half8_t*>(qhi_lds + ((size_t)(g0 + cb) * 16 + n16) * QPITCH + kg * SEG + c * 8);
+        float4_t sown[NCB];                                     // XCH: this wavefront's half of the scores
 #pragma unroll
-        for (int kt = 0; kt < 2; ++kt) {
+        for (int kt = 0; kt < NKT; ++kt) {
             half8_t ka[KS];
 #pragma unroll
             for (int c = 0; c < KS; ++c) {
@@ -298,24 +314,44 @@ __global__ __launch_bounds__((NCB == 1 && D <= 128) ? kPrefillOneHeadWaves * 64 
             }
 #pragma unroll
             for (int xx = 0; xx < KLD; ++xx)
-                kraw[sl][kt][xx] = __builtin_amdgcn_raw_buffer_load_b128(krsrc, lane_koff + xx * 16, noff + (uint32_t)(kt * 16) * row_stride, 0);
+                kraw[sl][kt][xx] = __builtin_amdgcn_raw_buffer_load_b128(krsrc, lane_koff + xx * 16, noff + ((uint32_t)kt + kt_own) * 16u * row_stride, 0);
 #pragma unroll
             for (int cb = 0; cb < NCB; ++cb) {
-                s[cb][kt] = float4_t{0.f, 0.f, 0.f, 0.f};
+                float4_t acc = float4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-                for (int c = 0; c < KS; ++c) s[cb][kt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ka[c], qhi[cb][c], s[cb][kt], 0, 0, 0);
+                for (int c = 0; c < KS; ++c) acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(ka[c], qhi[cb][c], acc, 0, 0, 0);
+                if (XCH) sown[cb] = acc; else s[cb][kt] = acc;
             }
             if (has_lo) {
 #pragma unroll
                 for (int cb = 0; cb < NCB; ++cb) {
                     const _Float16* lo_row = qlo_lds + ((size_t)(g0 + cb) * 16 + n16) * QPITCH + kg * SEG;
+                    float4_t acc = XCH ? sown[cb] : s[cb][kt];
 #pragma unroll
                     for (int c = 0; c < KS; ++c) {
                         const half8_t ql = *reinterpret_cast<const half8_t*>(lo_row + c * 8);
-                        s[cb][kt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ka[c], ql, s[cb][kt], 0, 0, 0);
+                        acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(ka[c], ql, acc, 0, 0, 0);
                     }
+                    if (XCH) sown[cb] = acc; else s[cb][kt] = acc;
                 }
             }
+        }
+        if constexpr (XCH) {
+            // swap halves with the partner wavefront (the other output slice of the same head and key split: w ^ 1).  Two
+            // buffers alternate, so one barrier per tile is enough: a buffer is rewritten two tiles later, after a barrier
+            // the partner can only have reached by finishing this tile's read.
+            float4_t* const xw = xbuf + ((size_t)(xpar * nwaves + w) * NCB) * 64 + lane;
+            const float4_t* const xr = xbuf + ((size_t)(xpar * nwaves + (w ^ 1)) * NCB) * 64 + lane;
+#pragma unroll
+            for (int cb = 0; cb < NCB; ++cb) xw[cb * 64] = sown[cb];
+            __syncthreads();
+#pragma unroll
+            for (int cb = 0; cb < NCB; ++cb) {
+                const float4_t other = xr[cb * 64];
+                s[cb][0] = kt_own == 0u ? sown[cb] : other;
+                s[cb][1] = kt_own == 0u ? other : sown[cb];
+            }
+            xpar ^= 1;
         }
     };
     // scores of the tile in log2 units (this lane owns keys tcur + kt*16 + kg*4 + i of query n16); returns whether one of
@@ -335,7 +371,7 @@ __global__ __launch_bounds__((NCB == 1 && D <= 128) ? kPrefillOneHeadWaves * 64 
                     if (CAP) y = cap_l2 * tanhf(y / cap_l2);
                     if (MASKED) {
                         const uint32_t t = tcur + kt * 16 + kg * 4 + i;
-                        y = (t < my_len && t >= a.kv_start) ? y : kMasked;
+                        y = (t < my_len && t >= a.kv_start && t < kmax) ? y : kMasked;    // (t >= kmax: padding tiles of a key chunk)
                     }
                     x[cb][kt * 4 + i] = y;
                     tmax[cb] = fmaxf(tmax[cb], y);
@@ -412,14 +448,14 @@ __global__ __launch_bounds__((NCB == 1 && D <= 128) ? kPrefillOneHeadWaves * 64 
     uint32_t tb = tb0;
     int first_slot = 0;          // slots of the group at tb that the inner loop has already finished
     bool s_ready = false;        // s[] of slot first_slot is already computed
-    while (tb < kmax) {
+    while (tb < kloop) {
 #pragma unroll
         for (int sl = 0; sl < PFD; ++sl) {
             const uint32_t tcur = tb + sl * step;
-            if (tcur >= kmax) break;                            // wavefront-uniform
+            if (tcur >= kloop) break;                           // wavefront-uniform
             if (sl < first_slot) continue;
             if (!(s_ready && sl == first_slot)) stage_and_first_product(sl, tcur);
-            if (tcur >= a.kv_start && tcur + KT <= full_len) {  // every query of the block sees the whole tile
+            if (tcur >= a.kv_start && tcur + KT <= fast_end) {  // every query of the block sees the whole tile (and it is this workgroup's)
                 if (__builtin_amdgcn_ballot_w64(scores(std::false_type{}, tcur)) != 0ull) move_maximum();
                 weights_and_second_product(std::false_type{}, std::integral_constant<bool, !F16W>{});
             } else {

@@ -42,8 +42,8 @@ PROFILED_TRAFFIC = {
         "bytes": (65635 + 520) * 1024, "profile": "profiles/decode_floor_calibration.md",
         "sources": ("attn_decode.hip", "attn_decode_mfma.h", "device_utils.h"), "sha256_16": "0145bfacb7bdfd49"},
     "prefill_fp8_512x4608_32layers": {
-        "bytes": (83362 + 10240) * 1024, "profile": "profiles/prefill_fp8_512x4608_batch_mfma2_kernel.md",
-        "sources": ("attn_prefill.hip", "attn_prefill_mfma2.h", "device_utils.h"), "sha256_16": "215be75768ec94e9"},
+        "bytes": (82484 + 10240) * 1024, "profile": "profiles/prefill_fp8_512x4608_batch_mfma2_kernel.md",
+        "sources": ("attn_prefill.hip", "attn_prefill_mfma2.h", "device_utils.h"), "sha256_16": "efc8ad4fabe74a13"},
 }
 
 

@@ -136,11 +136,15 @@ static hipError_t launch_batch_kernels(const BatchLaunch& L, hipStream_t stream,
         // per SIMD), 512 accumulator columns per wavefront need the whole register file of a SIMD (one wavefront per SIMD)
         const uint32_t reg_waves = (ncb == 1u && L.head_dim <= 128u) ? (uint32_t)kPrefillOneHeadWaves
                                  : (ncb * L.head_dim >= 512u || (L.dtype == kF16 && L.head_dim == 256u)) ? 4u : 8u;   // (always 4 at head_dim 512)
+        // FP8 rows of 128 elements, two heads per wavefront: three raw V tiles per wavefront (filled by loads that write LDS)
+        // instead of one f16 copy
+        const bool vdma = L.dtype == kF8 && L.head_dim == 128u && ncb == 2u;
         // the private V tiles and the two Q planes have to fit in 160 KiB of LDS
         auto waves_for = [&](uint32_t slices) -> uint32_t {
             const size_t qbytes = (size_t)2 * (slices / nh) * ncb * 16 * (L.head_dim + 8) * sizeof(_Float16);
             // private V tile, and with two wavefronts per head the two buffers through which they swap score halves
-            const size_t per_wave = (size_t)32 * (dv + 16) * sizeof(_Float16) + (nh == 2u ? (size_t)2 * ncb * 64 * 16 : 0u);   // (unused by the two-heads FP8 form)
+            const size_t per_wave = (vdma ? (size_t)3 * 32 * 128 : (size_t)32 * (dv + 16) * sizeof(_Float16)) +
+                                    (nh == 2u ? (size_t)2 * ncb * 64 * 16 : 0u);   // (unused by the two-heads FP8 form)
             const size_t fit = qbytes < 160u * 1024u ? (160u * 1024u - qbytes) / per_wave : 0u;
             return fit < reg_waves ? (uint32_t)fit : reg_waves;
         };
@@ -191,7 +195,7 @@ static hipError_t launch_batch_kernels(const BatchLaunch& L, hipStream_t stream,
                                        (((uintptr_t)L.gate->gate) & 15u) == 0u;
             if (gate_in_store) { a.gate = L.gate->gate; a.gchunk = L.gate->chunk; a.gstride = L.gate->stride; a.goff = L.gate->gate_offset; }
             const dim3 grid((L.m + 15u) / 16u, L.n_kv_heads, nz * nk), block(nwaves * kWave);
-            const size_t vbytes = (size_t)nwaves * 32 * (dv + 16) * sizeof(_Float16) +
+            const size_t vbytes = (size_t)nwaves * (vdma ? (size_t)3 * 32 * 128 : (size_t)32 * (dv + 16) * sizeof(_Float16)) +
                                   (size_t)2 * (hp / nh) * ncb * 16 * (L.head_dim + 8) * sizeof(_Float16) +
                                   (nh == 2u ? (size_t)2 * nwaves * ncb * 64 * 16 : 0u);
             const size_t mbytes = (size_t)(ns - 1) * hp * ncb * 64 * (dv / 4 + 2) * sizeof(float);

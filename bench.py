@@ -42,9 +42,18 @@ PROFILED_TRAFFIC = {
         "bytes": (65635 + 520) * 1024, "profile": "profiles/decode_floor_calibration.md",
         "sources": ("attn_decode.hip", "attn_decode_mfma.h", "device_utils.h"), "sha256_16": "0145bfacb7bdfd49"},
     "prefill_fp8_512x4608_32layers": {
-        "bytes": (82484 + 10240) * 1024, "profile": "profiles/prefill_fp8_512x4608_batch_mfma2_kernel.md",
-        "sources": ("attn_prefill.hip", "attn_prefill_mfma2.h", "device_utils.h"), "sha256_16": "efc8ad4fabe74a13"},
+        "bytes": (18572 + 9728) * 1024, "profile": "profiles/prefill_fp8_512x4608_batch_dma_kernel.md",
+        "sources": ("attn_prefill.hip", "attn_prefill_dma.h", "device_utils.h"), "sha256_16": "f491467e8ab047c7"},
 }
+
+
+def prefill_kernel_name(kv_label, head_dim, group):
+    """The kernel attn_prefill.hip launches for a shape with 16-byte aligned buffers."""
+    if kv_label == "FP32" or head_dim == 96:
+        return "batch_mfma_f32_kernel"
+    if kv_label == "FP8" and head_dim == 128 and group >= 2:
+        return "batch_dma_kernel"       # two heads per wavefront over FP8 rows: V loaded straight into LDS
+    return "batch_mfma2_kernel"
 
 
 def kernel_sources_digest(names):
@@ -483,7 +492,7 @@ def bench_prefill(args, wl):
         "data": "synthetic, seeded N(0,1); queries " + ("general f32" if args.f32_queries else "cast to fp16 as the configuration states") + "; K/V rows cast to fp16 and written through the append kernels",
         "config": {"workload": wl.name, "n_layers": L, "n_heads": H, "n_kv_heads": Hkv, "head_dim": D,
                    "m": wl.m, "q_start": wl.base_pos, "n_kv": max_seq, "flop_per_step": flops_step},
-        "roofline": {"bound": "mfma", "kernel": "batch_mfma_f32_kernel" if f32_cache else "batch_mfma2_kernel",
+        "roofline": {"bound": "mfma", "kernel": prefill_kernel_name(wl.dtype.label(), D, H // Hkv),
                      "achieved": achieved, "peak": peak,
                      "unit": "TFLOP/s", "frac": achieved / peak, "traffic": traffic, "traffic_source": traffic_source,
                      "avg_launch_us": avg_ms * 1e3},

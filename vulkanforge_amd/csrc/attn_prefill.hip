@@ -34,6 +34,7 @@ struct BatchArgs {
 
 }  // namespace vfkv
 #include "attn_prefill_mfma2.h"
+#include "attn_prefill_dma.h"
 #include "attn_prefill_f32.h"
 namespace vfkv {
 
@@ -163,7 +164,7 @@ static hipError_t launch_batch_kernels(const BatchLaunch& L, hipStream_t stream,
         }
         const uint32_t nz = (hp_group + hp - 1u) / hp;
         const uint32_t max_waves = waves_for(hp);
-        if (max_waves >= hp && nz <= 65535u) {
+        if (max_waves >= hp && nz <= 65535u && (L.m + 15u) / 16u <= 65535u) {
             const uint32_t ns = max_waves / hp;               // key splits: fill the workgroup
             const uint32_t nwaves = hp * ns;
             // Short chunks over long histories (the suffix of a request that reuses its prefix) still leave most compute
@@ -194,7 +195,9 @@ static hipError_t launch_batch_kernels(const BatchLaunch& L, hipStream_t stream,
                                        ((L.gate->chunk | L.gate->stride | L.gate->gate_offset) % 4u) == 0u &&
                                        (((uintptr_t)L.gate->gate) & 15u) == 0u;
             if (gate_in_store) { a.gate = L.gate->gate; a.gchunk = L.gate->chunk; a.gstride = L.gate->stride; a.goff = L.gate->gate_offset; }
-            const dim3 grid((L.m + 15u) / 16u, L.n_kv_heads, nz * nk), block(nwaves * kWave);
+            // the KV head is the fastest grid index: consecutive workgroups go to consecutive XCDs, so with eight KV heads all
+            // query blocks of a head share one XCD's L2 and its K / V rows come from memory once, not once per XCD
+            const dim3 grid(L.n_kv_heads, (L.m + 15u) / 16u, nz * nk), block(nwaves * kWave);
             const size_t vbytes = (size_t)nwaves * (vdma ? (size_t)3 * 32 * 128 : (size_t)32 * (dv + 16) * sizeof(_Float16)) +
                                   (size_t)2 * (hp / nh) * ncb * 16 * (L.head_dim + 8) * sizeof(_Float16) +
                                   (nh == 2u ? (size_t)2 * nwaves * ncb * 64 * 16 : 0u);
@@ -207,20 +210,24 @@ static hipError_t launch_batch_kernels(const BatchLaunch& L, hipStream_t stream,
         if (cap) hipLaunchKernelGGL((batch_mfma2_kernel<DT, DD, NCBV, PFDV, true>), grid, block, lds, stream, a, (int)hp, (int)ns);  \
         else hipLaunchKernelGGL((batch_mfma2_kernel<DT, DD, NCBV, PFDV, false>), grid, block, lds, stream, a, (int)hp, (int)ns);      \
     } else
-            // The options are built for the head_dim 128 forms the benchmark geometries run on; other shapes keep the default
-            // arithmetic.  f16_weights: one product with the weights instead of value + remainder.  fp8_scores: the first
-            // product on the FP8 matrix instruction (needs the Q block staged in one round: four key splits).
-            const bool f8s = L.fp8_scores && L.dtype == kF8 && L.head_dim == 128u && ncb == 2u && ns >= 4u;
-#define VFKV_P2_OPT(DT, NCBV, PFDV, F16WV, F8SV)                                                                       \
-    { if (cap) hipLaunchKernelGGL((batch_mfma2_kernel<DT, 128, NCBV, PFDV, true, 1, F16WV, F8SV>), grid, block, lds, stream, a, (int)hp, (int)ns);  \
-      else hipLaunchKernelGGL((batch_mfma2_kernel<DT, 128, NCBV, PFDV, false, 1, F16WV, F8SV>), grid, block, lds, stream, a, (int)hp, (int)ns); }
-            if (f8s && L.f16_weights) VFKV_P2_OPT(kF8, 2, 2, true, true)
-            else if (f8s) VFKV_P2_OPT(kF8, 2, 2, false, true)
-            else if (L.f16_weights && L.dtype == kF8 && L.head_dim == 128u && ncb == 2u) VFKV_P2_OPT(kF8, 2, 2, true, false)
-            else if (L.f16_weights && L.dtype == kF16 && L.head_dim == 128u && ncb == 4u) VFKV_P2_OPT(kF16, 4, 1, true, false)
-            else
-#undef VFKV_P2_OPT
-            VFKV_P2(kF8, 64, 2, 2) VFKV_P2(kF8, 64, 1, 2) VFKV_P2(kF8, 128, 2, 2) VFKV_P2(kF8, 128, 1, 2)
+            // FP8 rows of 128 elements, two heads per wavefront: the kernel that loads V straight into LDS.  Its options --
+            // f16_weights: one product with the weights instead of value + remainder; fp8_scores: the first product on the
+            // FP8 matrix instruction (needs the Q block staged in one round: four key splits).  Over F16 rows (four heads per
+            // wavefront) f16_weights is an instantiation of the general kernel; other shapes keep the default arithmetic.
+            const bool f8s = L.fp8_scores && vdma && ns >= 4u;
+#define VFKV_PDMA(F16WV, F8SV)                                                                                         \
+    { if (cap) hipLaunchKernelGGL((batch_dma_kernel<true, F16WV, F8SV>), grid, block, lds, stream, a, (int)hp, (int)ns);  \
+      else hipLaunchKernelGGL((batch_dma_kernel<false, F16WV, F8SV>), grid, block, lds, stream, a, (int)hp, (int)ns); }
+            if (vdma && f8s && L.f16_weights) VFKV_PDMA(true, true)
+            else if (vdma && f8s) VFKV_PDMA(false, true)
+            else if (vdma && L.f16_weights) VFKV_PDMA(true, false)
+            else if (vdma) VFKV_PDMA(false, false)
+#undef VFKV_PDMA
+            else if (L.f16_weights && L.dtype == kF16 && L.head_dim == 128u && ncb == 4u) {
+                if (cap) hipLaunchKernelGGL((batch_mfma2_kernel<kF16, 128, 4, 1, true, 1, true>), grid, block, lds, stream, a, (int)hp, (int)ns);
+                else hipLaunchKernelGGL((batch_mfma2_kernel<kF16, 128, 4, 1, false, 1, true>), grid, block, lds, stream, a, (int)hp, (int)ns);
+            } else
+            VFKV_P2(kF8, 64, 2, 2) VFKV_P2(kF8, 64, 1, 2) VFKV_P2(kF8, 128, 1, 2)
             VFKV_P2(kF16, 64, 2, 2) VFKV_P2(kF16, 64, 1, 2) VFKV_P2(kF16, 128, 1, 1) VFKV_P2(kF16, 128, 2, 1)
             VFKV_P2(kF8, 256, 1, 1) VFKV_P2(kF16, 256, 1, 1)
             VFKV_P2(kF16, 128, 4, 1) VFKV_P2(kF8, 256, 2, 1) VFKV_P2(kF16, 256, 2, 1)

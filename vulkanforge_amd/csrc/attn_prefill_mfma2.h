@@ -19,10 +19,6 @@
 //
 // Q is used as f16(q); when some q of the workgroup is not exactly representable the first product is
 // repeated with f16(q - f16(q)) kept in LDS, which restores f32-level accuracy.
-//
-// FP8 rows of 128 elements with two heads per wavefront (the form the long-prompt benchmark runs) differ in two ways (VDMA,
-// PAIR below): V tiles are loaded from global memory straight into LDS as FP8 and widened after the byte-transposing LDS
-// read, and the fast loop issues the first products of two tiles before their softmax.
 #pragma once
 #include <type_traits>
 
@@ -36,7 +32,7 @@ constexpr int kPrefillOneHeadWaves = 12;
 // workgroup barrier per tile, and each then
 // accumulates, merges and stores its own slice of D / NH output elements: the accumulators of a 512-wide head do not fit
 // one wavefront.  HP then counts (head, slice) units.
-template <int DT, int D, int NCB, int PFD, bool CAP, int NH = 1, bool F16W = false, bool F8S = false>
+template <int DT, int D, int NCB, int PFD, bool CAP, int NH = 1, bool F16W = false>
 __global__ __launch_bounds__((NCB == 1 && D <= 128) ? kPrefillOneHeadWaves * 64 : (NCB * D >= 512 || (DT == kF16 && D == 256)) ? 256 : 512) void batch_mfma2_kernel(BatchArgs a, int HP, int NS) {
     constexpr int DV = D / NH;                   // output elements (V columns) of this wavefront
     constexpr int ES = DT == kF16 ? 2 : 1;
@@ -56,21 +52,11 @@ __global__ __launch_bounds__((NCB == 1 && D <= 128) ? kPrefillOneHeadWaves * 64 
     // 16 / 2 / 512, 512 x 4 608: 218 us without, 245 us with)
     constexpr bool XCH = NH == 2 && !(DT == kF8 && NCB == 2);
     constexpr int NKT = XCH ? 1 : 2;             // 16-key halves of a tile this wavefront loads and scores
-    // VDMA (FP8 rows of 128 elements, two heads per wavefront): V tiles go from global memory straight into LDS as the cache
-    // holds them (buffer loads with the LDS bit, three tiles per wavefront in rotation: the one being read and the next two
-    // under way), and the second product's operand comes from the byte-transposing LDS read, widened to f16 in registers.
-    // The wavefront then holds no V registers and writes no f16 copy.  PAIR: the fast loop takes its tiles in groups whose
-    // first products are issued together (the registers that V no longer needs hold the second tile's scores).
-    constexpr bool VDMA = DT == kF8 && D == 128 && NH == 1 && NCB == 2 && PFD == 2;
-    constexpr bool PAIR = VDMA;
-    constexpr int VBUF = KT * D;                 // VDMA: bytes of a raw V tile
     static_assert(NH == 1 || NH == 2, "one or two wavefronts per head");
     static_assert(D % 32 == 0 && SEGB % 16 == 0 && VLD >= 1, "unsupported head_dim");
-    static_assert(!F8S || (DT == kF8 && D == 128 && NH == 1), "the fp8 first product is built for FP8 rows of 128 elements");
 
-    extern __shared__ __attribute__((aligned(16))) _Float16 lds[];      // [waves][KT][VPITCH] V tiles (VDMA: [waves][3][KT * D] bytes) | [GP][16][D + 8] f16(q) | [GP][16][D + 8] remainders
+    extern __shared__ __attribute__((aligned(16))) _Float16 lds[];      // [waves][KT][VPITCH] V tiles | [GP][16][D + 8] f16(q) | [GP][16][D + 8] remainders
     __shared__ int lds_haslo;
-    __shared__ uint32_t lds_qmax;                                // F8S: bits of the largest |q| of the workgroup's Q block
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -78,8 +64,8 @@ __global__ __launch_bounds__((NCB == 1 && D <= 128) ? kPrefillOneHeadWaves * 64 
     const int hp = w % HP, sp = w / HP;
     const int n16 = lane & 15, kg = lane >> 4;
     const int G = a.n_heads / a.n_kv_heads;
-    const uint32_t kvh = blockIdx.y;
-    const uint32_t q0 = blockIdx.x * 16;
+    const uint32_t kvh = blockIdx.x;
+    const uint32_t q0 = blockIdx.y * 16;
     const uint32_t qi = q0 + n16;                               // this lane's query (column of S^T)
     const bool q_ok = qi < a.m;
     const uint32_t row_stride = a.n_kv_heads * D * ES;
@@ -89,9 +75,8 @@ __global__ __launch_bounds__((NCB == 1 && D <= 128) ? kPrefillOneHeadWaves * 64 
     const int dslice = hp % NH;                                 // which D / NH output elements this wavefront owns
 
     _Float16* const vb = lds + (size_t)w * KT * VPITCH;
-    uint8_t* const v8 = reinterpret_cast<uint8_t*>(lds) + (size_t)w * 3 * VBUF;   // VDMA: [3][KT * D] raw V tiles of this wavefront
     constexpr int QPITCH = D + 8;
-    _Float16* const qhi_lds = lds + (VDMA ? (size_t)nwaves * 3 * VBUF / 2 : (size_t)nwaves * KT * VPITCH);   // [GP][16][D + 8] f16(q); the slots past G hold zeros
+    _Float16* const qhi_lds = lds + (size_t)nwaves * KT * VPITCH;   // [GP][16][D + 8] f16(q); the slots past G hold zeros
     const int GP = (HP / NH) * NCB;                                 // head slots of the workgroup: G rounded up to whole wavefronts
     _Float16* const qlo_lds = qhi_lds + (size_t)GP * 16 * QPITCH;   // [GP][16][D + 8] f16(q - f16(q))
     float4_t* const xbuf = reinterpret_cast<float4_t*>(qlo_lds + (size_t)GP * 16 * QPITCH);   // XCH: [2][waves][NCB][64] score halves
@@ -121,54 +106,17 @@ __global__ __launch_bounds__((NCB == 1 && D <= 128) ? kPrefillOneHeadWaves * 64 
 
     const uint32_t kt_own = XCH ? (uint32_t)dslice : 0u;         // XCH: the half this wavefront scores
     u32x4 kraw[PFD][NKT][KLD];
-    u32x4 vraw[VDMA ? 1 : PFD][VLD];
-    // VDMA.  A buffer load with the LDS bit writes lane L's 16 bytes at (LDS base) + 16 L, so one load lays down eight rows of
-    // 128 bytes; which 16-byte chunk of its row a lane fetches is free.  Lane L of the load for rows 8 b .. 8 b + 7 fetches
-    // chunk (L % 8) ^ rot(row) of row 8 b + L / 8, rot(row) = (row % 8) ^ (row >= 16 ? 4 : 0): the transposing read of the
-    // second product then takes one chunk index from eight rows (four consecutive ones and the four 16 rows further) and
-    // finds them in eight different bank groups.
-    const uint32_t lane_vdma = (uint32_t)(lane / 8) * row_stride + head_b;
-    const uint32_t vdma_lo = lane_vdma + (uint32_t)(((lane % 8) ^ (lane / 8)) * 16);          // rows 0..15 of a tile
-    const uint32_t vdma_hi = lane_vdma + (uint32_t)(((lane % 8) ^ (lane / 8) ^ 4) * 16);      // rows 16..31
-    const int vrow_rd = (n16 < 8 ? 0 : 16) + kg * 4 + (n16 / 2) % 4;        // the row this lane supplies to the transposing read
-    const uint32_t vdma_rd = (uint32_t)((vrow_rd >> 3) * 1024 + (vrow_rd & 7) * 128 + (n16 & 1) * 8 +
-                                        (((vrow_rd & 7) ^ (vrow_rd >= 16 ? 4 : 0)) << 4));   // chunk index dt enters by XOR
-    int vcur = 0;                                               // VDMA: buffer (0..2) of the tile the second product reads next
-    // The loads are written as assembly: the compiler would otherwise wait, before every LDS read, for the newest load that
-    // writes LDS -- the prefetch of the tile after next -- because it cannot tell the three buffers apart.  Here the wait in
-    // front of the transposing reads counts the loads issued since the tile they read: vmcnt(8), two tiles of four loads
-    // (loads into registers that the compiler places between them only make the count more patient than necessary).
-    const u32x4 vdesc = u32x4{(uint32_t)(uintptr_t)a.v, (uint32_t)((uintptr_t)a.v >> 32) & 0xFFFFu, a.n_kv * row_stride, 0x00020000u};
-    const uint32_t v8_addr = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) void*)v8;
-    auto v_dma = [&](int buf, uint32_t toff) {
-#pragma unroll
-        for (int b = 0; b < 4; ++b)
-            // (m0 is reserved: the compiler sets it itself in front of every instruction of its own that reads it)
-            asm volatile("s_mov_b32 m0, %0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
-                         :: "s"(v8_addr + (uint32_t)(buf * VBUF + b * 1024)), "v"(b < 2 ? vdma_lo : vdma_hi), "s"(vdesc),
-                            "s"(toff + (uint32_t)(b * 8) * row_stride) : "memory");
-    };
+    u32x4 vraw[PFD][VLD];
     auto issue = [&](int slot, uint32_t toff) {
 #pragma unroll
         for (int kt = 0; kt < NKT; ++kt)
 #pragma unroll
             for (int x = 0; x < KLD; ++x)
                 kraw[slot][kt][x] = __builtin_amdgcn_raw_buffer_load_b128(krsrc, lane_koff + x * 16, toff + ((uint32_t)kt + kt_own) * 16u * row_stride, 0);
-        if constexpr (VDMA) {
-            v_dma(slot, toff);
-        } else {
 #pragma unroll
-            for (int c = 0; c < VLD; ++c)
-                vraw[slot][c] = __builtin_amdgcn_raw_buffer_load_b128(vrsrc, lane_voff, toff + (uint32_t)(c * VROWS) * row_stride, 0);
-        }
+        for (int c = 0; c < VLD; ++c)
+            vraw[slot][c] = __builtin_amdgcn_raw_buffer_load_b128(vrsrc, lane_voff, toff + (uint32_t)(c * VROWS) * row_stride, 0);
     };
-    if constexpr (VDMA) {
-        // rows past the end of the cache are outside the buffer: whatever such a lane leaves in LDS only ever meets weights
-        // of zero, so it must be a finite number -- the buffers start as zeros
-#pragma unroll
-        for (int i = 0; i < 3 * VBUF / (64 * 16); ++i) *reinterpret_cast<u32x4*>(v8 + (i * 64 + lane) * 16) = u32x4{0u, 0u, 0u, 0u};
-        __builtin_amdgcn_s_waitcnt(0xC07F);                     // lgkmcnt(0): the zeros are in place before a load can overwrite them
-    }
     const uint32_t step = KT * NS;
     const uint32_t tb0 = t_first + sp * KT;                     // this wavefront's first tile (may already be past the end)
     // XCH: every tile has a workgroup barrier, so every wavefront walks the same number of tiles; the ones past the last key
@@ -182,55 +130,7 @@ __global__ __launch_bounds__((NCB == 1 && D <= 128) ? kPrefillOneHeadWaves * 64 
     constexpr int QLD = 4;                                      // query loads per thread and round
     const int nthreads = nwaves * 64;
     const int q4_total = 16 * GP * (D / 4);
-    // F8S: Q as three E4M3 planes q ~ 2^e (t1 + t2 / 16 + t3 / 256), every term the E4M3 rounding of what the terms before it
-    // left (12 significant bits: exact for f16-representable q; e keeps the largest |q| of the block below 256).  The first
-    // product then runs on the FP8 matrix instruction with the cache rows as they are.
-    constexpr int Q8PITCH = D + 16;                             // bytes per (head slot, query) row of a term plane
-    uint8_t* const q8_lds = reinterpret_cast<uint8_t*>(qhi_lds);    // [3][GP][16][Q8PITCH]
-    int q_exp = 0;
     bool has_lo = false;
-    if constexpr (F8S) {
-        if (tid == 0) lds_qmax = 0u;
-        float4 qf[QLD];                                         // the launcher guarantees q4_total <= QLD * nthreads
-        float amax = 0.f;
-#pragma unroll
-        for (int i = 0; i < QLD; ++i) {
-            const int idx = tid + i * nthreads;
-            const int qq = idx / (GP * (D / 4)), rem = idx - qq * (GP * (D / 4));
-            const bool ok = idx < q4_total && q0 + qq < a.m && rem < (G - gz) * (D / 4);
-            qf[i] = *reinterpret_cast<const float4*>(a.q + ((size_t)(ok ? q0 + qq : 0) * a.n_heads + kvh * G + gz) * D + (ok ? rem * 4 : 0));
-            if (!ok) qf[i] = make_float4(0.f, 0.f, 0.f, 0.f);
-            amax = fmaxf(fmaxf(amax, fmaxf(fabsf(qf[i].x), fabsf(qf[i].y))), fmaxf(fabsf(qf[i].z), fabsf(qf[i].w)));
-        }
-#pragma unroll
-        for (int sl = 0; sl < PFD; ++sl) issue(sl, tile_off(tb0 + sl * step));
-        __syncthreads();                                        // lds_qmax cleared
-        amax = wave_max_uniform(amax);
-        if (lane == 0) atomicMax(&lds_qmax, __builtin_bit_cast(uint32_t, amax));   // non-negative floats order like their bits
-        __syncthreads();
-        const uint32_t mb = lds_qmax;
-        q_exp = (int)((mb >> 23) & 0xFFu) - 127 - 7;            // floor(log2(max|q|)) - 7: max|q| * 2^-e < 256
-        q_exp = q_exp < -100 ? -100 : q_exp > 100 ? 100 : q_exp;
-        const float down = __builtin_bit_cast(float, (uint32_t)(127 - q_exp) << 23);
-#pragma unroll
-        for (int i = 0; i < QLD; ++i) {
-            const int idx = tid + i * nthreads;
-            if (idx >= q4_total) continue;
-            const int qq = idx / (GP * (D / 4)), rem = idx - qq * (GP * (D / 4));
-            const int g = rem / (D / 4), d = (rem - g * (D / 4)) * 4;
-            float r[4] = {qf[i].x * down, qf[i].y * down, qf[i].z * down, qf[i].w * down};
-#pragma unroll
-            for (int t = 0; t < 3; ++t) {
-                int w8 = __builtin_amdgcn_cvt_pk_fp8_f32(r[0], r[1], 0, false);
-                w8 = __builtin_amdgcn_cvt_pk_fp8_f32(r[2], r[3], w8, true);
-                *reinterpret_cast<uint32_t*>(q8_lds + ((size_t)(t * GP + g) * 16 + qq) * Q8PITCH + d) = (uint32_t)w8;
-                const float2_t d01 = __builtin_amdgcn_cvt_pk_f32_fp8(w8, false), d23 = __builtin_amdgcn_cvt_pk_f32_fp8(w8, true);
-                r[0] = (r[0] - d01[0]) * 16.f; r[1] = (r[1] - d01[1]) * 16.f;
-                r[2] = (r[2] - d23[0]) * 16.f; r[3] = (r[3] - d23[1]) * 16.f;
-            }
-        }
-        __syncthreads();                                        // planes written
-    } else {
     if (tid == 0) lds_haslo = 0;
     bool any_lo = false;
     for (int base = 0; base < q4_total; base += QLD * nthreads) {
@@ -265,7 +165,6 @@ __global__ __launch_bounds__((NCB == 1 && D <= 128) ? kPrefillOneHeadWaves * 64 
     if (any_lo) lds_haslo = 1;
     __syncthreads();
     has_lo = __builtin_amdgcn_readfirstlane(lds_haslo) != 0;   // workgroup-uniform
-    }
 
     float4_t oacc[NCB][DTILES];
 #pragma unroll
@@ -277,16 +176,12 @@ __global__ __launch_bounds__((NCB == 1 && D <= 128) ? kPrefillOneHeadWaves * 64 
     for (int cb = 0; cb < NCB; ++cb) { m_run[cb] = kMasked; l_run[cb] = 0.f; }
 
     // ---- pieces of one tile ----
-    float4_t s[PFD][NCB][2];
-    float x[PFD][NCB][8], tmax[PFD][NCB];
-    // V tile -> f16 row-major in this wavefront's LDS area (before the first product, so that the writes complete behind it
-    // and the softmax) and the slot's next tile requested; VDMA: only the request, for the tile after next
-    auto stage_v = [&](int sl, uint32_t tcur) {
+    float4_t s[NCB][2];
+    float x[NCB][8], tmax[NCB];
+    // V tile -> f16 row-major in this wavefront's LDS area (first: the writes complete behind the first product and the
+    // softmax), the slot's next tile requested, then S^T = K Q^T for the NCB heads (Q operands re-read from LDS every tile)
+    auto stage_and_first_product = [&](int sl, uint32_t tcur) {
         const uint32_t noff = tile_off(tcur + PFD * step);
-        if constexpr (VDMA) {                                   // the tile after next goes where the previous tile was
-            const int nb = vcur + 2 >= 3 ? vcur - 1 : vcur + 2;
-            v_dma(nb, noff);
-        } else {
 #pragma unroll
         for (int c = 0; c < VLD; ++c) {
             _Float16* dst = vb + (c * VROWS + vrow) * VPITCH + vcol * (16 / ES);
@@ -306,49 +201,6 @@ __global__ __launch_bounds__((NCB == 1 && D <= 128) ? kPrefillOneHeadWaves * 64 
                 *reinterpret_cast<u32x4*>(dst) = vraw[sl][c];
             }
             vraw[sl][c] = __builtin_amdgcn_raw_buffer_load_b128(vrsrc, lane_voff, noff + (uint32_t)(c * VROWS) * row_stride, 0);
-        }
-        }
-    };
-    // S^T = K Q^T for the NCB heads (Q operands re-read from LDS every tile); lo_tag: whether the remainder plane of Q takes
-    // part (a bool, or a type where the walk is compiled once per case)
-    auto first_product = [&](int sl, uint32_t tcur, auto lo_tag) {
-        bool with_lo;
-        if constexpr (std::is_same_v<decltype(lo_tag), bool>) with_lo = lo_tag; else with_lo = decltype(lo_tag)::value;
-        const uint32_t noff = tile_off(tcur + PFD * step);
-        if constexpr (F8S) {
-            // S^T = K Q^T on the FP8 matrix instruction: A = the lane's quarter row of K as loaded (32 codes), B = the same
-            // quarter of the query's three term planes, each with its power-of-two weight as the instruction's block scale
-#pragma unroll
-            for (int cb = 0; cb < NCB; ++cb)
-#pragma unroll
-                for (int kt = 0; kt < 2; ++kt) s[sl][cb][kt] = float4_t{0.f, 0.f, 0.f, 0.f};
-            typedef int v8i_t __attribute__((ext_vector_type(8)));
-            v8i_t ka8[2];
-#pragma unroll
-            for (int kt = 0; kt < 2; ++kt)
-#pragma unroll
-                for (int j = 0; j < 8; ++j) ka8[kt][j] = (int)kraw[sl][kt][j / 4][j % 4];
-#pragma unroll
-            for (int t = 0; t < 3; ++t) {
-                const int sb = 127 + q_exp - 4 * t;             // E8M0 code of 2^(e - 4t)
-#pragma unroll
-                for (int cb = 0; cb < NCB; ++cb) {
-                    const uint8_t* qrow = q8_lds + ((size_t)(t * GP + g0 + cb) * 16 + n16) * Q8PITCH + kg * 32;
-                    const u32x4 b0 = *reinterpret_cast<const u32x4*>(qrow), b1 = *reinterpret_cast<const u32x4*>(qrow + 16);
-                    v8i_t qb8;
-#pragma unroll
-                    for (int j = 0; j < 4; ++j) { qb8[j] = (int)b0[j]; qb8[4 + j] = (int)b1[j]; }
-#pragma unroll
-                    for (int kt = 0; kt < 2; ++kt)
-                        s[sl][cb][kt] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(ka8[kt], qb8, s[sl][cb][kt], 0, 0, 0, 127, 0, sb);
-                }
-            }
-#pragma unroll
-            for (int kt = 0; kt < 2; ++kt)
-#pragma unroll
-                for (int xx = 0; xx < KLD; ++xx)
-                    kraw[sl][kt][xx] = __builtin_amdgcn_raw_buffer_load_b128(krsrc, lane_koff + xx * 16, noff + (uint32_t)(kt * 16) * row_stride, 0);
-            return;
         }
         half8_t qhi[NCB][KS];
 #pragma unroll
@@ -382,19 +234,19 @@ __global__ __launch_bounds__((NCB == 1 && D <= 128) ? kPrefillOneHeadWaves * 64 
                 float4_t acc = float4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
                 for (int c = 0; c < KS; ++c) acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(ka[c], qhi[cb][c], acc, 0, 0, 0);
-                if (XCH) sown[cb] = acc; else s[sl][cb][kt] = acc;
+                if (XCH) sown[cb] = acc; else s[cb][kt] = acc;
             }
-            if (with_lo) {
+            if (has_lo) {
 #pragma unroll
                 for (int cb = 0; cb < NCB; ++cb) {
                     const _Float16* lo_row = qlo_lds + ((size_t)(g0 + cb) * 16 + n16) * QPITCH + kg * SEG;
-                    float4_t acc = XCH ? sown[cb] : s[sl][cb][kt];
+                    float4_t acc = XCH ? sown[cb] : s[cb][kt];
 #pragma unroll
                     for (int c = 0; c < KS; ++c) {
                         const half8_t ql = *reinterpret_cast<const half8_t*>(lo_row + c * 8);
                         acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(ka[c], ql, acc, 0, 0, 0);
                     }
-                    if (XCH) sown[cb] = acc; else s[sl][cb][kt] = acc;
+                    if (XCH) sown[cb] = acc; else s[cb][kt] = acc;
                 }
             }
         }
@@ -410,43 +262,43 @@ __global__ __launch_bounds__((NCB == 1 && D <= 128) ? kPrefillOneHeadWaves * 64 
 #pragma unroll
             for (int cb = 0; cb < NCB; ++cb) {
                 const float4_t other = xr[cb * 64];
-                s[sl][cb][0] = kt_own == 0u ? sown[cb] : other;
-                s[sl][cb][1] = kt_own == 0u ? other : sown[cb];
+                s[cb][0] = kt_own == 0u ? sown[cb] : other;
+                s[cb][1] = kt_own == 0u ? other : sown[cb];
             }
             xpar ^= 1;
         }
     };
     // scores of the tile in log2 units (this lane owns keys tcur + kt*16 + kg*4 + i of query n16); returns whether one of
     // them exceeds the lane's reference maximum by more than the slack
-    auto scores = [&](auto masked_tag, int sl, uint32_t tcur) -> bool {
+    auto scores = [&](auto masked_tag, uint32_t tcur) -> bool {
         constexpr bool MASKED = decltype(masked_tag)::value;
         constexpr bool FOLD = !MASKED && !CAP;                   // scores stay unscaled until the exponent's FMA
         bool moved = false;
 #pragma unroll
         for (int cb = 0; cb < NCB; ++cb) {
-            tmax[sl][cb] = kMasked;
+            tmax[cb] = kMasked;
 #pragma unroll
             for (int kt = 0; kt < 2; ++kt)
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
-                    float y = FOLD ? s[sl][cb][kt][i] : s[sl][cb][kt][i] * scale_l2;
+                    float y = FOLD ? s[cb][kt][i] : s[cb][kt][i] * scale_l2;
                     if (CAP) y = cap_l2 * tanhf(y / cap_l2);
                     if (MASKED) {
                         const uint32_t t = tcur + kt * 16 + kg * 4 + i;
                         y = (t < my_len && t >= a.kv_start && t < kmax) ? y : kMasked;    // (t >= kmax: padding tiles of a key chunk)
                     }
-                    x[sl][cb][kt * 4 + i] = y;
-                    tmax[sl][cb] = fmaxf(tmax[sl][cb], y);
+                    x[cb][kt * 4 + i] = y;
+                    tmax[cb] = fmaxf(tmax[cb], y);
                 }
-            if (FOLD) tmax[sl][cb] *= scale_l2;
-            moved |= tmax[sl][cb] > m_run[cb] + kMaxSlack;
+            if (FOLD) tmax[cb] *= scale_l2;
+            moved |= tmax[cb] > m_run[cb] + kMaxSlack;
         }
         return moved;
     };
-    auto move_maximum = [&](int sl) {
+    auto move_maximum = [&]() {
 #pragma unroll
         for (int cb = 0; cb < NCB; ++cb) {
-            float t = tmax[sl][cb];
+            float t = tmax[cb];
             { float y = t; swap16(t, y); t = fmaxf(t, y); y = t; swap32(t, y); t = fmaxf(t, y); }
             const float m_new = fmaxf(m_run[cb], t);
             const float alpha = __builtin_amdgcn_exp2f(m_run[cb] - m_new);
@@ -456,14 +308,14 @@ __global__ __launch_bounds__((NCB == 1 && D <= 128) ? kPrefillOneHeadWaves * 64 
             m_run[cb] = m_new;
         }
     };
-    // weights of a tile as f16 value + f16 remainder, kept per slot
+    // weights as f16 value + f16 remainder, then O^T += V^T P^T for the NCB heads
     // TWO: the weights enter the product as f16 value + f16 remainder (two MFMAs per d-tile and head: f32-level accuracy);
     // otherwise as the f16 value alone (the F16W instantiations).
-    u32x4 phi[PFD][NCB], plo[PFD][NCB];
-    auto weights = [&](auto masked_tag, auto two_tag, int sl) {
+    auto weights_and_second_product = [&](auto masked_tag, auto two_tag) {
         constexpr bool MASKED = decltype(masked_tag)::value;
         constexpr bool TWO = decltype(two_tag)::value;
         constexpr bool FOLD = !MASKED && !CAP;
+        u32x4 phi[NCB], plo[NCB];
 #pragma unroll
         for (int cb = 0; cb < NCB; ++cb)
 #pragma unroll
@@ -471,55 +323,32 @@ __global__ __launch_bounds__((NCB == 1 && D <= 128) ? kPrefillOneHeadWaves * 64 
                 float2_t pp;
 #pragma unroll
                 for (int e = 0; e < 2; ++e) {
-                    const float xe = x[sl][cb][2 * j2 + e];
+                    const float xe = x[cb][2 * j2 + e];
                     float pv = __builtin_amdgcn_exp2f(FOLD ? __builtin_fmaf(xe, scale_l2, -m_run[cb]) : xe - m_run[cb]);
                     if (MASKED) pv = xe > -1e29f ? pv : 0.f;
                     pp[e] = pv;
                 }
                 l_run[cb] += pp[0] + pp[1];
-                phi[sl][cb][j2] = __builtin_bit_cast(uint32_t, __builtin_convertvector(pp, half2_t));
-                if (TWO) plo[sl][cb][j2] = pack_f16_remainder(pp[0], pp[1], phi[sl][cb][j2]);
+                phi[cb][j2] = __builtin_bit_cast(uint32_t, __builtin_convertvector(pp, half2_t));
+                if (TWO) plo[cb][j2] = pack_f16_remainder(pp[0], pp[1], phi[cb][j2]);
             }
-    };
-    // O^T += V^T P^T for the NCB heads with the weights of slot sl.  VDMA: first the request for the tile after next (into
-    // the buffer of the tile before this one, whose second product is done), then the wait for this tile's rows.
-    auto second_product = [&](auto two_tag, int sl, uint32_t tcur) {
-        constexpr bool TWO = decltype(two_tag)::value;
-        typedef int v2i_t __attribute__((ext_vector_type(2)));
-        uint32_t vrd = 0u;
-        if constexpr (VDMA) {
-            stage_v(sl, tcur);
-            // supplier lane s of a 16-lane group points at the 8 bytes V[key][dt*16 + 8*(s%2) ..], key = 4*kg + s/2 for
-            // s < 8 and 16 + 4*kg + (s/2 - 4) above; the read hands lane n the bytes of the eight keys at d = dt*16 + n
-            vrd = vdma_rd + (uint32_t)(vcur * VBUF);
-            asm volatile("s_waitcnt vmcnt(8)" ::: "memory");   // this tile's V rows are in LDS
-        }
 #pragma unroll
         for (int dt = 0; dt < DTILES; ++dt) {
+            // supplier lane s of a 16-lane group points at V[key = 4*kg + s/4 (+16)][d = dt*16 + 4*(s%4)]
+            const _Float16* p0 = vb + (kg * 4 + n16 / 4) * VPITCH + dt * 16 + 4 * (n16 % 4);
+            const half4_t v0 = lds_read_tr16(p0);
+            const half4_t v1 = lds_read_tr16(p0 + 16 * VPITCH);
             half8_t va;
-            if constexpr (VDMA) {
-                const v2i_t raw = __builtin_amdgcn_ds_read_tr8_b64_v2i32((__attribute__((address_space(3))) v2i_t*)(v8 + (vrd ^ (uint32_t)(dt << 4))));
-                half2_t p0, p1, p2, p3;
-                e4m3x4_to_h2((uint32_t)raw[0], p0, p1);
-                e4m3x4_to_h2((uint32_t)raw[1], p2, p3);
-                va[0] = p0[0]; va[1] = p0[1]; va[2] = p1[0]; va[3] = p1[1]; va[4] = p2[0]; va[5] = p2[1]; va[6] = p3[0]; va[7] = p3[1];
-            } else {
-                // supplier lane s of a 16-lane group points at V[key = 4*kg + s/4 (+16)][d = dt*16 + 4*(s%4)]
-                const _Float16* p0 = vb + (kg * 4 + n16 / 4) * VPITCH + dt * 16 + 4 * (n16 % 4);
-                const half4_t v0 = lds_read_tr16(p0);
-                const half4_t v1 = lds_read_tr16(p0 + 16 * VPITCH);
-                va[0] = v0[0]; va[1] = v0[1]; va[2] = v0[2]; va[3] = v0[3]; va[4] = v1[0]; va[5] = v1[1]; va[6] = v1[2]; va[7] = v1[3];
-            }
+            va[0] = v0[0]; va[1] = v0[1]; va[2] = v0[2]; va[3] = v0[3]; va[4] = v1[0]; va[5] = v1[1]; va[6] = v1[2]; va[7] = v1[3];
 #pragma unroll
             for (int cb = 0; cb < NCB; ++cb)
-                oacc[cb][dt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(va, __builtin_bit_cast(half8_t, phi[sl][cb]), oacc[cb][dt], 0, 0, 0);
+                oacc[cb][dt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(va, __builtin_bit_cast(half8_t, phi[cb]), oacc[cb][dt], 0, 0, 0);
             if (TWO) {
 #pragma unroll
                 for (int cb = 0; cb < NCB; ++cb)
-                    oacc[cb][dt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(va, __builtin_bit_cast(half8_t, plo[sl][cb]), oacc[cb][dt], 0, 0, 0);
+                    oacc[cb][dt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(va, __builtin_bit_cast(half8_t, plo[cb]), oacc[cb][dt], 0, 0, 0);
             }
         }
-        if constexpr (VDMA) vcur = vcur == 2 ? 0 : vcur + 1;
     };
 
     // ---- the wavefront's tiles.  The reference maximum m of a query only moves when some score of a tile exceeds it by more
@@ -530,76 +359,42 @@ __global__ __launch_bounds__((NCB == 1 && D <= 128) ? kPrefillOneHeadWaves * 64 
     // two loops: the inner one only takes tiles that every query of the block sees completely and leaves as soon as a
     // maximum has to move, so that its accumulators have a single definition per tile and stay in place; the outer one
     // handles whatever the inner one left (first tiles, moved maxima, tiles on the causal diagonal or the window edge).
-    // The walk exists in two compiled forms where the fast loop is the grouped one: without the remainder product its
-    // first products are straight-line code.
-    auto walk = [&](auto lo_tag) {
-    constexpr bool GROUP = PAIR && std::is_same_v<decltype(lo_tag), std::false_type>;   // (the remainder product's registers leave no room for a second tile's scores)
     uint32_t tb = tb0;
     int first_slot = 0;          // slots of the group at tb that the inner loop has already finished
-    bool s_ready = false;        // the inner loop left the group at tb with scores computed: those of slot first_slot (and, except
-                                 // in the VDMA form, its V tile staged); GROUP: those of every slot
-    constexpr auto two_tag = std::integral_constant<bool, !F16W>{};
+    bool s_ready = false;        // s[] of slot first_slot is already computed
     while (tb < kloop) {
 #pragma unroll
         for (int sl = 0; sl < PFD; ++sl) {
             const uint32_t tcur = tb + sl * step;
             if (tcur >= kloop) break;                           // wavefront-uniform
             if (sl < first_slot) continue;
-            if (!(s_ready && (GROUP || sl == first_slot))) {
-                if constexpr (!VDMA) stage_v(sl, tcur);
-                first_product(sl, tcur, lo_tag);
-            }
+            if (!(s_ready && sl == first_slot)) stage_and_first_product(sl, tcur);
             if (tcur >= a.kv_start && tcur + KT <= fast_end) {  // every query of the block sees the whole tile (and it is this workgroup's)
-                if (__builtin_amdgcn_ballot_w64(scores(std::false_type{}, sl, tcur)) != 0ull) move_maximum(sl);
-                weights(std::false_type{}, two_tag, sl);
+                if (__builtin_amdgcn_ballot_w64(scores(std::false_type{}, tcur)) != 0ull) move_maximum();
+                weights_and_second_product(std::false_type{}, std::integral_constant<bool, !F16W>{});
             } else {
-                if (__builtin_amdgcn_ballot_w64(scores(std::true_type{}, sl, tcur)) != 0ull) move_maximum(sl);
-                weights(std::true_type{}, two_tag, sl);
+                if (__builtin_amdgcn_ballot_w64(scores(std::true_type{}, tcur)) != 0ull) move_maximum();
+                weights_and_second_product(std::true_type{}, std::integral_constant<bool, !F16W>{});
             }
-            second_product(two_tag, sl, tcur);
         }
         tb += PFD * step;
         first_slot = 0;
         s_ready = false;
-        if constexpr (GROUP) {
-            // a whole group per pass: the first products of its tiles do not depend on the softmax and the second product of
-            // the tiles before them, so the matrix pipe and the vector ALU have work from different tiles side by side
-            while (tb >= a.kv_start && tb + (PFD - 1) * step + KT <= fast_end) {
-                bool moved = false;
+        bool left = false;
+        while (!left && tb >= a.kv_start && tb + (PFD - 1) * step + KT <= fast_end) {
 #pragma unroll
-                for (int sl = 0; sl < PFD; ++sl) first_product(sl, tb + sl * step, lo_tag);
-#pragma unroll
-                for (int sl = 0; sl < PFD; ++sl) moved |= scores(std::false_type{}, sl, tb + sl * step);
-                if (__builtin_amdgcn_ballot_w64(moved) != 0ull) { s_ready = true; break; }
-#pragma unroll
-                for (int sl = 0; sl < PFD; ++sl) {
-                    weights(std::false_type{}, two_tag, sl);
-                    second_product(two_tag, sl, tb + sl * step);
+            for (int sl = 0; sl < PFD; ++sl) {
+                const uint32_t tcur = tb + sl * step;
+                stage_and_first_product(sl, tcur);
+                if (__builtin_amdgcn_ballot_w64(scores(std::false_type{}, tcur)) != 0ull) {
+                    first_slot = sl; s_ready = true; left = true;
+                    break;
                 }
-                tb += PFD * step;
+                weights_and_second_product(std::false_type{}, std::integral_constant<bool, !F16W>{});
             }
-        } else {
-            bool left = false;
-            while (!left && tb >= a.kv_start && tb + (PFD - 1) * step + KT <= fast_end) {
-#pragma unroll
-                for (int sl = 0; sl < PFD; ++sl) {
-                    const uint32_t tcur = tb + sl * step;
-                    if constexpr (!VDMA) stage_v(sl, tcur);
-                    first_product(sl, tcur, lo_tag);
-                    if (__builtin_amdgcn_ballot_w64(scores(std::false_type{}, sl, tcur)) != 0ull) {
-                        first_slot = sl; s_ready = true; left = true;
-                        break;
-                    }
-                    weights(std::false_type{}, two_tag, sl);
-                    second_product(two_tag, sl, tcur);
-                }
-                if (!left) tb += PFD * step;
-            }
+            if (!left) tb += PFD * step;
         }
     }
-    };
-    if constexpr (PAIR) { if (has_lo) walk(std::true_type{}); else walk(std::false_type{}); }
-    else walk(has_lo);
 #pragma unroll
     for (int cb = 0; cb < NCB; ++cb) l_run[cb] = xor32_sum(xor16_sum(l_run[cb]));   // every lane of a query column has its wavefront's sum
 

@@ -72,15 +72,14 @@ __global__ __launch_bounds__(256) void batch_mfma_f32_kernel(BatchArgs a) {
     const uint32_t lane_koff = n16 * row_stride + head_b + kg * QB;                      // key l % 16, quarter l / 16
     const uint32_t lane_voff = kg * row_stride + head_b + (half * DV + n16) * ES;        // key l / 16 of a group of four, element l % 16
 
-    uint32_t kraw[KDW];
+    constexpr int KV4 = WIDE ? KDW / 4 : 1;
+    u32x4 kraw4[KV4];                            // WIDE: the quarter row as 16-byte pieces
+    uint32_t kraw[WIDE ? 1 : KDW];
     uint32_t vraw[4][DTILES];
     auto issue = [&](uint32_t toff) {
-        if (WIDE) {
+        if constexpr (WIDE) {
 #pragma unroll
-            for (int x = 0; x < KDW / 4; ++x) {
-                const u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(krsrc, lane_koff + x * 16, toff, 0);
-                kraw[4 * x] = v[0]; kraw[4 * x + 1] = v[1]; kraw[4 * x + 2] = v[2]; kraw[4 * x + 3] = v[3];
-            }
+            for (int x = 0; x < KV4; ++x) kraw4[x] = __builtin_amdgcn_raw_buffer_load_b128(krsrc, lane_koff + x * 16, toff, 0);
         } else {
 #pragma unroll
             for (int x = 0; x < KDW; ++x) kraw[x] = __builtin_amdgcn_raw_buffer_load_b32(krsrc, lane_koff + x * 4, toff, 0);
@@ -123,8 +122,16 @@ __global__ __launch_bounds__(256) void batch_mfma_f32_kernel(BatchArgs a) {
         // ---- operands of this tile out of the load registers, next tile requested ----
         uint32_t kcur[KDW];
         float va[4][DTILES];
+        if constexpr (WIDE) {
 #pragma unroll
-        for (int x = 0; x < KDW; ++x) kcur[x] = kraw[x];
+            for (int x = 0; x < KV4; ++x) {
+                const u32x4 v = kraw4[x];                                // (the whole vector is copied before its elements are taken)
+                kcur[4 * x] = v[0]; kcur[4 * x + 1] = v[1]; kcur[4 * x + 2] = v[2]; kcur[4 * x + 3] = v[3];
+            }
+        } else {
+#pragma unroll
+            for (int x = 0; x < KDW; ++x) kcur[x] = kraw[x];
+        }
 #pragma unroll
         for (int g4 = 0; g4 < 4; ++g4)
 #pragma unroll

@@ -79,6 +79,9 @@ CASES = [
     (vf.KvDtype.F16, 8, 2, 256, 35, 260, 100, 0.0),   # head_dim 256, G = 4 on a 2-byte cache, window
     (vf.KvDtype.F8, 32, 4, 256, 18, 130, 0, 0.0),     # head_dim 256, G = 8: the group is spread over workgroups so that the Q planes fit
     (vf.KvDtype.F16, 16, 16, 256, 20, 90, 0, 20.0),   # head_dim 256, G = 1: seven key splits
+    (vf.KvDtype.F8, 32, 8, 128, 100, 2517, 0, 0.0),   # FP8 rows of 128 elements (V loaded straight into LDS): many two-tile passes, ragged end
+    (vf.KvDtype.F8, 16, 4, 128, 33, 6005, 4100, 30.0),  # the same kernel: window that starts inside a tile, soft-cap
+    (vf.KvDtype.F8, 40, 8, 128, 7, 1037, 0, 0.0),     # G = 5: a padded head slot beside the rotation of V buffers
 ]
 
 
@@ -98,6 +101,29 @@ def test_batch_matches_oracle(dtype, heads, hkv, d, m, q_start, kv_start, cap):
     assert np.isfinite(o).all()
     err = np.abs(o - ref).max()
     assert err < TOL[dtype], err
+
+
+@pytest.mark.parametrize("f32_queries", (False, True))
+@pytest.mark.parametrize("f16_weights,fp8_scores", ((False, False), (True, False), (False, True), (True, True)))
+def test_fp8_head_dim_128_long_context_with_moving_maximum(f32_queries, f16_weights, fp8_scores):
+    """The kernel that loads V tiles straight into LDS (FP8 rows of 128 elements, GQA group >= 2), every form of it: K
+    three times as wide as usual, so that the reference maximum moves in the middle of two-tile passes and the loop
+    leaves and re-enters its fast path with scores already computed; 3 000 keys, ragged last tile."""
+    H, HKV, D, m, q_start = 32, 8, 128, 48, 2953
+    r = rng(4242 + int(f32_queries))
+    n_kv = q_start + m
+    q = r.standard_normal((m, H, D)).astype(np.float32) if f32_queries else fp16_normal(r, (m, H, D))
+    k = encode_np(fp16_normal(r, (n_kv, HKV, D), 3.0), vf.KvDtype.F8)
+    v = encode_np(fp16_normal(r, (n_kv, HKV, D)), vf.KvDtype.F8)
+    scale = float(1.0 / np.sqrt(D))
+    o = torch.full((m, H, D), float("nan"), device=DEV)
+    vf.Forward.run_flash_attn_batch(to_dev(q), to_dev(k.reshape(n_kv, -1)), to_dev(v.reshape(n_kv, -1)), vf.KvDtype.F8, o, H, HKV, D,
+                                    m, q_start, n_kv, scale, f16_weights=f16_weights, fp8_scores=fp8_scores)
+    torch.cuda.synchronize()
+    ref = oracle.attn_batch_ref(q, k, v, int(vf.KvDtype.F8), m, n_kv, H, HKV, D, q_start, scale)
+    err = np.abs(to_np(o) - ref).max()
+    # default: f32-level; the options: weights to 11 bits (2^-11 max|v|, |v| <= 5 here) and scores through the FP8 instruction
+    assert err < (2e-4 if not (f16_weights or fp8_scores) else 6e-3), err
 
 
 @pytest.mark.parametrize("dtype", (vf.KvDtype.F8, vf.KvDtype.F16))

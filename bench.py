@@ -624,6 +624,51 @@ def copy_calibration(args):
             "launches": args.steps, "value": 2 * n * args.steps / dt / 1e9, "unit": "GB/s", "n_gpus": 1}
 
 
+def slab_reuse_calibration(args):
+    """The compute-free readers of libvfkv_calib.so over 64 MiB layer slabs (32 768 rows x 8 KV heads x 128 FP8 bytes, K and
+    V) when consecutive launches rotate over 32, 6, 4, 2 slabs or read one slab again and again: what the memory-side
+    cache (and, for slabs that fit them, the L2s) contribute to a read that follows another read of the same bytes."""
+    import ctypes as C
+    import torch
+    calib = C.CDLL(os.path.join(ROOT, "vulkanforge_amd", "libvfkv_calib.so"))
+    calib.vfkv_calib_stream_read.argtypes = [C.c_void_p, C.c_void_p, C.c_uint64, C.c_void_p, C.c_void_p]
+    calib.vfkv_calib_pattern_read.argtypes = [C.c_void_p, C.c_void_p, C.c_uint32, C.c_uint32, C.c_uint32, C.c_void_p, C.c_void_p]
+    L, ctx, hkv, d = 32, 32768, 8, 128
+    lb = ctx * hkv * d
+    k = torch.randint(0, 255, (L * lb,), dtype=torch.uint8, device="cuda")
+    v = torch.randint(0, 255, (L * lb + 256,), dtype=torch.uint8, device="cuda")[256:]
+    sink = torch.zeros(1024, dtype=torch.int32, device="cuda")
+
+    def timed(launch, n_slabs, frac=1.0):
+        def fn():
+            st = torch.cuda.current_stream().cuda_stream
+            for i in range(L):
+                launch(k.data_ptr() + (i % n_slabs) * lb, v.data_ptr() + (i % n_slabs) * lb, frac, st)
+        fn()
+        torch.cuda.synchronize()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            fn()
+        g.replay()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(max(args.steps, 5)):
+            g.replay()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) * 1e3 / max(args.steps, 5) / L
+
+    pattern = lambda kp, vp, frac, st: calib.vfkv_calib_pattern_read(kp, vp, ctx, hkv, 32, sink.data_ptr(), st)
+    stream = lambda kp, vp, frac, st: calib.vfkv_calib_stream_read(kp, vp, int(lb * frac) // 16 * 16, sink.data_ptr(), st)
+    out = {"metric": "slab_reuse_calibration", "unit": "us per launch", "slab_bytes": 2 * lb, "n_gpus": 1,
+           "pattern_read": {str(n): timed(pattern, n) for n in (32, 6, 4, 2, 1)},
+           "stream_read": {str(n): timed(stream, n) for n in (32, 6, 4, 2, 1)},
+           "stream_read_one_slab_half_and_quarter": [timed(stream, 1, 0.5), timed(stream, 1, 0.25)]}
+    out["value"] = out["pattern_read"]["1"]
+    return out
+
+
 HEADLINE = "decode_fp8_32k_32layers"
 # the other benchmark configurations, run briefly after the headline workload so that one invocation witnesses all five
 OTHER_CONFIGS = ("decode_f16_2k_1layer", "decode_fp8_8k_32layers", "decode_f16_hd256_sliding_12layers",
@@ -640,6 +685,8 @@ def run_workload(args, name):
         return bench_rope_append(args, workloads.ROPE_APPEND[name])
     if name == "copy_calibration":
         return copy_calibration(args)
+    if name == "slab_reuse_calibration":
+        return slab_reuse_calibration(args)
     return None
 
 
@@ -668,7 +715,7 @@ def main():
     from vulkanforge_amd import workloads
     res = run_workload(args, args.workload)
     if res is None:
-        print("unknown workload; choose from: " + ", ".join(list(workloads.DECODE) + list(workloads.PREFILL) + list(workloads.ROPE_APPEND) + ["copy_calibration"]),
+        print("unknown workload; choose from: " + ", ".join(list(workloads.DECODE) + list(workloads.PREFILL) + list(workloads.ROPE_APPEND) + ["copy_calibration", "slab_reuse_calibration"]),
               file=sys.stderr)
         sys.exit(2)
     if args.workload == HEADLINE and not args.no_other_workloads:

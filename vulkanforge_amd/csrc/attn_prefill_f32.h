@@ -44,7 +44,7 @@ __global__ __launch_bounds__(256) void batch_mfma_f32_kernel(BatchArgs a) {
     const uint32_t g = (blockIdx.z / NH) * 4u + (uint32_t)w;    // head inside the GQA group
     if (g >= G) return;                                         // wavefronts never meet at a barrier
     const uint32_t kvh = blockIdx.y, h = kvh * G + g;
-    const uint32_t q0 = blockIdx.x * 16u, qi = q0 + n16;        // this lane's query (column of S^T)
+    const uint32_t q0 = (gridDim.x - 1u - blockIdx.x) * 16u, qi = q0 + n16;   // this lane's query (column of S^T); later blocks see more keys: longest first
     const bool q_ok = qi < a.m;
     const uint32_t row_stride = a.n_kv_heads * D * ES;          // bytes between two keys
 

@@ -65,7 +65,7 @@ __global__ __launch_bounds__((NCB == 1 && D <= 128) ? kPrefillOneHeadWaves * 64 
     const int n16 = lane & 15, kg = lane >> 4;
     const int G = a.n_heads / a.n_kv_heads;
     const uint32_t kvh = blockIdx.x;
-    const uint32_t q0 = blockIdx.y * 16;
+    const uint32_t q0 = (gridDim.y - 1u - blockIdx.y) * 16;   // later query blocks see more keys: longest workgroups first
     const uint32_t qi = q0 + n16;                               // this lane's query (column of S^T)
     const bool q_ok = qi < a.m;
     const uint32_t row_stride = a.n_kv_heads * D * ES;

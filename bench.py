@@ -669,6 +669,53 @@ def slab_reuse_calibration(args):
     return out
 
 
+def issue_rate_calibration(args):
+    """What the vector instructions of the prefill loop cost a SIMD to issue, and how far matrix and vector instructions
+    overlap (compute-only kernels of libvfkv_calib.so, no memory traffic).  Per entry: ticks of the shader clock per
+    wavefront instruction as wavefront 0 saw them, and per instruction of the SIMD (kernel time x clock / instructions issued
+    on one SIMD) -- the two differ when the wavefronts of a SIMD run side by side."""
+    import ctypes as C
+    import torch
+    calib = C.CDLL(os.path.join(ROOT, "vulkanforge_amd", "libvfkv_calib.so"))
+    calib.vfkv_calib_issue.argtypes = [C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p]
+    calib.vfkv_calib_overlap.argtypes = [C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p]
+    sink = torch.zeros(1024, dtype=torch.int32, device="cuda")
+    clk = torch.zeros(2, dtype=torch.int64, device="cuda")
+
+    def timed(launch):
+        st = torch.cuda.current_stream().cuda_stream
+        assert launch(st) == 0
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        assert launch(st) == 0
+        e1.record()
+        torch.cuda.synchronize()
+        ticks, wall = (int(x) for x in clk.cpu())
+        return e0.elapsed_time(e1), ticks, ticks / wall * 100.0       # ms, shader-clock ticks of wavefront 0, MHz
+
+    iters = 4000
+    out = {"metric": "issue_rate_calibration", "unit": "shader-clock ticks", "n_gpus": 1, "instructions": {}, "overlap": {}}
+    names = ["v_fma_f32", "v_exp_f32", "v_cvt_scalef32_pk_f16_fp8", "v_max_f32", "v_fma_mixlo_f16", "v_xor_b32"]
+    for op, name in enumerate(names):
+        entry = {}
+        for waves in (1, 2):
+            ms, ticks, mhz = timed(lambda st: calib.vfkv_calib_issue(op, waves, iters, sink.data_ptr(), clk.data_ptr(), st))
+            entry[f"{waves}_per_simd"] = {"wavefront_0_ticks_per_instruction": ticks / (iters * 64),
+                                          "simd_ticks_per_instruction": ms * 1e-3 * mhz * 1e6 / (iters * 64 * waves),
+                                          "kernel_ms": ms, "clock_mhz": mhz}
+        out["instructions"][name] = entry
+    it2 = 20000
+    for label, nv, mode in (("48_mfma_only", 0, 0), ("48_mfma_then_100_fma", 100, 0), ("48_mfma_then_200_fma", 200, 0),
+                            ("48_mfma_then_400_fma", 400, 0), ("48_mfma_200_fma_opposite_phases_by_barrier", 200, 1),
+                            ("48_mfma_200_fma_one_block", 200, 2)):
+        ms, ticks, mhz = timed(lambda st: calib.vfkv_calib_overlap(nv, mode, it2, sink.data_ptr(), clk.data_ptr(), st))
+        out["overlap"][label] = {"simd_ticks_per_pass_of_both_wavefronts": ms * 1e-3 * mhz * 1e6 / it2, "kernel_ms": ms,
+                                 "clock_mhz": mhz}
+    out["value"] = out["overlap"]["48_mfma_only"]["simd_ticks_per_pass_of_both_wavefronts"] / 96.0
+    return out
+
+
 HEADLINE = "decode_fp8_32k_32layers"
 # the other benchmark configurations, run briefly after the headline workload so that one invocation witnesses all five
 OTHER_CONFIGS = ("decode_f16_2k_1layer", "decode_fp8_8k_32layers", "decode_f16_hd256_sliding_12layers",
@@ -687,6 +734,8 @@ def run_workload(args, name):
         return copy_calibration(args)
     if name == "slab_reuse_calibration":
         return slab_reuse_calibration(args)
+    if name == "issue_rate_calibration":
+        return issue_rate_calibration(args)
     return None
 
 
@@ -715,7 +764,7 @@ def main():
     from vulkanforge_amd import workloads
     res = run_workload(args, args.workload)
     if res is None:
-        print("unknown workload; choose from: " + ", ".join(list(workloads.DECODE) + list(workloads.PREFILL) + list(workloads.ROPE_APPEND) + ["copy_calibration", "slab_reuse_calibration"]),
+        print("unknown workload; choose from: " + ", ".join(list(workloads.DECODE) + list(workloads.PREFILL) + list(workloads.ROPE_APPEND) + ["copy_calibration", "slab_reuse_calibration", "issue_rate_calibration"]),
               file=sys.stderr)
         sys.exit(2)
     if args.workload == HEADLINE and not args.no_other_workloads:

@@ -43,7 +43,7 @@ PROFILED_TRAFFIC = {
         "sources": ("attn_decode.hip", "attn_decode_mfma.h", "device_utils.h"), "sha256_16": "0145bfacb7bdfd49"},
     "prefill_fp8_512x4608_32layers": {
         "bytes": (18572 + 9728) * 1024, "profile": "profiles/prefill_fp8_512x4608_batch_dma_kernel.md",
-        "sources": ("attn_prefill.hip", "attn_prefill_dma.h", "device_utils.h"), "sha256_16": "d6d75637b01e53ca"},
+        "sources": ("attn_prefill.hip", "attn_prefill_dma.h", "device_utils.h"), "sha256_16": "7be340169e27988f"},
 }
 
 
@@ -457,6 +457,8 @@ def bench_prefill(args, wl):
         variants = [("f16_weights", dict(f16_weights=True))]
         if wl.dtype.label() == "FP8":
             variants += [("fp8_scores", dict(fp8_scores=True)), ("f16_weights+fp8_scores", dict(f16_weights=True, fp8_scores=True))]
+        if args.f32_queries:     # general f32 queries: what rounding them to f16 inside the call saves (the remainder pass)
+            variants += [("f16_queries", dict(f16_queries=True))]
         for name, opts in variants:
             ms = time_steps(torch, step_with(**opts), args) * 1e3
             f16w[name] = {"ms_per_step": ms, "TFLOPs": wl.flops_layer() * L / (ms * 1e-3) / 1e12}

@@ -141,6 +141,35 @@ def test_batch_with_f32_queries_keeps_f32_accuracy(dtype):
     assert np.abs(o - ref).max() < 1e-3
 
 
+@pytest.mark.parametrize("dtype,heads,hkv,d", [(vf.KvDtype.F8, 32, 8, 128), (vf.KvDtype.F16, 32, 8, 128), (vf.KvDtype.F8, 16, 8, 256),
+                                                (vf.KvDtype.F16, 8, 2, 512), (vf.KvDtype.F8, 8, 4, 64)])
+def test_f16_queries_option_is_the_call_on_queries_rounded_to_f16(dtype, heads, hkv, d):
+    """VFKV_PREFILL_F16_QUERIES: general f32 queries take the path of f16-representable ones.  Bit-identical to rounding the
+    queries first; against the oracle on the unrounded queries a score is off by at most 2^-12 of the sum of its |k q|
+    products times scale, inside the path's tolerance on these inputs."""
+    m, q_start = 40, 700
+    r = rng(77)
+    n_kv = q_start + m
+    q = (r.standard_normal((m, heads, d)) * 2).astype(np.float32)
+    k = encode_np(fp16_normal(r, (n_kv, hkv, d)), dtype)
+    v = encode_np(fp16_normal(r, (n_kv, hkv, d)), dtype)
+    scale = float(1.0 / np.sqrt(d))
+
+    def run(qq, **kw):
+        o = torch.full((m, heads, d), float("nan"), device=DEV)
+        vf.Forward.run_flash_attn_batch(to_dev(qq), to_dev(k.reshape(n_kv, -1)), to_dev(v.reshape(n_kv, -1)), dtype, o, heads, hkv, d,
+                                        m, q_start, n_kv, scale, **kw)
+        torch.cuda.synchronize()
+        return to_np(o)
+
+    o_opt = run(q, f16_queries=True)
+    o_cast = run(q.astype(np.float16).astype(np.float32))
+    assert np.array_equal(o_opt, o_cast)
+    ref = oracle.attn_batch_ref(q, k, v, int(dtype), m, n_kv, heads, hkv, d, q_start, scale)
+    assert np.abs(o_opt - ref).max() < 2e-3             # 1.0e-3 measured on the first case (queries of standard deviation 2)
+    assert np.abs(run(q) - ref).max() < 2e-5            # the default keeps the remainder
+
+
 def test_config5_chunk_append_then_prefill_fp8_one_layer():
     # benchmark configuration 5, one of its 32 layers: FP8 cache filled to 4096, append 512 tokens, then
     # 512 causal queries over 4608 keys (32/8/128).  The oracle is run on a sample of query rows.

@@ -46,7 +46,7 @@ class Gate(C.Structure):
     _fields_ = [("gate", C.c_void_p), ("chunk", C.c_uint32), ("stride", C.c_uint32), ("gate_offset", C.c_uint32)]
 
 
-PREFILL_F16_WEIGHTS, PREFILL_FP8_SCORES = 1, 2   # VFKV_PREFILL_F16_WEIGHTS, VFKV_PREFILL_FP8_SCORES
+PREFILL_F16_WEIGHTS, PREFILL_FP8_SCORES, PREFILL_F16_QUERIES = 1, 2, 4   # the VFKV_PREFILL_* option bits
 ROPE_NORM, ROPE_NEOX = 0, 2   # GGML_ROPE_TYPE_NORMAL / _NEOX (rms_norm.comp:25-26)
 
 assert C.sizeof(SplitParams) == 32 and C.sizeof(BatchParams) == 32  # pipeline.rs:569,611

@@ -707,7 +707,7 @@ int vfkv_kv_write_decode_attention(vfkv_cache* c, uint32_t layer, uint32_t n_hea
 static int flash_attn_batch_impl(const float* q, const void* k_layer, const void* v_layer, uint32_t kv_dtype, float* o,
                                  const vfkv_batch_params* p, float softcap, vfkv_workspace* ws, vfkv_stream stream,
                                  const vfkv::GateArgs* gate = nullptr, uint32_t options = 0u) {
-    if ((options & ~(VFKV_PREFILL_F16_WEIGHTS | VFKV_PREFILL_FP8_SCORES)) != 0u) return fail(VFKV_ERR_INVALID_ARG, "flash_attn_batch: unknown option bits 0x%x", options);
+    if ((options & ~(VFKV_PREFILL_F16_WEIGHTS | VFKV_PREFILL_FP8_SCORES | VFKV_PREFILL_F16_QUERIES)) != 0u) return fail(VFKV_ERR_INVALID_ARG, "flash_attn_batch: unknown option bits 0x%x", options);
     if (!p) return fail(VFKV_ERR_INVALID_ARG, "flash_attn_batch: params is NULL");
     if (!q || !k_layer || !v_layer || !o) return fail(VFKV_ERR_INVALID_ARG, "flash_attn_batch: NULL buffer");
     if (kv_dtype > VFKV_F8E4M3) return fail(VFKV_ERR_INVALID_ARG, "flash_attn_batch: unknown kv dtype %u", kv_dtype);
@@ -732,6 +732,7 @@ static int flash_attn_batch_impl(const float* q, const void* k_layer, const void
     L.scale = p->scale; L.softcap = softcap;
     L.f16_weights = (options & VFKV_PREFILL_F16_WEIGHTS) != 0u;
     L.fp8_scores = (options & VFKV_PREFILL_FP8_SCORES) != 0u;
+    L.f16_queries = (options & VFKV_PREFILL_F16_QUERIES) != 0u;
     if (ws) {
         L.scratch_out = ws->scratch_out; L.scratch_max = ws->scratch_max; L.scratch_sum = ws->scratch_sum;
         L.scratch_ml_floats = (uint64_t)ws->n_heads * ws->max_tiles;

@@ -30,6 +30,7 @@ struct BatchArgs {
     // multiples of 4, a 16-byte aligned gate and fewer than 2^32 output elements.
     const float* gate;
     uint32_t gchunk, gstride, goff;
+    uint32_t q_f16;          // f16 matrix-core kernels: use f16(q) alone, whatever the queries hold
 };
 
 }  // namespace vfkv
@@ -109,6 +110,7 @@ static hipError_t launch_batch_kernels(const BatchLaunch& L, hipStream_t stream,
     a.scale = L.scale; a.softcap = L.softcap; a.dtype = L.dtype;
     a.so = nullptr; a.sm = nullptr; a.ss = nullptr; a.nk = 1u; a.chunk = 0u;
     a.gate = nullptr; a.gchunk = 1u; a.gstride = 0u; a.goff = 0u;
+    a.q_f16 = L.f16_queries ? 1u : 0u;
     const uint32_t g = L.n_heads / L.n_kv_heads;
     const uint64_t slab_bytes = (uint64_t)L.n_kv * L.n_kv_heads * L.head_dim * elem_size(L.dtype);
     const bool aligned = ((((uintptr_t)L.k) | ((uintptr_t)L.v) | ((uintptr_t)L.q) | ((uintptr_t)L.o)) & 15u) == 0u;

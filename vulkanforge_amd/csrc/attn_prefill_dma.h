@@ -206,7 +206,7 @@ __global__ __launch_bounds__(512) void batch_dma_kernel(BatchArgs a, int HP, int
         }
     }
     __syncthreads();                                            // lds_haslo cleared, planes written
-    if (any_lo) lds_haslo = 1;
+    if (any_lo && a.q_f16 == 0u) lds_haslo = 1;
     __syncthreads();
     has_lo = __builtin_amdgcn_readfirstlane(lds_haslo) != 0;   // workgroup-uniform
     }

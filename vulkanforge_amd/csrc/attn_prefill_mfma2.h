@@ -162,7 +162,7 @@ __global__ __launch_bounds__((NCB == 1 && D <= 128) ? kPrefillOneHeadWaves * 64 
         }
     }
     __syncthreads();                                            // lds_haslo cleared, planes written
-    if (any_lo) lds_haslo = 1;
+    if (any_lo && a.q_f16 == 0u) lds_haslo = 1;
     __syncthreads();
     has_lo = __builtin_amdgcn_readfirstlane(lds_haslo) != 0;   // workgroup-uniform
 

@@ -106,6 +106,9 @@ struct BatchLaunch {
     // FP8 caches at head_dim 128, GQA groups of 2-4 heads: the first product K Q^T runs on the FP8 matrix instruction, K rows as
     // stored and Q as three E4M3 terms (12 significant bits); no widening of K.  Other shapes ignore it.
     bool fp8_scores = false;
+    // f16 matrix-core kernels: the queries enter the first product as f16(q) only (no remainder pass for queries that f16
+    // cannot represent): scores off by up to 2^-12 of the sum of their |k q| products
+    bool f16_queries = false;
 };
 hipError_t launch_batch(const BatchLaunch& a, hipStream_t stream);
 

@@ -194,12 +194,15 @@ class Forward:
     # ---- prefill attention (runs.rs:933-1010, executor/attention.rs:2192-2390) ----
     @staticmethod
     def run_flash_attn_batch(q, k_layer, v_layer, kv_dtype, o, n_heads, n_kv_heads, head_dim, m, q_start, n_kv,
-                             scale, kv_start=0, softcap=0.0, stream=None, f16_weights=False, fp8_scores=False) -> None:
+                             scale, kv_start=0, softcap=0.0, stream=None, f16_weights=False, fp8_scores=False,
+                             f16_queries=False) -> None:
         """``f16_weights=True``: vfkv_flash_attn_batch_opt with VFKV_PREFILL_F16_WEIGHTS (softmax weights rounded to f16
         in the second product: faster, output off by up to 2^-11 * max|v|)."""
         p = _ffi.BatchParams(n_heads, n_kv_heads, head_dim, m, n_kv, q_start, scale, kv_start)
-        if f16_weights or fp8_scores:   # fp8_scores: VFKV_PREFILL_FP8_SCORES (first product on the FP8 matrix instruction)
-            opts = (_ffi.PREFILL_F16_WEIGHTS if f16_weights else 0) | (_ffi.PREFILL_FP8_SCORES if fp8_scores else 0)
+        if f16_weights or fp8_scores or f16_queries:   # fp8_scores: VFKV_PREFILL_FP8_SCORES (first product on the FP8 matrix
+            # instruction); f16_queries: VFKV_PREFILL_F16_QUERIES (queries rounded to f16: no remainder pass of the first product)
+            opts = ((_ffi.PREFILL_F16_WEIGHTS if f16_weights else 0) | (_ffi.PREFILL_FP8_SCORES if fp8_scores else 0) |
+                    (_ffi.PREFILL_F16_QUERIES if f16_queries else 0))
             _ffi.check(_ffi.lib().vfkv_flash_attn_batch_opt(_ptr(q), _ptr(k_layer), _ptr(v_layer), int(kv_dtype), _ptr(o),
                                                             C.byref(p), softcap, opts, _stream(stream)))
             return
@@ -209,15 +212,16 @@ class Forward:
     def b_step_attention(self, layer: int, base_pos: int, seq_len: int, q, o, kv_layer: int | None = None,
                          kv_start_window: int = 0, scale: float | None = None, softcap: float = 0.0,
                          stream=None, use_workspace: bool = False, f16_weights: bool = False,
-                         fp8_scores: bool = False) -> None:
+                         fp8_scores: bool = False, f16_queries: bool = False) -> None:
         """``use_workspace=True``: vfkv_prefill_attention_ws (key chunks over workgroups for short chunks over long
         histories, merged through the decode workspace).  ``f16_weights=True``: vfkv_prefill_attention_opt with
         VFKV_PREFILL_F16_WEIGHTS."""
         if scale is None:
             hd = self.kv_cache.head_dim_for(layer)
             scale = self.attn_scale if hd == self.kv_cache.config.head_dim else 1.0 / math.sqrt(hd)
-        if f16_weights or fp8_scores:
-            opts = (_ffi.PREFILL_F16_WEIGHTS if f16_weights else 0) | (_ffi.PREFILL_FP8_SCORES if fp8_scores else 0)
+        if f16_weights or fp8_scores or f16_queries:
+            opts = ((_ffi.PREFILL_F16_WEIGHTS if f16_weights else 0) | (_ffi.PREFILL_FP8_SCORES if fp8_scores else 0) |
+                    (_ffi.PREFILL_F16_QUERIES if f16_queries else 0))
             _ffi.check(_ffi.lib().vfkv_prefill_attention_opt(self.kv_cache.handle, layer,
                                                              layer if kv_layer is None else kv_layer, self.n_heads,
                                                              _ptr(q), _ptr(o), seq_len, base_pos, kv_start_window, scale,

@@ -107,7 +107,7 @@ extern "C" {
                                      ws: *mut VfkvWorkspace, stream: *mut c_void) -> c_int;
     pub fn vfkv_flash_attn_batch_opt(q: *const f32, k_layer: *const c_void, v_layer: *const c_void, kv_dtype: u32,
                                      o: *mut f32, p: *const VfkvBatchParams, softcap: f32, options: u32,
-                                     stream: *mut c_void) -> c_int;            // options: VFKV_PREFILL_F16_WEIGHTS = 1
+                                     stream: *mut c_void) -> c_int;            // options: VFKV_PREFILL_F16_WEIGHTS = 1, _FP8_SCORES = 2, _F16_QUERIES = 4
     pub fn vfkv_prefill_attention_opt(c: *mut VfkvCache, layer: u32, kv_layer: u32, n_heads: u32, q: *const f32,
                                       o: *mut f32, m: u32, base_pos: u32, window: u32, scale: f32, softcap: f32,
                                       options: u32, ws: *mut VfkvWorkspace, stream: *mut c_void) -> c_int;

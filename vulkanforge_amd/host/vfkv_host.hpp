@@ -211,8 +211,8 @@ public:
         check(vfkv_prefill_attention(kv_cache.handle(), layer, kv_layer, n_heads, q, o, seq_len, base_pos, kv_start_window,
                                      scale_for(layer), softcap, stream));
     }
-    // the same with the call's precision options (VFKV_PREFILL_F16_WEIGHTS | VFKV_PREFILL_FP8_SCORES): faster, weights to 11
-    // bits / scores through the FP8 matrix instruction; see include/vfkv.h for the bounds
+    // the same with the call's precision options (VFKV_PREFILL_F16_WEIGHTS | VFKV_PREFILL_FP8_SCORES | VFKV_PREFILL_F16_QUERIES):
+    // faster, weights to 11 bits / scores through the FP8 matrix instruction / queries to 11 bits; bounds in include/vfkv.h
     void b_step_attention_opt(uint32_t layer, uint32_t base_pos, uint32_t seq_len, const float* q, float* o, uint32_t kv_layer,
                               uint32_t kv_start_window, uint32_t options, float softcap = 0.f) {
         check(vfkv_prefill_attention_opt(kv_cache.handle(), layer, kv_layer, n_heads, q, o, seq_len, base_pos, kv_start_window,

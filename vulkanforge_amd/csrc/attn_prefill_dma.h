@@ -73,7 +73,6 @@ __global__ __launch_bounds__(512) void batch_dma_kernel(BatchArgs a, int HP, int
     const float cap_l2 = a.softcap * 1.44269504088896f;
 
     const __amdgpu_buffer_rsrc_t krsrc = __builtin_amdgcn_make_buffer_rsrc((void*)a.k, 0, a.n_kv * row_stride, 0x00020000);
-    const __amdgpu_buffer_rsrc_t vrsrc = __builtin_amdgcn_make_buffer_rsrc((void*)a.v, 0, a.n_kv * row_stride, 0x00020000);
     const uint32_t head_b = kvh * D;
     const uint32_t lane_koff = n16 * row_stride + head_b + kg * SEG;
 

@@ -167,7 +167,8 @@ static hipError_t launch_batch_kernels(const BatchLaunch& L, hipStream_t stream,
         const uint32_t nz = (hp_group + hp - 1u) / hp;
         const uint32_t max_waves = waves_for(hp);
         if (max_waves >= hp && nz <= 65535u && (L.m + 15u) / 16u <= 65535u) {
-            const uint32_t ns = max_waves / hp;               // key splits: fill the workgroup
+            uint32_t ns = max_waves / hp;                     // key splits: fill the workgroup
+            if (vdma) while (ns & (ns - 1u)) --ns;            // (that kernel's merge deals the 8 output tiles of a head to the splits)
             const uint32_t nwaves = hp * ns;
             // Short chunks over long histories (the suffix of a request that reuses its prefix) still leave most compute
             // units idle: with a workspace the keys are also cut into chunks over workgroups, every workgroup stores a
@@ -203,7 +204,10 @@ static hipError_t launch_batch_kernels(const BatchLaunch& L, hipStream_t stream,
             const size_t vbytes = (size_t)nwaves * (vdma ? (size_t)3 * 32 * 128 : (size_t)32 * (dv + 16) * sizeof(_Float16)) +
                                   (size_t)2 * (hp / nh) * ncb * 16 * (L.head_dim + 8) * sizeof(_Float16) +
                                   (nh == 2u ? (size_t)2 * nwaves * ncb * 64 * 16 : 0u);
-            const size_t mbytes = (size_t)(ns - 1) * hp * ncb * 64 * (dv / 4 + 2) * sizeof(float);
+            // merge area: the general kernel keeps the records of all splits but the first; the V-through-LDS kernel the
+            // output tiles and (m, l) of every wavefront
+            const size_t mbytes = vdma ? (size_t)nwaves * ncb * 64 * (dv / 4 + 2) * sizeof(float)
+                                       : (size_t)(ns - 1) * hp * ncb * 64 * (dv / 4 + 2) * sizeof(float);
             const size_t lds = vbytes > mbytes ? vbytes : mbytes;
             const bool cap = L.softcap > 0.f;
             bool launched = true;
@@ -217,9 +221,13 @@ static hipError_t launch_batch_kernels(const BatchLaunch& L, hipStream_t stream,
             // FP8 matrix instruction (needs the Q block staged in one round: four key splits).  Over F16 rows (four heads per
             // wavefront) f16_weights is an instantiation of the general kernel; other shapes keep the default arithmetic.
             const bool f8s = L.fp8_scores && vdma && ns >= 4u;
+            // eight wavefronts (two per SIMD) and an even number of key splits: the older wavefront of a SIMD gets 3 tiles
+            // for every 2 of the younger one
+            int deal_a = 1, deal_b = 1;
+            if (nwaves == 8u && ns % 2u == 0u) { deal_a = 3; deal_b = 2; }
 #define VFKV_PDMA(F16WV, F8SV)                                                                                         \
-    { if (cap) hipLaunchKernelGGL((batch_dma_kernel<true, F16WV, F8SV>), grid, block, lds, stream, a, (int)hp, (int)ns);  \
-      else hipLaunchKernelGGL((batch_dma_kernel<false, F16WV, F8SV>), grid, block, lds, stream, a, (int)hp, (int)ns); }
+    { if (cap) hipLaunchKernelGGL((batch_dma_kernel<true, F16WV, F8SV>), grid, block, lds, stream, a, (int)hp, (int)ns, deal_a, deal_b);  \
+      else hipLaunchKernelGGL((batch_dma_kernel<false, F16WV, F8SV>), grid, block, lds, stream, a, (int)hp, (int)ns, deal_a, deal_b); }
             if (vdma && f8s && L.f16_weights) VFKV_PDMA(true, true)
             else if (vdma && f8s) VFKV_PDMA(false, true)
             else if (vdma && L.f16_weights) VFKV_PDMA(true, false)

@@ -20,7 +20,7 @@
 namespace vfkv {
 
 template <bool CAP, bool F16W, bool F8S>
-__global__ __launch_bounds__(512) void batch_dma_kernel(BatchArgs a, int HP, int NS) {
+__global__ __launch_bounds__(512) void batch_dma_kernel(BatchArgs a, int HP, int NS, int DEAL_A, int DEAL_B) {
     constexpr int D = 128, NCB = 2, PFD = 2;     // head_dim, heads per wavefront, K tiles in flight
     constexpr int KT = 32;                       // keys per tile
     constexpr int KS = D / 32;                   // MFMA k-steps of the first product
@@ -116,8 +116,31 @@ __global__ __launch_bounds__(512) void batch_dma_kernel(BatchArgs a, int HP, int
 #pragma unroll
     for (int i = 0; i < 3 * VBUF / (64 * 16); ++i) *reinterpret_cast<u32x4*>(v8 + (i * 64 + lane) * 16) = u32x4{0u, 0u, 0u, 0u};
     __builtin_amdgcn_s_waitcnt(0xC07F);                         // lgkmcnt(0): the zeros are in place before a load can overwrite them
+    // Which tiles a wavefront takes.  The key splits deal the tiles round-robin, but not evenly: of two wavefronts on one
+    // SIMD the older one issues first whenever both are ready, so it advances about 1.5 times as fast, and an even deal
+    // leaves the younger one to finish alone at the single-wavefront rate.  Per period the splits of the older half of the
+    // workgroup take DEAL_A tiles each and the others DEAL_B (DEAL_A >= DEAL_B >= 1; equal: the even deal): DEAL_B rows of
+    // NS tiles, then DEAL_A - DEAL_B rows of NS / 2 tiles for the older half.  tp[] holds the positions of the wavefront's
+    // next four tiles (slot sl works on tp[sl]; its next one, already requested, is tp[sl + PFD]).
     const uint32_t step = KT * NS;
-    const uint32_t tb0 = t_first + sp * KT;                     // this wavefront's first tile (may already be past the end)
+    const bool older = sp * 2 < NS;
+    const uint32_t deal_n = older ? (uint32_t)DEAL_A : (uint32_t)DEAL_B;
+    const uint32_t deal_period = (uint32_t)DEAL_B * step + (uint32_t)(DEAL_A - DEAL_B) * (step / 2);
+    uint32_t deal_base = t_first + sp * KT, deal_r = 0;         // (a wavefront's first tile may already be past the end)
+    auto next_tile = [&]() -> uint32_t {
+        const uint32_t p = deal_base + (deal_r < (uint32_t)DEAL_B ? deal_r * step : (uint32_t)DEAL_B * step + (deal_r - (uint32_t)DEAL_B) * (step / 2));
+        if (++deal_r == deal_n) { deal_r = 0; deal_base += deal_period; }
+        return p;
+    };
+    uint32_t tp[2 * PFD];
+#pragma unroll
+    for (int i = 0; i < 2 * PFD; ++i) tp[i] = next_tile();
+    auto advance = [&]() {
+#pragma unroll
+        for (int i = 0; i < PFD; ++i) tp[i] = tp[i + PFD];
+#pragma unroll
+        for (int i = 0; i < PFD; ++i) tp[PFD + i] = next_tile();
+    };
     const uint32_t kloop = kmax;                                // where this wavefront's walk ends
     auto tile_off = [&](uint32_t t) -> uint32_t { return t < kmax ? t * row_stride : kNoTile; };
     // ---- Q block of the workgroup: 16 queries x G heads x D floats, loaded once with coalesced 16-byte loads (before the
@@ -146,7 +169,7 @@ __global__ __launch_bounds__(512) void batch_dma_kernel(BatchArgs a, int HP, int
             amax = fmaxf(fmaxf(amax, fmaxf(fabsf(qf[i].x), fabsf(qf[i].y))), fmaxf(fabsf(qf[i].z), fabsf(qf[i].w)));
         }
 #pragma unroll
-        for (int sl = 0; sl < PFD; ++sl) issue(sl, tile_off(tb0 + sl * step));
+        for (int sl = 0; sl < PFD; ++sl) issue(sl, tile_off(tp[sl]));
         __syncthreads();                                        // lds_qmax cleared
         amax = wave_max_uniform(amax);
         if (lane == 0) atomicMax(&lds_qmax, __builtin_bit_cast(uint32_t, amax));   // non-negative floats order like their bits
@@ -188,7 +211,7 @@ __global__ __launch_bounds__(512) void batch_dma_kernel(BatchArgs a, int HP, int
         }
         if (base == 0) {
 #pragma unroll
-            for (int sl = 0; sl < PFD; ++sl) issue(sl, tile_off(tb0 + sl * step));
+            for (int sl = 0; sl < PFD; ++sl) issue(sl, tile_off(tp[sl]));
         }
 #pragma unroll
         for (int i = 0; i < QLD; ++i) {
@@ -223,16 +246,16 @@ __global__ __launch_bounds__(512) void batch_dma_kernel(BatchArgs a, int HP, int
     float4_t s[PFD][NCB][2];
     float x[PFD][NCB][8], tmax[PFD][NCB];
     // the request for the V tile after next: it goes where the tile before the current one was
-    auto stage_v = [&](uint32_t tcur) {
+    auto stage_v = [&](int sl) {
         const int nb = vcur + 2 >= 3 ? vcur - 1 : vcur + 2;
-        v_dma(nb, tile_off(tcur + PFD * step));
+        v_dma(nb, tile_off(tp[sl + PFD]));
     };
     // S^T = K Q^T for the NCB heads (Q operands re-read from LDS every tile); lo_tag: whether the remainder plane of Q takes
     // part (a bool, or a type where the walk is compiled once per case)
     auto first_product = [&](int sl, uint32_t tcur, auto lo_tag) {
         bool with_lo;
         if constexpr (std::is_same_v<decltype(lo_tag), bool>) with_lo = lo_tag; else with_lo = decltype(lo_tag)::value;
-        const uint32_t noff = tile_off(tcur + PFD * step);
+        const uint32_t noff = tile_off(tp[sl + PFD]);
         if constexpr (F8S) {
             // S^T = K Q^T on the FP8 matrix instruction: A = the lane's quarter row of K as loaded (32 codes), B = the same
             // quarter of the query's three term planes, each with its power-of-two weight as the instruction's block scale
@@ -376,7 +399,7 @@ __global__ __launch_bounds__(512) void batch_dma_kernel(BatchArgs a, int HP, int
                 phi[cb][j2] = __builtin_bit_cast(uint32_t, __builtin_convertvector(pp, half2_t));
                 if (TWO) plo[cb][j2] = pack_f16_remainder(pp[0], pp[1], phi[cb][j2]);
             }
-        stage_v(tcur);
+        stage_v(sl);
         // supplier lane s of a 16-lane group points at the 8 bytes V[key][dt*16 + 8*(s%2) ..], key = 4*kg + s/2 for s < 8
         // and 16 + 4*kg + (s/2 - 4) above; the read hands lane n the bytes of the eight keys at d = dt*16 + n
         const uint32_t vrd = vdma_rd + (uint32_t)(vcur * VBUF);
@@ -408,15 +431,14 @@ __global__ __launch_bounds__(512) void batch_dma_kernel(BatchArgs a, int HP, int
     // are straight-line code and the inner loop is the grouped one.
     auto walk = [&](auto lo_tag) {
     constexpr bool GROUP = std::is_same_v<decltype(lo_tag), std::false_type>;   // (the remainder product's registers leave no room for a second tile's scores)
-    uint32_t tb = tb0;
     int first_slot = 0;          // slots of the group at tb that the inner loop has already finished
     bool s_ready = false;        // the inner loop left the group at tb with scores computed: those of slot first_slot; GROUP:
                                  // those of every slot
     constexpr auto two_tag = std::integral_constant<bool, !F16W>{};
-    while (tb < kloop) {
+    while (tp[0] < kloop) {
 #pragma unroll
         for (int sl = 0; sl < PFD; ++sl) {
-            const uint32_t tcur = tb + sl * step;
+            const uint32_t tcur = tp[sl];
             if (tcur >= kloop) break;                           // wavefront-uniform
             if (sl < first_slot) continue;
             if (!(s_ready && (GROUP || sl == first_slot))) first_product(sl, tcur, lo_tag);
@@ -428,29 +450,29 @@ __global__ __launch_bounds__(512) void batch_dma_kernel(BatchArgs a, int HP, int
                 weights_and_second_product(std::true_type{}, two_tag, sl, tcur);
             }
         }
-        tb += PFD * step;
+        advance();
         first_slot = 0;
         s_ready = false;
         if constexpr (GROUP) {
             // a whole group per pass: the first products of its tiles do not depend on the softmax and the second product of
             // the tiles before them, so the matrix pipe and the vector ALU have work from different tiles side by side
-            while (tb >= a.kv_start && tb + (PFD - 1) * step + KT <= fast_end) {
+            while (tp[0] >= a.kv_start && tp[PFD - 1] + KT <= fast_end) {
                 bool moved = false;
 #pragma unroll
-                for (int sl = 0; sl < PFD; ++sl) first_product(sl, tb + sl * step, lo_tag);
+                for (int sl = 0; sl < PFD; ++sl) first_product(sl, tp[sl], lo_tag);
 #pragma unroll
-                for (int sl = 0; sl < PFD; ++sl) moved |= scores(std::false_type{}, sl, tb + sl * step);
+                for (int sl = 0; sl < PFD; ++sl) moved |= scores(std::false_type{}, sl, tp[sl]);
                 if (__builtin_amdgcn_ballot_w64(moved) != 0ull) { s_ready = true; break; }
 #pragma unroll
-                for (int sl = 0; sl < PFD; ++sl) weights_and_second_product(std::false_type{}, two_tag, sl, tb + sl * step);
-                tb += PFD * step;
+                for (int sl = 0; sl < PFD; ++sl) weights_and_second_product(std::false_type{}, two_tag, sl, tp[sl]);
+                advance();
             }
         } else {
             bool left = false;
-            while (!left && tb >= a.kv_start && tb + (PFD - 1) * step + KT <= fast_end) {
+            while (!left && tp[0] >= a.kv_start && tp[PFD - 1] + KT <= fast_end) {
 #pragma unroll
                 for (int sl = 0; sl < PFD; ++sl) {
-                    const uint32_t tcur = tb + sl * step;
+                    const uint32_t tcur = tp[sl];
                     first_product(sl, tcur, lo_tag);
                     if (__builtin_amdgcn_ballot_w64(scores(std::false_type{}, sl, tcur)) != 0ull) {
                         first_slot = sl; s_ready = true; left = true;
@@ -458,7 +480,7 @@ __global__ __launch_bounds__(512) void batch_dma_kernel(BatchArgs a, int HP, int
                     }
                     weights_and_second_product(std::false_type{}, two_tag, sl, tcur);
                 }
-                if (!left) tb += PFD * step;
+                if (!left) advance();
             }
         }
     }
@@ -467,11 +489,82 @@ __global__ __launch_bounds__(512) void batch_dma_kernel(BatchArgs a, int HP, int
 #pragma unroll
     for (int cb = 0; cb < NCB; ++cb) l_run[cb] = xor32_sum(xor16_sum(l_run[cb]));   // every lane of a query column has its wavefront's sum
 
-    // ---- gated output (vk_shaders/sigmoid_mul.comp:44-52 in this kernel's store): the wavefronts that will store request
-    // their gate values and turn them into factors before the merge, so that the round trip overlaps it.  A head's D
-    // elements lie in one gate chunk.
+    // ---- merge the key splits through LDS, normalise and store: every wavefront leaves its (o, m, l) in LDS, then the NS
+    // wavefronts of a head pair each merge and store the d-tiles dt = sp, sp + NS, ... of the pair's NCB heads (gated
+    // output, vk_shaders/sigmoid_mul.comp:44-52, applied in that store: a head's D elements lie in one gate chunk).
+    // Layout: o as [wavefront slot][cb][dt][lane] float4 (16-byte accesses, consecutive lanes: no bank conflicts), then
+    // m and l as [wavefront slot][cb][2][lane].
+    if (NS > 1) {
+        __syncthreads();                                        // every wavefront is done with its V area
+        float4_t* obuf = reinterpret_cast<float4_t*>(lds);
+        float* mlbuf = reinterpret_cast<float*>(lds) + (size_t)nwaves * NCB * DTILES * 64 * 4;
+        const int slot = sp * HP + hp;
+#pragma unroll
+        for (int cb = 0; cb < NCB; ++cb) {
+#pragma unroll
+            for (int dt = 0; dt < DTILES; ++dt) obuf[((size_t)(slot * NCB + cb) * DTILES + dt) * 64 + lane] = oacc[cb][dt];
+            mlbuf[((size_t)(slot * NCB + cb) * 2 + 0) * 64 + lane] = m_run[cb];
+            mlbuf[((size_t)(slot * NCB + cb) * 2 + 1) * 64 + lane] = l_run[cb];
+        }
+        __syncthreads();
+        if (!q_ok) return;
+        // (compiled per split count so that the LDS reads of a head are independent instructions, not a chain of round trips)
+        auto merge_and_store = [&](auto ns_tag) {
+            constexpr int NSC = decltype(ns_tag)::value;
+#pragma unroll
+            for (int cb = 0; cb < NCB; ++cb) {
+                if (gz + g0 + cb >= G) continue;                // padding slot of an odd group
+                float f[NSC], lv[NSC];
+#pragma unroll
+                for (int s2 = 0; s2 < NSC; ++s2) {
+                    const float* ml = mlbuf + ((size_t)((s2 * HP + hp) * NCB + cb) * 2) * 64 + lane;
+                    f[s2] = ml[0]; lv[s2] = ml[64];
+                }
+                float mm = f[0];
+#pragma unroll
+                for (int s2 = 1; s2 < NSC; ++s2) mm = fmaxf(mm, f[s2]);
+                float lsum = 0.f;
+#pragma unroll
+                for (int s2 = 0; s2 < NSC; ++s2) { f[s2] = __builtin_amdgcn_exp2f(f[s2] - mm); lsum += lv[s2] * f[s2]; }
+                const uint32_t h = kvh * G + gz + g0 + cb;
+                const size_t pidx = ((size_t)qi * a.n_heads + h) * a.nk + kc;      // (key chunks: the partial of this chunk)
+                const float inv = a.so != nullptr ? 1.0f : 1.0f / lsum;
+                float* op = a.so != nullptr ? a.so + pidx * D + kg * 4 : a.o + ((size_t)qi * a.n_heads + h) * D + kg * 4;
+                const float* gp = nullptr;
+                if (a.gate != nullptr) {
+                    const uint32_t i0 = (qi * a.n_heads + h) * D;
+                    const uint32_t token = i0 / a.gchunk;
+                    gp = a.gate + (size_t)token * a.gstride + a.goff + (i0 - token * a.gchunk) + kg * 4;
+                }
+#pragma unroll
+                for (int j = 0; j < DTILES / NSC; ++j) {        // lane (query n16) holds d = dt*16 + kg*4 + i
+                    const int dt = sp + j * NSC;
+                    float4_t r = float4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                    for (int s2 = 0; s2 < NSC; ++s2)
+                        r += obuf[((size_t)((s2 * HP + hp) * NCB + cb) * DTILES + dt) * 64 + lane] * f[s2];
+                    r *= inv;
+                    if (gp != nullptr) {
+                        const float4 gv = *reinterpret_cast<const float4*>(gp + dt * 16);
+                        r *= float4_t{sigmoid_gate(1.0f, gv.x), sigmoid_gate(1.0f, gv.y), sigmoid_gate(1.0f, gv.z), sigmoid_gate(1.0f, gv.w)};
+                    }
+                    *reinterpret_cast<float4*>(op + dt * 16) = make_float4(r[0], r[1], r[2], r[3]);
+                }
+                if (a.so != nullptr && sp == 0 && kg == 0) {
+                    // key chunks: the unnormalised partial in the layout of the decode merge ([row][chunk][D], the maximum
+                    // in natural-log units); a query that sees no key of the chunk leaves (0, "minus infinity", 0)
+                    a.sm[pidx] = mm > -1e29f ? mm * 0.693147180559945f : kMasked;
+                    a.ss[pidx] = lsum;
+                }
+            }
+        };
+        if (NS == 4) merge_and_store(std::integral_constant<int, 4>{});
+        else if (NS == 2) merge_and_store(std::integral_constant<int, 2>{});
+        else merge_and_store(std::integral_constant<int, 8>{});  // (the launcher gives 2, 4 or 8 splits)
+        return;
+    }
     float4_t gfac[NCB][DTILES];
-    if (a.gate != nullptr && sp == 0 && q_ok) {
+    if (a.gate != nullptr && q_ok) {
 #pragma unroll
         for (int cb = 0; cb < NCB; ++cb) {
             if (gz + g0 + cb >= G) continue;
@@ -482,43 +575,6 @@ __global__ __launch_bounds__(512) void batch_dma_kernel(BatchArgs a, int HP, int
             for (int dt = 0; dt < DTILES; ++dt) {
                 const float4 gv = *reinterpret_cast<const float4*>(gp + dt * 16);
                 gfac[cb][dt] = float4_t{sigmoid_gate(1.0f, gv.x), sigmoid_gate(1.0f, gv.y), sigmoid_gate(1.0f, gv.z), sigmoid_gate(1.0f, gv.w)};
-            }
-        }
-    }
-
-    // ---- merge the key splits through LDS (split 0 collects), normalise and store ----
-    constexpr int REC = DTILES * 4 + 2;
-    if (NS > 1) {
-        __syncthreads();                                        // every wavefront is done with its V area
-        float* mbuf = reinterpret_cast<float*>(lds);            // [NS-1][HP][NCB][64][REC]
-        if (sp > 0) {
-#pragma unroll
-            for (int cb = 0; cb < NCB; ++cb) {
-                float* rec = mbuf + ((size_t)(((sp - 1) * HP + hp) * NCB + cb) * 64 + lane) * REC;
-#pragma unroll
-                for (int dt = 0; dt < DTILES; ++dt)
-#pragma unroll
-                    for (int i = 0; i < 4; ++i) rec[dt * 4 + i] = oacc[cb][dt][i];
-                rec[DTILES * 4] = m_run[cb];
-                rec[DTILES * 4 + 1] = l_run[cb];
-            }
-        }
-        __syncthreads();
-        if (sp > 0) return;
-#pragma unroll 1
-        for (int s2 = 1; s2 < NS; ++s2) {
-#pragma unroll
-            for (int cb = 0; cb < NCB; ++cb) {
-                const float* rec = mbuf + ((size_t)(((s2 - 1) * HP + hp) * NCB + cb) * 64 + lane) * REC;
-                const float m2 = rec[DTILES * 4], l2 = rec[DTILES * 4 + 1];
-                const float mm = fmaxf(m_run[cb], m2);
-                const float f1 = __builtin_amdgcn_exp2f(m_run[cb] - mm), f2 = __builtin_amdgcn_exp2f(m2 - mm);
-#pragma unroll
-                for (int dt = 0; dt < DTILES; ++dt)
-#pragma unroll
-                    for (int i = 0; i < 4; ++i) oacc[cb][dt][i] = oacc[cb][dt][i] * f1 + rec[dt * 4 + i] * f2;
-                l_run[cb] = l_run[cb] * f1 + l2 * f2;
-                m_run[cb] = mm;
             }
         }
     }

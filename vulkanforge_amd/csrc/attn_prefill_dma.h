@@ -38,11 +38,20 @@ __global__ __launch_bounds__(512) void batch_dma_kernel(BatchArgs a, int HP, int
     const int tid = threadIdx.x, lane = tid & 63;
     const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int nwaves = HP * NS;
-    const int hp = w % HP, sp = w / HP;
+    // Wavefront w: key split w / HP of head pair (w % HP) -- in a workgroup of eight the second four are turned by one
+    // head pair, so that the two wavefronts of a SIMD (w and w + 4) belong to different head pairs.
+    const int sp = w / HP;
+    const int hp = (nwaves == 8 && HP <= 4 && w >= 4 ? w + 1 : w) % HP;
     const int n16 = lane & 15, kg = lane >> 4;
     const int G = a.n_heads / a.n_kv_heads;
     const uint32_t kvh = blockIdx.x;
-    const uint32_t q0 = (gridDim.y - 1u - blockIdx.y) * 16;   // later query blocks see more keys: longest workgroups first
+    // Later query blocks see more keys.  The even head pairs of workgroup y take query block (last - y), the odd ones block
+    // y: every workgroup then has the same number of tiles, and with the turn above so has every SIMD (to within a tenth of
+    // the difference of the two blocks).  With an odd number of head pairs every wavefront takes block (last - y), the
+    // longest workgroups first.
+    const bool mirrored = HP % 2 == 0 && (hp & 1) != 0;
+    const uint32_t q0_even = (gridDim.y - 1u - blockIdx.y) * 16, q0_odd = HP % 2 == 0 ? blockIdx.y * 16 : q0_even;
+    const uint32_t q0 = mirrored ? q0_odd : q0_even;
     const uint32_t qi = q0 + n16;                               // this lane's query (column of S^T)
     const bool q_ok = qi < a.m;
     const uint32_t row_stride = a.n_kv_heads * D;
@@ -163,8 +172,9 @@ __global__ __launch_bounds__(512) void batch_dma_kernel(BatchArgs a, int HP, int
         for (int i = 0; i < QLD; ++i) {
             const int idx = tid + i * nthreads;
             const int qq = idx / (GP * (D / 4)), rem = idx - qq * (GP * (D / 4));
-            const bool ok = idx < q4_total && q0 + qq < a.m && rem < (G - gz) * (D / 4);
-            qf[i] = *reinterpret_cast<const float4*>(a.q + ((size_t)(ok ? q0 + qq : 0) * a.n_heads + kvh * G + gz) * D + (ok ? rem * 4 : 0));
+            const uint32_t qrow = (((rem / (D / 4)) / NCB) & 1 ? q0_odd : q0_even) + qq;     // the head slot's query block
+            const bool ok = idx < q4_total && qrow < a.m && rem < (G - gz) * (D / 4);
+            qf[i] = *reinterpret_cast<const float4*>(a.q + ((size_t)(ok ? qrow : 0) * a.n_heads + kvh * G + gz) * D + (ok ? rem * 4 : 0));
             if (!ok) qf[i] = make_float4(0.f, 0.f, 0.f, 0.f);
             amax = fmaxf(fmaxf(amax, fmaxf(fabsf(qf[i].x), fabsf(qf[i].y))), fmaxf(fabsf(qf[i].z), fabsf(qf[i].w)));
         }
@@ -205,8 +215,9 @@ __global__ __launch_bounds__(512) void batch_dma_kernel(BatchArgs a, int HP, int
         for (int i = 0; i < QLD; ++i) {
             const int idx = base + tid + i * nthreads;
             const int qq = idx / (GP * (D / 4)), rem = idx - qq * (GP * (D / 4));
-            const bool ok = idx < q4_total && q0 + qq < a.m && rem < (G - gz) * (D / 4);      // head slots past G read nothing
-            qf[i] = *reinterpret_cast<const float4*>(a.q + ((size_t)(ok ? q0 + qq : 0) * a.n_heads + kvh * G + gz) * D + (ok ? rem * 4 : 0));
+            const uint32_t qrow = (((rem / (D / 4)) / NCB) & 1 ? q0_odd : q0_even) + qq;     // the head slot's query block
+            const bool ok = idx < q4_total && qrow < a.m && rem < (G - gz) * (D / 4);      // head slots past G read nothing
+            qf[i] = *reinterpret_cast<const float4*>(a.q + ((size_t)(ok ? qrow : 0) * a.n_heads + kvh * G + gz) * D + (ok ? rem * 4 : 0));
             if (!ok) qf[i] = make_float4(0.f, 0.f, 0.f, 0.f);
         }
         if (base == 0) {

@@ -42,8 +42,8 @@ PROFILED_TRAFFIC = {
         "bytes": (65635 + 520) * 1024, "profile": "profiles/decode_floor_calibration.md",
         "sources": ("attn_decode.hip", "attn_decode_mfma.h", "device_utils.h"), "sha256_16": "0145bfacb7bdfd49"},
     "prefill_fp8_512x4608_32layers": {
-        "bytes": (18572 + 9728) * 1024, "profile": "profiles/prefill_fp8_512x4608_batch_dma_kernel.md",
-        "sources": ("attn_prefill.hip", "attn_prefill_dma.h", "device_utils.h"), "sha256_16": "8598cef9f505c863"},
+        "bytes": (19511 + 10240) * 1024, "profile": "profiles/prefill_fp8_512x4608_batch_dma_kernel.md",
+        "sources": ("attn_prefill.hip", "attn_prefill_dma.h", "device_utils.h"), "sha256_16": "2b0ad01b6d75d8a4"},
 }
 
 

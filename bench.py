@@ -43,7 +43,7 @@ PROFILED_TRAFFIC = {
         "sources": ("attn_decode.hip", "attn_decode_mfma.h", "device_utils.h"), "sha256_16": "0145bfacb7bdfd49"},
     "prefill_fp8_512x4608_32layers": {
         "bytes": (19511 + 10240) * 1024, "profile": "profiles/prefill_fp8_512x4608_batch_dma_kernel.md",
-        "sources": ("attn_prefill.hip", "attn_prefill_dma.h", "device_utils.h"), "sha256_16": "2b0ad01b6d75d8a4"},
+        "sources": ("attn_prefill.hip", "attn_prefill_dma.h", "device_utils.h"), "sha256_16": "782842a8167298a4"},
 }
 
 
@@ -714,7 +714,67 @@ def issue_rate_calibration(args):
         ms, ticks, mhz = timed(lambda st: calib.vfkv_calib_overlap(nv, mode, it2, sink.data_ptr(), clk.data_ptr(), st))
         out["overlap"][label] = {"simd_ticks_per_pass_of_both_wavefronts": ms * 1e-3 * mhz * 1e6 / it2, "kernel_ms": ms,
                                  "clock_mhz": mhz}
-    out["value"] = out["overlap"]["48_mfma_only"]["simd_ticks_per_pass_of_both_wavefronts"] / 96.0
+    # the same two-phase pass with 100 vector instructions of each kind: alone, and behind 48 matrix instructions
+    calib.vfkv_calib_overlap_kind.argtypes = [C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p]
+    out["overlap_by_kind"] = {}
+    base = out["overlap"]["48_mfma_only"]["simd_ticks_per_pass_of_both_wavefronts"]
+    for op, name in enumerate(names):
+        t = {}
+        for with_matrix in (0, 1):
+            ms, ticks, mhz = timed(lambda st: calib.vfkv_calib_overlap_kind(op, with_matrix, it2, sink.data_ptr(), clk.data_ptr(), st))
+            t[with_matrix] = ms * 1e-3 * mhz * 1e6 / it2
+        out["overlap_by_kind"][name] = {"100_vector_alone": t[0], "48_mfma_then_100_vector": t[1], "hidden": base + t[0] - t[1]}
+    out["value"] = base / 96.0
+    return out
+
+
+def prefill_phase_stamps(args):
+    """Where one launch of the FP8 prefill kernel spends its time outside the tile loop: the kernel compiled with wall-clock
+    stamps (libvfkv_calib.so, csrc/calibration_prefill.hip) on the 512 x 4 608 geometry; microseconds after the first
+    wavefront's start."""
+    import ctypes as C
+    import numpy as np
+    import torch
+    from vulkanforge_amd import workloads
+    cfg = workloads.PREFILL["prefill_fp8_512x4608_32layers"]
+    H, Hkv, D, m, base = cfg.n_heads, cfg.n_kv_heads, cfg.head_dim, cfg.m, cfg.base_pos
+    n_kv = base + m
+    calib = C.CDLL(os.path.join(ROOT, "vulkanforge_amd", "libvfkv_calib.so"))
+    calib.vfkv_calib_prefill_stamps.argtypes = [C.c_void_p] * 4 + [C.c_uint32] * 5 + [C.c_float, C.c_int, C.c_void_p, C.c_void_p]
+    g = torch.Generator(device="cuda").manual_seed(3)
+    # standard-normal rows rounded to E4M3, as the benchmark's prefill workload holds them
+    k = torch.randn((n_kv, Hkv * D), device="cuda", generator=g).to(torch.float8_e4m3fn).view(torch.uint8)
+    v = torch.randn((n_kv, Hkv * D), device="cuda", generator=g).to(torch.float8_e4m3fn).view(torch.uint8)
+    q = torch.randn((m, H, D), device="cuda", generator=g).half().float()
+    o = torch.empty_like(q)
+    nb = (m + 15) // 16
+    st = torch.zeros((nb, Hkv, 8, 8), dtype=torch.int64, device="cuda")
+    stream = torch.cuda.current_stream().cuda_stream
+    out = {"metric": "prefill_phase_stamps", "unit": "us after the first wavefront's start", "n_gpus": 1,
+           "config": {"workload": "prefill_fp8_512x4608 one layer, instrumented kernel"}, "variants": {}}
+    for label, f16w in (("default", 0), ("f16_weights", 1)):
+        for rep in range(4):                                 # the last of four launches is reported
+            st.zero_()
+            torch.cuda.synchronize()
+            rc = calib.vfkv_calib_prefill_stamps(q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), H, Hkv, m, n_kv, base,
+                                                 1.0 / D ** 0.5, f16w, st.data_ptr(), stream)
+            assert rc == 0, rc
+            torch.cuda.synchronize()
+        s = st.cpu().numpy().astype(np.float64) / 100.0
+        s = np.where(s > 0, s - s[..., 0].min(), np.nan)
+        med = lambda a: float(np.nanmedian(a))
+        wg_end = np.nanmax(s[..., 6], axis=2)                # [launch row][KV head]
+        walk_end = np.nanmax(s[..., 2], axis=2)
+        out["variants"][label] = {
+            "kernel_span": float(np.nanmax(s)),
+            "q_planes_ready": {"min": float(np.nanmin(s[..., 1])), "median": med(s[..., 1]), "max": float(np.nanmax(s[..., 1]))},
+            "last_tile_done_wavefronts_0_3_median": med(s[:, :, :4, 2]), "last_tile_done_wavefronts_4_7_median": med(s[:, :, 4:, 2]),
+            "last_tile_of_workgroup_to_workgroup_done_median": med(wg_end - walk_end),
+            "workgroup_done": {"min": float(wg_end.min()), "median": med(wg_end), "max": float(wg_end.max())},
+            "workgroup_done_by_launch_row_mean": [round(float(x), 2) for x in wg_end.mean(axis=1)],
+            "workgroup_done_by_kv_head_mean": [round(float(x), 2) for x in wg_end.mean(axis=0)],
+        }
+    out["value"] = out["variants"]["default"]["kernel_span"]
     return out
 
 
@@ -738,6 +798,8 @@ def run_workload(args, name):
         return slab_reuse_calibration(args)
     if name == "issue_rate_calibration":
         return issue_rate_calibration(args)
+    if name == "prefill_phase_stamps":
+        return prefill_phase_stamps(args)
     return None
 
 
@@ -766,7 +828,7 @@ def main():
     from vulkanforge_amd import workloads
     res = run_workload(args, args.workload)
     if res is None:
-        print("unknown workload; choose from: " + ", ".join(list(workloads.DECODE) + list(workloads.PREFILL) + list(workloads.ROPE_APPEND) + ["copy_calibration", "slab_reuse_calibration", "issue_rate_calibration"]),
+        print("unknown workload; choose from: " + ", ".join(list(workloads.DECODE) + list(workloads.PREFILL) + list(workloads.ROPE_APPEND) + ["copy_calibration", "slab_reuse_calibration", "issue_rate_calibration", "prefill_phase_stamps"]),
               file=sys.stderr)
         sys.exit(2)
     if args.workload == HEADLINE and not args.no_other_workloads:

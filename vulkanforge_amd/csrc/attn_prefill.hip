@@ -31,7 +31,13 @@ struct BatchArgs {
     const float* gate;
     uint32_t gchunk, gstride, goff;
     uint32_t q_f16;          // f16 matrix-core kernels: use f16(q) alone, whatever the queries hold
+#ifdef VFKV_PREFILL_STAMPS
+    unsigned long long* stamps;   // instrumented build (calibration_prefill.hip): [workgroup][8 wavefronts][8] wall-clock readings
+#endif
 };
+#ifdef VFKV_PREFILL_STAMPS
+static unsigned long long* g_prefill_stamps = nullptr;
+#endif
 
 }  // namespace vfkv
 #include "attn_prefill_mfma2.h"
@@ -221,6 +227,9 @@ static hipError_t launch_batch_kernels(const BatchLaunch& L, hipStream_t stream,
             // FP8 matrix instruction (needs the Q block staged in one round: four key splits).  Over F16 rows (four heads per
             // wavefront) f16_weights is an instantiation of the general kernel; other shapes keep the default arithmetic.
             const bool f8s = L.fp8_scores && vdma && ns >= 4u;
+#ifdef VFKV_PREFILL_STAMPS
+            a.stamps = vdma ? g_prefill_stamps : nullptr;
+#endif
             // eight wavefronts (two per SIMD) and an even number of key splits: the older wavefront of a SIMD gets 3 tiles
             // for every 2 of the younger one
             int deal_a = 1, deal_b = 1;

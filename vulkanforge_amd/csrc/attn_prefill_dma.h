@@ -19,6 +19,16 @@
 
 namespace vfkv {
 
+// Instrumented build only (calibration_prefill.hip): lane 0 of every wavefront stores the 100 MHz wall clock at seven points
+// of the kernel.  The library proper compiles these to nothing.
+#ifdef VFKV_PREFILL_STAMPS
+#define VFKV_STAMP(i)                                                                                                        \
+    do { if (a.stamps != nullptr && lane == 0)                                                                               \
+        a.stamps[((size_t)((blockIdx.z * gridDim.y + blockIdx.y) * gridDim.x + blockIdx.x) * 8 + w) * 8 + (i)] = wall_clock64(); } while (0)
+#else
+#define VFKV_STAMP(i) do { } while (0)
+#endif
+
 template <bool CAP, bool F16W, bool F8S>
 __global__ __launch_bounds__(512) void batch_dma_kernel(BatchArgs a, int HP, int NS, int DEAL_A, int DEAL_B) {
     constexpr int D = 128, NCB = 2, PFD = 2;     // head_dim, heads per wavefront, K tiles in flight
@@ -59,6 +69,7 @@ __global__ __launch_bounds__(512) void batch_dma_kernel(BatchArgs a, int HP, int
     const int gz = (blockIdx.z / a.nk) * HP * NCB;              // first head (inside the group) of this workgroup
     const int g0 = hp * NCB;                                    // first head slot (inside the workgroup) of this wavefront
 
+    VFKV_STAMP(0);                                              // start
     uint8_t* const v8 = reinterpret_cast<uint8_t*>(lds) + (size_t)w * 3 * VBUF;   // [3][KT * D] raw V tiles of this wavefront
     constexpr int QPITCH = D + 8;
     _Float16* const qhi_lds = lds + (size_t)nwaves * 3 * VBUF / 2;  // [GP][16][D + 8] f16(q); the slots past G hold zeros
@@ -243,6 +254,7 @@ __global__ __launch_bounds__(512) void batch_dma_kernel(BatchArgs a, int HP, int
     __syncthreads();
     has_lo = __builtin_amdgcn_readfirstlane(lds_haslo) != 0;   // workgroup-uniform
     }
+    VFKV_STAMP(1);                                              // Q planes ready
 
     float4_t oacc[NCB][DTILES];
 #pragma unroll
@@ -497,6 +509,7 @@ __global__ __launch_bounds__(512) void batch_dma_kernel(BatchArgs a, int HP, int
     }
     };
     if (has_lo) walk(std::true_type{}); else walk(std::false_type{});
+    VFKV_STAMP(2);                                              // last tile done
 #pragma unroll
     for (int cb = 0; cb < NCB; ++cb) l_run[cb] = xor32_sum(xor16_sum(l_run[cb]));   // every lane of a query column has its wavefront's sum
 
@@ -517,7 +530,9 @@ __global__ __launch_bounds__(512) void batch_dma_kernel(BatchArgs a, int HP, int
             mlbuf[((size_t)(slot * NCB + cb) * 2 + 0) * 64 + lane] = m_run[cb];
             mlbuf[((size_t)(slot * NCB + cb) * 2 + 1) * 64 + lane] = l_run[cb];
         }
+        VFKV_STAMP(3);                                          // (o, m, l) in LDS
         __syncthreads();
+        VFKV_STAMP(4);
         if (!q_ok) return;
         // (compiled per split count so that the LDS reads of a head are independent instructions, not a chain of round trips)
         auto merge_and_store = [&](auto ns_tag) {
@@ -572,6 +587,11 @@ __global__ __launch_bounds__(512) void batch_dma_kernel(BatchArgs a, int HP, int
         if (NS == 4) merge_and_store(std::integral_constant<int, 4>{});
         else if (NS == 2) merge_and_store(std::integral_constant<int, 2>{});
         else merge_and_store(std::integral_constant<int, 8>{});  // (the launcher gives 2, 4 or 8 splits)
+        VFKV_STAMP(5);                                          // merged, stores issued
+#ifdef VFKV_PREFILL_STAMPS
+        __builtin_amdgcn_s_waitcnt(0);
+#endif
+        VFKV_STAMP(6);                                          // stores complete
         return;
     }
     float4_t gfac[NCB][DTILES];
@@ -628,5 +648,7 @@ __global__ __launch_bounds__(512) void batch_dma_kernel(BatchArgs a, int HP, int
         }
     }
 }
+
+#undef VFKV_STAMP
 
 }  // namespace vfkv

@@ -82,6 +82,10 @@ CASES = [
     (vf.KvDtype.F8, 32, 8, 128, 100, 2517, 0, 0.0),   # FP8 rows of 128 elements (V loaded straight into LDS): many two-tile passes, ragged end
     (vf.KvDtype.F8, 16, 4, 128, 33, 6005, 4100, 30.0),  # the same kernel: window that starts inside a tile, soft-cap
     (vf.KvDtype.F8, 40, 8, 128, 7, 1037, 0, 0.0),     # G = 5: a padded head slot beside the rotation of V buffers
+    (vf.KvDtype.F8, 32, 8, 128, 45, 1300, 0, 0.0),    # the same kernel, three query blocks, the last one ragged: the head pairs of a workgroup take mirrored blocks (the middle one both)
+    (vf.KvDtype.F8, 16, 2, 128, 96, 700, 650, 0.0),   # G = 8: four head pairs in two key splits, six query blocks, window that starts after some blocks' first tile
+    (vf.KvDtype.F8, 8, 4, 128, 130, 37, 0, 20.0),     # G = 2: one head pair (no mirroring), eight key splits dealt 3:2, nine query blocks, soft-cap
+    (vf.KvDtype.F8, 32, 8, 128, 256, 0, 0, 0.0),      # from position 0: the first query blocks see fewer tiles than a workgroup has key splits
 ]
 
 

@@ -31,6 +31,7 @@ struct BatchArgs {
     const float* gate;
     uint32_t gchunk, gstride, goff;
     uint32_t q_f16;          // f16 matrix-core kernels: use f16(q) alone, whatever the queries hold
+    uint32_t merge_all;      // batch_mfma2_kernel: the LDS area holds the (o, m, l) of every wavefront, and every wavefront merges a share
 #ifdef VFKV_PREFILL_STAMPS
     unsigned long long* stamps;   // instrumented build (calibration_prefill.hip): [workgroup][8 wavefronts][8] wall-clock readings
 #endif
@@ -117,6 +118,10 @@ static hipError_t launch_batch_kernels(const BatchLaunch& L, hipStream_t stream,
     a.so = nullptr; a.sm = nullptr; a.ss = nullptr; a.nk = 1u; a.chunk = 0u;
     a.gate = nullptr; a.gchunk = 1u; a.gstride = 0u; a.goff = 0u;
     a.q_f16 = L.f16_queries ? 1u : 0u;
+    a.merge_all = 0u;
+#ifdef VFKV_PREFILL_STAMPS
+    a.stamps = nullptr;
+#endif
     const uint32_t g = L.n_heads / L.n_kv_heads;
     const uint64_t slab_bytes = (uint64_t)L.n_kv * L.n_kv_heads * L.head_dim * elem_size(L.dtype);
     const bool aligned = ((((uintptr_t)L.k) | ((uintptr_t)L.v) | ((uintptr_t)L.q) | ((uintptr_t)L.o)) & 15u) == 0u;
@@ -212,8 +217,9 @@ static hipError_t launch_batch_kernels(const BatchLaunch& L, hipStream_t stream,
                                   (nh == 2u ? (size_t)2 * nwaves * ncb * 64 * 16 : 0u);
             // merge area: the general kernel keeps the records of all splits but the first; the V-through-LDS kernel the
             // output tiles and (m, l) of every wavefront
-            const size_t mbytes = vdma ? (size_t)nwaves * ncb * 64 * (dv / 4 + 2) * sizeof(float)
-                                       : (size_t)(ns - 1) * hp * ncb * 64 * (dv / 4 + 2) * sizeof(float);
+            const size_t mbytes_all = (size_t)nwaves * ncb * 64 * (dv / 4 + 2) * sizeof(float);
+            a.merge_all = (!vdma && nh == 1u && mbytes_all + 64u <= 160u * 1024u) ? 1u : 0u;
+            const size_t mbytes = (vdma || a.merge_all) ? mbytes_all : (size_t)(ns - 1) * hp * ncb * 64 * (dv / 4 + 2) * sizeof(float);
             const size_t lds = vbytes > mbytes ? vbytes : mbytes;
             const bool cap = L.softcap > 0.f;
             bool launched = true;

@@ -417,8 +417,81 @@ __global__ __launch_bounds__((NCB == 1 && D <= 128) ? kPrefillOneHeadWaves * 64 
         }
     }
 
-    // ---- merge the key splits through LDS (split 0 collects), normalise and store ----
+    // ---- merge the key splits through LDS, normalise and store.  Where the launcher found room for it (a.merge_all) and
+    // the split count is 2, 4 or 8, every wavefront leaves its (o, m, l) in LDS -- o as [wavefront][cb][dt][lane] float4:
+    // 16-byte accesses of consecutive lanes, no bank conflicts -- and the NS wavefronts of a head unit each merge and store
+    // the d-tiles dt = sp, sp + NS, ... of the unit's NCB heads, compiled per split count so that the LDS reads of a head
+    // are independent instructions.  Otherwise split 0 collects the records of the others one after the other.
     constexpr int REC = DTILES * 4 + 2;
+    // (not compiled into the F16 head_dim 256 form: with it that instantiation's tile loop spills twice as many registers, 109 -> 137 us)
+    constexpr bool MERGE_ALL = NH == 1 && !(DT == kF16 && D == 256);
+    if (MERGE_ALL && NS > 1 && a.merge_all != 0u && (NS == 2 || NS == 4 || NS == 8)) {
+        __syncthreads();                                        // every wavefront is done with its V area
+        float4_t* obuf = reinterpret_cast<float4_t*>(lds);
+        float* mlbuf = reinterpret_cast<float*>(lds) + (size_t)nwaves * NCB * DTILES * 64 * 4;
+        const int slot = sp * HP + hp;
+#pragma unroll
+        for (int cb = 0; cb < NCB; ++cb) {
+#pragma unroll
+            for (int dt = 0; dt < DTILES; ++dt) obuf[((size_t)(slot * NCB + cb) * DTILES + dt) * 64 + lane] = oacc[cb][dt];
+            mlbuf[((size_t)(slot * NCB + cb) * 2 + 0) * 64 + lane] = m_run[cb];
+            mlbuf[((size_t)(slot * NCB + cb) * 2 + 1) * 64 + lane] = l_run[cb];
+        }
+        __syncthreads();
+        if (!q_ok) return;
+        auto merge_and_store = [&](auto ns_tag) {
+            constexpr int NSC = decltype(ns_tag)::value;
+#pragma unroll
+            for (int cb = 0; cb < NCB; ++cb) {
+                if (gz + g0 + cb >= G) continue;                // padding slot of an odd group
+                float f[NSC], lv[NSC];
+#pragma unroll
+                for (int s2 = 0; s2 < NSC; ++s2) {
+                    const float* ml = mlbuf + ((size_t)((s2 * HP + hp) * NCB + cb) * 2) * 64 + lane;
+                    f[s2] = ml[0]; lv[s2] = ml[64];
+                }
+                float mm = f[0];
+#pragma unroll
+                for (int s2 = 1; s2 < NSC; ++s2) mm = fmaxf(mm, f[s2]);
+                float lsum = 0.f;
+#pragma unroll
+                for (int s2 = 0; s2 < NSC; ++s2) { f[s2] = __builtin_amdgcn_exp2f(f[s2] - mm); lsum += lv[s2] * f[s2]; }
+                const uint32_t h = kvh * G + gz + g0 + cb;
+                const size_t pidx = ((size_t)qi * a.n_heads + h) * a.nk + kc;      // (key chunks: the partial of this chunk)
+                const float inv = a.so != nullptr ? 1.0f : 1.0f / lsum;
+                float* op = a.so != nullptr ? a.so + pidx * D + kg * 4 : a.o + ((size_t)qi * a.n_heads + h) * D + kg * 4;
+                const float* gp = nullptr;
+                if (a.gate != nullptr) {
+                    const uint32_t i0 = (qi * a.n_heads + h) * D;
+                    const uint32_t token = i0 / a.gchunk;
+                    gp = a.gate + (size_t)token * a.gstride + a.goff + (i0 - token * a.gchunk) + kg * 4;
+                }
+#pragma unroll
+                for (int j = 0; j < (DTILES + NSC - 1) / NSC; ++j) {   // lane (query n16) holds d = dt*16 + kg*4 + i
+                    const int dt = sp + j * NSC;
+                    if (DTILES % NSC != 0 && dt >= DTILES) break;
+                    float4_t r = float4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                    for (int s2 = 0; s2 < NSC; ++s2)
+                        r += obuf[((size_t)((s2 * HP + hp) * NCB + cb) * DTILES + dt) * 64 + lane] * f[s2];
+                    r *= inv;
+                    if (gp != nullptr) {
+                        const float4 gv = *reinterpret_cast<const float4*>(gp + dt * 16);
+                        r *= float4_t{sigmoid_gate(1.0f, gv.x), sigmoid_gate(1.0f, gv.y), sigmoid_gate(1.0f, gv.z), sigmoid_gate(1.0f, gv.w)};
+                    }
+                    *reinterpret_cast<float4*>(op + dt * 16) = make_float4(r[0], r[1], r[2], r[3]);
+                }
+                if (a.so != nullptr && sp == 0 && kg == 0) {
+                    a.sm[pidx] = mm > -1e29f ? mm * 0.693147180559945f : kMasked;
+                    a.ss[pidx] = lsum;
+                }
+            }
+        };
+        if (NS == 4) merge_and_store(std::integral_constant<int, 4>{});
+        else if (NS == 2) merge_and_store(std::integral_constant<int, 2>{});
+        else merge_and_store(std::integral_constant<int, 8>{});
+        return;
+    }
     if (NS > 1) {
         __syncthreads();                                        // every wavefront is done with its V area
         float* mbuf = reinterpret_cast<float*>(lds);            // [NS-1][HP][NCB][64][REC]

@@ -31,3 +31,17 @@ def test_workload_tables_state_the_configurations_algorithmic_work():
     sliding = workloads.DECODE["decode_f16_hd256_sliding_12layers"]
     assert [sliding.layer_window(i) for i in range(6)] == [4096] * 5 + [0]        # five sliding layers, then a global one
     assert json.dumps({"ok": True})                                               # (bench lines are plain JSON)
+
+
+def test_calibration_library_loads_and_exports_what_the_benchmark_calls():
+    # (no device work: symbols only; the library resolves libvfkv.so beside it)
+    import ctypes
+    lib = ctypes.CDLL(os.path.join(ROOT, "vulkanforge_amd", "libvfkv_calib.so"))
+    for name in ("vfkv_calib_stream_read", "vfkv_calib_pattern_read", "vfkv_calib_empty", "vfkv_calib_issue",
+                 "vfkv_calib_overlap", "vfkv_calib_overlap_kind", "vfkv_calib_prefill_stamps"):
+        assert hasattr(lib, name), name
+    with open(os.path.join(ROOT, "bench.py")) as f:
+        text = f.read()
+    import re
+    for name in set(re.findall(r"calib\.(vfkv_calib_\w+)", text)):
+        assert hasattr(lib, name), name

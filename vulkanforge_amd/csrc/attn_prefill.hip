@@ -174,6 +174,10 @@ static hipError_t launch_batch_kernels(const BatchLaunch& L, hipStream_t stream,
                 hp = (hp_group / nh + want - 1u) / want * nh;    // the output slices of a head stay in one workgroup
             }
             while (hp > nh && waves_for(hp) < hp) hp -= nh;      // one head always fits
+            // the V-through-LDS kernel runs best as two head pairs x four key splits (two wavefronts per SIMD, mirrored query
+            // blocks, the uneven deal): a group of four head pairs becomes two such workgroups instead of one workgroup of
+            // four wavefronts that each walk every key (512 queries over 4 608 keys, 64 / 8 / 128: 133.7 -> 120.0 us; 128 / 8 / 128: 352 -> 233 us)
+            if (vdma && hp > 2u && hp_group % 2u == 0u) hp = 2u;
         }
         const uint32_t nz = (hp_group + hp - 1u) / hp;
         const uint32_t max_waves = waves_for(hp);

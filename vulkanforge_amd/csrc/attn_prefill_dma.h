@@ -13,6 +13,12 @@
 //   tile stand between the vector instructions of the other.  (With general f32 queries the remainder product of Q leaves
 //   no room for it and the loop takes one tile per pass.)
 //
+// and three measures that even out the work inside a workgroup of eight wavefronts (two per SIMD): the key splits of the
+// older wavefront of a SIMD take three tiles for every two of the younger one's (the older one issues first whenever both
+// are ready); the head pairs of a workgroup take mirrored query blocks, so that every workgroup and every SIMD walks the
+// same number of tiles whatever the causal mask leaves each block; and every wavefront merges and stores a share of the
+// output tiles.
+//
 // Included by attn_prefill.hip after attn_prefill_mfma2.h.
 #pragma once
 #include <type_traits>

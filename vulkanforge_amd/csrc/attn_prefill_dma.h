@@ -487,12 +487,13 @@ __global__ __launch_bounds__(512) void batch_dma_kernel(BatchArgs a, int HP, int
             // the tiles before them, so the matrix pipe and the vector ALU have work from different tiles side by side
             while (tp[0] >= a.kv_start && tp[PFD - 1] + KT <= fast_end) {
                 bool moved = false;
-                // the first products issue ahead of the other wavefront's vector work (measured: 2 us of a 63 us launch;
-                // the same around the second products, or around the softmax instead, gains nothing)
-                __builtin_amdgcn_s_setprio(1);
+                // the first products issue ahead of the other wavefront's vector work (measured: 2 % of a 32-layer step; the
+                // same around the second products, or around the softmax instead, gains nothing, and the FP8 first product
+                // loses 1 % with it)
+                if constexpr (!F8S) __builtin_amdgcn_s_setprio(1);
 #pragma unroll
                 for (int sl = 0; sl < PFD; ++sl) first_product(sl, tp[sl], lo_tag);
-                __builtin_amdgcn_s_setprio(0);
+                if constexpr (!F8S) __builtin_amdgcn_s_setprio(0);
 #pragma unroll
                 for (int sl = 0; sl < PFD; ++sl) moved |= scores(std::false_type{}, sl, tp[sl]);
                 if (__builtin_amdgcn_ballot_w64(moved) != 0ull) { s_ready = true; break; }

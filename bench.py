@@ -43,7 +43,7 @@ PROFILED_TRAFFIC = {
         "sources": ("attn_decode.hip", "attn_decode_mfma.h", "device_utils.h"), "sha256_16": "0145bfacb7bdfd49"},
     "prefill_fp8_512x4608_32layers": {
         "bytes": (19511 + 10240) * 1024, "profile": "profiles/prefill_fp8_512x4608_batch_dma_kernel.md",
-        "sources": ("attn_prefill.hip", "attn_prefill_dma.h", "device_utils.h"), "sha256_16": "1982084227e23ad8"},
+        "sources": ("attn_prefill.hip", "attn_prefill_dma.h", "device_utils.h"), "sha256_16": "eac4a9fed6ede5bb"},
 }
 
 
@@ -767,6 +767,8 @@ def prefill_phase_stamps(args):
         walk_end = np.nanmax(s[..., 2], axis=2)
         out["variants"][label] = {
             "kernel_span": float(np.nanmax(s)),
+            "wavefront_start": {"median": med(s[..., 0]), "max": float(np.nanmax(s[..., 0]))},
+            "query_block_arrived": {"min": float(np.nanmin(s[..., 7])), "median": med(s[..., 7]), "max": float(np.nanmax(s[..., 7]))},
             "q_planes_ready": {"min": float(np.nanmin(s[..., 1])), "median": med(s[..., 1]), "max": float(np.nanmax(s[..., 1]))},
             "last_tile_done_wavefronts_0_3_median": med(s[:, :, :4, 2]), "last_tile_done_wavefronts_4_7_median": med(s[:, :, 4:, 2]),
             "last_tile_of_workgroup_to_workgroup_done_median": med(wg_end - walk_end),

@@ -241,6 +241,9 @@ __global__ __launch_bounds__(512) void batch_dma_kernel(BatchArgs a, int HP, int
 #pragma unroll
             for (int sl = 0; sl < PFD; ++sl) issue(sl, tile_off(tp[sl]));
         }
+#ifdef VFKV_PREFILL_STAMPS
+        if (base == 0) { asm volatile("s_waitcnt vmcnt(16)" ::: "memory"); VFKV_STAMP(7); }   // the query block has arrived (16 K / V requests behind it)
+#endif
 #pragma unroll
         for (int i = 0; i < QLD; ++i) {
             const int idx = base + tid + i * nthreads;

@@ -43,7 +43,7 @@ PROFILED_TRAFFIC = {
         "sources": ("attn_decode.hip", "attn_decode_mfma.h", "device_utils.h"), "sha256_16": "0145bfacb7bdfd49"},
     "prefill_fp8_512x4608_32layers": {
         "bytes": (19511 + 10240) * 1024, "profile": "profiles/prefill_fp8_512x4608_batch_dma_kernel.md",
-        "sources": ("attn_prefill.hip", "attn_prefill_dma.h", "device_utils.h"), "sha256_16": "eac4a9fed6ede5bb"},
+        "sources": ("attn_prefill.hip", "attn_prefill_dma.h", "device_utils.h"), "sha256_16": "2fb842f1b03337c1"},
 }
 
 

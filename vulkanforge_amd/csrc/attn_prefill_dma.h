@@ -544,6 +544,21 @@ __global__ __launch_bounds__(512) void batch_dma_kernel(BatchArgs a, int HP, int
             mlbuf[((size_t)(slot * NCB + cb) * 2 + 0) * 64 + lane] = m_run[cb];
             mlbuf[((size_t)(slot * NCB + cb) * 2 + 1) * 64 + lane] = l_run[cb];
         }
+        // the gate values of the tiles this wavefront will store are requested here, so that their round trip overlaps the
+        // barrier and the merge (tile j of its share is dt = sp + j NS)
+        float4 gpre[NCB][DTILES / 2];
+        if (a.gate != nullptr && q_ok) {
+#pragma unroll
+            for (int cb = 0; cb < NCB; ++cb) {
+                if (gz + g0 + cb >= G) continue;
+                const uint32_t i0 = (qi * a.n_heads + kvh * G + gz + g0 + cb) * D;
+                const uint32_t token = i0 / a.gchunk;
+                const float* gp = a.gate + (size_t)token * a.gstride + a.goff + (i0 - token * a.gchunk) + kg * 4;
+#pragma unroll
+                for (int j = 0; j < DTILES / 2; ++j)
+                    if (sp + j * NS < DTILES) gpre[cb][j] = *reinterpret_cast<const float4*>(gp + (sp + j * NS) * 16);
+            }
+        }
         VFKV_STAMP(3);                                          // (o, m, l) in LDS
         __syncthreads();
         VFKV_STAMP(4);
@@ -570,12 +585,6 @@ __global__ __launch_bounds__(512) void batch_dma_kernel(BatchArgs a, int HP, int
                 const size_t pidx = ((size_t)qi * a.n_heads + h) * a.nk + kc;      // (key chunks: the partial of this chunk)
                 const float inv = a.so != nullptr ? 1.0f : 1.0f / lsum;
                 float* op = a.so != nullptr ? a.so + pidx * D + kg * 4 : a.o + ((size_t)qi * a.n_heads + h) * D + kg * 4;
-                const float* gp = nullptr;
-                if (a.gate != nullptr) {
-                    const uint32_t i0 = (qi * a.n_heads + h) * D;
-                    const uint32_t token = i0 / a.gchunk;
-                    gp = a.gate + (size_t)token * a.gstride + a.goff + (i0 - token * a.gchunk) + kg * 4;
-                }
 #pragma unroll
                 for (int j = 0; j < DTILES / NSC; ++j) {        // lane (query n16) holds d = dt*16 + kg*4 + i
                     const int dt = sp + j * NSC;
@@ -584,8 +593,8 @@ __global__ __launch_bounds__(512) void batch_dma_kernel(BatchArgs a, int HP, int
                     for (int s2 = 0; s2 < NSC; ++s2)
                         r += obuf[((size_t)((s2 * HP + hp) * NCB + cb) * DTILES + dt) * 64 + lane] * f[s2];
                     r *= inv;
-                    if (gp != nullptr) {
-                        const float4 gv = *reinterpret_cast<const float4*>(gp + dt * 16);
+                    if (a.gate != nullptr) {
+                        const float4 gv = gpre[cb][j];
                         r *= float4_t{sigmoid_gate(1.0f, gv.x), sigmoid_gate(1.0f, gv.y), sigmoid_gate(1.0f, gv.z), sigmoid_gate(1.0f, gv.w)};
                     }
                     *reinterpret_cast<float4*>(op + dt * 16) = make_float4(r[0], r[1], r[2], r[3]);

@@ -744,7 +744,11 @@ def prefill_phase_stamps(args):
     g = torch.Generator(device="cuda").manual_seed(3)
     # standard-normal rows rounded to E4M3, as the benchmark's prefill workload holds them
     k = torch.randn((n_kv, Hkv * D), device="cuda", generator=g).to(torch.float8_e4m3fn).view(torch.uint8)
-    v = torch.randn((n_kv, Hkv * D), device="cuda", generator=g).to(torch.float8_e4m3fn).view(torch.uint8)
+    # V starts 256 bytes past an allocation boundary, as in a cache made by vfkv_cache_create (K and V rows at the same offsets make
+    # one KV head's loads slower than the others')
+    vpool = torch.randn((n_kv * Hkv * D + (1 << 21),), device="cuda", generator=g).to(torch.float8_e4m3fn).view(torch.uint8)
+    voff = (-vpool.data_ptr()) % (1 << 21) + 256
+    v = vpool[voff: voff + n_kv * Hkv * D].view(n_kv, Hkv * D)
     q = torch.randn((m, H, D), device="cuda", generator=g).half().float()
     o = torch.empty_like(q)
     nb = (m + 15) // 16
@@ -780,6 +784,73 @@ def prefill_phase_stamps(args):
     return out
 
 
+def decode_phase_stamps(args):
+    """Where one launch of the decode worker spends its time: split_mfma_kernel compiled with wall-clock stamps (libvfkv_calib.so,
+    csrc/calibration_decode.hip) on the headline geometry (32 / 8 / 128, FP8, 32 768 keys) and on 8 192 keys; eight launches over eight
+    layer slabs captured into one graph and replayed, as a step issues them; microseconds after the launch's first wavefront started,
+    means over the eight launches of the last replay."""
+    import ctypes as C
+    import numpy as np
+    import torch
+    import vulkanforge_amd as vf
+    calib = C.CDLL(os.path.join(ROOT, "vulkanforge_amd", "libvfkv_calib.so"))
+    calib.vfkv_calib_decode_stamps.argtypes = [C.c_void_p] * 6 + [C.c_uint32] * 7 + [C.c_float, C.c_void_p, C.c_void_p]
+    H, Hkv, D, NL, NW = 32, 8, 128, 8, 4
+    out = {"metric": "decode_phase_stamps", "unit": "us after the launch's first wavefront started", "n_gpus": 1,
+           "config": {"workload": "split_mfma_kernel, 32 / 8 / 128 FP8, instrumented kernel, 8 launches per graph replay"}, "contexts": {}}
+    g = torch.Generator(device="cuda").manual_seed(5)
+    # (seq_len, byte offset of the V slabs from a 2 MiB boundary; the K slabs start on one).  256 is what vfkv_cache_create gives V:
+    # with K and V rows at the same offsets one KV head's stream runs 10 % slower than the others and the launch waits for it
+    # (the head whose 128-byte pieces lie at addresses with bits 9:7 == 011, on whichever XCD it runs)
+    for seq, shift in ((32768, 256), (8192, 256), (32768, 0)):
+        tile = vf.lib().vfkv_decode_tile_for(seq, H, Hkv, D, int(vf.KvDtype.F8))
+        nt = (seq + tile - 1) // tile
+        slab = seq * Hkv * D
+        pool = [torch.randn(((NL * slab + (1 << 21)) // 4,), device="cuda", generator=g).to(torch.float8_e4m3fn).view(torch.uint8).repeat(4)
+                for _ in range(2)]
+        base = [(-pool[0].data_ptr()) % (1 << 21), (-pool[1].data_ptr()) % (1 << 21) + shift]      # offset of the first slab inside its pool
+        ks = [pool[0][base[0] + l * slab: base[0] + (l + 1) * slab] for l in range(NL)]
+        vs = [pool[1][base[1] + l * slab: base[1] + (l + 1) * slab] for l in range(NL)]
+        q = torch.randn((H, D), device="cuda", generator=g).half().float()
+        so = torch.empty((H, nt, D), device="cuda"); sm = torch.empty((H, nt), device="cuda"); ss = torch.empty((H, nt), device="cuda")
+        st = torch.zeros((NL, Hkv, nt, 1, NW, 4), dtype=torch.int64, device="cuda")
+
+        def launches():
+            stream = torch.cuda.current_stream().cuda_stream
+            for l in range(NL):
+                rc = calib.vfkv_calib_decode_stamps(q.data_ptr(), ks[l].data_ptr(), vs[l].data_ptr(), so.data_ptr(), sm.data_ptr(),
+                                                    ss.data_ptr(), int(vf.KvDtype.F8), H, Hkv, D, seq, tile, nt, 1.0 / D ** 0.5,
+                                                    st[l].data_ptr(), stream)
+                assert rc == 0, rc
+        launches()
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            launches()
+        for _ in range(3):
+            graph.replay()
+        torch.cuda.synchronize()
+        s = st.cpu().numpy().astype(np.float64) / 100.0                  # [launch][KV head][workgroup][1][wavefront][stamp]
+        names = ("wavefront_start", "loop_start", "loop_end", "partial_stored")
+        pct = lambda a: {"min": float(a.min()), "p50": float(np.percentile(a, 50)), "p90": float(np.percentile(a, 90)), "max": float(a.max())}
+        rel = s - s[..., 0].min(axis=(1, 2, 3, 4), keepdims=True)[..., None]
+        entry = {n: pct(rel[..., i]) for i, n in enumerate(names)}
+        entry["loop_per_wavefront"] = pct(rel[..., 2] - rel[..., 1])
+        entry["epilogue_per_wavefront"] = pct(rel[..., 3] - rel[..., 2])
+        entry["loop_start_by_kv_head_mean"] = [round(float(x), 2) for x in rel[..., 1].mean(axis=(0, 2, 3, 4))]
+        entry["loop_per_wavefront_by_kv_head_mean"] = [round(float(x), 2) for x in (rel[..., 2] - rel[..., 1]).mean(axis=(0, 2, 3, 4))]
+        entry["finish_by_kv_head_mean"] = [round(float(x), 2) for x in rel[..., 3].mean(axis=(0, 2, 3, 4))]
+        starts = s[..., 0].min(axis=(1, 2, 3, 4)); ends = s[..., 3].max(axis=(1, 2, 3, 4))
+        entry["launch_span_mean"] = float((ends - starts).mean())
+        entry["next_launch_start_after_last_store_mean"] = float((starts[1:] - ends[:-1]).mean())
+        entry["tile"] = int(tile); entry["workgroups_per_kv_head"] = int(nt)
+        if shift != 256:
+            entry = {k: entry[k] for k in ("loop_per_wavefront_by_kv_head_mean", "finish_by_kv_head_mean", "launch_span_mean")}
+        out["contexts"][str(seq) if shift == 256 else f"{seq}_v_slabs_not_offset"] = entry
+    out["value"] = out["contexts"]["32768"]["launch_span_mean"]
+    return out
+
+
 HEADLINE = "decode_fp8_32k_32layers"
 # the other benchmark configurations, run briefly after the headline workload so that one invocation witnesses all five
 OTHER_CONFIGS = ("decode_f16_2k_1layer", "decode_fp8_8k_32layers", "decode_f16_hd256_sliding_12layers",
@@ -802,6 +873,8 @@ def run_workload(args, name):
         return issue_rate_calibration(args)
     if name == "prefill_phase_stamps":
         return prefill_phase_stamps(args)
+    if name == "decode_phase_stamps":
+        return decode_phase_stamps(args)
     return None
 
 
@@ -830,7 +903,7 @@ def main():
     from vulkanforge_amd import workloads
     res = run_workload(args, args.workload)
     if res is None:
-        print("unknown workload; choose from: " + ", ".join(list(workloads.DECODE) + list(workloads.PREFILL) + list(workloads.ROPE_APPEND) + ["copy_calibration", "slab_reuse_calibration", "issue_rate_calibration", "prefill_phase_stamps"]),
+        print("unknown workload; choose from: " + ", ".join(list(workloads.DECODE) + list(workloads.PREFILL) + list(workloads.ROPE_APPEND) + ["copy_calibration", "slab_reuse_calibration", "issue_rate_calibration", "prefill_phase_stamps", "decode_phase_stamps"]),
               file=sys.stderr)
         sys.exit(2)
     if args.workload == HEADLINE and not args.no_other_workloads:

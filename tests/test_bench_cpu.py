@@ -38,7 +38,7 @@ def test_calibration_library_loads_and_exports_what_the_benchmark_calls():
     import ctypes
     lib = ctypes.CDLL(os.path.join(ROOT, "vulkanforge_amd", "libvfkv_calib.so"))
     for name in ("vfkv_calib_stream_read", "vfkv_calib_pattern_read", "vfkv_calib_empty", "vfkv_calib_issue",
-                 "vfkv_calib_overlap", "vfkv_calib_overlap_kind", "vfkv_calib_prefill_stamps"):
+                 "vfkv_calib_overlap", "vfkv_calib_overlap_kind", "vfkv_calib_prefill_stamps", "vfkv_calib_decode_stamps"):
         assert hasattr(lib, name), name
     with open(os.path.join(ROOT, "bench.py")) as f:
         text = f.read()

@@ -40,7 +40,7 @@ MFMA_F32_PEAK_TFLOPS = 157.3      # dense f32 matrix rate: what an F32 cache is 
 PROFILED_TRAFFIC = {
     "decode_fp8_32k_32layers": {
         "bytes": (65635 + 520) * 1024, "profile": "profiles/decode_floor_calibration.md",
-        "sources": ("attn_decode.hip", "attn_decode_mfma.h", "device_utils.h"), "sha256_16": "0145bfacb7bdfd49"},
+        "sources": ("attn_decode.hip", "attn_decode_mfma.h", "device_utils.h"), "sha256_16": "b27ea68dc2e8f205"},
     "prefill_fp8_512x4608_32layers": {
         "bytes": (19511 + 10240) * 1024, "profile": "profiles/prefill_fp8_512x4608_batch_dma_kernel.md",
         "sources": ("attn_prefill.hip", "attn_prefill_dma.h", "device_utils.h"), "sha256_16": "2fb842f1b03337c1"},

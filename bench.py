@@ -110,6 +110,7 @@ def parse_args():
                     help="leave the queries as general f32 values instead of casting them to fp16 first")
     ap.add_argument("--no-graph", action="store_true",
                     help="launch every kernel from Python instead of replaying one captured HIP graph per step")
+    ap.add_argument("--v-offsets", default="", help="decode_phase_stamps: further byte offsets of the V slabs to time at 32 768 keys, comma-separated")
     ap.add_argument("--no-other-workloads", action="store_true",
                     help="headline run only: skip the short runs of the other benchmark configurations ('workloads' array)")
     return ap.parse_args()
@@ -802,7 +803,8 @@ def decode_phase_stamps(args):
     # (seq_len, byte offset of the V slabs from a 2 MiB boundary; the K slabs start on one).  256 is what vfkv_cache_create gives V:
     # with K and V rows at the same offsets one KV head's stream runs 10 % slower than the others and the launch waits for it
     # (the head whose 128-byte pieces lie at addresses with bits 9:7 == 011, on whichever XCD it runs)
-    for seq, shift in ((32768, 256), (8192, 256), (32768, 0)):
+    cases = [(32768, 256), (8192, 256), (32768, 0)] + [(32768, int(x)) for x in args.v_offsets.split(",") if x.strip()]
+    for seq, shift in cases:
         tile = vf.lib().vfkv_decode_tile_for(seq, H, Hkv, D, int(vf.KvDtype.F8))
         nt = (seq + tile - 1) // tile
         slab = seq * Hkv * D
@@ -846,7 +848,9 @@ def decode_phase_stamps(args):
         entry["tile"] = int(tile); entry["workgroups_per_kv_head"] = int(nt)
         if shift != 256:
             entry = {k: entry[k] for k in ("loop_per_wavefront_by_kv_head_mean", "finish_by_kv_head_mean", "launch_span_mean")}
-        out["contexts"][str(seq) if shift == 256 else f"{seq}_v_slabs_not_offset"] = entry
+        name = str(seq) if shift == 256 else f"{seq}_v_slabs_not_offset" if shift == 0 else f"{seq}_v_slabs_offset_by_{shift}"
+        if name not in out["contexts"]:
+            out["contexts"][name] = entry
     out["value"] = out["contexts"]["32768"]["launch_span_mean"]
     return out
 

@@ -31,6 +31,10 @@
 #ifdef __cplusplus
 extern "C" {
 #endif
+/* The library is built with hidden symbol visibility; the declarations of this header are its whole exported surface. */
+#if defined(__GNUC__) || defined(__clang__)
+#pragma GCC visibility push(default)
+#endif
 
 #define VFKV_ABI_VERSION 1u
 
@@ -52,6 +56,10 @@ typedef enum vfkv_dtype { VFKV_F32 = 0, VFKV_F16 = 1, VFKV_F8E4M3 = 2 } vfkv_dty
 
 const char* vfkv_status_string(int status);
 const char* vfkv_last_error(void);
+/* Advisory left by the last attention call of this thread ("" when there is none; never an error and never mixed into
+ * vfkv_last_error): set when the shape fell to the generic fallback kernels (head_dim outside {64, 96, 128, 256, 512},
+ * pointers not 16-byte aligned, or a layer slab of 2 GiB or more), which are 50-100x slower than the tiled kernels. */
+const char* vfkv_last_note(void);
 uint32_t vfkv_abi_version(void);
 /* Number of visible HIP devices (0 when there is none or the runtime cannot initialise). */
 int vfkv_device_count(void);
@@ -83,10 +91,13 @@ int vfkv_cache_create(const vfkv_cache_config* cfg, vfkv_cache** out);
 /* Same layout object over caller-owned buffers (either may be NULL for layout-only use, e.g. on a
  * host without a GPU).  No allocation happens and destroy() leaves the buffers alone.  For speed give
  * the two buffers different alignment modulo 512 bytes (e.g. v_buffer = allocation + 256): results are
- * identical either way, but equally aligned buffers cost the attention kernels up to 8 %.  The call
- * still returns VFKV_OK then and leaves a one-line note in vfkv_last_error() (empty otherwise). */
+ * identical either way, but equally aligned buffers cost the attention kernels up to 8 %;
+ * vfkv_cache_kv_alignment_note() tells. */
 int vfkv_cache_create_external(const vfkv_cache_config* cfg, void* k_buffer, void* v_buffer,
                                vfkv_cache** out);
+/* "" when the two buffers of the cache differ in address bits 7-8 (or one is NULL), else a one-line advisory that says
+ * what to change.  No counterpart in the reference (its allocator places the buffers, kv_cache.rs:293-339). */
+const char* vfkv_cache_kv_alignment_note(const vfkv_cache* c);
 /* KvCache::destroy (kv_cache.rs:496-499). */
 void vfkv_cache_destroy(vfkv_cache* c);
 /* KvCache::zero_fill (kv_cache.rs:357-380) / zero_layer (kv_cache.rs:389-407).  Both enqueue fill
@@ -436,6 +447,9 @@ int vfkv_prefill_attention_gated(vfkv_cache* c, uint32_t layer, uint32_t kv_laye
                                  const float* q, float* o, uint32_t m, uint32_t base_pos, uint32_t window,
                                  float scale, float softcap, const vfkv_gate* gate, vfkv_stream stream);
 
+#if defined(__GNUC__) || defined(__clang__)
+#pragma GCC visibility pop
+#endif
 #ifdef __cplusplus
 }
 #endif

@@ -373,9 +373,21 @@ def test_external_buffers_of_equal_alignment_leave_a_note_not_an_error():
     L = _ffi.lib()
     cfg = _ffi.CacheConfig(1, 8, 128, 64, None, None, 2)
     h = C.c_void_p()
+    assert L.vfkv_flash_attn_reduce(None, None, None, None, 1, 1, 1, None) == -1     # leaves an error text behind
+    err = L.vfkv_last_error()
     assert L.vfkv_cache_create_external(C.byref(cfg), 0x10000, 0x20000, C.byref(h)) == 0
-    assert b"256 bytes" in L.vfkv_last_error()
+    assert b"256 bytes" in L.vfkv_cache_kv_alignment_note(h)
+    assert L.vfkv_last_error() == err                  # a successful call neither writes nor clears the error text
     L.vfkv_cache_destroy(h)
     assert L.vfkv_cache_create_external(C.byref(cfg), 0x10000, 0x20100, C.byref(h)) == 0
-    assert L.vfkv_last_error() == b""
+    assert L.vfkv_cache_kv_alignment_note(h) == b""
     L.vfkv_cache_destroy(h)
+    assert L.vfkv_cache_kv_alignment_note(None) == b"" and L.vfkv_last_note() == b""
+
+
+def test_dynamic_symbol_table_holds_the_declared_entry_points_only():
+    import subprocess
+    so = os.path.join(ROOT, "vulkanforge_amd", "libvfkv.so")
+    out = subprocess.run(["nm", "-D", "--defined-only", so], check=True, capture_output=True, text=True).stdout
+    exported = sorted(line.split()[-1] for line in out.splitlines() if line.strip())
+    assert exported == _declared_symbols()

@@ -22,7 +22,8 @@ def calib():
     return lib
 
 
-@pytest.mark.parametrize("m,q_start,f16w", [(64, 300, 0), (45, 1300, 0), (100, 2517, 1)])
+# (shapes the launcher runs as one workgroup per (KV head, query block): the layout of the stamp buffer)
+@pytest.mark.parametrize("m,q_start,f16w", [(512, 300, 0), (500, 1300, 0), (520, 2517, 1)])
 def test_instrumented_prefill_kernel_equals_the_library_kernel(m, q_start, f16w):
     heads, hkv, d = 32, 8, 128
     n_kv = q_start + m
@@ -56,6 +57,9 @@ def test_calibration_entry_points_reject_bad_arguments():
     x = torch.zeros(16, device=DEV)
     # 16 heads over 8 KV heads: not the two-head-pairs form the instrumented copy is for
     assert lib.vfkv_calib_prefill_stamps(x.data_ptr(), x.data_ptr(), x.data_ptr(), x.data_ptr(), 16, 8, 16, 32, 16, 0.1, 0,
+                                         x.data_ptr(), None) == -1
+    # 64 queries x 8 KV heads: the launcher would use a third grid dimension that the stamp buffer has no room for
+    assert lib.vfkv_calib_prefill_stamps(x.data_ptr(), x.data_ptr(), x.data_ptr(), x.data_ptr(), 32, 8, 64, 364, 300, 0.1, 0,
                                          x.data_ptr(), None) == -1
 
 

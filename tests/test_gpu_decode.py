@@ -421,7 +421,7 @@ def test_short_context_goes_through_the_same_path():
 @pytest.mark.parametrize("dtype,heads,hkv,d,ctx", [(vf.KvDtype.F8, 32, 8, 128, 4097), (vf.KvDtype.F16, 16, 8, 256, 1500)])
 def test_caller_owned_buffers_give_the_same_output_at_any_relative_alignment(dtype, heads, hkv, d, ctx):
     # KvCache over buffers the caller allocated (kv_cache.rs:224-339 with the host's own allocator): equal alignment of K
-    # and V modulo 512 bytes only costs speed (vfkv_cache_create_external leaves a note), the bytes and the output of decode
+    # and V modulo 512 bytes only costs speed (vfkv_cache_kv_alignment_note says so), the bytes and the output of decode
     # and prefill attention are the same as with V offset by 256 bytes
     from gpu_util import read_device
     fill = outlier_normal if dtype == vf.KvDtype.F8 else fp16_normal
@@ -437,7 +437,7 @@ def test_caller_owned_buffers_give_the_same_output_at_any_relative_alignment(dty
         kp = (kbuf.data_ptr() + 511) // 512 * 512
         vp = (vbuf.data_ptr() + 511) // 512 * 512 + skew
         cache = vf.KvCache(vf.KvCacheConfig(1, hkv, d, ctx, dtype=dtype), k_buffer=kp, v_buffer=vp)
-        note = vf._ffi.lib().vfkv_last_error()
+        note = vf._ffi.lib().vfkv_cache_kv_alignment_note(cache.handle)
         assert (b"256 bytes" in note) == (skew == 0)
         fwd = vf.Forward(cache, heads)
         fwd.b_step_kv_write(0, 0, ctx, to_dev(k), to_dev(v))
@@ -453,3 +453,22 @@ def test_caller_owned_buffers_give_the_same_output_at_any_relative_alignment(dty
     ke, ve = encode_np(k, dtype).reshape(-1, hkv, d), encode_np(v, dtype).reshape(-1, hkv, d)
     ref = oracle.attn_decode_ref(q, ke, ve, int(dtype), heads, hkv, d, ctx, 1.0 / np.sqrt(d))
     assert np.abs(outs[0][0] - ref).max() < TOL[dtype]
+
+
+def test_shapes_on_the_generic_fallback_leave_a_note():
+    # head_dim 80 has no tiled kernel: the result is still right, and vfkv_last_note says that the call was a slow one;
+    # a shape on the tiled kernels clears it
+    L = vf._ffi.lib()
+    r = rng(80)
+    for d, slow in ((80, True), (128, False)):
+        heads, hkv, seq = 8, 2, 300
+        q = fp16_normal(r, (heads, d))
+        k, v = encode_np(fp16_normal(r, (seq, hkv, d)), vf.KvDtype.F16), encode_np(fp16_normal(r, (seq, hkv, d)), vf.KvDtype.F16)
+        scale = float(1.0 / np.sqrt(d))
+        o, *_ = gpu_split_reduce(q, k, v, vf.KvDtype.F16, heads, hkv, d, seq, scale, tile=64)
+        ref = oracle.attn_decode_ref(q, k, v, int(vf.KvDtype.F16), heads, hkv, d, seq, scale)
+        assert np.abs(o - ref).max() < TOL[vf.KvDtype.F16]
+    # (gpu_split_reduce's last library call is the merge, which leaves the note of the split alone)
+        note = L.vfkv_last_note()
+        assert (b"generic fallback" in note) == slow, note
+    assert L.vfkv_last_error() is not None

@@ -82,10 +82,16 @@ CASES = [
     (vf.KvDtype.F8, 32, 8, 128, 100, 2517, 0, 0.0),   # FP8 rows of 128 elements (V loaded straight into LDS): many two-tile passes, ragged end
     (vf.KvDtype.F8, 16, 4, 128, 33, 6005, 4100, 30.0),  # the same kernel: window that starts inside a tile, soft-cap
     (vf.KvDtype.F8, 40, 8, 128, 7, 1037, 0, 0.0),     # G = 5: a padded head slot beside the rotation of V buffers
-    (vf.KvDtype.F8, 32, 8, 128, 45, 1300, 0, 0.0),    # the same kernel, three query blocks, the last one ragged: the head pairs of a workgroup take mirrored blocks (the middle one both)
-    (vf.KvDtype.F8, 16, 2, 128, 96, 700, 650, 0.0),   # G = 8: four head pairs in two key splits, six query blocks, window that starts after some blocks' first tile
+    (vf.KvDtype.F8, 32, 8, 128, 45, 1300, 0, 0.0),    # the same kernel, three query blocks, the last one ragged (24 workgroups: launched as one head pair x eight key splits)
+    (vf.KvDtype.F8, 16, 2, 128, 96, 700, 650, 0.0),   # G = 8, six query blocks (12 workgroups: one head pair x eight key splits per workgroup), window that starts after some blocks' first tile
     (vf.KvDtype.F8, 8, 4, 128, 130, 37, 0, 20.0),     # G = 2: one head pair (no mirroring), eight key splits dealt 3:2, nine query blocks, soft-cap
     (vf.KvDtype.F8, 32, 8, 128, 256, 0, 0, 0.0),      # from position 0: the first query blocks see fewer tiles than a workgroup has key splits
+    # launches of at least 256 workgroups take the form the 512 x 4 608 benchmark runs: two head pairs x four key splits per
+    # workgroup, mirrored query blocks, wavefronts 4-7 turned by one head pair, tiles dealt 3:2
+    (vf.KvDtype.F8, 128, 32, 128, 125, 300, 0, 0.0),  # G = 4: 8 query blocks x 32 KV heads, ragged last block
+    (vf.KvDtype.F8, 128, 32, 128, 125, 700, 519, 30.0),  # the same with a window that starts inside a tile, and the soft-cap
+    (vf.KvDtype.F8, 128, 16, 128, 250, 100, 0, 0.0),  # G = 8: two such workgroups per (KV head, query block)
+    (vf.KvDtype.F8, 128, 32, 128, 128, 0, 0, 0.0),    # from position 0: query blocks with fewer tiles than key splits
 ]
 
 
@@ -105,6 +111,29 @@ def test_batch_matches_oracle(dtype, heads, hkv, d, m, q_start, kv_start, cap):
     assert np.isfinite(o).all()
     err = np.abs(o - ref).max()
     assert err < TOL[dtype], err
+
+
+@pytest.mark.parametrize("f32_queries", (False, True))
+@pytest.mark.parametrize("f16_weights,fp8_scores", ((False, False), (True, False), (False, True), (True, True)))
+def test_fp8_head_dim_128_two_head_pairs_per_workgroup_every_option(f32_queries, f16_weights, fp8_scores):
+    """The form of the V-through-LDS kernel that a full launch takes (two head pairs x four key splits per workgroup: 256
+    workgroups and more), with general f32 queries (remainder pass of the first product) and with each precision option; K
+    three times as wide as usual so that the reference maximum moves inside two-tile passes; 125 queries, ragged last block."""
+    H, HKV, D, m, q_start = 128, 32, 128, 125, 1100
+    r = rng(977 + int(f32_queries))
+    n_kv = q_start + m
+    q = r.standard_normal((m, H, D)).astype(np.float32) if f32_queries else fp16_normal(r, (m, H, D))
+    k = encode_np(fp16_normal(r, (n_kv, HKV, D), 3.0), vf.KvDtype.F8)
+    v = encode_np(fp16_normal(r, (n_kv, HKV, D)), vf.KvDtype.F8)
+    scale = float(1.0 / np.sqrt(D))
+    o = torch.full((m, H, D), float("nan"), device=DEV)
+    print(f"case f32_queries={f32_queries} f16_weights={f16_weights} fp8_scores={fp8_scores}", flush=True)
+    vf.Forward.run_flash_attn_batch(to_dev(q), to_dev(k.reshape(n_kv, -1)), to_dev(v.reshape(n_kv, -1)), vf.KvDtype.F8, o, H, HKV, D,
+                                    m, q_start, n_kv, scale, f16_weights=f16_weights, fp8_scores=fp8_scores)
+    torch.cuda.synchronize()
+    ref = oracle.attn_batch_ref(q, k, v, int(vf.KvDtype.F8), m, n_kv, H, HKV, D, q_start, scale)
+    err = np.abs(to_np(o) - ref).max()
+    assert err < (2e-4 if not (f16_weights or fp8_scores) else 6e-3), err
 
 
 @pytest.mark.parametrize("f32_queries", (False, True))

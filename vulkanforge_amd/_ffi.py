@@ -58,10 +58,12 @@ _u32p = C.POINTER(C.c_uint32)
 SIGNATURES = {
     "vfkv_status_string": (C.c_char_p, [C.c_int]),
     "vfkv_last_error": (C.c_char_p, []),
+    "vfkv_last_note": (C.c_char_p, []),
     "vfkv_abi_version": (_u32, []),
     "vfkv_device_count": (C.c_int, []),
     "vfkv_cache_create": (C.c_int, [C.POINTER(CacheConfig), C.POINTER(_vp)]),
     "vfkv_cache_create_external": (C.c_int, [C.POINTER(CacheConfig), _vp, _vp, C.POINTER(_vp)]),
+    "vfkv_cache_kv_alignment_note": (C.c_char_p, [_vp]),
     "vfkv_cache_destroy": (None, [_vp]),
     "vfkv_cache_zero_fill": (C.c_int, [_vp, _vp]),
     "vfkv_cache_zero_layer": (C.c_int, [_vp, _u32, _vp]),

@@ -18,6 +18,13 @@
 namespace {
 
 thread_local char g_err[512] = "";
+// Advisory of the last attention call on this thread (vfkv_last_note): never an error, never touches g_err.
+thread_local char g_note[256] = "";
+
+void note_generic(const char* who, uint32_t dtype, uint32_t head_dim) {
+    snprintf(g_note, sizeof(g_note), "%s: this shape (kv dtype %u, head_dim %u, or unaligned pointers / a layer slab of 2 GiB or more) "
+             "ran on the generic fallback kernel, 50-100x slower than the tiled kernels", who, dtype, head_dim);
+}
 
 int fail(int status, const char* fmt, ...) {
     va_list ap;
@@ -189,14 +196,19 @@ int vfkv_cache_create_external(const vfkv_cache_config* cfg, void* k_buffer, voi
     c->v_alloc = nullptr;
     c->owns = false;
     *out = c;
-    g_err[0] = '\0';
-    // Not an error, but worth telling the caller once: K and V buffers whose addresses agree in bits 7-8 cost the
-    // attention kernels up to 8 % (see vfkv_cache_create).  The note is readable through vfkv_last_error().
-    if (k_buffer && v_buffer && ((((uintptr_t)k_buffer) ^ ((uintptr_t)v_buffer)) & 0x180u) == 0u)
-        snprintf(g_err, sizeof(g_err), "note: k_buffer and v_buffer have the same alignment modulo 512 bytes; "
-                 "offsetting v_buffer by 256 bytes inside its allocation makes decode attention up to 8 %% faster");
     return VFKV_OK;
 }
+
+// Not an error, but worth telling the caller: K and V buffers whose addresses agree in bits 7-8 cost the attention
+// kernels up to 8 % (see vfkv_cache_create).
+const char* vfkv_cache_kv_alignment_note(const vfkv_cache* c) {
+    if (c && c->k && c->v && ((((uintptr_t)c->k) ^ ((uintptr_t)c->v)) & 0x180u) == 0u)
+        return "k_buffer and v_buffer have the same alignment modulo 512 bytes; offsetting v_buffer by 256 bytes inside its "
+               "allocation makes decode attention up to 8 % faster";
+    return "";
+}
+
+const char* vfkv_last_note(void) { return g_note; }
 
 int vfkv_cache_create(const vfkv_cache_config* cfg, vfkv_cache** out) {
     if (!out) return fail(VFKV_ERR_INVALID_ARG, "out is NULL");
@@ -488,7 +500,10 @@ static int flash_attn_split_impl(const float* q, const void* k_layer, const void
     L.dtype = kv_dtype; L.n_heads = p->n_heads; L.n_kv_heads = p->n_kv_heads; L.head_dim = p->head_dim;
     L.seq_len = p->seq_len; L.kv_start = p->kv_start; L.tile = tile; L.tile_first = 0; L.n_tiles = p->n_tiles;
     L.scale = p->scale; L.softcap = softcap; L.interleave = interleave;
-    VFKV_HIP(vfkv::launch_split(L, S(stream)));
+    bool generic = false;
+    g_note[0] = '\0';
+    VFKV_HIP(vfkv::launch_split(L, S(stream), &generic));
+    if (generic) note_generic("flash_attn_split", kv_dtype, p->head_dim);
     return VFKV_OK;
 }
 
@@ -569,7 +584,19 @@ void vfkv_workspace_destroy(vfkv_workspace* w) {
     delete w;
 }
 
-// Tile length for the convenience path: enough workgroups to cover the 256 CUs about twice, tiles a
+// Compute units of the current device, asked once (256 on MI355X; the same figure when no device answers, so that the
+// layout-only helpers keep working on a host without a GPU).
+static uint32_t device_cus() {
+    static const uint32_t n = [] {
+        int dev = 0, cus = 0;
+        if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
+            return 256u;
+        return (uint32_t)cus;
+    }();
+    return n;
+}
+
+// Tile length for the convenience path: enough workgroups to cover the CUs once (matrix-core worker) or twice, tiles a
 // multiple of 64 keys (so they never exceed the workspace's ceil(max_seq / 64) rows).
 static uint32_t choose_tile(uint32_t span, uint32_t n_kv_heads, uint32_t groups, uint32_t target_wgs) {
     static const uint32_t forced = [] {
@@ -599,10 +626,10 @@ uint32_t vfkv_decode_tile_for(uint32_t span, uint32_t n_heads, uint32_t n_kv_hea
         // 22.7 us in one tile against 13.6 us in four).
         static const bool forced = getenv("VFKV_DECODE_TILE") != nullptr;
         if (span <= (head_dim == 512u ? 64u : 256u) && !forced) return 256u;
-        return choose_tile(span, n_kv_heads, (g + 7u) / 8u, 256u);
+        return choose_tile(span, n_kv_heads, (g + 7u) / 8u, device_cus());
     }
     const uint32_t groups = (g % 4u == 0u) ? g / 4u : (g % 2u == 0u) ? g / 2u : g;
-    return choose_tile(span, n_kv_heads, groups, 512u);
+    return choose_tile(span, n_kv_heads, groups, 2u * device_cus());
 }
 
 static int decode_attention_impl(vfkv_cache* c, uint32_t layer, uint32_t kv_layer, uint32_t n_heads, const float* q, float* o,
@@ -666,13 +693,16 @@ static int decode_attention_impl(vfkv_cache* c, uint32_t layer, uint32_t kv_laye
             if (rc != VFKV_OK) return rc;
         }
     }
+    bool generic = false;
+    g_note[0] = '\0';
     if (vfkv::split_writes_output(L) && ((uintptr_t)o & 15u) == 0u) {   // one tile sees every key: the worker normalises and writes o itself
         L.o_direct = o;
         VFKV_HIP(vfkv::launch_split(L, S(stream)));
         if (gate) VFKV_HIP(vfkv::launch_sigmoid_mul(o, n_heads * hd, *gate, S(stream)));
         return VFKV_OK;
     }
-    VFKV_HIP(vfkv::launch_split(L, S(stream)));
+    VFKV_HIP(vfkv::launch_split(L, S(stream), &generic));
+    if (generic) note_generic(who, c->dtype, hd);
     bool gate_applied = false;
     VFKV_HIP(vfkv::launch_reduce(ws->scratch_out, ws->scratch_max, ws->scratch_sum, o, n_heads, hd, n_tiles, S(stream), gate,
                                  &gate_applied));
@@ -738,7 +768,10 @@ static int flash_attn_batch_impl(const float* q, const void* k_layer, const void
         L.scratch_ml_floats = (uint64_t)ws->n_heads * ws->max_tiles;
         L.scratch_out_floats = L.scratch_ml_floats * ws->head_dim;
     }
-    VFKV_HIP(vfkv::launch_batch(L, S(stream)));
+    bool generic = false;
+    g_note[0] = '\0';
+    VFKV_HIP(vfkv::launch_batch(L, S(stream), &generic));
+    if (generic) note_generic("flash_attn_batch", kv_dtype, p->head_dim);
     return VFKV_OK;
 }
 

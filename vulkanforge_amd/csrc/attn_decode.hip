@@ -737,7 +737,8 @@ bool split_writes_output(const SplitLaunch& L) {
     return aligned && slab_bytes < 0x7FFF0000ull && mfma_worker_enabled() && mfma_shape;
 }
 
-hipError_t launch_split(const SplitLaunch& L, hipStream_t stream) {
+hipError_t launch_split(const SplitLaunch& L, hipStream_t stream, bool* generic_used) {
+    if (generic_used) *generic_used = false;
     if (L.dtype > kF8 || L.head_dim == 0u || L.head_dim > 512u) return hipErrorInvalidValue;
     if (L.n_tiles == 0u) return hipSuccess;
     SplitArgs a;
@@ -784,6 +785,7 @@ hipError_t launch_split(const SplitLaunch& L, hipStream_t stream) {
         VFKV_CASE(kF32, 64) VFKV_CASE(kF32, 128) VFKV_CASE(kF32, 256)
 #undef VFKV_CASE
     }
+    if (generic_used) *generic_used = true;
     dim3 grid(L.n_tiles, L.n_heads, 1);
     hipLaunchKernelGGL(split_generic_kernel, grid, dim3(kWave), 0, stream, a, L.dtype, L.head_dim);
     return hipGetLastError();

@@ -108,7 +108,7 @@ __global__ __launch_bounds__(kWave) void batch_generic_kernel(BatchArgs a) {
 }
 
 // Launches the attention kernel(s) for L.  *gate_applied tells whether L.gate went into their stores.
-static hipError_t launch_batch_kernels(const BatchLaunch& L, hipStream_t stream, bool* gate_applied) {
+static hipError_t launch_batch_kernels(const BatchLaunch& L, hipStream_t stream, bool* gate_applied, bool* generic_used) {
     *gate_applied = false;
     BatchArgs a;
     a.q = L.q; a.k = (const uint8_t*)L.k; a.v = (const uint8_t*)L.v; a.o = L.o;
@@ -297,17 +297,19 @@ static hipError_t launch_batch_kernels(const BatchLaunch& L, hipStream_t stream,
         VFKV_PF32(kF16, 96, 1) VFKV_PF32(kF8, 96, 1) VFKV_PF32(kF32, 512, 2)
 #undef VFKV_PF32
     }
+    if (generic_used) *generic_used = true;
     hipLaunchKernelGGL(batch_generic_kernel, dim3(L.n_heads, L.m), dim3(kWave), 0, stream, a);
     return hipGetLastError();
 }
 
-hipError_t launch_batch(const BatchLaunch& L, hipStream_t stream) {
+hipError_t launch_batch(const BatchLaunch& L, hipStream_t stream, bool* generic_used) {
+    if (generic_used) *generic_used = false;
     if (L.dtype > kF8 || L.head_dim == 0u || L.head_dim > 512u) return hipErrorInvalidValue;
     if (L.m == 0u) return hipSuccess;
     const uint64_t ne = (uint64_t)L.m * L.n_heads * L.head_dim;
     if (L.gate != nullptr && (L.gate->gate == nullptr || L.gate->chunk == 0u || ne > 0xFFFFFFFFull)) return hipErrorInvalidValue;
     bool gate_applied = false;
-    hipError_t e = launch_batch_kernels(L, stream, &gate_applied);
+    hipError_t e = launch_batch_kernels(L, stream, &gate_applied, generic_used);
     if (e == hipSuccess && L.gate != nullptr && !gate_applied) e = launch_sigmoid_mul(L.o, (uint32_t)ne, *L.gate, stream);
     return e;
 }

@@ -124,10 +124,10 @@ __global__ __launch_bounds__(512) void batch_dma_kernel(BatchArgs a, int HP, int
     auto v_dma = [&](int buf, uint32_t toff) {
 #pragma unroll
         for (int b = 0; b < 4; ++b)
-            // (m0 is reserved: the compiler sets it itself in front of every instruction of its own that reads it)
+            // (m0 is listed as clobbered, so the compiler sets it again in front of any instruction of its own that reads it)
             asm volatile("s_mov_b32 m0, %0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
                          :: "s"(v8_addr + (uint32_t)(buf * VBUF + b * 1024)), "v"(b < 2 ? vdma_lo : vdma_hi), "s"(vdesc),
-                            "s"(toff + (uint32_t)(b * 8) * row_stride) : "memory");
+                            "s"(toff + (uint32_t)(b * 8) * row_stride) : "memory", "m0");
     };
     auto issue = [&](int slot, uint32_t toff) {
 #pragma unroll

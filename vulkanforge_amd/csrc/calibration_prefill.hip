@@ -10,11 +10,13 @@ extern "C" {
 // One launch of the FP8 head_dim-128 prefill kernel (flash_attn_batch.comp:105-208) with stamps: q [m, n_heads, 128] f32, k / v
 // FP8 layer slabs of n_kv rows, o [m, n_heads, 128] f32, stamps [n_kv_heads * ceil(m / 16)][8][8] uint64 (device, zeroed by the
 // caller; entry i of wavefront w of workgroup (x = KV head, y): 100 MHz wall clock at point i, 0 where a wavefront left before it).
-// n_heads / n_kv_heads must be 4 (two head pairs per workgroup).  One caller at a time: the stamp buffer reaches the launcher
+// n_heads / n_kv_heads must be 4 (two head pairs per workgroup) and ceil(m / 16) * n_kv_heads at least 256: below that the launcher
+// spreads the head pairs of a KV head over a third grid dimension, which the stamp layout has no room for (-1).  One caller at a time: the stamp buffer reaches the launcher
 // through a file-scope pointer.  0 on success.
 int vfkv_calib_prefill_stamps(const float* q, const void* k, const void* v, float* o, uint32_t n_heads, uint32_t n_kv_heads,
                               uint32_t m, uint32_t n_kv, uint32_t q_start, float scale, int f16_weights, void* stamps, void* stream) {
-    if (!q || !k || !v || !o || !stamps || n_kv_heads == 0 || n_heads != 4u * n_kv_heads || m == 0 || q_start + m > n_kv) return -1;
+    if (!q || !k || !v || !o || !stamps || n_kv_heads == 0 || n_heads != 4u * n_kv_heads || m == 0 || q_start + m > n_kv ||
+        (uint64_t)((m + 15u) / 16u) * n_kv_heads < 256u) return -1;
     vfkv::BatchLaunch L{};
     L.q = q; L.k = k; L.v = v; L.o = o;
     L.dtype = vfkv::kF8; L.n_heads = n_heads; L.n_kv_heads = n_kv_heads; L.head_dim = 128;

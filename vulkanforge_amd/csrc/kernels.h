@@ -61,7 +61,8 @@ struct SplitLaunch {
 };
 // Returns hipErrorInvalidValue when no kernel covers the shape (or when k_new / v_new are given although
 // split_appends() is false: then the caller appends the row with launch_kv_append and leaves them NULL).
-hipError_t launch_split(const SplitLaunch& a, hipStream_t stream);
+// *generic_used (optional) is set when the shape fell to the one-wavefront-per-(head, tile) fallback kernel.
+hipError_t launch_split(const SplitLaunch& a, hipStream_t stream, bool* generic_used = nullptr);
 bool split_appends(const SplitLaunch& a);
 bool split_writes_output(const SplitLaunch& a);
 // Gate of the attention output (vk_shaders/sigmoid_mul.comp:30-53): element i of the output is multiplied by
@@ -110,6 +111,7 @@ struct BatchLaunch {
     // cannot represent): scores off by up to 2^-12 of the sum of their |k q| products
     bool f16_queries = false;
 };
-hipError_t launch_batch(const BatchLaunch& a, hipStream_t stream);
+// *generic_used (optional) is set when the shape fell to the one-wavefront-per-(query, head) fallback kernel.
+hipError_t launch_batch(const BatchLaunch& a, hipStream_t stream, bool* generic_used = nullptr);
 
 }  // namespace vfkv

@@ -26,12 +26,14 @@ use std::os::raw::{c_char, c_int, c_void};
 pub enum VfkvCache {} pub enum VfkvWorkspace {}
 extern "C" {
     pub fn vfkv_last_error() -> *const c_char;
+    pub fn vfkv_last_note() -> *const c_char;
     pub fn vfkv_status_string(status: c_int) -> *const c_char;
     pub fn vfkv_abi_version() -> u32;
     pub fn vfkv_device_count() -> c_int;
     pub fn vfkv_cache_create(cfg: *const VfkvCacheConfig, out: *mut *mut VfkvCache) -> c_int;
     pub fn vfkv_cache_create_external(cfg: *const VfkvCacheConfig, k_buffer: *mut c_void, v_buffer: *mut c_void,
                                       out: *mut *mut VfkvCache) -> c_int;
+    pub fn vfkv_cache_kv_alignment_note(c: *const VfkvCache) -> *const c_char;
     pub fn vfkv_cache_destroy(c: *mut VfkvCache);
     pub fn vfkv_cache_zero_fill(c: *mut VfkvCache, stream: *mut c_void) -> c_int;
     pub fn vfkv_cache_zero_layer(c: *mut VfkvCache, layer: u32, stream: *mut c_void) -> c_int;

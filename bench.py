@@ -148,10 +148,51 @@ V_SKEW = 256
 STEP_SPREAD = {}   # filled by time_steps: percentiles of single event-timed steps, microseconds
 
 
-def time_steps(torch, step, args):
+def time_steps(torch, step, args, rotating=False):
     """W untimed steps, then exactly K timed steps between two device synchronisations.  One step's
     launches are captured once into a HIP graph and replayed, so the host's per-launch cost (Python
-    and ctypes here) does not gate a step that is only a few hundred microseconds of GPU work."""
+    and ctypes here) does not gate a step that is only a few hundred microseconds of GPU work.
+    rotating: steps of a handful of launches (fewer than 8 layers).  Replaying a graph of one or two kernels measures
+    the graph launch, not the kernels, so all K steps are captured into ONE graph -- step(i) works on cache instance
+    i % 4, so that no step finds its rows in a cache -- and the timed region is one replay of it (the warm-up is another
+    replay: K >= W steps)."""
+    if rotating and not args.no_graph:
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            step(0)
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            for i in range(args.steps):
+                step(i)
+        graph.replay()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        graph.replay()
+        torch.cuda.synchronize()
+        mean = (time.perf_counter() - t0) / args.steps
+        stream = torch.cuda.current_stream()
+        pairs = []
+        for _ in range(20):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record(stream)
+            graph.replay()
+            e1.record(stream)
+            pairs.append((e0, e1))
+        torch.cuda.synchronize()
+        us = sorted(e0.elapsed_time(e1) * 1e3 / args.steps for e0, e1 in pairs)
+        STEP_SPREAD.clear()
+        STEP_SPREAD.update({"p10": us[2], "p50": us[10], "p90": us[18], "samples": 20,
+                            "note": f"per step of {args.steps}-step graph replays"})
+        return mean
+    if rotating:
+        step0 = step
+        counter = [0]
+        def step():
+            step0(counter[0])
+            counter[0] += 1
     run = step
     if not args.no_graph:
         side = torch.cuda.Stream()
@@ -200,14 +241,21 @@ def bench_decode(args, wl):
     L, H, Hkv, D = wl.n_layers, wl.n_heads, wl.n_kv_heads, wl.head_dim
     max_seq = wl.context
     es = wl.dtype.element_size()
-    nbytes = L * max_seq * Hkv * D * es
+    # A model of fewer than 8 layers is a step of a handful of launches: it is timed as K steps inside one graph, each on
+    # one of four cache instances in rotation (instance r = layers [r L, (r + 1) L) of one larger cache)
+    rotating = L < 8
+    inst = 4 if rotating else 1
+    nbytes = L * inst * max_seq * Hkv * D * es
     kbuf = torch.empty(nbytes, dtype=torch.uint8, device=dev)
     vbuf = torch.empty(nbytes + V_SKEW, dtype=torch.uint8, device=dev)[V_SKEW:]
-    cache = vf.KvCache(vf.KvCacheConfig(L, Hkv, D, max_seq, dtype=wl.dtype), k_buffer=kbuf.data_ptr(),
+    cache = vf.KvCache(vf.KvCacheConfig(L * inst, Hkv, D, max_seq, dtype=wl.dtype), k_buffer=kbuf.data_ptr(),
                        v_buffer=vbuf.data_ptr())
     fwd = vf.Forward(cache, H)
     outliers = wl.name == "decode_fp8_8k_32layers"
-    fill_cache(torch, vf, fwd, wl, max_seq, args.seed, outliers)
+
+    class _AllInstances:
+        n_layers = L * inst
+    fill_cache(torch, vf, fwd, _AllInstances, max_seq, args.seed, outliers)
 
     g = torch.Generator(device="cuda").manual_seed(args.seed + 1)
     q = torch.randn((L, H, D), device=dev, generator=g)
@@ -227,21 +275,22 @@ def bench_decode(args, wl):
             fwd.run_scalar_attn(layer, pos, q[layer], o[layer], kv_start=starts[layer], scale=scale, softcap=wl.softcap)
             fwd.run_sigmoid_mul(gate[layer], o[layer], H * D, H * D, H * D, 0)
 
-    def step():
+    def step(i=0):
+        base = (i % inst) * L       # first layer of the cache instance this step works on
         for layer in range(L):
             if wl.gated:        # step_attention + step_attn_gated_output: the merge applies the gate
-                fwd.step_attention_gated(layer, pos, q[layer], o[layer], gate[layer], H * D, H * D, 0,
+                fwd.step_attention_gated(base + layer, pos, q[layer], o[layer], gate[layer], H * D, H * D, 0,
                                          k_src=k_new[layer] if wl.append else None, v_src=v_new[layer] if wl.append else None,
                                          kv_start=starts[layer], scale=scale, softcap=wl.softcap)
             elif wl.append:     # step_kv_write + step_attention of the new token, issued as one call
-                fwd.step_kv_write_attention(layer, pos, q[layer], k_new[layer], v_new[layer], o[layer],
+                fwd.step_kv_write_attention(base + layer, pos, q[layer], k_new[layer], v_new[layer], o[layer],
                                             kv_start=starts[layer], scale=scale, softcap=wl.softcap)
             else:
-                fwd.run_scalar_attn(layer, pos, q[layer], o[layer], kv_start=starts[layer], scale=scale,
+                fwd.run_scalar_attn(base + layer, pos, q[layer], o[layer], kv_start=starts[layer], scale=scale,
                                     softcap=wl.softcap)
 
     gate_separate_us = time_steps(torch, step_gate_separate, args) * 1e6 if wl.gated and not wl.append else None
-    sec_per_step = time_steps(torch, step, args)
+    sec_per_step = time_steps(torch, step, args, rotating=rotating)
     step_spread = dict(STEP_SPREAD)
     bytes_step = wl.kv_bytes_step()
 
@@ -255,17 +304,23 @@ def bench_decode(args, wl):
     sm = torch.empty((H * max_tiles,), device=dev)
     ss = torch.empty((H * max_tiles,), device=dev)
 
+    # (fewer than 8 layers: the launches of at least 32 steps over the rotating cache instances, so that the pair of events
+    # brackets kernels and not one graph launch)
+    split_reps = (32 + L - 1) // L if rotating else 1
+
     def split_only():
-        for layer in range(L):
-            span = wl.context - starts[layer]
-            tile = lib.vfkv_decode_tile_for(span, H, Hkv, D, int(wl.dtype))
-            # the step's own launch starts at the tile that holds kv_start; the standalone split call numbers its tiles
-            # from row 0 (flash_attn_split.comp), so a windowed layer is handed the slab from that tile on
-            skip = starts[layer] // tile * tile
-            klay = cache.k_ptr + cache.layer_offset_bytes(layer) + skip * cache.row_bytes(layer)
-            vlay = cache.v_ptr + cache.layer_offset_bytes(layer) + skip * cache.row_bytes(layer)
-            fwd.run_flash_attn_split(q[layer], klay, vlay, wl.dtype, so, sm, ss, H, Hkv, D, wl.context - skip, scale,
-                                     kv_start=starts[layer] - skip, tile=tile, softcap=wl.softcap, interleaved=True)
+        for rep in range(split_reps):
+            for layer in range(L):
+                span = wl.context - starts[layer]
+                tile = lib.vfkv_decode_tile_for(span, H, Hkv, D, int(wl.dtype))
+                # the step's own launch starts at the tile that holds kv_start; the standalone split call numbers its tiles
+                # from row 0 (flash_attn_split.comp), so a windowed layer is handed the slab from that tile on
+                skip = starts[layer] // tile * tile
+                phys = (rep % inst) * L + layer
+                klay = cache.k_ptr + cache.layer_offset_bytes(phys) + skip * cache.row_bytes(phys)
+                vlay = cache.v_ptr + cache.layer_offset_bytes(phys) + skip * cache.row_bytes(phys)
+                fwd.run_flash_attn_split(q[layer], klay, vlay, wl.dtype, so, sm, ss, H, Hkv, D, wl.context - skip, scale,
+                                         kv_start=starts[layer] - skip, tile=tile, softcap=wl.softcap, interleaved=True)
 
     def event_timed(fn, reps):
         """Total milliseconds of `reps` replays of fn's launches (captured once into a graph) between two events."""
@@ -291,7 +346,7 @@ def bench_decode(args, wl):
 
     n_ev = min(max(args.steps, 5), 20)
     split_ms = event_timed(split_only, n_ev)
-    launches = n_ev * L
+    launches = n_ev * L * split_reps
     bytes_launch = bytes_step / L          # mean over the layers of the step
     avg_ms = split_ms / launches
     achieved = bytes_launch / (avg_ms * 1e-3) / 1e9
@@ -324,9 +379,9 @@ def bench_decode(args, wl):
                     assert rc == 0, rc
             return run
 
-        stream_us = event_timed(per_layer(lambda kp, vp, st: calib.vfkv_calib_stream_read(kp, vp, layer_bytes // 16 * 16, sink.data_ptr(), st)), n_ev) * 1e3 / launches
-        pattern_us = event_timed(per_layer(lambda kp, vp, st: calib.vfkv_calib_pattern_read(kp, vp, wl.context, Hkv, n_tiles, sink.data_ptr(), st)), n_ev) * 1e3 / launches
-        empty_us = event_timed(per_layer(lambda kp, vp, st: calib.vfkv_calib_empty(Hkv, n_tiles, sink.data_ptr(), st)), n_ev) * 1e3 / launches
+        stream_us = event_timed(per_layer(lambda kp, vp, st: calib.vfkv_calib_stream_read(kp, vp, layer_bytes // 16 * 16, sink.data_ptr(), st)), n_ev) * 1e3 / (n_ev * L)
+        pattern_us = event_timed(per_layer(lambda kp, vp, st: calib.vfkv_calib_pattern_read(kp, vp, wl.context, Hkv, n_tiles, sink.data_ptr(), st)), n_ev) * 1e3 / (n_ev * L)
+        empty_us = event_timed(per_layer(lambda kp, vp, st: calib.vfkv_calib_empty(Hkv, n_tiles, sink.data_ptr(), st)), n_ev) * 1e3 / (n_ev * L)
         floors = {"stream_floor_us": stream_us, "pattern_floor_us": pattern_us, "empty_launch_us": empty_us}
 
     mfma_worker = mfma_decode_worker(wl.dtype.label(), D)

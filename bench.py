@@ -385,7 +385,8 @@ def bench_decode(args, wl):
         floors = {"stream_floor_us": stream_us, "pattern_floor_us": pattern_us, "empty_launch_us": empty_us}
 
     mfma_worker = mfma_decode_worker(wl.dtype.label(), D)
-    worker_name = "split_mfma_kernel" if mfma_worker else "split_kernel"
+    f32_mfma = wl.dtype.label() == "FP32" and D in (64, 128, 256) and os.environ.get("VFKV_DECODE_WORKER", "m")[:1] != "v"
+    worker_name = "split_mfma_kernel" if mfma_worker else "split_mfma_f32_kernel" if f32_mfma else "split_kernel"
     traffic, traffic_source = profiled_traffic(wl.name) if mfma_worker else (None, None)   # the profiles cover the default worker
     result = {
         "metric": "kv_read_GBps_decode_step",
@@ -400,7 +401,7 @@ def bench_decode(args, wl):
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": MFMA_DTYPE if mfma_worker else "f32",
+        "dtype": MFMA_DTYPE if mfma_worker else "f32 mfma, f32 accumulate" if f32_mfma else "f32",
         "kv_dtype": wl.dtype.label(),
         "launch": "eager" if args.no_graph else "hip_graph",
         "data": "synthetic, seeded N(0,1); queries " + ("general f32" if args.f32_queries else "cast to fp16 as the configuration states") + "; K/V rows cast to fp16 and written through the append kernels",
@@ -850,7 +851,7 @@ def decode_phase_stamps(args):
     import torch
     import vulkanforge_amd as vf
     calib = C.CDLL(os.path.join(ROOT, "vulkanforge_amd", "libvfkv_calib.so"))
-    calib.vfkv_calib_decode_stamps.argtypes = [C.c_void_p] * 6 + [C.c_uint32] * 7 + [C.c_float, C.c_void_p, C.c_void_p]
+    calib.vfkv_calib_decode_stamps.argtypes = [C.c_void_p] * 6 + [C.c_uint32] * 7 + [C.c_float, C.c_void_p, C.c_void_p, C.c_void_p, C.c_uint32, C.c_int]
     H, Hkv, D, NL, NW = 32, 8, 128, 8, 4
     out = {"metric": "decode_phase_stamps", "unit": "us after the launch's first wavefront started", "n_gpus": 1,
            "config": {"workload": "split_mfma_kernel, 32 / 8 / 128 FP8, instrumented kernel, 8 launches per graph replay"}, "contexts": {}}
@@ -858,10 +859,20 @@ def decode_phase_stamps(args):
     # (seq_len, byte offset of the V slabs from a 2 MiB boundary; the K slabs start on one).  256 is what vfkv_cache_create gives V:
     # with K and V rows at the same offsets one KV head's stream runs 10 % slower than the others and the launch waits for it
     # (the head whose 128-byte pieces lie at addresses with bits 9:7 == 011, on whichever XCD it runs)
-    cases = [(32768, 256), (8192, 256), (32768, 0)] + [(32768, int(x)) for x in args.v_offsets.split(",") if x.strip()]
+    cases = [(32768, 256), (8192, 256), (8193, 256), (32768, 0)] + [(32768, int(x)) for x in args.v_offsets.split(",") if x.strip()]
+    # the counter-dealt worker, with the library's own environment switches and its choice of static rounds
+    dyn_rounds = int(os.environ.get("VFKV_DECODE_DYN_ROUNDS", "2"))
+    dyn_half = int(os.environ.get("VFKV_DECODE_DYN_HALF", "0") != "0")
+    out["config"]["dyn_rounds"], out["config"]["dyn_half_units"] = dyn_rounds, dyn_half
+    tickets = torch.zeros(4096, dtype=torch.int32, device="cuda")
     for seq, shift in cases:
         tile = vf.lib().vfkv_decode_tile_for(seq, H, Hkv, D, int(vf.KvDtype.F8))
         nt = (seq + tile - 1) // tile
+        static_rounds = 0
+        if dyn_rounds:
+            tile, nt = 64, 32
+            rounds = -(-((seq + 31) // 32) // (4 * nt))
+            static_rounds = max(rounds - dyn_rounds, 1)
         slab = seq * Hkv * D
         pool = [torch.randn(((NL * slab + (1 << 21)) // 4,), device="cuda", generator=g).to(torch.float8_e4m3fn).view(torch.uint8).repeat(4)
                 for _ in range(2)]
@@ -877,7 +888,8 @@ def decode_phase_stamps(args):
             for l in range(NL):
                 rc = calib.vfkv_calib_decode_stamps(q.data_ptr(), ks[l].data_ptr(), vs[l].data_ptr(), so.data_ptr(), sm.data_ptr(),
                                                     ss.data_ptr(), int(vf.KvDtype.F8), H, Hkv, D, seq, tile, nt, 1.0 / D ** 0.5,
-                                                    st[l].data_ptr(), stream)
+                                                    st[l].data_ptr(), stream, tickets.data_ptr() if dyn_rounds else None,
+                                                    static_rounds, dyn_half)
                 assert rc == 0, rc
         launches()
         torch.cuda.synchronize()

@@ -628,6 +628,13 @@ uint32_t vfkv_decode_tile_for(uint32_t span, uint32_t n_heads, uint32_t n_kv_hea
         if (span <= (head_dim == 512u ? 64u : 256u) && !forced) return 256u;
         return choose_tile(span, n_kv_heads, (g + 7u) / 8u, device_cus());
     }
+    // F32 caches on the f32 matrix instruction: one workgroup per CU as well, up to 16 heads of a group per workgroup
+    static const bool valu_forced = [] { const char* e = getenv("VFKV_DECODE_WORKER"); return e && e[0] == 'v'; }();
+    if (kv_dtype == VFKV_F32 && !valu_forced && (head_dim == 64u || head_dim == 128u || head_dim == 256u)) {
+        static const bool forced = getenv("VFKV_DECODE_TILE") != nullptr;
+        if (span <= 256u && !forced) return 256u;
+        return choose_tile(span, n_kv_heads, (g + 15u) / 16u, device_cus());
+    }
     const uint32_t groups = (g % 4u == 0u) ? g / 4u : (g % 2u == 0u) ? g / 2u : g;
     return choose_tile(span, n_kv_heads, groups, 2u * device_cus());
 }
@@ -654,9 +661,31 @@ static int decode_attention_impl(vfkv_cache* c, uint32_t layer, uint32_t kv_laye
     if (ws && (n_heads > ws->n_heads || hd > ws->head_dim))
         return fail(VFKV_ERR_WORKSPACE, "%s: workspace built for %u heads x %u dims, need %u x %u", who,
                     ws->n_heads, ws->head_dim, n_heads, hd);
-    const uint32_t tile = vfkv_decode_tile_for(seq_len - kv_start, n_heads, kvh, hd, c->dtype);
-    const uint32_t first = kv_start / tile;
-    const uint32_t n_tiles = (seq_len + tile - 1u) / tile - first;
+    uint32_t tile = vfkv_decode_tile_for(seq_len - kv_start, n_heads, kvh, hd, c->dtype);
+    uint32_t first = kv_start / tile;
+    uint32_t n_tiles = (seq_len + tile - 1u) / tile - first;
+    // Late rebalancing (attn_decode_dyn.h): launches of several workgroups per KV head on the matrix-core worker deal the
+    // last runs of the span statically and hand the front out through counters.  The workgroup count is then chosen directly
+    // (one per CU), independent of a tile length: the launch covers the rows from the 64-row boundary at or below kv_start.
+    static const uint32_t dyn_rounds = [] { const char* e = getenv("VFKV_DECODE_DYN_ROUNDS"); return e ? (uint32_t)strtoul(e, nullptr, 10) : 2u; }();
+    static const bool dyn_half = [] { const char* e = getenv("VFKV_DECODE_DYN_HALF"); return e ? e[0] != '0' : false; }();
+    uint32_t static_rounds = 0u;
+    const uint32_t run_rows = vfkv::split_run_rows(c->dtype, hd);
+    const uint32_t nz = (n_heads / kvh + 7u) / 8u;
+    if (dyn_rounds != 0u && n_tiles > 1u && run_rows != 0u && (hd == 128u || hd == 256u)) {
+        const uint32_t base_row = kv_start / 64u * 64u;
+        const uint32_t nv = (seq_len - base_row + run_rows - 1u) / run_rows;
+        uint32_t wgs = device_cus() / (kvh * nz);
+        if (wgs < 1u) wgs = 1u;
+        if (wgs > (nv + 3u) / 4u) wgs = (nv + 3u) / 4u;              // four run streams per workgroup: no workgroup without a run
+        const uint32_t cap_tiles = static_ws ? 0xFFFFFFFFu : ws->max_tiles;
+        if (wgs > cap_tiles) wgs = cap_tiles;
+        if (wgs >= 2u) {
+            const uint32_t rounds = (nv + 4u * wgs - 1u) / (4u * wgs);
+            static_rounds = rounds > dyn_rounds ? rounds - dyn_rounds : 1u;
+            tile = 64u; first = kv_start / 64u; n_tiles = wgs;
+        }
+    }
     vfkv_workspace fixed;
     if (static_ws) {
         // the partials of this launch laid out in the static array: [out | max | sum], each part 256-byte aligned
@@ -685,6 +714,7 @@ static int decode_attention_impl(vfkv_cache* c, uint32_t layer, uint32_t kv_laye
     L.scale = scale; L.softcap = softcap;
     // the partials stay inside the workspace, so they need not correspond to tiles
     L.interleave = true;
+    if (static_rounds != 0u) { L.static_rounds = static_rounds; L.half_units = dyn_half; }
     if (k_new) {
         L.k_new = k_new; L.v_new = v_new; L.append_pos = position;
         if (!vfkv::split_appends(L)) {          // this shape's worker cannot write the row itself: append in its own launch

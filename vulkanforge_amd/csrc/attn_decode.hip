@@ -48,6 +48,7 @@ struct SplitArgs {
     uint32_t group;          // n_heads / n_kv_heads
     uint32_t interleave;     // matrix-core worker: deal the runs of the launched span round-robin instead of by tile
     float scale, softcap;
+    uint32_t static_rounds;  // attn_decode_dyn.h: runs per run stream dealt from the end of the span (0: the other workers)
 #ifdef VFKV_DECODE_STAMPS
     unsigned long long* stamps;   // instrumented build (calibration_decode.hip): [KV head][workgroup of the head][head slice][wavefront][4] wall-clock readings
 #endif
@@ -655,6 +656,8 @@ __global__ __launch_bounds__(kWave) void reduce_generic_kernel(const float* __re
 
 }  // namespace vfkv
 #include "attn_decode_mfma.h"
+#include "attn_decode_dyn.h"
+#include "attn_decode_f32.h"
 namespace vfkv {
 
 // ---- dispatch -----------------------------------------------------------------------------------
@@ -675,6 +678,38 @@ static hipError_t launch_split_mfma(const SplitArgs& a, uint32_t g, hipStream_t 
     else
         hipLaunchKernelGGL((split_mfma_kernel<DT, D, RUN, PF, NW, false, NH>), grid, dim3(NW * kWave), 0, stream, a, gt);
     return hipGetLastError();
+}
+
+template <int DT, int D, int RUN>
+static hipError_t launch_split_dyn(const SplitArgs& a, uint32_t g, bool half_units, hipStream_t stream) {
+    constexpr int NW = kMfmaWaves;
+    const uint32_t gt = g < 8u ? g : 8u;
+    dim3 grid(a.n_kv_heads, a.n_tiles, (g + gt - 1u) / gt);
+#define VFKV_DYN(CAPV, HUV) hipLaunchKernelGGL((split_mfma_dyn_kernel<DT, D, RUN, NW, CAPV, HUV>), grid, dim3(NW * kWave), 0, stream, a, gt)
+    if (a.softcap > 0.f) { if (half_units) VFKV_DYN(true, true); else VFKV_DYN(true, false); }
+    else { if (half_units) VFKV_DYN(false, true); else VFKV_DYN(false, false); }
+#undef VFKV_DYN
+    return hipGetLastError();
+}
+
+uint32_t split_run_rows(uint32_t dtype, uint32_t D) {
+    if ((dtype != kF8 && dtype != kF16) || (D != 64u && D != 128u && D != 256u && D != 512u)) return 0u;
+    return D == 64u ? 64u : 32u;
+}
+
+template <int D>
+static hipError_t launch_split_f32(const SplitArgs& a, uint32_t g, hipStream_t stream) {
+    constexpr int NW = kMfmaWaves;
+    const uint32_t gt = g < 16u ? g : 16u;          // up to 16 heads of a group share a workgroup's K / V stream
+    dim3 grid(a.n_kv_heads, a.n_tiles, (g + gt - 1u) / gt);
+    if (a.softcap > 0.f) hipLaunchKernelGGL((split_mfma_f32_kernel<D, NW, true>), grid, dim3(NW * kWave), 0, stream, a, gt);
+    else hipLaunchKernelGGL((split_mfma_f32_kernel<D, NW, false>), grid, dim3(NW * kWave), 0, stream, a, gt);
+    return hipGetLastError();
+}
+
+// F32 caches on the f32 matrix instruction (attn_decode_f32.h)
+static bool f32_mfma_shape(uint32_t dtype, uint32_t D) {
+    return dtype == kF32 && (D == 64u || D == 128u || D == 256u);
 }
 
 // Shapes the matrix-core worker is built for (head_dim 512: two wavefronts per run, each half of the output columns).
@@ -733,8 +768,16 @@ bool split_writes_output(const SplitLaunch& L) {
     if (L.n_tiles != 1u || L.n_kv_heads == 0u) return false;
     const bool aligned = ((((uintptr_t)L.k) | ((uintptr_t)L.v) | ((uintptr_t)L.q) | ((uintptr_t)L.scratch_out)) & 15u) == 0u;
     const uint64_t slab_bytes = (uint64_t)L.seq_len * L.n_kv_heads * L.head_dim * elem_size(L.dtype);
-    const bool mfma_shape = mfma_worker_shape(L.dtype, L.head_dim);
+    const bool mfma_shape = mfma_worker_shape(L.dtype, L.head_dim) || f32_mfma_shape(L.dtype, L.head_dim);
     return aligned && slab_bytes < 0x7FFF0000ull && mfma_worker_enabled() && mfma_shape;
+}
+
+bool split_deals_dynamically(const SplitLaunch& L) {
+    if (!L.interleave || L.static_rounds == 0u || L.n_tiles < 2u || L.o_direct || L.n_kv_heads == 0u) return false;
+    const bool aligned = ((((uintptr_t)L.k) | ((uintptr_t)L.v) | ((uintptr_t)L.q) | ((uintptr_t)L.scratch_out)) & 15u) == 0u;
+    const uint64_t slab_bytes = (uint64_t)L.seq_len * L.n_kv_heads * L.head_dim * elem_size(L.dtype);
+    return aligned && slab_bytes < 0x7FFF0000ull && mfma_worker_enabled() && (L.dtype == kF8 || L.dtype == kF16) &&
+           (L.head_dim == 128u || L.head_dim == 256u);
 }
 
 hipError_t launch_split(const SplitLaunch& L, hipStream_t stream, bool* generic_used) {
@@ -750,6 +793,7 @@ hipError_t launch_split(const SplitLaunch& L, hipStream_t stream, bool* generic_
     a.scale = L.scale; a.softcap = L.softcap;
     a.k_new = nullptr; a.v_new = nullptr; a.append_pos = 0u; a.o_direct = nullptr;
     a.interleave = L.interleave ? 1u : 0u;
+    a.static_rounds = 0u;
 #ifdef VFKV_DECODE_STAMPS
     a.stamps = g_decode_stamps;
 #endif
@@ -767,6 +811,13 @@ hipError_t launch_split(const SplitLaunch& L, hipStream_t stream, bool* generic_
     }
     // the matrix-core worker also stores its partials (or the output) 16 bytes at a time
     const bool out_aligned = ((((uintptr_t)L.scratch_out) | ((uintptr_t)L.o_direct)) & 15u) == 0u;
+    if (split_deals_dynamically(L) && out_aligned) {
+        a.static_rounds = L.static_rounds;
+        if (L.dtype == kF8 && L.head_dim == 128u) return launch_split_dyn<kF8, 128, 32>(a, g, L.half_units, stream);
+        if (L.dtype == kF16 && L.head_dim == 128u) return launch_split_dyn<kF16, 128, 32>(a, g, L.half_units, stream);
+        if (L.dtype == kF8 && L.head_dim == 256u) return launch_split_dyn<kF8, 256, 32>(a, g, L.half_units, stream);
+        if (L.dtype == kF16 && L.head_dim == 256u) return launch_split_dyn<kF16, 256, 32>(a, g, L.half_units, stream);
+    }
     if (aligned && out_aligned && slab_bytes < 0x7FFF0000ull && mfma_worker_enabled()) {
         if (L.dtype == kF8 && L.head_dim == 64u) return launch_split_mfma<kF8, 64, 64, 1>(a, g, stream);
         if (L.dtype == kF8 && L.head_dim == 128u) return launch_split_mfma<kF8, 128, 32, 1>(a, g, stream);
@@ -776,6 +827,11 @@ hipError_t launch_split(const SplitLaunch& L, hipStream_t stream, bool* generic_
         if (L.dtype == kF16 && L.head_dim == 256u) return launch_split_mfma<kF16, 256, 32, 1>(a, g, stream);
         if (L.dtype == kF8 && L.head_dim == 512u) return launch_split_mfma<kF8, 512, 32, 1, 2>(a, g, stream);
         if (L.dtype == kF16 && L.head_dim == 512u) return launch_split_mfma<kF16, 512, 32, 1, 2>(a, g, stream);
+    }
+    if (aligned && out_aligned && slab_bytes < 0x7FFF0000ull && mfma_worker_enabled() && f32_mfma_shape(L.dtype, L.head_dim)) {
+        if (L.head_dim == 64u) return launch_split_f32<64>(a, g, stream);
+        if (L.head_dim == 128u) return launch_split_f32<128>(a, g, stream);
+        return launch_split_f32<256>(a, g, stream);
     }
     if (fast_shape(L.dtype, L.head_dim) && aligned && slab_bytes < 0x7FFF0000ull) {
 #define VFKV_CASE(DT, DD) \

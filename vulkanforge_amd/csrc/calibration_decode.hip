@@ -14,9 +14,10 @@ extern "C" {
 // a file-scope pointer.  0 on success.
 int vfkv_calib_decode_stamps(const float* q, const void* k, const void* v, float* so, float* sm, float* ss, uint32_t kv_dtype,
                              uint32_t n_heads, uint32_t n_kv_heads, uint32_t head_dim, uint32_t seq_len, uint32_t tile,
-                             uint32_t n_tiles, float scale, void* stamps, void* stream) {
+                             uint32_t n_tiles, float scale, void* stamps, void* stream, void* tickets, uint32_t static_rounds,
+                             int half_units) {
     if (!q || !k || !v || !so || !sm || !ss || !stamps || n_kv_heads == 0 || n_heads % n_kv_heads != 0 || seq_len == 0 || tile == 0 ||
-        n_tiles != (seq_len + tile - 1) / tile || (kv_dtype != vfkv::kF16 && kv_dtype != vfkv::kF8) ||
+        (static_rounds == 0 && n_tiles != (seq_len + tile - 1) / tile) || (kv_dtype != vfkv::kF16 && kv_dtype != vfkv::kF8) ||
         (head_dim != 64 && head_dim != 128 && head_dim != 256))
         return -1;
     vfkv::SplitLaunch L;
@@ -26,6 +27,8 @@ int vfkv_calib_decode_stamps(const float* q, const void* k, const void* v, float
     L.seq_len = seq_len; L.kv_start = 0; L.tile = tile; L.tile_first = 0; L.n_tiles = n_tiles;
     L.scale = scale; L.softcap = 0.f;
     L.interleave = true;
+    // static_rounds > 0: the worker of attn_decode_dyn.h (tickets is unused)
+    (void)tickets; L.static_rounds = static_rounds; L.half_units = half_units != 0;
     vfkv::g_decode_stamps = (unsigned long long*)stamps;
     const hipError_t e = vfkv::launch_split(L, (hipStream_t)stream);
     vfkv::g_decode_stamps = nullptr;

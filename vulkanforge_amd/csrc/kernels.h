@@ -58,6 +58,11 @@ struct SplitLaunch {
     // partial j need not be tile j: the matrix-core worker then deals the rows of the launched tiles to its
     // workgroups in interleaved runs (other workers ignore the flag); the merge is the same either way
     bool interleave = false;
+    // interleaved launches of more than one workgroup per KV head on the matrix-core worker: static_rounds > 0 selects the
+    // worker of attn_decode_dyn.h, whose run streams take that many runs each from the END of the span (the ragged last run
+    // and an appended row first) and the rest from the front; half_units halves the units of the front part
+    uint32_t static_rounds = 0;
+    bool half_units = false;
 };
 // Returns hipErrorInvalidValue when no kernel covers the shape (or when k_new / v_new are given although
 // split_appends() is false: then the caller appends the row with launch_kv_append and leaves them NULL).
@@ -78,6 +83,10 @@ hipError_t launch_reduce(const float* scratch_out, const float* scratch_max, con
                          const GateArgs* gate = nullptr, bool* gate_applied = nullptr);
 // ---- gated_output.hip ----
 hipError_t launch_sigmoid_mul(float* data, uint32_t ne, const GateArgs& gate, hipStream_t stream);
+// True when launch_split would run the worker of attn_decode_dyn.h for L (static_rounds given, shape covered).
+bool split_deals_dynamically(const SplitLaunch& a);
+// Rows per run of the matrix-core worker for this shape (0: the shape is not the matrix-core worker's).
+uint32_t split_run_rows(uint32_t dtype, uint32_t head_dim);
 // Smallest tile granule (keys) the split kernel for this shape works in; 0 if unsupported.
 uint32_t split_tile_granule(uint32_t dtype, uint32_t head_dim);
 

@@ -65,11 +65,17 @@ DECODE = {
     "decode_f16_2k_1layer": DecodeWorkload("decode_f16_2k_1layer", 1, 32, 8, 128, 2049, KvDtype.F16, True),
     "decode_fp8_8k_32layers": DecodeWorkload("decode_fp8_8k_32layers", 32, 32, 8, 128, 8193, KvDtype.F8, True),
     "decode_fp8_32k_32layers": DecodeWorkload("decode_fp8_32k_32layers", 32, 32, 8, 128, 32768, KvDtype.F8, False),
+    # configuration 2 without the append (what the append inside the attention launch costs; not a reference configuration)
+    "decode_fp8_8k_32layers_no_append": DecodeWorkload("decode_fp8_8k_32layers_no_append", 32, 32, 8, 128, 8193, KvDtype.F8, False),
+    "decode_fp8_8192_32layers_no_append": DecodeWorkload("decode_fp8_8192_32layers_no_append", 32, 32, 8, 128, 8192, KvDtype.F8, False),
     # the headline geometry over an F16 cache (not one of the reference configurations; used to tune the F16 variant)
     "decode_f16_32k_32layers": DecodeWorkload("decode_f16_32k_32layers", 32, 32, 8, 128, 32768, KvDtype.F16, False),
     # the headline geometry with the gated output of the Qwen3.6 full-attention layers (not a reference configuration)
     "decode_fp8_32k_32layers_gated": DecodeWorkload("decode_fp8_32k_32layers_gated", 32, 32, 8, 128, 32768, KvDtype.F8, False,
                                                     gated=True),
+    # the configuration-2 geometry over an F32 cache (the reference's VULKANFORGE_FP16_KV=0 mode; not a reference configuration):
+    # the same bytes per layer as the headline workload
+    "decode_f32_8k_32layers": DecodeWorkload("decode_f32_8k_32layers", 32, 32, 8, 128, 8193, KvDtype.F32, True),
     "decode_f16_hd256_sliding_12layers": DecodeWorkload("decode_f16_hd256_sliding_12layers", 12, 16, 8, 256, 16384,
                                                         KvDtype.F16, False, softcap=50.0, window=4096,
                                                         sliding_pattern=5),

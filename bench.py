@@ -275,10 +275,26 @@ def bench_decode(args, wl):
             fwd.run_scalar_attn(layer, pos, q[layer], o[layer], kv_start=starts[layer], scale=scale, softcap=wl.softcap)
             fwd.run_sigmoid_mul(gate[layer], o[layer], H * D, H * D, H * D, 0)
 
+    rope_kw = None
+    if wl.rope:
+        import oracle as _o
+        rope_kw = dict(q_norm_weight=(1 + 0.1 * torch.randn(D, device=dev, generator=g)), k_norm_weight=(1 + 0.1 * torch.randn(D, device=dev, generator=g)),
+                       eps=1e-6)
+        theta_scale = float(_o.rope_theta_scale(10000.0, D))
+        q_rot = torch.zeros((L, H, D), device=dev)
+
+    def step_rope_separate():   # QNormRope + KNormRope + KvWrite as one launch, then attention (split + merge)
+        for layer in range(L):
+            fwd.step_qk_rope_kv_write(layer, pos, 1, q[layer], k_new[layer], v_new[layer], D, theta_scale, q_out=q_rot[layer], **rope_kw)
+            fwd.run_scalar_attn(layer, pos, q_rot[layer], o[layer], kv_start=starts[layer], scale=scale, softcap=wl.softcap)
+
     def step(i=0):
         base = (i % inst) * L       # first layer of the cache instance this step works on
         for layer in range(L):
-            if wl.gated:        # step_attention + step_attn_gated_output: the merge applies the gate
+            if wl.rope:         # norm + RoPE of the token's Q and K rows, append and attention in one call
+                fwd.step_qk_rope_kv_write_attention(base + layer, pos, q[layer], k_new[layer], v_new[layer], o[layer], D, theta_scale,
+                                                    kv_start=starts[layer], scale=scale, softcap=wl.softcap, **rope_kw)
+            elif wl.gated:        # step_attention + step_attn_gated_output: the merge applies the gate
                 fwd.step_attention_gated(base + layer, pos, q[layer], o[layer], gate[layer], H * D, H * D, 0,
                                          k_src=k_new[layer] if wl.append else None, v_src=v_new[layer] if wl.append else None,
                                          kv_start=starts[layer], scale=scale, softcap=wl.softcap)
@@ -290,6 +306,7 @@ def bench_decode(args, wl):
                                     softcap=wl.softcap)
 
     gate_separate_us = time_steps(torch, step_gate_separate, args) * 1e6 if wl.gated and not wl.append else None
+    rope_separate_us = time_steps(torch, step_rope_separate, args) * 1e6 if wl.rope else None
     sec_per_step = time_steps(torch, step, args, rotating=rotating)
     step_spread = dict(STEP_SPREAD)
     bytes_step = wl.kv_bytes_step()
@@ -419,6 +436,8 @@ def bench_decode(args, wl):
 
     if gate_separate_us is not None:
         result["config"]["us_per_step_with_separate_gate_launch"] = gate_separate_us
+    if rope_separate_us is not None:
+        result["config"]["us_per_step_with_separate_rope_append_launch"] = rope_separate_us
 
     if not args.no_cpu_baseline:
         import numpy as np
@@ -431,7 +450,7 @@ def bench_decode(args, wl):
             lo = layer * per_layer
             kh = kbuf[lo:lo + per_layer].cpu().numpy().view(oracle.NP_DTYPE[int(wl.dtype)]).reshape(max_seq, Hkv, D)
             vh = vbuf[lo:lo + per_layer].cpu().numpy().view(oracle.NP_DTYPE[int(wl.dtype)]).reshape(max_seq, Hkv, D)
-            qh = q[layer].cpu().numpy()
+            qh = (q_rot if wl.rope else q)[layer].cpu().numpy()      # (rope: the rotated queries that the separate launch left)
             c0 = time.perf_counter()
             ref = oracle.attn_decode_ref(qh, kh, vh, int(wl.dtype), H, Hkv, D, wl.context, scale,
                                          kv_start=starts[layer], softcap=wl.softcap, threads=threads)
@@ -851,7 +870,7 @@ def decode_phase_stamps(args):
     import torch
     import vulkanforge_amd as vf
     calib = C.CDLL(os.path.join(ROOT, "vulkanforge_amd", "libvfkv_calib.so"))
-    calib.vfkv_calib_decode_stamps.argtypes = [C.c_void_p] * 6 + [C.c_uint32] * 7 + [C.c_float, C.c_void_p, C.c_void_p, C.c_void_p, C.c_uint32, C.c_int]
+    calib.vfkv_calib_decode_stamps.argtypes = [C.c_void_p] * 6 + [C.c_uint32] * 7 + [C.c_float, C.c_void_p, C.c_void_p]
     H, Hkv, D, NL, NW = 32, 8, 128, 8, 4
     out = {"metric": "decode_phase_stamps", "unit": "us after the launch's first wavefront started", "n_gpus": 1,
            "config": {"workload": "split_mfma_kernel, 32 / 8 / 128 FP8, instrumented kernel, 8 launches per graph replay"}, "contexts": {}}
@@ -860,19 +879,10 @@ def decode_phase_stamps(args):
     # with K and V rows at the same offsets one KV head's stream runs 10 % slower than the others and the launch waits for it
     # (the head whose 128-byte pieces lie at addresses with bits 9:7 == 011, on whichever XCD it runs)
     cases = [(32768, 256), (8192, 256), (8193, 256), (32768, 0)] + [(32768, int(x)) for x in args.v_offsets.split(",") if x.strip()]
-    # the counter-dealt worker, with the library's own environment switches and its choice of static rounds
-    dyn_rounds = int(os.environ.get("VFKV_DECODE_DYN_ROUNDS", "2"))
-    dyn_half = int(os.environ.get("VFKV_DECODE_DYN_HALF", "0") != "0")
-    out["config"]["dyn_rounds"], out["config"]["dyn_half_units"] = dyn_rounds, dyn_half
-    tickets = torch.zeros(4096, dtype=torch.int32, device="cuda")
     for seq, shift in cases:
         tile = vf.lib().vfkv_decode_tile_for(seq, H, Hkv, D, int(vf.KvDtype.F8))
         nt = (seq + tile - 1) // tile
-        static_rounds = 0
-        if dyn_rounds:
-            tile, nt = 64, 32
-            rounds = -(-((seq + 31) // 32) // (4 * nt))
-            static_rounds = max(rounds - dyn_rounds, 1)
+        tile, nt = 64, 32            # vfkv_decode_attention's launch: one workgroup per CU, the rows dealt to them in runs
         slab = seq * Hkv * D
         pool = [torch.randn(((NL * slab + (1 << 21)) // 4,), device="cuda", generator=g).to(torch.float8_e4m3fn).view(torch.uint8).repeat(4)
                 for _ in range(2)]
@@ -888,8 +898,7 @@ def decode_phase_stamps(args):
             for l in range(NL):
                 rc = calib.vfkv_calib_decode_stamps(q.data_ptr(), ks[l].data_ptr(), vs[l].data_ptr(), so.data_ptr(), sm.data_ptr(),
                                                     ss.data_ptr(), int(vf.KvDtype.F8), H, Hkv, D, seq, tile, nt, 1.0 / D ** 0.5,
-                                                    st[l].data_ptr(), stream, tickets.data_ptr() if dyn_rounds else None,
-                                                    static_rounds, dyn_half)
+                                                    st[l].data_ptr(), stream)
                 assert rc == 0, rc
         launches()
         torch.cuda.synchronize()

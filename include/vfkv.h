@@ -331,6 +331,23 @@ int vfkv_kv_write_decode_attention(vfkv_cache* c, uint32_t layer, uint32_t n_hea
                                    uint32_t kv_start, float scale, float softcap, vfkv_workspace* ws,
                                    vfkv_stream stream);
 
+/* The whole attention block of a decode layer as the executor issues it back to back (executor/attention.rs:360-625):
+ * step_q_norm_rope / step_q_rope, step_k_norm_rope / step_k_rope, step_kv_write and step_attention of one token.
+ * `q` [n_heads, head_dim] and `k_src` [kv_heads * head_dim] are the rows BEFORE norm and rotation; they are
+ * RMS-normalised per head times q_norm_weight / k_norm_weight (NULL: no norm) and rotated for `position` exactly as
+ * vfkv_qk_rope_kv_write does (same arithmetic: the cache bytes and k_out are bit-identical to that call), K and V are
+ * appended at `position`, and the rotated queries attend over keys [kv_start, position].  Where the decode worker can,
+ * all of this is ONE launch plus the merge: every workgroup rotates its query heads while its first K rows are in
+ * flight, and the wavefront that reads the new row rotates, converts and stores it itself; otherwise the call is
+ * vfkv_qk_rope_kv_write + vfkv_decode_attention.  `q_out` (may be NULL; must not overlap `q`) receives the rotated
+ * queries, `k_out` (may be NULL, may be k_src) the rotated K row as f32 (what the reference leaves in q_buf / k_buf). */
+int vfkv_qk_rope_kv_write_decode_attention(vfkv_cache* c, uint32_t layer, uint32_t n_heads, const float* q,
+                                           const float* q_norm_weight, float* q_out, const float* k_src,
+                                           const float* v_src, const float* k_norm_weight,
+                                           const float* freq_factors, const vfkv_rope_params* p, float* k_out,
+                                           float* o, uint32_t position, uint32_t kv_start, float scale,
+                                           float softcap, vfkv_workspace* ws, vfkv_stream stream);
+
 /* ------------------------------------------------------------------------------------------ */
 /* Chunked-prefill causal attention over the cache.                                           */
 /* ------------------------------------------------------------------------------------------ */

@@ -18,7 +18,7 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 def calib():
     lib = C.CDLL(os.path.join(ROOT, "vulkanforge_amd", "libvfkv_calib.so"))
     lib.vfkv_calib_prefill_stamps.argtypes = [C.c_void_p] * 4 + [C.c_uint32] * 5 + [C.c_float, C.c_int, C.c_void_p, C.c_void_p]
-    lib.vfkv_calib_decode_stamps.argtypes = [C.c_void_p] * 6 + [C.c_uint32] * 7 + [C.c_float, C.c_void_p, C.c_void_p, C.c_void_p, C.c_uint32, C.c_int]
+    lib.vfkv_calib_decode_stamps.argtypes = [C.c_void_p] * 6 + [C.c_uint32] * 7 + [C.c_float, C.c_void_p, C.c_void_p]
     return lib
 
 
@@ -78,7 +78,7 @@ def test_instrumented_decode_worker_equals_the_library_worker(dtype, heads, hkv,
     stamps = torch.zeros((hkv, nt, 1, 4, 4), dtype=torch.int64, device=DEV)
     print(f"case {dtype.label()} H={heads} Hkv={hkv} D={d} seq={seq} tile={tile}", flush=True)
     rc = calib().vfkv_calib_decode_stamps(qd.data_ptr(), kd.data_ptr(), vd.data_ptr(), *(b.data_ptr() for b in bufs[1]), int(dtype), heads,
-                                          hkv, d, seq, tile, nt, scale, stamps.data_ptr(), torch.cuda.current_stream().cuda_stream, None, 0, 0)
+                                          hkv, d, seq, tile, nt, scale, stamps.data_ptr(), torch.cuda.current_stream().cuda_stream)
     assert rc == 0
     torch.cuda.synchronize()
     for a, b in zip(*bufs):

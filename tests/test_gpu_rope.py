@@ -251,3 +251,107 @@ def test_qk_rope_kv_write_is_the_two_calls_in_one(dtype, h, hkv, d, m, pos0):
     q_ref = oracle.rms_norm_rope(q, pos, d, d, ts, weight=wq, eps=1e-6)
     assert (np.abs(to_np(qa) - q_ref) <= k_tolerance(q_ref, pos)[:, None, None]).all()
     a.destroy(); b.destroy()
+
+
+FOLD_CASES = [
+    # dtype, heads, hkv, d, ctx, rotary, mode, norm, ff, window, cap
+    (vf.KvDtype.F8, 32, 8, 128, 8193, 128, _ffi.ROPE_NEOX, True, False, 0, 0.0),     # the decode step of a Qwen3-style layer
+    (vf.KvDtype.F8, 32, 8, 128, 4097, 128, _ffi.ROPE_NORM, False, False, 0, 0.0),    # plain QRope / KRope, adjacent pairs
+    (vf.KvDtype.F8, 32, 8, 128, 3000, 64, _ffi.ROPE_NEOX, True, True, 1000, 0.0),    # partial rotary, frequency factors, window
+    (vf.KvDtype.F16, 16, 8, 256, 5000, 256, _ffi.ROPE_NEOX, True, False, 0, 30.0),   # head_dim 256, soft-cap
+    (vf.KvDtype.F16, 16, 4, 64, 2500, 64, _ffi.ROPE_NORM, True, False, 0, 0.0),      # head_dim 64 (runs of 64 rows)
+    (vf.KvDtype.F8, 8, 8, 64, 1300, 32, _ffi.ROPE_NEOX, False, False, 0, 0.0),       # FP8 rows of 64 bytes: two KV heads share a line
+    (vf.KvDtype.F8, 32, 8, 128, 200, 128, _ffi.ROPE_NEOX, True, False, 0, 0.0),      # one workgroup per KV head writes the output itself
+    (vf.KvDtype.F8, 32, 8, 128, 8209, 128, _ffi.ROPE_NEOX, True, False, 0, 0.0),     # 17 rows in the last run: a unit of its own
+    (vf.KvDtype.F8, 96, 8, 128, 2049, 128, _ffi.ROPE_NEOX, True, False, 0, 0.0),     # 12 heads per KV head: two head slices
+    (vf.KvDtype.F8, 4, 1, 512, 700, 128, _ffi.ROPE_NEOX, True, False, 0, 0.0),       # head_dim 512: the separate RoPE launch
+    (vf.KvDtype.F32, 8, 2, 128, 600, 128, _ffi.ROPE_NEOX, True, False, 0, 0.0),      # F32 cache: the separate RoPE launch
+]
+
+
+@pytest.mark.parametrize("dtype,heads,hkv,d,ctx,rotary,mode,norm,ff,window,cap", FOLD_CASES)
+def test_qk_rope_kv_write_decode_attention_equals_the_separate_calls(dtype, heads, hkv, d, ctx, rotary, mode, norm, ff, window, cap):
+    """vfkv_qk_rope_kv_write_decode_attention (norm + RoPE of the token inside the decode worker where it can) against
+    vfkv_qk_rope_kv_write followed by vfkv_decode_attention: cache bytes, rotated queries and rotated K row bit-identical, the
+    output within f32 rounding of the two-call output and within this path's tolerance of the oracle
+    (vfo_rms_norm_rope -> cache encoding -> vfo_attn_decode_ref)."""
+    from gpu_util import TOL, encode_np, outlier_normal
+    r = rng(ctx * 3 + d)
+    fill = outlier_normal if dtype == vf.KvDtype.F8 else fp16_normal
+    k_hist, v_hist = fill(r, (ctx - 1, hkv * d)), fill(r, (ctx - 1, hkv * d))
+    q = (r.standard_normal((heads, d)) * 1.2).astype(np.float32)
+    k_new = (r.standard_normal((hkv, d)) * 1.5).astype(np.float32)
+    v_new = fp16_normal(r, (hkv, d))
+    qw = (1 + 0.2 * r.standard_normal(d)).astype(np.float32) if norm else None
+    kw = (1 + 0.2 * r.standard_normal(d)).astype(np.float32) if norm else None
+    ffv = (1 + 2 * r.random(rotary // 2)).astype(np.float32) if ff else None
+    ts = float(oracle.rope_theta_scale(10000.0, rotary))
+    pos = ctx - 1
+    kv_start = max(0, pos + 1 - window) if window else 0
+    scale = float(1.0 / np.sqrt(d))
+    es = dtype.element_size()
+    got = []
+    for fused in (True, False):
+        cache = vf.KvCache(vf.KvCacheConfig(1, hkv, d, ctx + 4, dtype=dtype))
+        cache.zero_fill()
+        fwd = vf.Forward(cache, heads)
+        fwd.b_step_kv_write(0, 0, ctx - 1, to_dev(k_hist), to_dev(v_hist))
+        qd, kd, vd = to_dev(q), to_dev(k_new), to_dev(v_new)
+        q_out = torch.full((heads, d), float("nan"), device=DEV)
+        k_out = torch.full((hkv, d), float("nan"), device=DEV)
+        o = torch.full((heads, d), float("nan"), device=DEV)
+        kwargs = dict(q_norm_weight=to_dev(qw) if norm else None, k_norm_weight=to_dev(kw) if norm else None,
+                      freq_factors=to_dev(ffv) if ff else None, rope_mode=mode, eps=1e-6, k_out=k_out)
+        print(f"case {dtype.label()} H={heads} Hkv={hkv} D={d} ctx={ctx} rotary={rotary} mode={mode} norm={norm} fused={fused}", flush=True)
+        if fused:
+            fwd.step_qk_rope_kv_write_attention(0, pos, qd, kd, vd, o, rotary, ts, q_out=q_out, kv_start=kv_start, scale=scale,
+                                                softcap=cap, **kwargs)
+        else:
+            fwd.step_qk_rope_kv_write(0, pos, 1, qd, kd, vd, rotary, ts, q_out=q_out, **kwargs)
+            fwd.run_scalar_attn(0, pos, q_out, o, kv_start=kv_start, scale=scale, softcap=cap)
+        torch.cuda.synchronize()
+        row = read_device(cache.k_ptr + cache.pos_offset_bytes(0, pos), hkv * d * es).copy()
+        vrow = read_device(cache.v_ptr + cache.pos_offset_bytes(0, pos), hkv * d * es).copy()
+        got.append((row, vrow, to_np(q_out).copy(), to_np(k_out).copy(), to_np(o).copy()))
+        assert (to_np(qd) == q).all()                       # the caller's rows are left alone
+        cache.destroy()
+    (rk, rv, rq, rko, ro), (sk, sv, sq, sko, so_) = got
+    assert (rk == sk).all() and (rv == sv).all()            # cache bytes
+    assert (rq == sq).all() and (rko == sko).all()          # rotated queries and K row
+    assert np.abs(ro - so_).max() < 2e-6
+    # against the oracle.  The rotation: within one ulp of the f32 angle of the oracle's (the slack the reference grants its own GPU
+    # at tests/correctness.rs:799-815), the stored K code a correct rounding of a value inside that band
+    q_ref = oracle.rms_norm_rope(q[None], np.array([pos], np.int32), d, rotary, ts, mode=mode, weight=qw, ff=ffv, eps=1e-6)[0]
+    k_ref = oracle.rms_norm_rope(k_new[None], np.array([pos], np.int32), d, rotary, ts, mode=mode, weight=kw, ff=ffv, eps=1e-6)[0]
+    assert (np.abs(rq - q_ref) <= k_tolerance(q_ref, pos)).all()
+    tol = k_tolerance(k_ref, pos)
+    assert (np.abs(rko - k_ref) <= tol).all()
+    if dtype == vf.KvDtype.F8:
+        k_code, enc = rk, oracle.f32_to_e4m3
+    elif dtype == vf.KvDtype.F16:
+        k_code, enc = rk.view(np.uint16), oracle.f32_to_f16_bits
+    else:
+        k_code, enc = rk.view(np.float32), lambda x: x                                      # noqa: E731
+    assert (k_code == enc(rko.reshape(-1))).all()           # the cache holds the conversion of exactly what k_out holds
+    # The attention: the oracle over the rotated queries and the row as the GPU produced them (the angle's ulp, times K entries of
+    # +-40, would otherwise move a score by more than this path's output tolerance)
+    ke = np.concatenate([encode_np(k_hist.reshape(ctx - 1, hkv, d), dtype), k_code.reshape(1, hkv, d)])
+    ve = encode_np(np.concatenate([v_hist.reshape(ctx - 1, hkv, d), v_new[None]]), dtype)
+    assert (ve[ctx - 1].reshape(-1).view(np.uint8) == rv).all()      # V bytes: what vfkv_kv_write stores
+    ref = oracle.attn_decode_ref(rq, ke, ve, int(dtype), heads, hkv, d, ctx, scale, kv_start=kv_start, softcap=cap)
+    assert np.abs(ro - ref).max() < TOL[dtype]
+
+
+def test_qk_rope_kv_write_decode_attention_rejects_bad_arguments():
+    cache = vf.KvCache(vf.KvCacheConfig(1, 2, 64, 64, dtype=vf.KvDtype.F16))
+    fwd = vf.Forward(cache, 4)
+    q, o, kv = torch.zeros((4, 64), device=DEV), torch.zeros((4, 64), device=DEV), torch.zeros((2, 64), device=DEV)
+    with pytest.raises(vf.VfkvError):
+        fwd.step_qk_rope_kv_write_attention(0, 3, q, kv, kv, o, 64, 0.9, q_out=q)            # q_out overlaps q
+    with pytest.raises(vf.VfkvError):
+        fwd.step_qk_rope_kv_write_attention(0, 3, q, kv, kv, o, 63, 0.9)                     # odd rotary_dim
+    with pytest.raises(vf.VfkvError):
+        fwd.step_qk_rope_kv_write_attention(0, 3, q, kv, kv, o, 64, 0.9, rope_mode=1)        # unsupported mode
+    with pytest.raises(vf.VfkvError):
+        fwd.step_qk_rope_kv_write_attention(0, 3, q, None, kv, o, 64, 0.9)                   # no K row
+    cache.destroy()

@@ -102,6 +102,8 @@ SIGNATURES = {
     "vfkv_workspace_create": (C.c_int, [_u32, _u32, _u32, C.POINTER(_vp)]),
     "vfkv_workspace_destroy": (None, [_vp]),
     "vfkv_kv_write_decode_attention": (C.c_int, [_vp, _u32, _u32, _vp, _vp, _vp, _vp, _u32, _u32, _f, _f, _vp, _vp]),
+    "vfkv_qk_rope_kv_write_decode_attention": (C.c_int, [_vp, _u32, _u32, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _u32, _u32, _f, _f,
+                                                        _vp, _vp]),
     "vfkv_decode_tile_for": (_u32, [_u32, _u32, _u32, _u32, _u32]),
     "vfkv_decode_attention": (C.c_int, [_vp, _u32, _u32, _u32, _vp, _vp, _u32, _u32, _f, _f, _vp, _vp]),
     "vfkv_decode_attention_static": (C.c_int, [_vp, _u32, _u32, _u32, _vp, _vp, _u32, _u32, _f, _f, _vp]),

@@ -69,6 +69,8 @@ struct vfkv_workspace {
     float* scratch_out;
     float* scratch_max;
     float* scratch_sum;
+    float* q_rot;          // n_heads * head_dim floats: rotated queries of vfkv_qk_rope_kv_write_decode_attention when the caller
+                           // does not want them and the shape takes the separate RoPE launch
 };
 
 // Decode partials of vfkv_decode_attention_static: device memory that exists from the moment the library is loaded, so
@@ -550,11 +552,13 @@ int vfkv_workspace_create(uint32_t n_heads, uint32_t head_dim, uint32_t max_seq_
     // one allocation: [out | max | sum], each 256-byte aligned
     const uint64_t out_b = (n_out * 4u + 255u) & ~255ull, ml_b = (n_ml * 4u + 255u) & ~255ull;
     void* base = nullptr;
-    hipError_t e = hipMalloc(&base, out_b + 2u * ml_b);
+    const uint64_t q_b = ((uint64_t)n_heads * head_dim * 4u + 255u) & ~255ull;
+    hipError_t e = hipMalloc(&base, out_b + 2u * ml_b + q_b);
     if (e != hipSuccess) { delete w; return hip_fail(e, "hipMalloc(workspace)"); }
     w->scratch_out = (float*)base;
     w->scratch_max = (float*)((char*)base + out_b);
     w->scratch_sum = (float*)((char*)base + out_b + ml_b);
+    w->q_rot = (float*)((char*)base + out_b + 2u * ml_b);
     *out = w;
     return VFKV_OK;
 }
@@ -598,12 +602,18 @@ static uint32_t device_cus() {
 
 // Tile length for the convenience path: enough workgroups to cover the CUs once (matrix-core worker) or twice, tiles a
 // multiple of 64 keys (so they never exceed the workspace's ceil(max_seq / 64) rows).
-static uint32_t choose_tile(uint32_t span, uint32_t n_kv_heads, uint32_t groups, uint32_t target_wgs) {
+// VFKV_DECODE_TILE: keys per workgroup forced by the environment (0: the library chooses)
+static uint32_t forced_tile() {
     static const uint32_t forced = [] {
         const char* e = getenv("VFKV_DECODE_TILE");
-        return e ? (uint32_t)strtoul(e, nullptr, 10) : 0u;
+        const uint32_t v = e ? (uint32_t)strtoul(e, nullptr, 10) : 0u;
+        return (v >= 64u && v % 64u == 0u) ? v : 0u;
     }();
-    if (forced >= 64u && forced % 64u == 0u) return forced;
+    return forced;
+}
+
+static uint32_t choose_tile(uint32_t span, uint32_t n_kv_heads, uint32_t groups, uint32_t target_wgs) {
+    if (forced_tile() != 0u) return forced_tile();
     uint32_t tiles = (target_wgs + n_kv_heads * groups - 1u) / (n_kv_heads * groups);
     if (tiles == 0u) tiles = 1u;
     uint32_t tile = (span + tiles - 1u) / tiles;
@@ -642,7 +652,8 @@ uint32_t vfkv_decode_tile_for(uint32_t span, uint32_t n_heads, uint32_t n_kv_hea
 static int decode_attention_impl(vfkv_cache* c, uint32_t layer, uint32_t kv_layer, uint32_t n_heads, const float* q, float* o,
                                  uint32_t position, uint32_t kv_start, float scale, float softcap, vfkv_workspace* ws,
                                  const float* k_new, const float* v_new, vfkv_stream stream, const char* who,
-                                 const vfkv::GateArgs* gate = nullptr, bool static_ws = false) {
+                                 const vfkv::GateArgs* gate = nullptr, bool static_ws = false, const vfkv::RopeFold* rope = nullptr,
+                                 const vfkv_rope_params* rope_params = nullptr) {
     if (!c || !c->k || !c->v) return fail(VFKV_ERR_INVALID_ARG, "%s: cache has no buffers", who);
     if (!ws && !static_ws) return fail(VFKV_ERR_INVALID_ARG, "%s: workspace is NULL", who);
     if (!q || !o) return fail(VFKV_ERR_INVALID_ARG, "%s: NULL buffer", who);
@@ -664,27 +675,26 @@ static int decode_attention_impl(vfkv_cache* c, uint32_t layer, uint32_t kv_laye
     uint32_t tile = vfkv_decode_tile_for(seq_len - kv_start, n_heads, kvh, hd, c->dtype);
     uint32_t first = kv_start / tile;
     uint32_t n_tiles = (seq_len + tile - 1u) / tile - first;
-    // Late rebalancing (attn_decode_dyn.h): launches of several workgroups per KV head on the matrix-core worker deal the
-    // last runs of the span statically and hand the front out through counters.  The workgroup count is then chosen directly
-    // (one per CU), independent of a tile length: the launch covers the rows from the 64-row boundary at or below kv_start.
-    static const uint32_t dyn_rounds = [] { const char* e = getenv("VFKV_DECODE_DYN_ROUNDS"); return e ? (uint32_t)strtoul(e, nullptr, 10) : 2u; }();
-    static const bool dyn_half = [] { const char* e = getenv("VFKV_DECODE_DYN_HALF"); return e ? e[0] != '0' : false; }();
-    uint32_t static_rounds = 0u;
-    const uint32_t run_rows = vfkv::split_run_rows(c->dtype, hd);
-    const uint32_t nz = (n_heads / kvh + 7u) / 8u;
-    if (dyn_rounds != 0u && n_tiles > 1u && run_rows != 0u && (hd == 128u || hd == 256u)) {
-        const uint32_t base_row = kv_start / 64u * 64u;
-        const uint32_t nv = (seq_len - base_row + run_rows - 1u) / run_rows;
+    const uint64_t off = layer_off(c, kv_layer);
+    vfkv::SplitLaunch L;
+    L.q = q; L.k = (char*)c->k + off; L.v = (char*)c->v + off;
+    L.dtype = c->dtype; L.n_heads = n_heads; L.n_kv_heads = kvh; L.head_dim = hd;
+    L.seq_len = seq_len; L.kv_start = kv_start; L.tile = tile; L.tile_first = first; L.n_tiles = n_tiles;
+    L.scale = scale; L.softcap = softcap;
+    // the partials stay inside the workspace, so they need not correspond to tiles
+    L.interleave = true;
+    // The interleaved worker deals the runs of the span to its workgroups whatever the tile length says: the workgroup count
+    // is chosen directly (one per CU, none without a run), and the launch covers the rows from the 64-row boundary at or
+    // below kv_start.
+    if (n_tiles > 1u && forced_tile() == 0u && vfkv::split_interleaves(L)) {
+        const uint32_t run_rows = vfkv::split_run_rows(c->dtype, hd), nz = (n_heads / kvh + 7u) / 8u;
+        const uint32_t runs = (seq_len - kv_start / 64u * 64u + run_rows - 1u) / run_rows;
         uint32_t wgs = device_cus() / (kvh * nz);
+        if (wgs > (runs + 3u) / 4u) wgs = (runs + 3u) / 4u;             // four run streams per workgroup
+        if (!static_ws && wgs > ws->max_tiles) wgs = ws->max_tiles;
         if (wgs < 1u) wgs = 1u;
-        if (wgs > (nv + 3u) / 4u) wgs = (nv + 3u) / 4u;              // four run streams per workgroup: no workgroup without a run
-        const uint32_t cap_tiles = static_ws ? 0xFFFFFFFFu : ws->max_tiles;
-        if (wgs > cap_tiles) wgs = cap_tiles;
-        if (wgs >= 2u) {
-            const uint32_t rounds = (nv + 4u * wgs - 1u) / (4u * wgs);
-            static_rounds = rounds > dyn_rounds ? rounds - dyn_rounds : 1u;
-            tile = 64u; first = kv_start / 64u; n_tiles = wgs;
-        }
+        tile = 64u; first = kv_start / 64u; n_tiles = wgs;
+        L.tile = tile; L.tile_first = first; L.n_tiles = n_tiles;
     }
     vfkv_workspace fixed;
     if (static_ws) {
@@ -702,19 +712,24 @@ static int decode_attention_impl(vfkv_cache* c, uint32_t layer, uint32_t kv_laye
         fixed.scratch_out = (float*)base;
         fixed.scratch_max = (float*)((char*)base + out_b);
         fixed.scratch_sum = (float*)((char*)base + out_b + ml_b);
+        fixed.q_rot = nullptr;
         ws = &fixed;
     }
     if (n_tiles > ws->max_tiles) return fail(VFKV_ERR_WORKSPACE, "%s: %u tiles > workspace capacity %u", who, n_tiles, ws->max_tiles);
-    const uint64_t off = layer_off(c, kv_layer);
-    vfkv::SplitLaunch L;
-    L.q = q; L.k = (char*)c->k + off; L.v = (char*)c->v + off;
     L.scratch_out = ws->scratch_out; L.scratch_max = ws->scratch_max; L.scratch_sum = ws->scratch_sum;
-    L.dtype = c->dtype; L.n_heads = n_heads; L.n_kv_heads = kvh; L.head_dim = hd;
-    L.seq_len = seq_len; L.kv_start = kv_start; L.tile = tile; L.tile_first = first; L.n_tiles = n_tiles;
-    L.scale = scale; L.softcap = softcap;
-    // the partials stay inside the workspace, so they need not correspond to tiles
-    L.interleave = true;
-    if (static_rounds != 0u) { L.static_rounds = static_rounds; L.half_units = dyn_half; }
+    // Q / K norm + RoPE of the token: inside the worker where it can (then q and k_new are the rows before rotation), else
+    // as the launch of its own that vfkv_qk_rope_kv_write makes (which also appends)
+    if (rope) {
+        L.k_new = k_new; L.v_new = v_new; L.append_pos = position; L.rope = rope;
+        if (!vfkv::split_folds_rope(L)) {
+            float* const q_rot = rope->q_out ? rope->q_out : ws->q_rot;
+            if (!q_rot) return fail(VFKV_ERR_WORKSPACE, "%s: no room for the rotated queries (give q_out)", who);
+            rc = rope_kv_write_impl(c, layer, position, 1, q, n_heads, rope->q_weight, q_rot, k_new, v_new, rope->k_weight, nullptr,
+                                    rope->freq_factors, rope_params, rope->k_out, stream);
+            if (rc != VFKV_OK) return rc;
+            L.q = q_rot; L.rope = nullptr; L.k_new = nullptr; L.v_new = nullptr; k_new = nullptr;
+        }
+    }
     if (k_new) {
         L.k_new = k_new; L.v_new = v_new; L.append_pos = position;
         if (!vfkv::split_appends(L)) {          // this shape's worker cannot write the row itself: append in its own launch
@@ -761,6 +776,35 @@ int vfkv_kv_write_decode_attention(vfkv_cache* c, uint32_t layer, uint32_t n_hea
         return fail(VFKV_ERR_ALIGNMENT, "kv_write_decode_attention: dst_byte_offset must be uint-aligned");
     return decode_attention_impl(c, layer, layer, n_heads, q, o, position, kv_start, scale, softcap, ws, k_src, v_src, stream,
                                  "kv_write_decode_attention");
+}
+
+int vfkv_qk_rope_kv_write_decode_attention(vfkv_cache* c, uint32_t layer, uint32_t n_heads, const float* q,
+                                           const float* q_norm_weight, float* q_out, const float* k_src, const float* v_src,
+                                           const float* k_norm_weight, const float* freq_factors, const vfkv_rope_params* p,
+                                           float* k_out, float* o, uint32_t position, uint32_t kv_start, float scale, float softcap,
+                                           vfkv_workspace* ws, vfkv_stream stream) {
+    const char* who = "qk_rope_kv_write_decode_attention";
+    if (!p) return fail(VFKV_ERR_INVALID_ARG, "%s: params is NULL", who);
+    if (!k_src || !v_src) return fail(VFKV_ERR_INVALID_ARG, "%s: NULL source row", who);
+    if (!c || layer >= c->n_layers) return fail(VFKV_ERR_INVALID_ARG, "%s: layer out of range", who);
+    const uint32_t hd = hd_for(c, layer);
+    if (p->rope_mode != VFKV_ROPE_NORM && p->rope_mode != VFKV_ROPE_NEOX)
+        return fail(VFKV_ERR_UNSUPPORTED, "%s: rope_mode %u (0 = NORM and 2 = NEOX are built)", who, p->rope_mode);
+    if (p->rotary_dim % 2u != 0u || p->rotary_dim > hd)
+        return fail(VFKV_ERR_INVALID_ARG, "%s: rotary_dim %u must be even and <= head_dim %u", who, p->rotary_dim, hd);
+    if (!(p->freq_scale > 0.f)) return fail(VFKV_ERR_INVALID_ARG, "%s: freq_scale must be > 0", who);
+    if ((layer_off(c, layer) + (uint64_t)position * row_b(c, layer)) % 4u != 0u)
+        return fail(VFKV_ERR_ALIGNMENT, "%s: dst_byte_offset must be uint-aligned", who);
+    if (q_out != nullptr && q != nullptr) {
+        const uintptr_t a0 = (uintptr_t)q, a1 = a0 + (uintptr_t)n_heads * hd * 4u, b0 = (uintptr_t)q_out, b1 = b0 + (uintptr_t)n_heads * hd * 4u;
+        if (a0 < b1 && b0 < a1) return fail(VFKV_ERR_INVALID_ARG, "%s: q_out must not overlap q (every workgroup reads q while one writes q_out)", who);
+    }
+    vfkv::RopeFold rf;
+    rf.q_weight = q_norm_weight; rf.k_weight = k_norm_weight; rf.freq_factors = freq_factors; rf.q_out = q_out; rf.k_out = k_out;
+    rf.rotary_dim = p->rotary_dim; rf.mode = p->rope_mode; rf.theta_scale = p->theta_scale; rf.freq_scale = p->freq_scale;
+    rf.attn_factor = p->attn_factor; rf.eps = p->eps;
+    return decode_attention_impl(c, layer, layer, n_heads, q, o, position, kv_start, scale, softcap, ws, k_src, v_src, stream, who,
+                                 nullptr, false, &rf, p);
 }
 
 // ---- prefill attention -------------------------------------------------------------------------------

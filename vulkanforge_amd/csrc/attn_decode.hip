@@ -26,6 +26,8 @@
 // loads of one phase are in flight during the other.  Loads are raw buffer loads whose descriptor
 // ends at the last populated row: rows past it read as zero without touching memory, which is also
 // how the ring is "refilled" when there is no next run.
+#include <cstdio>
+#include <cstdlib>
 #include "device_utils.h"
 #include "kernels.h"
 
@@ -48,7 +50,6 @@ struct SplitArgs {
     uint32_t group;          // n_heads / n_kv_heads
     uint32_t interleave;     // matrix-core worker: deal the runs of the launched span round-robin instead of by tile
     float scale, softcap;
-    uint32_t static_rounds;  // attn_decode_dyn.h: runs per run stream dealt from the end of the span (0: the other workers)
 #ifdef VFKV_DECODE_STAMPS
     unsigned long long* stamps;   // instrumented build (calibration_decode.hip): [KV head][workgroup of the head][head slice][wavefront][4] wall-clock readings
 #endif
@@ -656,7 +657,7 @@ __global__ __launch_bounds__(kWave) void reduce_generic_kernel(const float* __re
 
 }  // namespace vfkv
 #include "attn_decode_mfma.h"
-#include "attn_decode_dyn.h"
+#include "attn_decode_il.h"
 #include "attn_decode_f32.h"
 namespace vfkv {
 
@@ -681,14 +682,21 @@ static hipError_t launch_split_mfma(const SplitArgs& a, uint32_t g, hipStream_t 
 }
 
 template <int DT, int D, int RUN>
-static hipError_t launch_split_dyn(const SplitArgs& a, uint32_t g, bool half_units, hipStream_t stream) {
+static hipError_t launch_split_il(const SplitArgs& a, uint32_t g, const RopeFold* rope, hipStream_t stream) {
     constexpr int NW = kMfmaWaves;
     const uint32_t gt = g < 8u ? g : 8u;
     dim3 grid(a.n_kv_heads, a.n_tiles, (g + gt - 1u) / gt);
-#define VFKV_DYN(CAPV, HUV) hipLaunchKernelGGL((split_mfma_dyn_kernel<DT, D, RUN, NW, CAPV, HUV>), grid, dim3(NW * kWave), 0, stream, a, gt)
-    if (a.softcap > 0.f) { if (half_units) VFKV_DYN(true, true); else VFKV_DYN(true, false); }
-    else { if (half_units) VFKV_DYN(false, true); else VFKV_DYN(false, false); }
-#undef VFKV_DYN
+    if (rope != nullptr) {
+        RopeFoldArgs rf;
+        rf.q_weight = rope->q_weight; rf.k_weight = rope->k_weight; rf.freq_factors = rope->freq_factors;
+        rf.q_out = rope->q_out; rf.k_out = rope->k_out; rf.rotary_dim = rope->rotary_dim; rf.mode = rope->mode;
+        rf.theta_scale = rope->theta_scale; rf.freq_scale = rope->freq_scale; rf.attn_factor = rope->attn_factor; rf.eps = rope->eps;
+        if (a.softcap > 0.f) hipLaunchKernelGGL((split_mfma_il_rope_kernel<DT, D, RUN, NW, true>), grid, dim3(NW * kWave), 0, stream, a, gt, rf);
+        else hipLaunchKernelGGL((split_mfma_il_rope_kernel<DT, D, RUN, NW, false>), grid, dim3(NW * kWave), 0, stream, a, gt, rf);
+    } else {
+        if (a.softcap > 0.f) hipLaunchKernelGGL((split_mfma_il_kernel<DT, D, RUN, NW, true>), grid, dim3(NW * kWave), 0, stream, a, gt);
+        else hipLaunchKernelGGL((split_mfma_il_kernel<DT, D, RUN, NW, false>), grid, dim3(NW * kWave), 0, stream, a, gt);
+    }
     return hipGetLastError();
 }
 
@@ -750,13 +758,16 @@ uint32_t split_tile_granule(uint32_t dtype, uint32_t D) {
     return (uint32_t)kRun;
 }
 
-// True when launch_split would write the token row (k_new, v_new) itself: the matrix-core worker with a single head
-// slice, where one workgroup per KV head owns the new row and can store it before anything reads it.
+// True when launch_split would write the token row (k_new, v_new) itself.  The interleaved worker (attn_decode_il.h) does
+// so for the last row of the span (the wavefront that reads the row converts it into its own registers and stores it);
+// split_mfma_kernel with a single head slice, where one workgroup per KV head owns the new row and can store it before
+// anything reads it.
 bool split_appends(const SplitLaunch& L) {
     if (!L.k_new || !L.v_new || L.n_kv_heads == 0u) return false;
     const uint32_t g = L.n_heads / L.n_kv_heads;
     const bool aligned = ((((uintptr_t)L.k) | ((uintptr_t)L.v) | ((uintptr_t)L.q) | ((uintptr_t)L.k_new) | ((uintptr_t)L.v_new) |
                            ((uintptr_t)L.scratch_out)) & 15u) == 0u;
+    if (split_interleaves(L)) return aligned && L.append_pos + 1u == L.seq_len && L.append_pos >= L.kv_start;
     const uint64_t slab_bytes = (uint64_t)L.seq_len * L.n_kv_heads * L.head_dim * elem_size(L.dtype);
     const bool mfma_shape = mfma_worker_shape(L.dtype, L.head_dim);
     return aligned && slab_bytes < 0x7FFF0000ull && mfma_worker_enabled() && mfma_shape && g <= 8u &&
@@ -772,12 +783,19 @@ bool split_writes_output(const SplitLaunch& L) {
     return aligned && slab_bytes < 0x7FFF0000ull && mfma_worker_enabled() && mfma_shape;
 }
 
-bool split_deals_dynamically(const SplitLaunch& L) {
-    if (!L.interleave || L.static_rounds == 0u || L.n_tiles < 2u || L.o_direct || L.n_kv_heads == 0u) return false;
-    const bool aligned = ((((uintptr_t)L.k) | ((uintptr_t)L.v) | ((uintptr_t)L.q) | ((uintptr_t)L.scratch_out)) & 15u) == 0u;
+bool split_interleaves(const SplitLaunch& L) {
+    if (!L.interleave || L.n_kv_heads == 0u || L.n_tiles == 0u) return false;
+    const bool aligned = ((((uintptr_t)L.k) | ((uintptr_t)L.v) | ((uintptr_t)L.q) | ((uintptr_t)L.scratch_out) | ((uintptr_t)L.o_direct)) & 15u) == 0u;
     const uint64_t slab_bytes = (uint64_t)L.seq_len * L.n_kv_heads * L.head_dim * elem_size(L.dtype);
     return aligned && slab_bytes < 0x7FFF0000ull && mfma_worker_enabled() && (L.dtype == kF8 || L.dtype == kF16) &&
-           (L.head_dim == 128u || L.head_dim == 256u);
+           (L.head_dim == 64u || L.head_dim == 128u || L.head_dim == 256u);
+}
+
+bool split_folds_rope(const SplitLaunch& L) {
+    if (!L.rope || !split_interleaves(L) || !split_appends(L)) return false;
+    const RopeFold& r = *L.rope;
+    const bool aligned = ((((uintptr_t)r.q_out) | ((uintptr_t)r.k_out)) & 3u) == 0u;
+    return aligned && r.rotary_dim % 2u == 0u && r.rotary_dim <= L.head_dim && (r.mode == 0u || r.mode == 2u);
 }
 
 hipError_t launch_split(const SplitLaunch& L, hipStream_t stream, bool* generic_used) {
@@ -793,7 +811,6 @@ hipError_t launch_split(const SplitLaunch& L, hipStream_t stream, bool* generic_
     a.scale = L.scale; a.softcap = L.softcap;
     a.k_new = nullptr; a.v_new = nullptr; a.append_pos = 0u; a.o_direct = nullptr;
     a.interleave = L.interleave ? 1u : 0u;
-    a.static_rounds = 0u;
 #ifdef VFKV_DECODE_STAMPS
     a.stamps = g_decode_stamps;
 #endif
@@ -811,12 +828,14 @@ hipError_t launch_split(const SplitLaunch& L, hipStream_t stream, bool* generic_
     }
     // the matrix-core worker also stores its partials (or the output) 16 bytes at a time
     const bool out_aligned = ((((uintptr_t)L.scratch_out) | ((uintptr_t)L.o_direct)) & 15u) == 0u;
-    if (split_deals_dynamically(L) && out_aligned) {
-        a.static_rounds = L.static_rounds;
-        if (L.dtype == kF8 && L.head_dim == 128u) return launch_split_dyn<kF8, 128, 32>(a, g, L.half_units, stream);
-        if (L.dtype == kF16 && L.head_dim == 128u) return launch_split_dyn<kF16, 128, 32>(a, g, L.half_units, stream);
-        if (L.dtype == kF8 && L.head_dim == 256u) return launch_split_dyn<kF8, 256, 32>(a, g, L.half_units, stream);
-        if (L.dtype == kF16 && L.head_dim == 256u) return launch_split_dyn<kF16, 256, 32>(a, g, L.half_units, stream);
+    if (L.rope != nullptr && !split_folds_rope(L)) return hipErrorInvalidValue;      // the caller rotates in a launch of its own then
+    if (split_interleaves(L) && out_aligned) {
+        if (L.dtype == kF8 && L.head_dim == 64u) return launch_split_il<kF8, 64, 64>(a, g, L.rope, stream);
+        if (L.dtype == kF16 && L.head_dim == 64u) return launch_split_il<kF16, 64, 64>(a, g, L.rope, stream);
+        if (L.dtype == kF8 && L.head_dim == 128u) return launch_split_il<kF8, 128, 32>(a, g, L.rope, stream);
+        if (L.dtype == kF16 && L.head_dim == 128u) return launch_split_il<kF16, 128, 32>(a, g, L.rope, stream);
+        if (L.dtype == kF8 && L.head_dim == 256u) return launch_split_il<kF8, 256, 32>(a, g, L.rope, stream);
+        if (L.dtype == kF16 && L.head_dim == 256u) return launch_split_il<kF16, 256, 32>(a, g, L.rope, stream);
     }
     if (aligned && out_aligned && slab_bytes < 0x7FFF0000ull && mfma_worker_enabled()) {
         if (L.dtype == kF8 && L.head_dim == 64u) return launch_split_mfma<kF8, 64, 64, 1>(a, g, stream);

@@ -8,16 +8,15 @@
 extern "C" {
 
 // One launch of the decode worker as vfkv_decode_attention issues it (flash_attn_split.comp:82-162; rows dealt in interleaved runs)
-// with stamps: q [n_heads, head_dim] f32, k / v layer slabs of seq_len rows (kv_dtype 1 = F16, 2 = FP8), partials into
+// (the rows are dealt to the n_tiles workgroups per KV head whatever `tile` says) with stamps: q [n_heads, head_dim] f32, k / v layer slabs of seq_len rows (kv_dtype 1 = F16, 2 = FP8), partials into
 // so [n_heads][n_tiles][head_dim] / sm, ss [n_heads][n_tiles]; stamps [n_kv_heads][n_tiles][head slices][4 wavefronts][4] uint64
 // (device, zeroed by the caller; head slices = ceil(group / 8)).  One caller at a time: the stamp buffer reaches the launcher through
 // a file-scope pointer.  0 on success.
 int vfkv_calib_decode_stamps(const float* q, const void* k, const void* v, float* so, float* sm, float* ss, uint32_t kv_dtype,
                              uint32_t n_heads, uint32_t n_kv_heads, uint32_t head_dim, uint32_t seq_len, uint32_t tile,
-                             uint32_t n_tiles, float scale, void* stamps, void* stream, void* tickets, uint32_t static_rounds,
-                             int half_units) {
+                             uint32_t n_tiles, float scale, void* stamps, void* stream) {
     if (!q || !k || !v || !so || !sm || !ss || !stamps || n_kv_heads == 0 || n_heads % n_kv_heads != 0 || seq_len == 0 || tile == 0 ||
-        (static_rounds == 0 && n_tiles != (seq_len + tile - 1) / tile) || (kv_dtype != vfkv::kF16 && kv_dtype != vfkv::kF8) ||
+        n_tiles == 0 || (kv_dtype != vfkv::kF16 && kv_dtype != vfkv::kF8) ||
         (head_dim != 64 && head_dim != 128 && head_dim != 256))
         return -1;
     vfkv::SplitLaunch L;
@@ -27,8 +26,6 @@ int vfkv_calib_decode_stamps(const float* q, const void* k, const void* v, float
     L.seq_len = seq_len; L.kv_start = 0; L.tile = tile; L.tile_first = 0; L.n_tiles = n_tiles;
     L.scale = scale; L.softcap = 0.f;
     L.interleave = true;
-    // static_rounds > 0: the worker of attn_decode_dyn.h (tickets is unused)
-    (void)tickets; L.static_rounds = static_rounds; L.half_units = half_units != 0;
     vfkv::g_decode_stamps = (unsigned long long*)stamps;
     const hipError_t e = vfkv::launch_split(L, (hipStream_t)stream);
     vfkv::g_decode_stamps = nullptr;

@@ -35,19 +35,29 @@ struct RopeAppendLaunch {
 hipError_t launch_rope_append(const RopeAppendLaunch& L, hipStream_t stream);
 
 // ---- attn_decode.hip ----
+// Q-norm / RoPE and K-norm / RoPE of the decode token, folded into the decode worker (attn_decode_il.h).
+struct RopeFold {
+    const float* q_weight = nullptr;       // [head_dim] or NULL
+    const float* k_weight = nullptr;       // [head_dim] or NULL
+    const float* freq_factors = nullptr;   // [rotary_dim / 2] or NULL
+    float* q_out = nullptr;                // rotated queries [n_heads][head_dim] (must not overlap q), or NULL
+    float* k_out = nullptr;                // rotated K row [n_kv_heads][head_dim] as f32, or NULL
+    uint32_t rotary_dim = 0, mode = 2;
+    float theta_scale = 1.f, freq_scale = 1.f, attn_factor = 1.f, eps = 0.f;
+};
 struct SplitLaunch {
-    const float* q;        // [n_heads, head_dim] f32
-    const void* k;         // layer slab, [pos][kv_head][d] in `dtype`
-    const void* v;
-    float* scratch_out;    // [(h * n_tiles + j) * head_dim + d]
-    float* scratch_max;    // [h * n_tiles + j]
-    float* scratch_sum;
-    uint32_t dtype, n_heads, n_kv_heads, head_dim;
-    uint32_t seq_len, kv_start;
-    uint32_t tile;         // keys per tile
-    uint32_t tile_first;   // absolute index of the first tile launched
-    uint32_t n_tiles;      // tiles launched == row length of the scratch arrays
-    float scale, softcap;
+    const float* q = nullptr;        // [n_heads, head_dim] f32
+    const void* k = nullptr;         // layer slab, [pos][kv_head][d] in `dtype`
+    const void* v = nullptr;
+    float* scratch_out = nullptr;    // [(h * n_tiles + j) * head_dim + d]
+    float* scratch_max = nullptr;    // [h * n_tiles + j]
+    float* scratch_sum = nullptr;
+    uint32_t dtype = 0, n_heads = 0, n_kv_heads = 0, head_dim = 0;
+    uint32_t seq_len = 0, kv_start = 0;
+    uint32_t tile = 0;         // keys per tile
+    uint32_t tile_first = 0;   // absolute index of the first tile launched
+    uint32_t n_tiles = 0;      // tiles launched == row length of the scratch arrays
+    float scale = 0.f, softcap = 0.f;
     // optional fused append of one token (f32 rows of n_kv_heads * head_dim elements) at row append_pos of the slab
     const float* k_new = nullptr;
     const float* v_new = nullptr;
@@ -58,11 +68,9 @@ struct SplitLaunch {
     // partial j need not be tile j: the matrix-core worker then deals the rows of the launched tiles to its
     // workgroups in interleaved runs (other workers ignore the flag); the merge is the same either way
     bool interleave = false;
-    // interleaved launches of more than one workgroup per KV head on the matrix-core worker: static_rounds > 0 selects the
-    // worker of attn_decode_dyn.h, whose run streams take that many runs each from the END of the span (the ragged last run
-    // and an appended row first) and the rest from the front; half_units halves the units of the front part
-    uint32_t static_rounds = 0;
-    bool half_units = false;
+    // optional (interleaved launches that split_folds_rope() accepts): q and k_new are the rows BEFORE norm and rotation; the
+    // worker RMS-normalises (weights may be NULL) and rotates them for position append_pos itself
+    const struct RopeFold* rope = nullptr;
 };
 // Returns hipErrorInvalidValue when no kernel covers the shape (or when k_new / v_new are given although
 // split_appends() is false: then the caller appends the row with launch_kv_append and leaves them NULL).
@@ -83,8 +91,11 @@ hipError_t launch_reduce(const float* scratch_out, const float* scratch_max, con
                          const GateArgs* gate = nullptr, bool* gate_applied = nullptr);
 // ---- gated_output.hip ----
 hipError_t launch_sigmoid_mul(float* data, uint32_t ne, const GateArgs& gate, hipStream_t stream);
-// True when launch_split would run the worker of attn_decode_dyn.h for L (static_rounds given, shape covered).
-bool split_deals_dynamically(const SplitLaunch& a);
+// True when launch_split would run the interleaved worker of attn_decode_il.h for L (it deals the runs to n_tiles
+// workgroups per KV head whatever L.tile says, so the caller may choose n_tiles freely), and when that worker would also
+// fold L.rope (which needs k_new / v_new as well).
+bool split_interleaves(const SplitLaunch& a);
+bool split_folds_rope(const SplitLaunch& a);
 // Rows per run of the matrix-core worker for this shape (0: the shape is not the matrix-core worker's).
 uint32_t split_run_rows(uint32_t dtype, uint32_t head_dim);
 // Smallest tile granule (keys) the split kernel for this shape works in; 0 if unsupported.

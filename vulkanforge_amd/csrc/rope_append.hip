@@ -14,6 +14,7 @@
 // HBM / launch bound: 4 bytes read and 1, 2 or 4 written per element.
 #include "device_utils.h"
 #include "kernels.h"
+#include "rope_device.h"
 
 namespace vfkv {
 
@@ -70,48 +71,15 @@ __global__ __launch_bounds__(kRopeWaves * kWave) void rope_append_kernel(RopeApp
             wt[j] = (normed && d < D) ? weight[d] : 1.f;
         }
     }
-    // rope_funcs.glsl:63-67,97-101: theta = pos * theta_scale^p / freq_factor[p] * freq_scale, results scaled by attn_factor
+    // the token's cos / sin table (rope_device.h)
     if (blockIdx.y * kRopeWaves < nq + a.n_kv_heads) {     // workgroup-uniform: workgroups that only hold V rows skip it
         const float pos = (float)(a.positions ? a.positions[tok] : (int32_t)(a.pos0 + tok));
-        for (uint32_t p = tid; p < half; p += kRopeWaves * kWave) {
-            const float theta_base = pos * powf(a.theta_scale, (float)p);
-            const float ff = a.freq_factors ? a.freq_factors[p] : 1.0f;
-            const float theta = a.freq_scale * (theta_base / ff);
-            float sn, cs;
-            sincosf(theta, &sn, &cs);
-            cs_lds[p] = cs * a.attn_factor;
-            sn_lds[p] = sn * a.attn_factor;
-        }
+        rope_table(cs_lds, sn_lds, half, pos, a.theta_scale, a.freq_scale, a.attn_factor, a.freq_factors, (uint32_t)tid, kRopeWaves * kWave);
     }
     __syncthreads();
     if (!active) return;
-    if (normed) {                                          // rms_norm.comp:61-112: scale * x * w, f32
-        float ss = 0.f;
-#pragma unroll
-        for (int j = 0; j < kRopeMaxPerLane; ++j) ss = fmaf(x[j], x[j], ss);
-        ss = wave_sum_all(ss);
-        const float scale = 1.0f / sqrtf(ss / (float)D + a.eps);
-#pragma unroll
-        for (int j = 0; j < kRopeMaxPerLane; ++j) x[j] = (scale * x[j]) * wt[j];
-    }
-    // the LDS row is private to the wavefront and LDS operations of a wavefront execute in order, so the fences below only
-    // have to keep the compiler from moving accesses across them
-#pragma unroll
-    for (int j = 0; j < kRopeMaxPerLane; ++j) {
-        const uint32_t d = lane + j * kWave;
-        if (d < D) row[d] = x[j];
-    }
-    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+    rope_row<kRopeMaxPerLane>(x, wt, normed, a.eps, D, half, a.mode, !is_v, cs_lds, sn_lds, row, lane);
     if (!is_v) {
-        // rope_funcs.glsl:39-112: pair p of the rotary part is (2p, 2p + 1) in NORM mode, (p, p + n_dims / 2) in NEOX mode
-        for (uint32_t p = lane; p < half; p += kWave) {
-            const float cs = cs_lds[p], sn = sn_lds[p];
-            const uint32_t i0 = a.mode == 2u ? p : 2u * p, i1 = a.mode == 2u ? p + half : 2u * p + 1u;
-            const float x0 = row[i0], x1 = row[i1];
-            row[i0] = x0 * cs - x1 * sn;
-            row[i1] = x0 * sn + x1 * cs;
-        }
-        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
         float* const out = is_q ? a.q_out : a.k_out;
         if (out != nullptr)
             for (uint32_t d = lane; d < D; d += kWave) out[src_off + d] = row[d];

@@ -191,6 +191,23 @@ class Forward:
                                                              _ptr(k_src), _ptr(v_src), _ptr(o), position, kv_start,
                                                              scale, softcap, self.workspace._h, _stream(stream)))
 
+    def step_qk_rope_kv_write_attention(self, layer: int, position: int, q, k_src, v_src, o, rotary_dim: int, theta_scale: float,
+                                        q_norm_weight=None, k_norm_weight=None, q_out=None, k_out=None, freq_factors=None,
+                                        rope_mode: int = _ffi.ROPE_NEOX, freq_scale: float = 1.0, attn_factor: float = 1.0,
+                                        eps: float = 1e-6, kv_start: int = 0, scale: float | None = None, softcap: float = 0.0,
+                                        stream=None) -> None:
+        """step_q_norm_rope + step_k_norm_rope + step_kv_write + step_attention of one decode token
+        (executor/attention.rs:360-625) as one call: ``q`` and ``k_src`` are the rows before norm and rotation; where the
+        decode worker can, it rotates them itself and no separate RoPE / append launch runs."""
+        if scale is None:
+            hd = self.kv_cache.head_dim_for(layer)
+            scale = self.attn_scale if hd == self.kv_cache.config.head_dim else 1.0 / math.sqrt(hd)
+        p = _ffi.RopeParams(rope_mode, rotary_dim, theta_scale, freq_scale, attn_factor, eps)
+        _ffi.check(_ffi.lib().vfkv_qk_rope_kv_write_decode_attention(
+            self.kv_cache.handle, layer, self.n_heads, _ptr(q), _ptr(q_norm_weight), _ptr(q_out), _ptr(k_src), _ptr(v_src),
+            _ptr(k_norm_weight), _ptr(freq_factors), C.byref(p), _ptr(k_out), _ptr(o), position, kv_start, scale, softcap,
+            self.workspace._h, _stream(stream)))
+
     # ---- prefill attention (runs.rs:933-1010, executor/attention.rs:2192-2390) ----
     @staticmethod
     def run_flash_attn_batch(q, k_layer, v_layer, kv_dtype, o, n_heads, n_kv_heads, head_dim, m, q_start, n_kv,

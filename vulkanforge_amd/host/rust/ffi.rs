@@ -100,6 +100,11 @@ extern "C" {
     pub fn vfkv_prefill_attention(c: *mut VfkvCache, layer: u32, kv_layer: u32, n_heads: u32, q: *const f32,
                                   o: *mut f32, m: u32, base_pos: u32, window: u32, scale: f32, softcap: f32,
                                   stream: *mut c_void) -> c_int;               // b_step_attention
+    pub fn vfkv_qk_rope_kv_write_decode_attention(c: *mut VfkvCache, layer: u32, n_heads: u32, q: *const f32, q_norm_weight: *const f32,
+                                                  q_out: *mut f32, k_src: *const f32, v_src: *const f32, k_norm_weight: *const f32,
+                                                  freq_factors: *const f32, p: *const VfkvRopeParams, k_out: *mut f32, o: *mut f32,
+                                                  position: u32, kv_start: u32, scale: f32, softcap: f32, ws: *mut VfkvWorkspace,
+                                                  stream: *mut c_void) -> c_int;
     pub fn vfkv_kv_write_decode_attention(c: *mut VfkvCache, layer: u32, n_heads: u32, q: *const f32,
                                           k_src: *const f32, v_src: *const f32, o: *mut f32, position: u32,
                                           kv_start: u32, scale: f32, softcap: f32, ws: *mut VfkvWorkspace,

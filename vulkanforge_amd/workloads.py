@@ -21,6 +21,7 @@ class DecodeWorkload:
     window: int = 0         # sliding window of the sliding layers (0 = none)
     sliding_pattern: int = 0  # k sliding layers followed by one global layer, repeated
     gated: bool = False     # the output is multiplied by sigmoid(gate), the gate sitting behind Q (Qwen3.6 full attention)
+    rope: bool = False      # the step also RMS-normalises and rotates the token's Q and K rows (QNormRope + KNormRope + KvWrite + attention)
 
     def layer_window(self, layer: int) -> int:
         if not self.window or not self.sliding_pattern:
@@ -65,6 +66,9 @@ DECODE = {
     "decode_f16_2k_1layer": DecodeWorkload("decode_f16_2k_1layer", 1, 32, 8, 128, 2049, KvDtype.F16, True),
     "decode_fp8_8k_32layers": DecodeWorkload("decode_fp8_8k_32layers", 32, 32, 8, 128, 8193, KvDtype.F8, True),
     "decode_fp8_32k_32layers": DecodeWorkload("decode_fp8_32k_32layers", 32, 32, 8, 128, 32768, KvDtype.F8, False),
+    # configuration 2 with the Q / K norm + RoPE of the token in front of the append, as a Qwen3-style decode layer issues it
+    # (QNormRope, KNormRope, KvWrite, attention: executor/attention.rs:360-625); not a reference configuration
+    "decode_fp8_8k_32layers_rope": DecodeWorkload("decode_fp8_8k_32layers_rope", 32, 32, 8, 128, 8193, KvDtype.F8, True, rope=True),
     # configuration 2 without the append (what the append inside the attention launch costs; not a reference configuration)
     "decode_fp8_8k_32layers_no_append": DecodeWorkload("decode_fp8_8k_32layers_no_append", 32, 32, 8, 128, 8193, KvDtype.F8, False),
     "decode_fp8_8192_32layers_no_append": DecodeWorkload("decode_fp8_8192_32layers_no_append", 32, 32, 8, 128, 8192, KvDtype.F8, False),

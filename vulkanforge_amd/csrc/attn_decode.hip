@@ -682,8 +682,17 @@ static hipError_t launch_split_mfma(const SplitArgs& a, uint32_t g, hipStream_t 
 }
 
 template <int DT, int D, int RUN>
-static hipError_t launch_split_il(const SplitArgs& a, uint32_t g, const RopeFold* rope, hipStream_t stream) {
+static hipError_t launch_split_il(const SplitArgs& a_in, uint32_t g, const RopeFold* rope, hipStream_t stream) {
     constexpr int NW = kMfmaWaves;
+    SplitArgs a = a_in;
+    {   // A ragged last run of at most 16 rows rides with the run before it when that saves the launch a round: when, without
+        // it as a unit of its own, the units divide evenly among the run streams of a KV head.
+        const uint32_t tile_base = a.tile_first * a.tile, span = a.seq_len > tile_base ? a.seq_len - tile_base : 0u;
+        const uint32_t lo = tile_base > a.kv_start ? tile_base : a.kv_start;
+        const uint32_t n_runs = (span + RUN - 1u) / RUN, first_run = (lo - tile_base) / RUN, r_tail = span % RUN;
+        const uint32_t S = NW * a.n_tiles;
+        if (r_tail != 0u && r_tail <= 16u && n_runs >= first_run + 2u && (n_runs - first_run - 1u) % S == 0u) a.interleave |= 2u;
+    }
     const uint32_t gt = g < 8u ? g : 8u;
     dim3 grid(a.n_kv_heads, a.n_tiles, (g + gt - 1u) / gt);
     if (rope != nullptr) {
@@ -784,7 +793,8 @@ bool split_writes_output(const SplitLaunch& L) {
 }
 
 bool split_interleaves(const SplitLaunch& L) {
-    if (!L.interleave || L.n_kv_heads == 0u || L.n_tiles == 0u) return false;
+    static const bool off = [] { const char* e = getenv("VFKV_DECODE_IL"); return e && e[0] == '0'; }();
+    if (off || !L.interleave || L.n_kv_heads == 0u || L.n_tiles == 0u) return false;
     const bool aligned = ((((uintptr_t)L.k) | ((uintptr_t)L.v) | ((uintptr_t)L.q) | ((uintptr_t)L.scratch_out) | ((uintptr_t)L.o_direct)) & 15u) == 0u;
     const uint64_t slab_bytes = (uint64_t)L.seq_len * L.n_kv_heads * L.head_dim * elem_size(L.dtype);
     return aligned && slab_bytes < 0x7FFF0000ull && mfma_worker_enabled() && (L.dtype == kF8 || L.dtype == kF16) &&

@@ -48,9 +48,10 @@ struct RopeFoldArgs {
 template <int DT, int D, int RUN, int NW, bool CAP, bool ROPE>
 __device__ __forceinline__ void split_mfma_il_body(const SplitArgs& a, uint32_t gt, const RopeFoldArgs* rf) {
     constexpr int ES = DT == kF16 ? 2 : 1;
-    constexpr int EPP = 16 / ES;                 // elements per 16-byte piece
     constexpr int RT = RUN / 16;                 // 16-row tiles per run
-    constexpr int XT = RT + 1;                   // tiles of the long first unit
+    constexpr int KLD0 = (D / 4) * ES / 16, VLT0 = 16 / (64 / (D * ES / 16));
+    constexpr bool LONG = (RT + 1) * (KLD0 + VLT0) <= 24;   // the long first unit costs KLD + VLT more 16-byte registers: not where rows are 512 bytes wide
+    constexpr int XT = LONG ? RT + 1 : RT;       // tiles of the first unit of stream 0 at most
     constexpr int KS = D / 32;                   // k-steps of the first product
     constexpr int DTILES = D / 16;
     constexpr int SEG = D / 4, SEGB = SEG * ES;  // a lane group's quarter of a K row
@@ -70,6 +71,7 @@ __device__ __forceinline__ void split_mfma_il_body(const SplitArgs& a, uint32_t 
     __shared__ __attribute__((aligned(16))) _Float16 qlds[16][D + 8];   // rows 0-7: f16(q) per head, rows 8-15: remainders
     __shared__ __attribute__((aligned(16))) float rot[ROPE ? 9 : 1][ROPE ? D : 4];   // ROPE: rotated query heads, then the K row
     __shared__ float cs_lds[ROPE ? D / 2 : 1], sn_lds[ROPE ? D / 2 : 1];
+    __shared__ __attribute__((aligned(16))) uint8_t newrow[2][D * ES];   // the decode token's K and V row in the cache's format (stream 0's wavefront)
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -101,7 +103,8 @@ __device__ __forceinline__ void split_mfma_il_body(const SplitArgs& a, uint32_t 
     const uint32_t n_runs = (span + RUN - 1) / RUN;
     const uint32_t first_run = (lo - tile_base) / RUN;
     const uint32_t r_tail = span % RUN;                                         // rows of a ragged last run (0: none)
-    const bool long_first = r_tail != 0u && r_tail <= 16u && n_runs >= first_run + 2u;
+    // (the launcher sets bit 1 of a.interleave when that saves a round: when the units then divide evenly among the streams)
+    const bool long_first = LONG && (a.interleave & 2u) != 0u && r_tail != 0u && r_tail <= 16u && n_runs >= first_run + 2u;
     const uint32_t n_eff = n_runs - (long_first ? 1u : 0u);                     // units of the span
     const uint32_t nv = n_eff > first_run ? n_eff - first_run : 0u;            // units that reach the window
     const uint32_t S = NW * a.n_tiles, sidx = jl * NW + (uint32_t)w;            // run streams of the KV head, this one
@@ -130,35 +133,22 @@ __device__ __forceinline__ void split_mfma_il_body(const SplitArgs& a, uint32_t 
         const uint32_t off0 = unit_off(cur_rb);
 #pragma unroll
         for (int t = 0; t < RT; ++t) issue_k(t, off0);
-        issue_k(RT, first_long ? off0 : kOOB);
+        if (LONG && first_long) issue_k(XT - 1, off0);      // (a uniform branch: the other wavefronts never touch that tile's registers)
     }
 
-    // ---- the new row of the decode token, in the wavefront that reads it (stream 0: the last row lies in its first unit)
+    // ---- the new row of the decode token, in the wavefront that reads it (stream 0: the last row lies in its first unit).
+    // Without ROPE its f32 values come straight from global memory: requested here (four elements per lane), converted after
+    // the queries have arrived (loads return in order), parked in LDS in the cache's format, and fetched from there by the
+    // lanes whose K / V registers hold pieces of that row.
     const bool appends = a.k_new != nullptr && active && sidx == 0u;            // wavefront-uniform
     const uint32_t rn = appends ? a.append_pos - cur_rb : 0u;                   // the row's index inside the unit
-    // (without ROPE the row's f32 values come straight from global memory: requested here, used after the queries)
-    float knew[KLD][EPP], vnew[EPP];
     const bool k_mine = appends && (uint32_t)n16 == (rn & 15u);                 // lanes whose K registers hold a piece of the row
     const bool v_mine = appends && (uint32_t)vrow == rn % VROWS;                // lanes whose V registers (load rn / VROWS) do
-    if (!ROPE) {
-        if (k_mine) {
-#pragma unroll
-            for (int x = 0; x < KLD; ++x) {
-                const int e0 = (KIL ? x * 4 + kg : kg * KLD + x) * EPP;
-#pragma unroll
-                for (int j4 = 0; j4 < EPP / 4; ++j4) {
-                    const float4 f = *reinterpret_cast<const float4*>(a.k_new + (size_t)kvh * D + e0 + 4 * j4);
-                    knew[x][4 * j4] = f.x; knew[x][4 * j4 + 1] = f.y; knew[x][4 * j4 + 2] = f.z; knew[x][4 * j4 + 3] = f.w;
-                }
-            }
-        }
-    }
-    if (v_mine) {
-#pragma unroll
-        for (int j4 = 0; j4 < EPP / 4; ++j4) {
-            const float4 f = *reinterpret_cast<const float4*>(a.v_new + (size_t)kvh * D + vcol * EPP + 4 * j4);
-            vnew[4 * j4] = f.x; vnew[4 * j4 + 1] = f.y; vnew[4 * j4 + 2] = f.z; vnew[4 * j4 + 3] = f.w;
-        }
+    const bool row_lane = appends && lane * 4 < D;                              // lanes that convert four elements of the row
+    float4 knew4 = make_float4(0.f, 0.f, 0.f, 0.f), vnew4 = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (row_lane) {
+        if (!ROPE) knew4 = *reinterpret_cast<const float4*>(a.k_new + (size_t)kvh * D + lane * 4);
+        vnew4 = *reinterpret_cast<const float4*>(a.v_new + (size_t)kvh * D + lane * 4);
     }
 
     // ---- Q^T operands.  The workgroup converts its heads' queries once into f16 value / remainder planes in LDS; lane
@@ -194,8 +184,10 @@ __device__ __forceinline__ void split_mfma_il_body(const SplitArgs& a, uint32_t 
         const uint32_t off0 = unit_off(cur_rb);
 #pragma unroll
         for (int c = 0; c < RT * VLT; ++c) issue_v(c, off0);
+        if (LONG && first_long) {
 #pragma unroll
-        for (int c = RT * VLT; c < XT * VLT; ++c) issue_v(c, first_long ? off0 : kOOB);
+            for (int c = RT * VLT; c < XT * VLT; ++c) issue_v(c, off0);
+        }
     }
     if (ROPE) {
         const uint32_t half = rf->rotary_dim / 2u;
@@ -221,14 +213,7 @@ __device__ __forceinline__ void split_mfma_il_body(const SplitArgs& a, uint32_t 
             const int ii = idx < nq4 ? idx : 0;
             qf[i] = *reinterpret_cast<const float4*>(&rot[(ii * 4) / D][(ii * 4) % D]);
         }
-        if (k_mine) {                                              // the rotated K row is in rot[gcount] (this is workgroup 0)
-#pragma unroll
-            for (int x = 0; x < KLD; ++x) {
-                const int e0 = (KIL ? x * 4 + kg : kg * KLD + x) * EPP;
-#pragma unroll
-                for (int j = 0; j < EPP; ++j) knew[x][j] = rot[gcount][e0 + j];
-            }
-        }
+        if (row_lane) knew4 = *reinterpret_cast<const float4*>(&rot[gcount][lane * 4]);    // the rotated K row (this is workgroup 0)
     }
     {
 #pragma unroll
@@ -258,44 +243,26 @@ __device__ __forceinline__ void split_mfma_il_body(const SplitArgs& a, uint32_t 
         }
     }
 
-    // ---- the new row: converted (the f32 values have arrived with the queries: loads return in order), put into the
-    // registers of the unit's loads, and stored to the cache ----
+    // ---- the new row in the cache's format: four elements per lane (kept for the store to the cache after the last unit:
+    // stores count in the same in-order counter as the loads, so issued now, every later wait for rows would also wait for
+    // their acknowledgement) and as a whole in LDS for the lanes that patch their registers inside the first unit.
+    uint32_t kw0 = 0u, kw1 = 0u, vw0 = 0u, vw1 = 0u;
+    const uint32_t tk = rn >> 4, cv = rn / VROWS;               // the tile / the V load that hold the row (wavefront-uniform)
     if (appends) {
-        auto pack_piece = [&](const float (&f)[EPP]) -> u32x4 {
-            u32x4 p;
+        if (row_lane) {
             if (DT == kF8) {
-#pragma unroll
-                for (int q4 = 0; q4 < 4; ++q4) p[q4] = pack4_e4m3(f[4 * q4], f[4 * q4 + 1], f[4 * q4 + 2], f[4 * q4 + 3]);
+                kw0 = pack4_e4m3(knew4.x, knew4.y, knew4.z, knew4.w);
+                vw0 = pack4_e4m3(vnew4.x, vnew4.y, vnew4.z, vnew4.w);
+                reinterpret_cast<uint32_t*>(&newrow[0][0])[lane] = kw0;
+                reinterpret_cast<uint32_t*>(&newrow[1][0])[lane] = vw0;
             } else {
-#pragma unroll
-                for (int q4 = 0; q4 < 4; ++q4) p[q4] = f32_to_h16_bits(f[2 * q4]) | (f32_to_h16_bits(f[2 * q4 + 1]) << 16);
+                kw0 = f32_to_h16_bits(knew4.x) | (f32_to_h16_bits(knew4.y) << 16); kw1 = f32_to_h16_bits(knew4.z) | (f32_to_h16_bits(knew4.w) << 16);
+                vw0 = f32_to_h16_bits(vnew4.x) | (f32_to_h16_bits(vnew4.y) << 16); vw1 = f32_to_h16_bits(vnew4.z) | (f32_to_h16_bits(vnew4.w) << 16);
+                reinterpret_cast<u32x2*>(&newrow[0][0])[lane] = u32x2{kw0, kw1};
+                reinterpret_cast<u32x2*>(&newrow[1][0])[lane] = u32x2{vw0, vw1};
             }
-            return p;
-        };
-        uint8_t* const krow = const_cast<uint8_t*>(a.k) + (size_t)a.append_pos * row_stride + head_b;
-        uint8_t* const vrowp = const_cast<uint8_t*>(a.v) + (size_t)a.append_pos * row_stride + head_b;
-        const uint32_t tk = rn >> 4, cv = rn / VROWS;           // the tile / the V load that hold the row (wavefront-uniform)
-#pragma unroll
-        for (int x = 0; x < KLD; ++x) {
-            u32x4 p = u32x4{0u, 0u, 0u, 0u};
-            if (k_mine) {
-                p = pack_piece(knew[x]);
-                *reinterpret_cast<u32x4*>(krow + (KIL ? x * 4 + kg : kg * KLD + x) * 16) = p;
-            }
-#pragma unroll
-            for (int t = 0; t < XT; ++t)
-                if ((uint32_t)t == tk) { const u32x4 old = kraw[t][x]; kraw[t][x] = k_mine ? p : old; }
         }
-        {
-            u32x4 p = u32x4{0u, 0u, 0u, 0u};
-            if (v_mine) {
-                p = pack_piece(vnew);
-                *reinterpret_cast<u32x4*>(vrowp + vcol * 16) = p;
-            }
-#pragma unroll
-            for (int c = 0; c < XT * VLT; ++c)
-                if ((uint32_t)c == cv) { const u32x4 old = vraw[c]; vraw[c] = v_mine ? p : old; }
-        }
+        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");     // (the row is read back by lanes of this wavefront only)
     }
 
     float4_t oacc[DTILES];
@@ -305,14 +272,25 @@ __device__ __forceinline__ void split_mfma_il_body(const SplitArgs& a, uint32_t 
     _Float16* const vb = &vlds[w][0];
     VFKV_DSTAMP(1);                              // queries staged, first unit requested
 
-    // One unit: NT tiles of 16 rows from row rb on.  The K / V registers it consumes are refilled at once with the rows of
-    // the next unit (RT tiles from byte offset noff, or nothing: loads past the end of the slab return zeros without traffic).
-    auto process = [&](auto nt_tag, uint32_t rb, uint32_t noff) {
-        constexpr int NT = decltype(nt_tag)::value;
-        constexpr int NPK = (NT * 16 + 31) / 32;             // k-steps of 32 rows (the last one half empty when NT is odd)
-        float4_t s[NT];
+    // One unit: RUN rows from row rb on, plus 16 more when `extra` (the long first unit; wavefront-uniform).  The K / V registers
+    // it consumes are refilled at once with the rows of the next unit (RUN rows from byte offset noff, or nothing: loads past
+    // the end of the slab return zeros without traffic).  One body for both forms, so that the loop has a single shape.
+    auto process = [&](uint32_t rb, uint32_t noff, bool extra, bool patch) {
+        constexpr int PKS = RUN / 32;                        // k-steps of 32 rows of the second product
+        if (patch) {                                         // the new row's pieces replace what the loads found there
 #pragma unroll
-        for (int t = 0; t < NT; ++t) {
+            for (int t = 0; t < XT; ++t)
+                if ((uint32_t)t == tk) {
+#pragma unroll
+                    for (int x = 0; x < KLD; ++x) {
+                        const u32x4 old = kraw[t][x];
+                        const u32x4 nw = *reinterpret_cast<const u32x4*>(&newrow[0][(KIL ? x * 4 + kg : kg * KLD + x) * 16]);
+                        kraw[t][x] = k_mine ? nw : old;
+                    }
+                }
+        }
+        float4_t s[XT];
+        auto score_tile = [&](int t) {
             half8_t ka[KS];
 #pragma unroll
             for (int c = 0; c < KS; ++c) {
@@ -332,20 +310,20 @@ __device__ __forceinline__ void split_mfma_il_body(const SplitArgs& a, uint32_t 
             s[t] = float4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
             for (int c = 0; c < KS; ++c) s[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ka[c], qb[c], s[t], 0, 0, 0);
-        }
-        const bool interior = rb >= lo && rb + NT * 16 <= tile_end;      // wavefront-uniform
-        uint32_t pbits[NPK][4];
+        };
 #pragma unroll
-        for (int ks = 0; ks < NPK; ++ks)
-#pragma unroll
-            for (int r4 = 0; r4 < 4; ++r4) pbits[ks][r4] = 0u;
+        for (int t = 0; t < RT; ++t) score_tile(t);          // (one basic block: the widening of one tile overlaps the products of another)
+        if (LONG) { s[XT - 1] = float4_t{0.f, 0.f, 0.f, 0.f}; if (extra) score_tile(XT - 1); }
+        const bool interior = rb >= lo && rb + RUN <= tile_end && !extra;      // wavefront-uniform
+        uint32_t pbits[PKS][4], pext[2] = {0u, 0u};
         auto softmax = [&](auto masked_tag) {
             constexpr bool MASKED = decltype(masked_tag)::value;
             constexpr bool FOLD = !MASKED && !CAP;                   // scores stay unscaled until the exponent
-            float x[NT][4];
+            constexpr int NTS = MASKED ? XT : RT;                    // the extra tile only exists in the masked form
+            float x[NTS][4];
             float tmax = kMasked;
 #pragma unroll
-            for (int t = 0; t < NT; ++t)
+            for (int t = 0; t < NTS; ++t)
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
                     float y = s[t][i];
@@ -354,7 +332,7 @@ __device__ __forceinline__ void split_mfma_il_body(const SplitArgs& a, uint32_t 
                     if (CAP) y = cap_l2 * tanhf(y / cap_l2);
                     if (MASKED) {
                         const uint32_t row = rb + t * 16 + kg * 4 + i;
-                        y = (row >= lo && row < tile_end) ? y : kMasked;
+                        y = (row >= lo && row < tile_end && (t < RT || extra)) ? y : kMasked;
                     }
                     x[t][i] = y;
                     tmax = fmaxf(tmax, y);
@@ -371,7 +349,8 @@ __device__ __forceinline__ void split_mfma_il_body(const SplitArgs& a, uint32_t 
             }
             // weights as f16 value (columns 0-7) or f16 remainder (columns 8-15), two rows per register
 #pragma unroll
-            for (int t = 0; t < NT; ++t)
+            for (int t = 0; t < NTS; ++t) {
+                if (t >= RT && !extra) continue;
 #pragma unroll
                 for (int i2 = 0; i2 < 2; ++i2) {
                     float2_t pp;
@@ -385,13 +364,23 @@ __device__ __forceinline__ void split_mfma_il_body(const SplitArgs& a, uint32_t 
                     l_run += pp[0] + pp[1];
                     const uint32_t ph = __builtin_bit_cast(uint32_t, __builtin_convertvector(pp, half2_t));
                     const uint32_t pl = pack_f16_remainder(pp[0], pp[1], ph);
-                    pbits[t / 2][(t % 2) * 2 + i2] = is_lo ? pl : ph;
+                    if (t < RT) pbits[t / 2][(t % 2) * 2 + i2] = is_lo ? pl : ph;
+                    else pext[i2] = is_lo ? pl : ph;
                 }
+            }
         };
         if (interior) softmax(std::false_type{}); else softmax(std::true_type{});
         // ---------------- V rows -> f16 row-major in LDS ----------------
+        if (patch) {
 #pragma unroll
-        for (int c = 0; c < NT * VLT; ++c) {
+            for (int c = 0; c < XT * VLT; ++c)
+                if ((uint32_t)c == cv) {
+                    const u32x4 old = vraw[c];
+                    const u32x4 nw = *reinterpret_cast<const u32x4*>(&newrow[1][vcol * 16]);
+                    vraw[c] = v_mine ? nw : old;
+                }
+        }
+        auto stage_v = [&](int c) {
             _Float16* dst = vb + (c * VROWS + vrow) * VPITCH + vcol * (16 / ES);
             if (DT == kF8) {
                 uint32_t out[8];
@@ -409,37 +398,59 @@ __device__ __forceinline__ void split_mfma_il_body(const SplitArgs& a, uint32_t 
                 *reinterpret_cast<u32x4*>(dst) = vraw[c];
             }
             if (c < RT * VLT) issue_v(c, noff);
+        };
+#pragma unroll
+        for (int c = 0; c < RT * VLT; ++c) stage_v(c);
+        if (LONG && extra) {
+#pragma unroll
+            for (int c = RT * VLT; c < XT * VLT; ++c) stage_v(c);
         }
         // ---------------- O^T += V^T P ----------------
 #pragma unroll
-        for (int ks = 0; ks < NPK; ++ks)
+        for (int ks = 0; ks < PKS; ++ks)
 #pragma unroll
             for (int dt = 0; dt < DTILES; ++dt) {
                 // supplier lane s of a 16-lane group points at V[row = ks*32 + 4*kg + s/4 (+16)][d = dt*16 + 4*(s%4)]
                 const _Float16* p0 = vb + (ks * 32 + kg * 4 + n16 / 4) * VPITCH + dt * 16 + 4 * (n16 % 4);
                 const half4_t v0 = lds_read_tr16(p0);
-                if (NT * 16 >= ks * 32 + 32) {
-                    const half4_t v1 = lds_read_tr16(p0 + 16 * VPITCH);
-                    half8_t va;
-                    va[0] = v0[0]; va[1] = v0[1]; va[2] = v0[2]; va[3] = v0[3]; va[4] = v1[0]; va[5] = v1[1]; va[6] = v1[2]; va[7] = v1[3];
-                    const u32x4 pw = u32x4{pbits[ks][0], pbits[ks][1], pbits[ks][2], pbits[ks][3]};
-                    oacc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(va, __builtin_bit_cast(half8_t, pw), oacc[dt], 0, 0, 0);
-                } else {                   // the last 16 rows of an odd number of tiles: the 16-deep product
-                    const u32x2 pw = u32x2{pbits[ks][0], pbits[ks][1]};
-                    oacc[dt] = __builtin_amdgcn_mfma_f32_16x16x16f16(v0, __builtin_bit_cast(half4_t, pw), oacc[dt], 0, 0, 0);
-                }
+                const half4_t v1 = lds_read_tr16(p0 + 16 * VPITCH);
+                half8_t va;
+                va[0] = v0[0]; va[1] = v0[1]; va[2] = v0[2]; va[3] = v0[3]; va[4] = v1[0]; va[5] = v1[1]; va[6] = v1[2]; va[7] = v1[3];
+                const u32x4 pw = u32x4{pbits[ks][0], pbits[ks][1], pbits[ks][2], pbits[ks][3]};
+                oacc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(va, __builtin_bit_cast(half8_t, pw), oacc[dt], 0, 0, 0);
             }
+        if (LONG && extra) {               // the 16 rows behind the run: the 16-deep product
+#pragma unroll
+            for (int dt = 0; dt < DTILES; ++dt) {
+                const _Float16* p0 = vb + (RUN + kg * 4 + n16 / 4) * VPITCH + dt * 16 + 4 * (n16 % 4);
+                const half4_t v0 = lds_read_tr16(p0);
+                const u32x2 pw = u32x2{pext[0], pext[1]};
+                oacc[dt] = __builtin_amdgcn_mfma_f32_16x16x16f16(v0, __builtin_bit_cast(half4_t, pw), oacc[dt], 0, 0, 0);
+            }
+        }
     };
 
     if (active) {
         uint32_t jnext = 1;
-        uint32_t nxt_rb = unit_rb(jnext);
-        if (first_long) process(std::integral_constant<int, XT>{}, cur_rb, unit_off(nxt_rb));
-        else process(std::integral_constant<int, RT>{}, cur_rb, unit_off(nxt_rb));
-        while (nxt_rb != kNone) {
+        bool extra = first_long, patch = appends;
+        for (;;) {
+            const uint32_t nxt_rb = unit_rb(jnext);
+            ++jnext;
+            process(cur_rb, unit_off(nxt_rb), extra, patch);
+            if (nxt_rb == kNone) break;
             cur_rb = nxt_rb;
-            nxt_rb = unit_rb(++jnext);
-            process(std::integral_constant<int, RT>{}, cur_rb, unit_off(nxt_rb));
+            extra = false; patch = false;
+        }
+    }
+    if (row_lane) {                                    // the new row's bytes to the cache
+        uint8_t* const krow = const_cast<uint8_t*>(a.k) + (size_t)a.append_pos * row_stride + head_b;
+        uint8_t* const vrowp = const_cast<uint8_t*>(a.v) + (size_t)a.append_pos * row_stride + head_b;
+        if (DT == kF8) {
+            reinterpret_cast<uint32_t*>(krow)[lane] = kw0;
+            reinterpret_cast<uint32_t*>(vrowp)[lane] = vw0;
+        } else {
+            reinterpret_cast<u32x2*>(krow)[lane] = u32x2{kw0, kw1};
+            reinterpret_cast<u32x2*>(vrowp)[lane] = u32x2{vw0, vw1};
         }
     }
 

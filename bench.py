@@ -446,6 +446,9 @@ def bench_decode(args, wl):
         threads = len(os.sched_getaffinity(0))
         per_layer = L * max_seq * Hkv * D * es // L
         done_bytes, spent, layers_done = 0, 0.0, 0
+        if rotating:        # the timed steps ended on some cache instance: one more step on instance 0, which the oracle reads below
+            step(0)
+            torch.cuda.synchronize()
         for layer in range(L):
             lo = layer * per_layer
             kh = kbuf[lo:lo + per_layer].cpu().numpy().view(oracle.NP_DTYPE[int(wl.dtype)]).reshape(max_seq, Hkv, D)

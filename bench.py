@@ -110,7 +110,6 @@ def parse_args():
                     help="leave the queries as general f32 values instead of casting them to fp16 first")
     ap.add_argument("--no-graph", action="store_true",
                     help="launch every kernel from Python instead of replaying one captured HIP graph per step")
-    ap.add_argument("--v-offsets", default="", help="decode_phase_stamps: further byte offsets of the V slabs to time at 32 768 keys, comma-separated")
     ap.add_argument("--no-other-workloads", action="store_true",
                     help="headline run only: skip the short runs of the other benchmark configurations ('workloads' array)")
     return ap.parse_args()
@@ -403,7 +402,9 @@ def bench_decode(args, wl):
 
     mfma_worker = mfma_decode_worker(wl.dtype.label(), D)
     f32_mfma = wl.dtype.label() == "FP32" and D in (64, 128, 256) and os.environ.get("VFKV_DECODE_WORKER", "m")[:1] != "v"
-    worker_name = "split_mfma_kernel" if mfma_worker else "split_mfma_f32_kernel" if f32_mfma else "split_kernel"
+    il_worker = mfma_worker and D != 512 and os.environ.get("VFKV_DECODE_IL", "1")[:1] != "0"   # (mirrors split_interleaves() of the library)
+    worker_name = (("split_mfma_il_rope_kernel" if wl.rope else "split_mfma_il_kernel") if il_worker else "split_mfma_kernel" if mfma_worker
+                   else "split_mfma_f32_kernel" if f32_mfma else "split_kernel")
     traffic, traffic_source = profiled_traffic(wl.name) if mfma_worker else (None, None)   # the profiles cover the default worker
     result = {
         "metric": "kv_read_GBps_decode_step",
@@ -705,235 +706,6 @@ def copy_calibration(args):
             "launches": args.steps, "value": 2 * n * args.steps / dt / 1e9, "unit": "GB/s", "n_gpus": 1}
 
 
-def slab_reuse_calibration(args):
-    """The compute-free readers of libvfkv_calib.so over 64 MiB layer slabs (32 768 rows x 8 KV heads x 128 FP8 bytes, K and
-    V) when consecutive launches rotate over 32, 6, 4, 2 slabs or read one slab again and again: what the memory-side
-    cache (and, for slabs that fit them, the L2s) contribute to a read that follows another read of the same bytes."""
-    import ctypes as C
-    import torch
-    calib = C.CDLL(os.path.join(ROOT, "vulkanforge_amd", "libvfkv_calib.so"))
-    calib.vfkv_calib_stream_read.argtypes = [C.c_void_p, C.c_void_p, C.c_uint64, C.c_void_p, C.c_void_p]
-    calib.vfkv_calib_pattern_read.argtypes = [C.c_void_p, C.c_void_p, C.c_uint32, C.c_uint32, C.c_uint32, C.c_void_p, C.c_void_p]
-    L, ctx, hkv, d = 32, 32768, 8, 128
-    lb = ctx * hkv * d
-    k = torch.randint(0, 255, (L * lb,), dtype=torch.uint8, device="cuda")
-    v = torch.randint(0, 255, (L * lb + 256,), dtype=torch.uint8, device="cuda")[256:]
-    sink = torch.zeros(1024, dtype=torch.int32, device="cuda")
-
-    def timed(launch, n_slabs, frac=1.0):
-        def fn():
-            st = torch.cuda.current_stream().cuda_stream
-            for i in range(L):
-                launch(k.data_ptr() + (i % n_slabs) * lb, v.data_ptr() + (i % n_slabs) * lb, frac, st)
-        fn()
-        torch.cuda.synchronize()
-        g = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(g):
-            fn()
-        g.replay()
-        torch.cuda.synchronize()
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        e0.record()
-        for _ in range(max(args.steps, 5)):
-            g.replay()
-        e1.record()
-        torch.cuda.synchronize()
-        return e0.elapsed_time(e1) * 1e3 / max(args.steps, 5) / L
-
-    pattern = lambda kp, vp, frac, st: calib.vfkv_calib_pattern_read(kp, vp, ctx, hkv, 32, sink.data_ptr(), st)
-    stream = lambda kp, vp, frac, st: calib.vfkv_calib_stream_read(kp, vp, int(lb * frac) // 16 * 16, sink.data_ptr(), st)
-    out = {"metric": "slab_reuse_calibration", "unit": "us per launch", "slab_bytes": 2 * lb, "n_gpus": 1,
-           "pattern_read": {str(n): timed(pattern, n) for n in (32, 6, 4, 2, 1)},
-           "stream_read": {str(n): timed(stream, n) for n in (32, 6, 4, 2, 1)},
-           "stream_read_one_slab_half_and_quarter": [timed(stream, 1, 0.5), timed(stream, 1, 0.25)]}
-    out["value"] = out["pattern_read"]["1"]
-    return out
-
-
-def issue_rate_calibration(args):
-    """What the vector instructions of the prefill loop cost a SIMD to issue, and how far matrix and vector instructions
-    overlap (compute-only kernels of libvfkv_calib.so, no memory traffic).  Per entry: ticks of the shader clock per
-    wavefront instruction as wavefront 0 saw them, and per instruction of the SIMD (kernel time x clock / instructions issued
-    on one SIMD) -- the two differ when the wavefronts of a SIMD run side by side."""
-    import ctypes as C
-    import torch
-    calib = C.CDLL(os.path.join(ROOT, "vulkanforge_amd", "libvfkv_calib.so"))
-    calib.vfkv_calib_issue.argtypes = [C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p]
-    calib.vfkv_calib_overlap.argtypes = [C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p]
-    sink = torch.zeros(1024, dtype=torch.int32, device="cuda")
-    clk = torch.zeros(2, dtype=torch.int64, device="cuda")
-
-    def timed(launch):
-        st = torch.cuda.current_stream().cuda_stream
-        assert launch(st) == 0
-        torch.cuda.synchronize()
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        e0.record()
-        assert launch(st) == 0
-        e1.record()
-        torch.cuda.synchronize()
-        ticks, wall = (int(x) for x in clk.cpu())
-        return e0.elapsed_time(e1), ticks, ticks / wall * 100.0       # ms, shader-clock ticks of wavefront 0, MHz
-
-    iters = 4000
-    out = {"metric": "issue_rate_calibration", "unit": "shader-clock ticks", "n_gpus": 1, "instructions": {}, "overlap": {}}
-    names = ["v_fma_f32", "v_exp_f32", "v_cvt_scalef32_pk_f16_fp8", "v_max_f32", "v_fma_mixlo_f16", "v_xor_b32"]
-    for op, name in enumerate(names):
-        entry = {}
-        for waves in (1, 2):
-            ms, ticks, mhz = timed(lambda st: calib.vfkv_calib_issue(op, waves, iters, sink.data_ptr(), clk.data_ptr(), st))
-            entry[f"{waves}_per_simd"] = {"wavefront_0_ticks_per_instruction": ticks / (iters * 64),
-                                          "simd_ticks_per_instruction": ms * 1e-3 * mhz * 1e6 / (iters * 64 * waves),
-                                          "kernel_ms": ms, "clock_mhz": mhz}
-        out["instructions"][name] = entry
-    it2 = 20000
-    for label, nv, mode in (("48_mfma_only", 0, 0), ("48_mfma_then_100_fma", 100, 0), ("48_mfma_then_200_fma", 200, 0),
-                            ("48_mfma_then_400_fma", 400, 0), ("48_mfma_200_fma_opposite_phases_by_barrier", 200, 1),
-                            ("48_mfma_200_fma_one_block", 200, 2)):
-        ms, ticks, mhz = timed(lambda st: calib.vfkv_calib_overlap(nv, mode, it2, sink.data_ptr(), clk.data_ptr(), st))
-        out["overlap"][label] = {"simd_ticks_per_pass_of_both_wavefronts": ms * 1e-3 * mhz * 1e6 / it2, "kernel_ms": ms,
-                                 "clock_mhz": mhz}
-    # the same two-phase pass with 100 vector instructions of each kind: alone, and behind 48 matrix instructions
-    calib.vfkv_calib_overlap_kind.argtypes = [C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p]
-    out["overlap_by_kind"] = {}
-    base = out["overlap"]["48_mfma_only"]["simd_ticks_per_pass_of_both_wavefronts"]
-    for op, name in enumerate(names):
-        t = {}
-        for with_matrix in (0, 1):
-            ms, ticks, mhz = timed(lambda st: calib.vfkv_calib_overlap_kind(op, with_matrix, it2, sink.data_ptr(), clk.data_ptr(), st))
-            t[with_matrix] = ms * 1e-3 * mhz * 1e6 / it2
-        out["overlap_by_kind"][name] = {"100_vector_alone": t[0], "48_mfma_then_100_vector": t[1], "hidden": base + t[0] - t[1]}
-    out["value"] = base / 96.0
-    return out
-
-
-def prefill_phase_stamps(args):
-    """Where one launch of the FP8 prefill kernel spends its time outside the tile loop: the kernel compiled with wall-clock
-    stamps (libvfkv_calib.so, csrc/calibration_prefill.hip) on the 512 x 4 608 geometry; microseconds after the first
-    wavefront's start."""
-    import ctypes as C
-    import numpy as np
-    import torch
-    from vulkanforge_amd import workloads
-    cfg = workloads.PREFILL["prefill_fp8_512x4608_32layers"]
-    H, Hkv, D, m, base = cfg.n_heads, cfg.n_kv_heads, cfg.head_dim, cfg.m, cfg.base_pos
-    n_kv = base + m
-    calib = C.CDLL(os.path.join(ROOT, "vulkanforge_amd", "libvfkv_calib.so"))
-    calib.vfkv_calib_prefill_stamps.argtypes = [C.c_void_p] * 4 + [C.c_uint32] * 5 + [C.c_float, C.c_int, C.c_void_p, C.c_void_p]
-    g = torch.Generator(device="cuda").manual_seed(3)
-    # standard-normal rows rounded to E4M3, as the benchmark's prefill workload holds them
-    k = torch.randn((n_kv, Hkv * D), device="cuda", generator=g).to(torch.float8_e4m3fn).view(torch.uint8)
-    # V starts 256 bytes past an allocation boundary, as in a cache made by vfkv_cache_create (K and V rows at the same offsets make
-    # one KV head's loads slower than the others')
-    vpool = torch.randn((n_kv * Hkv * D + (1 << 21),), device="cuda", generator=g).to(torch.float8_e4m3fn).view(torch.uint8)
-    voff = (-vpool.data_ptr()) % (1 << 21) + 256
-    v = vpool[voff: voff + n_kv * Hkv * D].view(n_kv, Hkv * D)
-    q = torch.randn((m, H, D), device="cuda", generator=g).half().float()
-    o = torch.empty_like(q)
-    nb = (m + 15) // 16
-    st = torch.zeros((nb, Hkv, 8, 8), dtype=torch.int64, device="cuda")
-    stream = torch.cuda.current_stream().cuda_stream
-    out = {"metric": "prefill_phase_stamps", "unit": "us after the first wavefront's start", "n_gpus": 1,
-           "config": {"workload": "prefill_fp8_512x4608 one layer, instrumented kernel"}, "variants": {}}
-    for label, f16w in (("default", 0), ("f16_weights", 1)):
-        for rep in range(4):                                 # the last of four launches is reported
-            st.zero_()
-            torch.cuda.synchronize()
-            rc = calib.vfkv_calib_prefill_stamps(q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), H, Hkv, m, n_kv, base,
-                                                 1.0 / D ** 0.5, f16w, st.data_ptr(), stream)
-            assert rc == 0, rc
-            torch.cuda.synchronize()
-        s = st.cpu().numpy().astype(np.float64) / 100.0
-        s = np.where(s > 0, s - s[..., 0].min(), np.nan)
-        med = lambda a: float(np.nanmedian(a))
-        wg_end = np.nanmax(s[..., 6], axis=2)                # [launch row][KV head]
-        walk_end = np.nanmax(s[..., 2], axis=2)
-        out["variants"][label] = {
-            "kernel_span": float(np.nanmax(s)),
-            "wavefront_start": {"median": med(s[..., 0]), "max": float(np.nanmax(s[..., 0]))},
-            "query_block_arrived": {"min": float(np.nanmin(s[..., 7])), "median": med(s[..., 7]), "max": float(np.nanmax(s[..., 7]))},
-            "q_planes_ready": {"min": float(np.nanmin(s[..., 1])), "median": med(s[..., 1]), "max": float(np.nanmax(s[..., 1]))},
-            "last_tile_done_wavefronts_0_3_median": med(s[:, :, :4, 2]), "last_tile_done_wavefronts_4_7_median": med(s[:, :, 4:, 2]),
-            "last_tile_of_workgroup_to_workgroup_done_median": med(wg_end - walk_end),
-            "workgroup_done": {"min": float(wg_end.min()), "median": med(wg_end), "max": float(wg_end.max())},
-            "workgroup_done_by_launch_row_mean": [round(float(x), 2) for x in wg_end.mean(axis=1)],
-            "workgroup_done_by_kv_head_mean": [round(float(x), 2) for x in wg_end.mean(axis=0)],
-        }
-    out["value"] = out["variants"]["default"]["kernel_span"]
-    return out
-
-
-def decode_phase_stamps(args):
-    """Where one launch of the decode worker spends its time: split_mfma_kernel compiled with wall-clock stamps (libvfkv_calib.so,
-    csrc/calibration_decode.hip) on the headline geometry (32 / 8 / 128, FP8, 32 768 keys) and on 8 192 keys; eight launches over eight
-    layer slabs captured into one graph and replayed, as a step issues them; microseconds after the launch's first wavefront started,
-    means over the eight launches of the last replay."""
-    import ctypes as C
-    import numpy as np
-    import torch
-    import vulkanforge_amd as vf
-    calib = C.CDLL(os.path.join(ROOT, "vulkanforge_amd", "libvfkv_calib.so"))
-    calib.vfkv_calib_decode_stamps.argtypes = [C.c_void_p] * 6 + [C.c_uint32] * 7 + [C.c_float, C.c_void_p, C.c_void_p]
-    H, Hkv, D, NL, NW = 32, 8, 128, 8, 4
-    out = {"metric": "decode_phase_stamps", "unit": "us after the launch's first wavefront started", "n_gpus": 1,
-           "config": {"workload": "split_mfma_kernel, 32 / 8 / 128 FP8, instrumented kernel, 8 launches per graph replay"}, "contexts": {}}
-    g = torch.Generator(device="cuda").manual_seed(5)
-    # (seq_len, byte offset of the V slabs from a 2 MiB boundary; the K slabs start on one).  256 is what vfkv_cache_create gives V:
-    # with K and V rows at the same offsets one KV head's stream runs 10 % slower than the others and the launch waits for it
-    # (the head whose 128-byte pieces lie at addresses with bits 9:7 == 011, on whichever XCD it runs)
-    cases = [(32768, 256), (8192, 256), (8193, 256), (32768, 0)] + [(32768, int(x)) for x in args.v_offsets.split(",") if x.strip()]
-    for seq, shift in cases:
-        tile = vf.lib().vfkv_decode_tile_for(seq, H, Hkv, D, int(vf.KvDtype.F8))
-        nt = (seq + tile - 1) // tile
-        tile, nt = 64, 32            # vfkv_decode_attention's launch: one workgroup per CU, the rows dealt to them in runs
-        slab = seq * Hkv * D
-        pool = [torch.randn(((NL * slab + (1 << 21)) // 4,), device="cuda", generator=g).to(torch.float8_e4m3fn).view(torch.uint8).repeat(4)
-                for _ in range(2)]
-        base = [(-pool[0].data_ptr()) % (1 << 21), (-pool[1].data_ptr()) % (1 << 21) + shift]      # offset of the first slab inside its pool
-        ks = [pool[0][base[0] + l * slab: base[0] + (l + 1) * slab] for l in range(NL)]
-        vs = [pool[1][base[1] + l * slab: base[1] + (l + 1) * slab] for l in range(NL)]
-        q = torch.randn((H, D), device="cuda", generator=g).half().float()
-        so = torch.empty((H, nt, D), device="cuda"); sm = torch.empty((H, nt), device="cuda"); ss = torch.empty((H, nt), device="cuda")
-        st = torch.zeros((NL, Hkv, nt, 1, NW, 4), dtype=torch.int64, device="cuda")
-
-        def launches():
-            stream = torch.cuda.current_stream().cuda_stream
-            for l in range(NL):
-                rc = calib.vfkv_calib_decode_stamps(q.data_ptr(), ks[l].data_ptr(), vs[l].data_ptr(), so.data_ptr(), sm.data_ptr(),
-                                                    ss.data_ptr(), int(vf.KvDtype.F8), H, Hkv, D, seq, tile, nt, 1.0 / D ** 0.5,
-                                                    st[l].data_ptr(), stream)
-                assert rc == 0, rc
-        launches()
-        torch.cuda.synchronize()
-        graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(graph):
-            launches()
-        for _ in range(3):
-            graph.replay()
-        torch.cuda.synchronize()
-        s = st.cpu().numpy().astype(np.float64) / 100.0                  # [launch][KV head][workgroup][1][wavefront][stamp]
-        names = ("wavefront_start", "loop_start", "loop_end", "partial_stored")
-        pct = lambda a: {"min": float(a.min()), "p50": float(np.percentile(a, 50)), "p90": float(np.percentile(a, 90)), "max": float(a.max())}
-        rel = s - s[..., 0].min(axis=(1, 2, 3, 4), keepdims=True)[..., None]
-        entry = {n: pct(rel[..., i]) for i, n in enumerate(names)}
-        entry["loop_per_wavefront"] = pct(rel[..., 2] - rel[..., 1])
-        entry["epilogue_per_wavefront"] = pct(rel[..., 3] - rel[..., 2])
-        entry["loop_start_by_kv_head_mean"] = [round(float(x), 2) for x in rel[..., 1].mean(axis=(0, 2, 3, 4))]
-        entry["loop_per_wavefront_by_kv_head_mean"] = [round(float(x), 2) for x in (rel[..., 2] - rel[..., 1]).mean(axis=(0, 2, 3, 4))]
-        entry["finish_by_kv_head_mean"] = [round(float(x), 2) for x in rel[..., 3].mean(axis=(0, 2, 3, 4))]
-        starts = s[..., 0].min(axis=(1, 2, 3, 4)); ends = s[..., 3].max(axis=(1, 2, 3, 4))
-        entry["launch_span_mean"] = float((ends - starts).mean())
-        entry["next_launch_start_after_last_store_mean"] = float((starts[1:] - ends[:-1]).mean())
-        entry["tile"] = int(tile); entry["workgroups_per_kv_head"] = int(nt)
-        if shift != 256:
-            entry = {k: entry[k] for k in ("loop_per_wavefront_by_kv_head_mean", "finish_by_kv_head_mean", "launch_span_mean")}
-        name = str(seq) if shift == 256 else f"{seq}_v_slabs_not_offset" if shift == 0 else f"{seq}_v_slabs_offset_by_{shift}"
-        if name not in out["contexts"]:
-            out["contexts"][name] = entry
-    out["value"] = out["contexts"]["32768"]["launch_span_mean"]
-    return out
-
-
 HEADLINE = "decode_fp8_32k_32layers"
 # the other benchmark configurations, run briefly after the headline workload so that one invocation witnesses all five
 OTHER_CONFIGS = ("decode_f16_2k_1layer", "decode_fp8_8k_32layers", "decode_f16_hd256_sliding_12layers",
@@ -950,14 +722,6 @@ def run_workload(args, name):
         return bench_rope_append(args, workloads.ROPE_APPEND[name])
     if name == "copy_calibration":
         return copy_calibration(args)
-    if name == "slab_reuse_calibration":
-        return slab_reuse_calibration(args)
-    if name == "issue_rate_calibration":
-        return issue_rate_calibration(args)
-    if name == "prefill_phase_stamps":
-        return prefill_phase_stamps(args)
-    if name == "decode_phase_stamps":
-        return decode_phase_stamps(args)
     return None
 
 
@@ -986,7 +750,7 @@ def main():
     from vulkanforge_amd import workloads
     res = run_workload(args, args.workload)
     if res is None:
-        print("unknown workload; choose from: " + ", ".join(list(workloads.DECODE) + list(workloads.PREFILL) + list(workloads.ROPE_APPEND) + ["copy_calibration", "slab_reuse_calibration", "issue_rate_calibration", "prefill_phase_stamps", "decode_phase_stamps"]),
+        print("unknown workload; choose from: " + ", ".join(list(workloads.DECODE) + list(workloads.PREFILL) + list(workloads.ROPE_APPEND) + ["copy_calibration"]),
               file=sys.stderr)
         sys.exit(2)
     if args.workload == HEADLINE and not args.no_other_workloads:

@@ -34,11 +34,10 @@ def test_workload_tables_state_the_configurations_algorithmic_work():
 
 
 def test_calibration_library_loads_and_exports_what_the_benchmark_calls():
-    # (no device work: symbols only; the library resolves libvfkv.so beside it)
+    # (no device work: symbols only)
     import ctypes
     lib = ctypes.CDLL(os.path.join(ROOT, "vulkanforge_amd", "libvfkv_calib.so"))
-    for name in ("vfkv_calib_stream_read", "vfkv_calib_pattern_read", "vfkv_calib_empty", "vfkv_calib_issue",
-                 "vfkv_calib_overlap", "vfkv_calib_overlap_kind", "vfkv_calib_prefill_stamps", "vfkv_calib_decode_stamps"):
+    for name in ("vfkv_calib_stream_read", "vfkv_calib_pattern_read", "vfkv_calib_empty"):
         assert hasattr(lib, name), name
     with open(os.path.join(ROOT, "bench.py")) as f:
         text = f.read()

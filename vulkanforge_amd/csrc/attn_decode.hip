@@ -50,13 +50,7 @@ struct SplitArgs {
     uint32_t group;          // n_heads / n_kv_heads
     uint32_t interleave;     // matrix-core worker: deal the runs of the launched span round-robin instead of by tile
     float scale, softcap;
-#ifdef VFKV_DECODE_STAMPS
-    unsigned long long* stamps;   // instrumented build (calibration_decode.hip): [KV head][workgroup of the head][head slice][wavefront][4] wall-clock readings
-#endif
 };
-#ifdef VFKV_DECODE_STAMPS
-static unsigned long long* g_decode_stamps = nullptr;
-#endif
 
 template <int DT>
 struct ElemBytes { static constexpr int value = DT == kF32 ? 4 : DT == kF16 ? 2 : 1; };
@@ -821,9 +815,6 @@ hipError_t launch_split(const SplitLaunch& L, hipStream_t stream, bool* generic_
     a.scale = L.scale; a.softcap = L.softcap;
     a.k_new = nullptr; a.v_new = nullptr; a.append_pos = 0u; a.o_direct = nullptr;
     a.interleave = L.interleave ? 1u : 0u;
-#ifdef VFKV_DECODE_STAMPS
-    a.stamps = g_decode_stamps;
-#endif
     if (L.o_direct) {
         if (!split_writes_output(L) || ((uintptr_t)L.o_direct & 15u) != 0u) return hipErrorInvalidValue;
         a.o_direct = L.o_direct;

@@ -37,14 +37,6 @@ struct RopeFoldArgs {
     float theta_scale, freq_scale, attn_factor, eps;
 };
 
-#ifdef VFKV_DECODE_STAMPS
-#define VFKV_DSTAMP(i)                                                                                                       \
-    do { if (a.stamps != nullptr && lane == 0)                                                                               \
-        a.stamps[((((size_t)blockIdx.x * gridDim.y + blockIdx.y) * gridDim.z + blockIdx.z) * NW + w) * 4 + (i)] = wall_clock64(); } while (0)
-#else
-#define VFKV_DSTAMP(i) do { } while (0)
-#endif
-
 template <int DT, int D, int RUN, int NW, bool CAP, bool ROPE>
 __device__ __forceinline__ void split_mfma_il_body(const SplitArgs& a, uint32_t gt, const RopeFoldArgs* rf) {
     constexpr int ES = DT == kF16 ? 2 : 1;
@@ -75,7 +67,6 @@ __device__ __forceinline__ void split_mfma_il_body(const SplitArgs& a, uint32_t 
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
-    VFKV_DSTAMP(0);                              // wavefront start
     const int n16 = lane & 15, kg = lane >> 4;
     const int col = n16 & 7;
     const bool is_lo = n16 >= 8;
@@ -270,7 +261,6 @@ __device__ __forceinline__ void split_mfma_il_body(const SplitArgs& a, uint32_t 
     for (int dt = 0; dt < DTILES; ++dt) oacc[dt] = float4_t{0.f, 0.f, 0.f, 0.f};
     float m_run = kMasked, l_run = 0.f;
     _Float16* const vb = &vlds[w][0];
-    VFKV_DSTAMP(1);                              // queries staged, first unit requested
 
     // One unit: RUN rows from row rb on, plus 16 more when `extra` (the long first unit; wavefront-uniform).  The K / V registers
     // it consumes are refilled at once with the rows of the next unit (RUN rows from byte offset noff, or nothing: loads past
@@ -454,7 +444,6 @@ __device__ __forceinline__ void split_mfma_il_body(const SplitArgs& a, uint32_t 
         }
     }
 
-    VFKV_DSTAMP(2);                              // last unit done
     // ---------------- wavefront totals, then the workgroup merge through LDS (as in split_mfma_kernel) ----------------
     l_run = xor32_sum(xor16_sum(l_run));
 #pragma unroll
@@ -508,12 +497,7 @@ __device__ __forceinline__ void split_mfma_il_body(const SplitArgs& a, uint32_t 
         a.sm[pidx] = M > -1e29f ? M * 0.693147180559945f : kMasked;
         a.ss[pidx] = l;
     }
-#ifdef VFKV_DECODE_STAMPS
-    __builtin_amdgcn_s_waitcnt(0);
-#endif
-    VFKV_DSTAMP(3);                              // partial stored and acknowledged
 }
-#undef VFKV_DSTAMP
 
 template <int DT, int D, int RUN, int NW, bool CAP>
 __global__ __launch_bounds__(NW * 64) void split_mfma_il_kernel(SplitArgs a, uint32_t gt) {

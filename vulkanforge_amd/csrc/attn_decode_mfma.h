@@ -34,16 +34,6 @@ namespace vfkv {
 // NH > 1 (head_dim 512): NH wavefronts walk the same runs.  Each computes the scores over the whole head_dim and stages,
 // accumulates, merges and stores its own slice of D / NH output columns (the accumulators of a 512-wide head do not fit
 // one wavefront); the workgroup then walks NW / NH runs at a time.
-// Instrumented build only (calibration_decode.hip): lane 0 of every wavefront stores the 100 MHz wall clock at four points of
-// the kernel.  The library proper compiles these to nothing.
-#ifdef VFKV_DECODE_STAMPS
-#define VFKV_DSTAMP(i)                                                                                                       \
-    do { if (a.stamps != nullptr && lane == 0)                                                                               \
-        a.stamps[((((size_t)blockIdx.x * gridDim.y + blockIdx.y) * gridDim.z + blockIdx.z) * NW + w) * 4 + (i)] = wall_clock64(); } while (0)
-#else
-#define VFKV_DSTAMP(i) do { } while (0)
-#endif
-
 template <int DT, int D, int RUN, int PF, int NW, bool CAP, int NH = 1>
 __global__ __launch_bounds__(NW * 64) void split_mfma_kernel(SplitArgs a, uint32_t gt) {
     constexpr int ES = DT == kF16 ? 2 : 1;
@@ -76,7 +66,6 @@ __global__ __launch_bounds__(NW * 64) void split_mfma_kernel(SplitArgs a, uint32
     const int tid = threadIdx.x, lane = tid & 63;
     const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wp = w / NH, ds = w % NH;          // run stream of this wavefront, its slice of the output columns
-    VFKV_DSTAMP(0);                              // wavefront start
     const int n16 = lane & 15, kg = lane >> 4;
     const int col = n16 & 7;
     const bool is_lo = n16 >= 8;
@@ -231,7 +220,6 @@ __global__ __launch_bounds__(NW * 64) void split_mfma_kernel(SplitArgs a, uint32
     for (int dt = 0; dt < DTILES; ++dt) oacc[dt] = float4_t{0.f, 0.f, 0.f, 0.f};
     float m_run = kMasked, l_run = 0.f;
     _Float16* const vb = &vlds[w][0];
-    VFKV_DSTAMP(1);                              // queries staged, first run requested
 
     if (active) {
         for (uint32_t it = 0; nth_run(it) < n_runs; it += PF) {
@@ -359,7 +347,6 @@ __global__ __launch_bounds__(NW * 64) void split_mfma_kernel(SplitArgs a, uint32
         }
     }
 
-    VFKV_DSTAMP(2);                              // last run done
     // ---------------- wavefront totals, then the workgroup merge through LDS ----------------
     // Every wavefront parks its accumulators in LDS in register order (lane-major: conflict-free 16-byte accesses),
     // then wavefront w merges the d-tiles w, w + NW, ... of all wavefronts and stores them straight from registers
@@ -418,11 +405,6 @@ __global__ __launch_bounds__(NW * 64) void split_mfma_kernel(SplitArgs a, uint32
         a.sm[pidx] = M > -1e29f ? M * 0.693147180559945f : kMasked;
         a.ss[pidx] = l;
     }
-#ifdef VFKV_DECODE_STAMPS
-    __builtin_amdgcn_s_waitcnt(0);
-#endif
-    VFKV_DSTAMP(3);                              // partial stored and acknowledged
 }
-#undef VFKV_DSTAMP
 
 }  // namespace vfkv

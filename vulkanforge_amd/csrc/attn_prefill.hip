@@ -32,13 +32,7 @@ struct BatchArgs {
     uint32_t gchunk, gstride, goff;
     uint32_t q_f16;          // f16 matrix-core kernels: use f16(q) alone, whatever the queries hold
     uint32_t merge_all;      // batch_mfma2_kernel: the LDS area holds the (o, m, l) of every wavefront, and every wavefront merges a share
-#ifdef VFKV_PREFILL_STAMPS
-    unsigned long long* stamps;   // instrumented build (calibration_prefill.hip): [workgroup][8 wavefronts][8] wall-clock readings
-#endif
 };
-#ifdef VFKV_PREFILL_STAMPS
-static unsigned long long* g_prefill_stamps = nullptr;
-#endif
 
 }  // namespace vfkv
 #include "attn_prefill_mfma2.h"
@@ -119,9 +113,6 @@ static hipError_t launch_batch_kernels(const BatchLaunch& L, hipStream_t stream,
     a.gate = nullptr; a.gchunk = 1u; a.gstride = 0u; a.goff = 0u;
     a.q_f16 = L.f16_queries ? 1u : 0u;
     a.merge_all = 0u;
-#ifdef VFKV_PREFILL_STAMPS
-    a.stamps = nullptr;
-#endif
     const uint32_t g = L.n_heads / L.n_kv_heads;
     const uint64_t slab_bytes = (uint64_t)L.n_kv * L.n_kv_heads * L.head_dim * elem_size(L.dtype);
     const bool aligned = ((((uintptr_t)L.k) | ((uintptr_t)L.v) | ((uintptr_t)L.q) | ((uintptr_t)L.o)) & 15u) == 0u;
@@ -155,7 +146,8 @@ static hipError_t launch_batch_kernels(const BatchLaunch& L, hipStream_t stream,
         const bool vdma = L.dtype == kF8 && L.head_dim == 128u && ncb == 2u;
         // the private V tiles and the two Q planes have to fit in 160 KiB of LDS
         auto waves_for = [&](uint32_t slices) -> uint32_t {
-            const size_t qbytes = (size_t)2 * (slices / nh) * ncb * 16 * (L.head_dim + 8) * sizeof(_Float16);
+            const size_t qbytes = (size_t)2 * (slices / nh) * ncb * 16 * (L.head_dim + 8) * sizeof(_Float16) +
+                                  (vdma ? (size_t)slices * ncb * 16 * (L.head_dim + 16) : 0u);   // (that kernel: a third plane of one byte per element)
             // private V tile, and with two wavefronts per head the two buffers through which they swap score halves
             const size_t per_wave = (vdma ? (size_t)3 * 32 * 128 : (size_t)32 * (dv + 16) * sizeof(_Float16)) +
                                     (nh == 2u ? (size_t)2 * ncb * 64 * 16 : 0u);   // (unused by the two-heads FP8 form)
@@ -218,6 +210,7 @@ static hipError_t launch_batch_kernels(const BatchLaunch& L, hipStream_t stream,
             const dim3 grid(L.n_kv_heads, (L.m + 15u) / 16u, nz * nk), block(nwaves * kWave);
             const size_t vbytes = (size_t)nwaves * (vdma ? (size_t)3 * 32 * 128 : (size_t)32 * (dv + 16) * sizeof(_Float16)) +
                                   (size_t)2 * (hp / nh) * ncb * 16 * (L.head_dim + 8) * sizeof(_Float16) +
+                                  (vdma ? (size_t)hp * ncb * 16 * (L.head_dim + 16) : 0u) +
                                   (nh == 2u ? (size_t)2 * nwaves * ncb * 64 * 16 : 0u);
             // merge area: the general kernel keeps the records of all splits but the first; the V-through-LDS kernel the
             // output tiles and (m, l) of every wavefront
@@ -237,9 +230,6 @@ static hipError_t launch_batch_kernels(const BatchLaunch& L, hipStream_t stream,
             // FP8 matrix instruction (needs the Q block staged in one round: four key splits).  Over F16 rows (four heads per
             // wavefront) f16_weights is an instantiation of the general kernel; other shapes keep the default arithmetic.
             const bool f8s = L.fp8_scores && vdma && ns >= 4u;
-#ifdef VFKV_PREFILL_STAMPS
-            a.stamps = vdma ? g_prefill_stamps : nullptr;
-#endif
             // eight wavefronts (two per SIMD) and an even number of key splits: the older wavefront of a SIMD gets 3 tiles
             // for every 2 of the younger one
             int deal_a = 1, deal_b = 1;

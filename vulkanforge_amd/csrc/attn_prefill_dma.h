@@ -25,16 +25,6 @@
 
 namespace vfkv {
 
-// Instrumented build only (calibration_prefill.hip): lane 0 of every wavefront stores the 100 MHz wall clock at seven points
-// of the kernel.  The library proper compiles these to nothing.
-#ifdef VFKV_PREFILL_STAMPS
-#define VFKV_STAMP(i)                                                                                                        \
-    do { if (a.stamps != nullptr && lane == 0)                                                                               \
-        a.stamps[((size_t)((blockIdx.z * gridDim.y + blockIdx.y) * gridDim.x + blockIdx.x) * 8 + w) * 8 + (i)] = wall_clock64(); } while (0)
-#else
-#define VFKV_STAMP(i) do { } while (0)
-#endif
-
 template <bool CAP, bool F16W, bool F8S>
 __global__ __launch_bounds__(512) void batch_dma_kernel(BatchArgs a, int HP, int NS, int DEAL_A, int DEAL_B) {
     constexpr int D = 128, NCB = 2, PFD = 2;     // head_dim, heads per wavefront, K tiles in flight
@@ -75,12 +65,12 @@ __global__ __launch_bounds__(512) void batch_dma_kernel(BatchArgs a, int HP, int
     const int gz = (blockIdx.z / a.nk) * HP * NCB;              // first head (inside the group) of this workgroup
     const int g0 = hp * NCB;                                    // first head slot (inside the workgroup) of this wavefront
 
-    VFKV_STAMP(0);                                              // start
     uint8_t* const v8 = reinterpret_cast<uint8_t*>(lds) + (size_t)w * 3 * VBUF;   // [3][KT * D] raw V tiles of this wavefront
     constexpr int QPITCH = D + 8;
     _Float16* const qhi_lds = lds + (size_t)nwaves * 3 * VBUF / 2;  // [GP][16][D + 8] f16(q); the slots past G hold zeros
     const int GP = HP * NCB;                                        // head slots of the workgroup: G rounded up to whole wavefronts
     _Float16* const qlo_lds = qhi_lds + (size_t)GP * 16 * QPITCH;   // [GP][16][D + 8] f16(q - f16(q))
+    uint8_t* const qlo8_lds = reinterpret_cast<uint8_t*>(qlo_lds + (size_t)GP * 16 * QPITCH);   // [GP][16][D + 16] the remainders as E4M3 codes
 
     // ---- key range ----
     uint32_t kmax = a.q_start + q0 + 16;                        // one past the last key any of the 16 queries sees
@@ -224,8 +214,9 @@ __global__ __launch_bounds__(512) void batch_dma_kernel(BatchArgs a, int HP, int
         }
         __syncthreads();                                        // planes written
     } else {
-    if (tid == 0) lds_haslo = 0;
+    if (tid == 0) { lds_haslo = 0; lds_qmax = 0u; }
     bool any_lo = false;
+    float lo_max = 0.f;                                         // largest |q - f16(q)| this thread has seen
     for (int base = 0; base < q4_total; base += QLD * nthreads) {
         float4 qf[QLD];
 #pragma unroll
@@ -241,9 +232,6 @@ __global__ __launch_bounds__(512) void batch_dma_kernel(BatchArgs a, int HP, int
 #pragma unroll
             for (int sl = 0; sl < PFD; ++sl) issue(sl, tile_off(tp[sl]));
         }
-#ifdef VFKV_PREFILL_STAMPS
-        if (base == 0) { asm volatile("s_waitcnt vmcnt(16)" ::: "memory"); VFKV_STAMP(7); }   // the query block has arrived (16 K / V requests behind it)
-#endif
 #pragma unroll
         for (int i = 0; i < QLD; ++i) {
             const int idx = base + tid + i * nthreads;
@@ -253,17 +241,41 @@ __global__ __launch_bounds__(512) void batch_dma_kernel(BatchArgs a, int HP, int
             const float v[4] = {qf[i].x, qf[i].y, qf[i].z, qf[i].w};
             _Float16 hv[4], lv[4];
 #pragma unroll
-            for (int j = 0; j < 4; ++j) { hv[j] = (_Float16)v[j]; lv[j] = (_Float16)(v[j] - (float)hv[j]); any_lo |= lv[j] != (_Float16)0; }
+            for (int j = 0; j < 4; ++j) {
+                hv[j] = (_Float16)v[j]; lv[j] = (_Float16)(v[j] - (float)hv[j]); any_lo |= lv[j] != (_Float16)0;
+                lo_max = fmaxf(lo_max, fabsf((float)lv[j]));
+            }
             *reinterpret_cast<half4_t*>(qhi_lds + ((size_t)g * 16 + qq) * QPITCH + d) = half4_t{hv[0], hv[1], hv[2], hv[3]};
             *reinterpret_cast<half4_t*>(qlo_lds + ((size_t)g * 16 + qq) * QPITCH + d) = half4_t{lv[0], lv[1], lv[2], lv[3]};
         }
     }
     __syncthreads();                                            // lds_haslo cleared, planes written
     if (any_lo && a.q_f16 == 0u) lds_haslo = 1;
+    lo_max = wave_max_uniform(lo_max);
+    if (lane == 0) atomicMax(&lds_qmax, __builtin_bit_cast(uint32_t, lo_max));   // non-negative floats order like their bits
     __syncthreads();
     has_lo = __builtin_amdgcn_readfirstlane(lds_haslo) != 0;   // workgroup-uniform
+    if (has_lo) {
+        // General f32 queries.  The cache rows are E4M3 codes, so K (q - f16(q))^T can run on the FP8 matrix instruction with
+        // the rows as loaded: one instruction spans the whole row where the f16 one needs four, and the remainders only
+        // need the few bits E4M3 gives them (q is then carried with 15 significant bits).  Every thread turns the remainders
+        // it wrote above into codes 2^-e (q - f16(q)), e keeping the largest of the block below 256; 2^e rides in the
+        // instruction's block-scale operand.
+        const uint32_t mb = lds_qmax;
+        q_exp = (int)((mb >> 23) & 0xFFu) - 127 - 7;
+        q_exp = q_exp < -100 ? -100 : q_exp > 100 ? 100 : q_exp;
+        const float down = __builtin_bit_cast(float, (uint32_t)(127 - q_exp) << 23);
+        for (int idx = tid; idx < q4_total; idx += nthreads) {
+            const int qq = idx / (GP * (D / 4)), rem = idx - qq * (GP * (D / 4));
+            const int g = rem / (D / 4), d = (rem - g * (D / 4)) * 4;
+            const half4_t lv = *reinterpret_cast<const half4_t*>(qlo_lds + ((size_t)g * 16 + qq) * QPITCH + d);
+            int w8 = __builtin_amdgcn_cvt_pk_fp8_f32((float)lv[0] * down, (float)lv[1] * down, 0, false);
+            w8 = __builtin_amdgcn_cvt_pk_fp8_f32((float)lv[2] * down, (float)lv[3] * down, w8, true);
+            *reinterpret_cast<uint32_t*>(qlo8_lds + ((size_t)g * 16 + qq) * Q8PITCH + d) = (uint32_t)w8;
+        }
+        __syncthreads();
     }
-    VFKV_STAMP(1);                                              // Q planes ready
+    }
 
     float4_t oacc[NCB][DTILES];
 #pragma unroll
@@ -331,6 +343,23 @@ __global__ __launch_bounds__(512) void batch_dma_kernel(BatchArgs a, int HP, int
                 qhi[cb][c] = *reinterpret_cast<const half8_t*>(qhi_lds + ((size_t)(g0 + cb) * 16 + n16) * QPITCH + kg * SEG + c * 8);
 #pragma unroll
         for (int kt = 0; kt < 2; ++kt) {
+            if (with_lo) {
+                // K (q - f16(q))^T first: A = the lane's quarter row of K as loaded (32 codes), B = the same quarter of the
+                // query's remainder codes, their power of two as the block scale; the f16 products below add to it
+                typedef int v8i_t __attribute__((ext_vector_type(8)));
+                v8i_t ka8;
+#pragma unroll
+                for (int j = 0; j < 8; ++j) ka8[j] = (int)kraw[sl][kt][j / 4][j % 4];
+#pragma unroll
+                for (int cb = 0; cb < NCB; ++cb) {
+                    const uint8_t* qrow = qlo8_lds + ((size_t)(g0 + cb) * 16 + n16) * Q8PITCH + kg * 32;
+                    const u32x4 b0 = *reinterpret_cast<const u32x4*>(qrow), b1 = *reinterpret_cast<const u32x4*>(qrow + 16);
+                    v8i_t qb8;
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) { qb8[j] = (int)b0[j]; qb8[4 + j] = (int)b1[j]; }
+                    s[sl][cb][kt] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(ka8, qb8, float4_t{0.f, 0.f, 0.f, 0.f}, 0, 0, 0, 127, 0, 127 + q_exp);
+                }
+            }
             half8_t ka[KS];
 #pragma unroll
             for (int c = 0; c < KS; ++c) {
@@ -346,23 +375,10 @@ __global__ __launch_bounds__(512) void batch_dma_kernel(BatchArgs a, int HP, int
                 kraw[sl][kt][xx] = __builtin_amdgcn_raw_buffer_load_b128(krsrc, lane_koff + xx * 16, noff + (uint32_t)kt * 16u * row_stride, 0);
 #pragma unroll
             for (int cb = 0; cb < NCB; ++cb) {
-                float4_t acc = float4_t{0.f, 0.f, 0.f, 0.f};
+                float4_t acc = with_lo ? s[sl][cb][kt] : float4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
                 for (int c = 0; c < KS; ++c) acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(ka[c], qhi[cb][c], acc, 0, 0, 0);
                 s[sl][cb][kt] = acc;
-            }
-            if (with_lo) {
-#pragma unroll
-                for (int cb = 0; cb < NCB; ++cb) {
-                    const _Float16* lo_row = qlo_lds + ((size_t)(g0 + cb) * 16 + n16) * QPITCH + kg * SEG;
-                    float4_t acc = s[sl][cb][kt];
-#pragma unroll
-                    for (int c = 0; c < KS; ++c) {
-                        const half8_t ql = *reinterpret_cast<const half8_t*>(lo_row + c * 8);
-                        acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(ka[c], ql, acc, 0, 0, 0);
-                    }
-                    s[sl][cb][kt] = acc;
-                }
             }
         }
     };
@@ -462,7 +478,7 @@ __global__ __launch_bounds__(512) void batch_dma_kernel(BatchArgs a, int HP, int
     // else).  The walk is compiled once with and once without the remainder product of Q: without it the first products
     // are straight-line code and the inner loop is the grouped one.
     auto walk = [&](auto lo_tag) {
-    constexpr bool GROUP = std::is_same_v<decltype(lo_tag), std::false_type>;   // (the remainder product's registers leave no room for a second tile's scores)
+    constexpr bool GROUP = std::is_same_v<decltype(lo_tag), std::false_type>;   // (with the remainder product in it the two-tile loop spills in both walks)
     int first_slot = 0;          // slots of the group at tb that the inner loop has already finished
     bool s_ready = false;        // the inner loop left the group at tb with scores computed: those of slot first_slot; GROUP:
                                  // those of every slot
@@ -523,7 +539,6 @@ __global__ __launch_bounds__(512) void batch_dma_kernel(BatchArgs a, int HP, int
     }
     };
     if (has_lo) walk(std::true_type{}); else walk(std::false_type{});
-    VFKV_STAMP(2);                                              // last tile done
 #pragma unroll
     for (int cb = 0; cb < NCB; ++cb) l_run[cb] = xor32_sum(xor16_sum(l_run[cb]));   // every lane of a query column has its wavefront's sum
 
@@ -559,9 +574,7 @@ __global__ __launch_bounds__(512) void batch_dma_kernel(BatchArgs a, int HP, int
                     if (sp + j * NS < DTILES) gpre[cb][j] = *reinterpret_cast<const float4*>(gp + (sp + j * NS) * 16);
             }
         }
-        VFKV_STAMP(3);                                          // (o, m, l) in LDS
         __syncthreads();
-        VFKV_STAMP(4);
         if (!q_ok) return;
         // (compiled per split count so that the LDS reads of a head are independent instructions, not a chain of round trips)
         auto merge_and_store = [&](auto ns_tag) {
@@ -610,11 +623,6 @@ __global__ __launch_bounds__(512) void batch_dma_kernel(BatchArgs a, int HP, int
         if (NS == 4) merge_and_store(std::integral_constant<int, 4>{});
         else if (NS == 2) merge_and_store(std::integral_constant<int, 2>{});
         else merge_and_store(std::integral_constant<int, 8>{});  // (the launcher gives 2, 4 or 8 splits)
-        VFKV_STAMP(5);                                          // merged, stores issued
-#ifdef VFKV_PREFILL_STAMPS
-        __builtin_amdgcn_s_waitcnt(0);
-#endif
-        VFKV_STAMP(6);                                          // stores complete
         return;
     }
     float4_t gfac[NCB][DTILES];
@@ -672,6 +680,5 @@ __global__ __launch_bounds__(512) void batch_dma_kernel(BatchArgs a, int HP, int
     }
 }
 
-#undef VFKV_STAMP
 
 }  // namespace vfkv

@@ -11,17 +11,6 @@
 //   calib_empty          the same grid with no work: the cost of a launch
 //
 // The loaded values are folded into an XOR that is stored only if it equals a constant, so the compiler keeps the loads.
-//
-// Two more, for the prefill kernels' roofline entry (no memory traffic at all): what the instructions of their inner loop
-// cost a SIMD to issue, and how far matrix and vector instructions overlap:
-//
-//   calib_issue          one kind of vector instruction, 64 per loop pass on eight independent registers, in workgroups of one
-//                        or two wavefronts per SIMD; wavefront 0 reports its shader-clock and 100 MHz wall-clock ticks
-//   calib_overlap        per loop pass 48 v_mfma_f32_16x16x32_f16 and NV v_fma_f32 per wavefront, two wavefronts per SIMD:
-//                        in two phases, the same with the two wavefronts of a SIMD held in opposite phases by workgroup
-//                        barriers, or in one basic block left to the compiler's scheduler
-//   calib_overlap_kind   the two-phase pass with 100 vector instructions of one of calib_issue's kinds
-// (calibration_prefill.hip adds the FP8 prefill kernel compiled with wall-clock stamps.)
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
@@ -105,119 +94,6 @@ __global__ __launch_bounds__(256) void calib_empty(uint32_t* __restrict__ sink, 
     if (never == 0x12345678u) sink[threadIdx.x] = never;
 }
 
-typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
-typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
-typedef float float4_t __attribute__((ext_vector_type(4)));
-
-// OP: 0 v_fma_f32, 1 v_exp_f32, 2 v_cvt_scalef32_pk_f16_fp8, 3 v_max_f32, 4 v_fma_mixlo_f16, 5 v_xor_b32
-template <int OP>
-__global__ __launch_bounds__(512) void calib_issue(uint32_t* __restrict__ sink, uint64_t* __restrict__ clk, int iters, float seed) {
-    float v[8];
-    uint32_t u[8];
-    for (int i = 0; i < 8; ++i) { v[i] = seed + i + threadIdx.x; u[i] = 0x38404448u + i + threadIdx.x; }
-    const float c0 = seed * 1.0001f, c1 = seed * 0.37f;
-    const uint64_t t0 = __builtin_readcyclecounter(), r0 = wall_clock64();
-    for (int it = 0; it < iters; ++it) {
-#pragma unroll
-        for (int n = 0; n < 64; ++n) {
-            const int i = n % 8, j = (n + 1) % 8;
-            if (OP == 0) v[i] = __builtin_fmaf(v[i], c0, c1);
-            if (OP == 1) v[i] = __builtin_amdgcn_exp2f(v[i]);
-            if (OP == 2) asm volatile("v_cvt_scalef32_pk_f16_fp8 %0, %1, 1.0" : "=v"(u[i]) : "v"(u[j]));
-            if (OP == 3) v[i] = fmaxf(v[i], v[(n + 3) % 8]);
-            if (OP == 4) asm volatile("v_fma_mixlo_f16 %0, %1, 1.0, -%2 op_sel:[0,0,0] op_sel_hi:[0,0,1]" : "=v"(u[i]) : "v"(v[i]), "v"(u[j]));
-            if (OP == 5) u[i] ^= u[j];
-        }
-    }
-    const uint64_t t1 = __builtin_readcyclecounter(), r1 = wall_clock64();
-    float r = 0.f;
-    for (int i = 0; i < 8; ++i) r += v[i] + (float)u[i];
-    if (r == 1234.5f) sink[threadIdx.x] = (uint32_t)r;
-    if (blockIdx.x == 0 && threadIdx.x == 0) { clk[0] = t1 - t0; clk[1] = r1 - r0; }
-}
-
-// MODE 0: 48 matrix instructions, then NV vector instructions; 1: the same, the second wavefront of every SIMD (threads
-// 256..511) starting with the vector phase and a workgroup barrier after every phase; 2: both kinds in one basic block
-template <int NV, int MODE>
-__global__ __launch_bounds__(512) void calib_overlap(uint32_t* __restrict__ sink, uint64_t* __restrict__ clk, int iters, float seed) {
-    constexpr int NM = 48;
-    half8_t a, b;
-    for (int i = 0; i < 8; ++i) { a[i] = (_Float16)(seed + threadIdx.x * 0.001f + i); b[i] = (_Float16)(seed * 0.5f + i); }
-    float4_t acc[8];
-    for (int i = 0; i < 8; ++i) acc[i] = float4_t{0.f, 0.f, 0.f, 0.f};
-    float v[8];
-    for (int i = 0; i < 8; ++i) v[i] = seed + i + threadIdx.x;
-    const float c0 = seed * 1.0001f, c1 = seed * 0.37f;
-    const bool second = (threadIdx.x >> 8) & 1;
-    auto matrix = [&]() {
-#pragma unroll
-        for (int m = 0; m < NM; ++m) acc[m % 8] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, acc[m % 8], 0, 0, 0);
-    };
-    auto vector = [&]() {
-#pragma unroll
-        for (int n = 0; n < NV; ++n) v[n % 8] = __builtin_fmaf(v[n % 8], c0, c1);
-    };
-    const uint64_t t0 = __builtin_readcyclecounter(), r0 = wall_clock64();
-    for (int it = 0; it < iters; ++it) {
-        if (MODE == 0) {
-            matrix();
-            __builtin_amdgcn_sched_barrier(0);
-            vector();
-            __builtin_amdgcn_sched_barrier(0);
-        } else if (MODE == 1) {
-            if (second) vector(); else matrix();
-            __syncthreads();
-            if (second) matrix(); else vector();
-            __syncthreads();
-        } else {
-            matrix();
-            vector();
-        }
-    }
-    const uint64_t t1 = __builtin_readcyclecounter(), r1 = wall_clock64();
-    float r = 0.f;
-    for (int i = 0; i < 8; ++i) r += acc[i][0] + acc[i][1] + acc[i][2] + acc[i][3] + v[i];
-    if (r == 1234.5f) sink[threadIdx.x] = (uint32_t)r;
-    if (blockIdx.x == 0 && threadIdx.x == 0) { clk[0] = t1 - t0; clk[1] = r1 - r0; }
-}
-
-// Per pass NM v_mfma_f32_16x16x32_f16 (0 or 48), then 100 vector instructions of kind OP (the kinds of calib_issue) per
-// wavefront, two wavefronts per SIMD, free running: how much of each kind of vector work hides behind the other wavefront's
-// matrix instructions.
-template <int OP, int NM>
-__global__ __launch_bounds__(512) void calib_overlap_kind(uint32_t* __restrict__ sink, uint64_t* __restrict__ clk, int iters, float seed) {
-    half8_t a, b;
-    for (int i = 0; i < 8; ++i) { a[i] = (_Float16)(seed + threadIdx.x * 0.001f + i); b[i] = (_Float16)(seed * 0.5f + i); }
-    float4_t acc[8];
-    for (int i = 0; i < 8; ++i) acc[i] = float4_t{0.f, 0.f, 0.f, 0.f};
-    float v[8];
-    uint32_t u[8];
-    for (int i = 0; i < 8; ++i) { v[i] = seed + i + threadIdx.x; u[i] = 0x38404448u + i + threadIdx.x; }
-    const float c0 = seed * 1.0001f, c1 = seed * 0.37f;
-    const uint64_t t0 = __builtin_readcyclecounter(), r0 = wall_clock64();
-    for (int it = 0; it < iters; ++it) {
-#pragma unroll
-        for (int m = 0; m < NM; ++m) acc[m % 8] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, acc[m % 8], 0, 0, 0);
-        __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-        for (int n = 0; n < 100; ++n) {
-            const int i = n % 8, j = (n + 3) % 8;
-            if (OP == 0) v[i] = __builtin_fmaf(v[i], c0, c1);
-            if (OP == 1) v[i] = __builtin_amdgcn_exp2f(v[i]);
-            if (OP == 2) asm volatile("v_cvt_scalef32_pk_f16_fp8 %0, %1, 1.0" : "=v"(u[i]) : "v"(u[j]));
-            if (OP == 3) v[i] = fmaxf(v[i], v[j]);
-            if (OP == 4) asm volatile("v_fma_mixlo_f16 %0, %1, 1.0, -%2 op_sel:[0,0,0] op_sel_hi:[0,0,1]" : "=v"(u[i]) : "v"(v[i]), "v"(u[j]));
-            if (OP == 5) u[i] ^= u[j];
-        }
-        __builtin_amdgcn_sched_barrier(0);
-    }
-    const uint64_t t1 = __builtin_readcyclecounter(), r1 = wall_clock64();
-    float r = 0.f;
-    for (int i = 0; i < 8; ++i) r += acc[i][0] + acc[i][1] + acc[i][2] + acc[i][3] + v[i] + (float)u[i];
-    if (r == 1234.5f) sink[threadIdx.x] = (uint32_t)r;
-    if (blockIdx.x == 0 && threadIdx.x == 0) { clk[0] = t1 - t0; clk[1] = r1 - r0; }
-}
-
 }  // namespace
 
 #pragma GCC visibility push(default)    // the library is built with hidden visibility: only these entry points are exported
@@ -249,52 +125,6 @@ int vfkv_calib_pattern_read(const void* k, const void* v, uint32_t seq_len, uint
 int vfkv_calib_empty(uint32_t n_kv_heads, uint32_t n_tiles, void* sink, void* stream) {
     if (!sink || n_kv_heads == 0 || n_tiles == 0) return -1;
     hipLaunchKernelGGL(calib_empty, dim3(n_kv_heads, n_tiles), dim3(256), 0, (hipStream_t)stream, (uint32_t*)sink, 0u);
-    return hipGetLastError() == hipSuccess ? 0 : -5;
-}
-
-// 256 workgroups of `waves_per_simd` x 256 threads issue `iters` x 64 instructions of kind `op` (0 v_fma_f32, 1 v_exp_f32,
-// 2 v_cvt_scalef32_pk_f16_fp8, 3 v_max_f32, 4 v_fma_mixlo_f16, 5 v_xor_b32).  clk (device, two uint64): shader-clock and 100 MHz
-// ticks of wavefront 0 of workgroup 0.  0 on success.
-int vfkv_calib_issue(int op, int waves_per_simd, int iters, void* sink, void* clk, void* stream) {
-    if (!sink || !clk || iters <= 0 || (waves_per_simd != 1 && waves_per_simd != 2)) return -1;
-    const dim3 grid(256), block(256 * waves_per_simd);
-#define VFKV_CALIB_OP(N) case N: hipLaunchKernelGGL((calib_issue<N>), grid, block, 0, (hipStream_t)stream, (uint32_t*)sink, (uint64_t*)clk, iters, 1.0f); break;
-    switch (op) {
-        VFKV_CALIB_OP(0) VFKV_CALIB_OP(1) VFKV_CALIB_OP(2) VFKV_CALIB_OP(3) VFKV_CALIB_OP(4) VFKV_CALIB_OP(5)
-        default: return -1;
-    }
-#undef VFKV_CALIB_OP
-    return hipGetLastError() == hipSuccess ? 0 : -5;
-}
-
-// 256 workgroups of two wavefronts per SIMD run `iters` passes of 48 matrix instructions + `n_vector` (0, 100, 200 or 400)
-// v_fma_f32 per wavefront; mode 0: two phases, 1: the wavefronts of a SIMD in opposite phases behind barriers, 2: one basic
-// block.  clk as above.  0 on success.
-int vfkv_calib_overlap(int n_vector, int mode, int iters, void* sink, void* clk, void* stream) {
-    if (!sink || !clk || iters <= 0 || mode < 0 || mode > 2) return -1;
-    const dim3 grid(256), block(512);
-#define VFKV_CALIB_OV(NV, M) if (n_vector == NV && mode == M) { hipLaunchKernelGGL((calib_overlap<NV, M>), grid, block, 0, (hipStream_t)stream, (uint32_t*)sink, (uint64_t*)clk, iters, 1.0f); return hipGetLastError() == hipSuccess ? 0 : -5; }
-    VFKV_CALIB_OV(0, 0) VFKV_CALIB_OV(100, 0) VFKV_CALIB_OV(200, 0) VFKV_CALIB_OV(400, 0)
-    VFKV_CALIB_OV(200, 1) VFKV_CALIB_OV(200, 2)
-#undef VFKV_CALIB_OV
-    return -1;
-}
-
-// 256 workgroups of two wavefronts per SIMD run `iters` passes of (48 matrix instructions if with_matrix) + 100 vector
-// instructions of kind `op` (as in vfkv_calib_issue) per wavefront.  clk as above.  0 on success.
-int vfkv_calib_overlap_kind(int op, int with_matrix, int iters, void* sink, void* clk, void* stream) {
-    if (!sink || !clk || iters <= 0) return -1;
-    const dim3 grid(256), block(512);
-#define VFKV_CALIB_OK(N)                                                                                                     \
-    case N:                                                                                                                  \
-        if (with_matrix) hipLaunchKernelGGL((calib_overlap_kind<N, 48>), grid, block, 0, (hipStream_t)stream, (uint32_t*)sink, (uint64_t*)clk, iters, 1.0f); \
-        else hipLaunchKernelGGL((calib_overlap_kind<N, 0>), grid, block, 0, (hipStream_t)stream, (uint32_t*)sink, (uint64_t*)clk, iters, 1.0f);  \
-        break;
-    switch (op) {
-        VFKV_CALIB_OK(0) VFKV_CALIB_OK(1) VFKV_CALIB_OK(2) VFKV_CALIB_OK(3) VFKV_CALIB_OK(4) VFKV_CALIB_OK(5)
-        default: return -1;
-    }
-#undef VFKV_CALIB_OK
     return hipGetLastError() == hipSuccess ? 0 : -5;
 }
 

@@ -548,17 +548,36 @@ def bench_prefill(args, wl):
     step_spread = dict(STEP_SPREAD)
     flops_step = wl.flops_layer() * L
 
+    # ---- duration of the attention kernel (the dominant kernel): the step's attention launches without the appends, back
+    # to back on the benchmark's stream (one graph), bracketed by one pair of HIP events per replay and averaged, as the
+    # decode workloads time their worker.  (Events around every single launch add their own packets between the kernels.)
     stream = torch.cuda.current_stream()
-    pairs = []
-    for _ in range(min(args.steps, 5)):
+
+    def attention_only():
         for layer in range(L):
-            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            e0.record(stream)
             attention(layer)
-            e1.record(stream)
-            pairs.append((e0, e1))
+
+    run = attention_only
+    if not args.no_graph:
+        attention_only()
+        torch.cuda.synchronize()
+        gr = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(gr):
+            attention_only()
+        run = gr.replay
+    run()
     torch.cuda.synchronize()
-    avg_ms = sum(a.elapsed_time(b) for a, b in pairs) / len(pairs)
+    pairs = []
+    n_ev = min(max(args.steps, 5), 20)
+    for _ in range(n_ev):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record(stream)
+        run()
+        e1.record(stream)
+        pairs.append((e0, e1))
+    torch.cuda.synchronize()
+    launches = n_ev * L
+    avg_ms = sum(a.elapsed_time(b) for a, b in pairs) / launches
     achieved = wl.flops_layer() / (avg_ms * 1e-3) / 1e12
     f32_cache = wl.dtype.label() == "FP32"
     peak = MFMA_F32_PEAK_TFLOPS if f32_cache else MFMA_F16_PEAK_TFLOPS
@@ -577,7 +596,8 @@ def bench_prefill(args, wl):
         "roofline": {"bound": "mfma", "kernel": prefill_kernel_name(wl.dtype.label(), D, H // Hkv),
                      "achieved": achieved, "peak": peak,
                      "unit": "TFLOP/s", "frac": achieved / peak, "traffic": traffic, "traffic_source": traffic_source,
-                     "avg_launch_us": avg_ms * 1e3},
+                     "avg_launch_us": avg_ms * 1e3, "launches_timed": launches,
+                     "algorithmic_flop_per_launch": wl.flops_layer()},
     }
     if gate_separate_ms is not None:
         result["config"]["ms_per_step_gate_as_separate_launch"] = gate_separate_ms

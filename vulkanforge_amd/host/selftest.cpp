@@ -97,6 +97,28 @@ int main() {
         }
         hipFree(dko);
     }
+    // The whole attention block of a decode token in one call (Q / K norm + RoPE, append, attention), closed form: no norm,
+    // theta_scale = 1, so every NEOX pair (1, 1) of q turns by `ctx` radians into (cos - sin, sin + cos); the new K row is zero,
+    // row 123 still dominates (score 16 * 128 * cos(ctx) * scale, about 100 above the rest), so O = V[123] again.
+    {
+        float *dqo, *dz; hipMalloc(&dqo, q.size() * 4); hipMalloc(&dz, row * 4);
+        hipMemset(dz, 0, row * 4);
+        vfkv_rope_params rp{VFKV_ROPE_NEOX, D, 1.0f, 1.0f, 1.0f, 1e-6f};
+        fwd.step_qk_rope_kv_write_attention(1, ctx, dq, nullptr, dqo, dz, dv + ctx * row, nullptr, rp, dout);
+        hipDeviceSynchronize();
+        std::vector<float> qo(q.size());
+        hipMemcpy(qo.data(), dqo, qo.size() * 4, hipMemcpyDeviceToHost);
+        hipMemcpy(o.data(), dout, o.size() * 4, hipMemcpyDeviceToHost);
+        const double c = std::cos((double)ctx), sn = std::sin((double)ctx);
+        double wq = 0; worst = 0;
+        for (uint32_t h = 0; h < H; ++h) for (uint32_t d = 0; d < D; ++d) {
+            wq = std::fmax(wq, std::fabs(qo[h * D + d] - (d < D / 2 ? c - sn : sn + c)));
+            worst = std::fmax(worst, std::fabs(o[h * D + d] - v[123 * row + (h / 4) * D + d]));
+        }
+        std::printf("fused decode block: max |q_rot - closed form| = %.3g, max |O - V[123]| = %.3g\n", wq, worst);
+        REQUIRE(wq < 2e-4 && worst < 1e-6);
+        hipFree(dqo); hipFree(dz);
+    }
     bool threw = false;
     try { fwd.step_attention(1, ctx + 1, dq, dout); } catch (const Error& e) { threw = e.status == VFKV_ERR_INVALID_ARG; }
     REQUIRE(threw);

@@ -196,6 +196,16 @@ public:
         check(vfkv_kv_write_decode_attention(kv_cache.handle(), layer, n_heads, q, k_src, v_src, attn_out, position, kv_start,
                                              scale_for(layer), softcap, ws_, stream));
     }
+    // step_q_norm_rope + step_k_norm_rope + step_kv_write + step_attention of one decode token (attention.rs:360-625) in one
+    // call: q and k_src are the rows before norm and rotation; q_out / k_out receive what the reference leaves in q_buf / k_buf
+    void step_qk_rope_kv_write_attention(uint32_t layer, uint32_t position, const float* q, const float* q_norm_weight,
+                                         float* q_out, const float* k_src, const float* v_src, const float* k_norm_weight,
+                                         const vfkv_rope_params& rope, float* attn_out, uint32_t kv_start = 0, float softcap = 0.f,
+                                         const float* freq_factors = nullptr, float* k_out = nullptr) {
+        check(vfkv_qk_rope_kv_write_decode_attention(kv_cache.handle(), layer, n_heads, q, q_norm_weight, q_out, k_src, v_src,
+                                                     k_norm_weight, freq_factors, &rope, k_out, attn_out, position, kv_start,
+                                                     scale_for(layer), softcap, ws_, stream));
+    }
     // runs.rs:933-1010
     void run_flash_attn_batch(uint32_t layer, const float* q_buf, float* o_buf, uint32_t m, uint32_t q_start, uint32_t n_kv,
                               uint32_t kv_layer, uint32_t kv_start, float softcap = 0.f) {

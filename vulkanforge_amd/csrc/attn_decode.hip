@@ -703,9 +703,33 @@ static hipError_t launch_split_il(const SplitArgs& a_in, uint32_t g, const RopeF
     return hipGetLastError();
 }
 
+// Rows per run of the interleaved worker.  The full run is 32 rows (64 at head_dim 64): 8 KiB of K and V per wavefront in
+// flight over FP8 rows of 64 / 128 elements, 16 KiB over F16 rows of 64 / 128 and FP8 rows of 256, 32 KiB over F16 rows of 256.
+// Every shape also has a worker with runs of half that, and a launch takes whichever measured faster for its shape and its
+// number of full runs per run stream (us per layer inside graphs that stream at least 768 MB per replay, so that nothing is
+// left in the memory-side cache; 32 / 8 heads, 16 / 8 at head_dim 256; S = run streams of a KV head):
+//   * where a stream has at most one and a half full runs (300 to 6 144 keys with 128 streams) half runs win on every shape,
+//     4-12 % per layer: the launch is a latency chain there and a smaller unit shortens it;
+//   * 32 KiB in flight per wavefront is too much at every length (F16 256: 13.8 -> 11.7 us at 4 096 keys, 28.9 -> 26.9 at 16 384);
+//   * the 8 KiB shapes lose with half runs from two full runs per stream on (FP8 128: 8.8 -> 9.3 us at 8 192 keys, 10.0 -> 11.2
+//     at 12 288, 16.4 -> 18.6 at 32 768), the 16 KiB shapes are level or 1-4 % ahead there (F16 128 at 32 768: 26.6 -> 25.7).
+static uint32_t il_full_run(uint32_t D) { return D == 64u ? 64u : 32u; }
+
+static bool il_half_runs(uint32_t dtype, uint32_t D, uint32_t span_rows, uint32_t n_tiles) {
+    static const bool off = [] { const char* e = getenv("VFKV_DECODE_HALF_RUNS"); return e && e[0] == '0'; }();   // for comparisons
+    if (off) return false;
+    const uint32_t full = il_full_run(D), units = (span_rows + full - 1u) / full, S = (uint32_t)kMfmaWaves * n_tiles;
+    if (dtype == kF16 && D == 256u) return true;
+    if (dtype == kF8 && D != 256u) return 2u * units <= 3u * S;
+    if (dtype == kF16 && D == 128u) return 2u * units <= 3u * S || units >= 4u * S;
+    return true;
+}
+
+// The shortest run the worker may take for this shape: what the caller sizes its workgroup count by.
 uint32_t split_run_rows(uint32_t dtype, uint32_t D) {
     if ((dtype != kF8 && dtype != kF16) || (D != 64u && D != 128u && D != 256u && D != 512u)) return 0u;
-    return D == 64u ? 64u : 32u;
+    if (D == 512u) return 32u;
+    return il_full_run(D) / 2u;
 }
 
 template <int D>
@@ -831,12 +855,14 @@ hipError_t launch_split(const SplitLaunch& L, hipStream_t stream, bool* generic_
     const bool out_aligned = ((((uintptr_t)L.scratch_out) | ((uintptr_t)L.o_direct)) & 15u) == 0u;
     if (L.rope != nullptr && !split_folds_rope(L)) return hipErrorInvalidValue;      // the caller rotates in a launch of its own then
     if (split_interleaves(L) && out_aligned) {
-        if (L.dtype == kF8 && L.head_dim == 64u) return launch_split_il<kF8, 64, 64>(a, g, L.rope, stream);
-        if (L.dtype == kF16 && L.head_dim == 64u) return launch_split_il<kF16, 64, 64>(a, g, L.rope, stream);
-        if (L.dtype == kF8 && L.head_dim == 128u) return launch_split_il<kF8, 128, 32>(a, g, L.rope, stream);
-        if (L.dtype == kF16 && L.head_dim == 128u) return launch_split_il<kF16, 128, 32>(a, g, L.rope, stream);
-        if (L.dtype == kF8 && L.head_dim == 256u) return launch_split_il<kF8, 256, 32>(a, g, L.rope, stream);
-        if (L.dtype == kF16 && L.head_dim == 256u) return launch_split_il<kF16, 256, 32>(a, g, L.rope, stream);
+        const uint32_t base_row = a.tile_first * a.tile;
+        const bool half = il_half_runs(L.dtype, L.head_dim, a.seq_len > base_row ? a.seq_len - base_row : 0u, a.n_tiles);
+#define VFKV_IL(DT, DD, FULL) \
+    if (L.dtype == DT && L.head_dim == DD) \
+        return half ? launch_split_il<DT, DD, FULL / 2>(a, g, L.rope, stream) : launch_split_il<DT, DD, FULL>(a, g, L.rope, stream);
+        VFKV_IL(kF8, 64u, 64) VFKV_IL(kF16, 64u, 64) VFKV_IL(kF8, 128u, 32) VFKV_IL(kF16, 128u, 32) VFKV_IL(kF8, 256u, 32)
+#undef VFKV_IL
+        if (L.dtype == kF16 && L.head_dim == 256u) return launch_split_il<kF16, 256, 16>(a, g, L.rope, stream);
     }
     if (aligned && out_aligned && slab_bytes < 0x7FFF0000ull && mfma_worker_enabled()) {
         if (L.dtype == kF8 && L.head_dim == 64u) return launch_split_mfma<kF8, 64, 64, 1>(a, g, stream);

@@ -41,8 +41,9 @@ template <int DT, int D, int RUN, int NW, bool CAP, bool ROPE>
 __device__ __forceinline__ void split_mfma_il_body(const SplitArgs& a, uint32_t gt, const RopeFoldArgs* rf) {
     constexpr int ES = DT == kF16 ? 2 : 1;
     constexpr int RT = RUN / 16;                 // 16-row tiles per run
+    constexpr bool HALF = RUN == 16;             // runs of one tile: the second product is the 16-deep matrix instruction
     constexpr int KLD0 = (D / 4) * ES / 16, VLT0 = 16 / (64 / (D * ES / 16));
-    constexpr bool LONG = (RT + 1) * (KLD0 + VLT0) <= 24;   // the long first unit costs KLD + VLT more 16-byte registers: not where rows are 512 bytes wide
+    constexpr bool LONG = RUN % 32 == 0 && (RT + 1) * (KLD0 + VLT0) <= 24;   // the long first unit costs KLD + VLT more 16-byte registers: not where rows are 512 bytes wide
     constexpr int XT = LONG ? RT + 1 : RT;       // tiles of the first unit of stream 0 at most
     constexpr int KS = D / 32;                   // k-steps of the first product
     constexpr int DTILES = D / 16;
@@ -54,7 +55,8 @@ __device__ __forceinline__ void split_mfma_il_body(const SplitArgs& a, uint32_t 
     constexpr int VROWS = 64 / VCHUNK_ROW;       // rows covered by one V load of the wavefront
     constexpr int VLT = 16 / VROWS;              // V loads per lane per tile of 16 rows
     constexpr int MAXJ = (D + 63) / 64;          // elements of a row per lane in the norm / RoPE stage
-    static_assert(D % 32 == 0 && SEGB % 16 == 0 && RUN % 32 == 0 && VCHUNK_ROW >= 4 && VCHUNK_ROW <= 64, "unsupported shape");
+    static_assert(D % 32 == 0 && SEGB % 16 == 0 && (RUN % 32 == 0 || HALF) && VCHUNK_ROW >= 4 && VCHUNK_ROW <= 64, "unsupported shape");
+    static_assert(!(HALF && LONG), "the long first unit needs runs of whole k-steps");
     static_assert(NW * (RUN + 16) * VPITCH * 2 >= NW * (D / 16) * 64 * 16, "merge buffer must fit in the V staging area");
     static_assert(DTILES % NW == 0, "d-tiles must divide evenly among the wavefronts");
 
@@ -305,7 +307,7 @@ __device__ __forceinline__ void split_mfma_il_body(const SplitArgs& a, uint32_t 
         for (int t = 0; t < RT; ++t) score_tile(t);          // (one basic block: the widening of one tile overlaps the products of another)
         if (LONG) { s[XT - 1] = float4_t{0.f, 0.f, 0.f, 0.f}; if (extra) score_tile(XT - 1); }
         const bool interior = rb >= lo && rb + RUN <= tile_end && !extra;      // wavefront-uniform
-        uint32_t pbits[PKS][4], pext[2] = {0u, 0u};
+        uint32_t pbits[PKS > 0 ? PKS : 1][4], pext[2] = {0u, 0u};
         auto softmax = [&](auto masked_tag) {
             constexpr bool MASKED = decltype(masked_tag)::value;
             constexpr bool FOLD = !MASKED && !CAP;                   // scores stay unscaled until the exponent
@@ -354,7 +356,7 @@ __device__ __forceinline__ void split_mfma_il_body(const SplitArgs& a, uint32_t 
                     l_run += pp[0] + pp[1];
                     const uint32_t ph = __builtin_bit_cast(uint32_t, __builtin_convertvector(pp, half2_t));
                     const uint32_t pl = pack_f16_remainder(pp[0], pp[1], ph);
-                    if (t < RT) pbits[t / 2][(t % 2) * 2 + i2] = is_lo ? pl : ph;
+                    if (t < RT && !HALF) pbits[t / 2][(t % 2) * 2 + i2] = is_lo ? pl : ph;
                     else pext[i2] = is_lo ? pl : ph;
                 }
             }
@@ -409,10 +411,10 @@ __device__ __forceinline__ void split_mfma_il_body(const SplitArgs& a, uint32_t 
                 const u32x4 pw = u32x4{pbits[ks][0], pbits[ks][1], pbits[ks][2], pbits[ks][3]};
                 oacc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(va, __builtin_bit_cast(half8_t, pw), oacc[dt], 0, 0, 0);
             }
-        if (LONG && extra) {               // the 16 rows behind the run: the 16-deep product
+        if (HALF || (LONG && extra)) {     // the 16 rows behind the run (or a run of 16 rows): the 16-deep product
 #pragma unroll
             for (int dt = 0; dt < DTILES; ++dt) {
-                const _Float16* p0 = vb + (RUN + kg * 4 + n16 / 4) * VPITCH + dt * 16 + 4 * (n16 % 4);
+                const _Float16* p0 = vb + ((HALF ? 0 : RUN) + kg * 4 + n16 / 4) * VPITCH + dt * 16 + 4 * (n16 % 4);
                 const half4_t v0 = lds_read_tr16(p0);
                 const u32x2 pw = u32x2{pext[0], pext[1]};
                 oacc[dt] = __builtin_amdgcn_mfma_f32_16x16x16f16(v0, __builtin_bit_cast(half4_t, pw), oacc[dt], 0, 0, 0);

@@ -109,6 +109,29 @@ def test_split_reduce_matches_oracle(dtype, heads, hkv, d, seq, tile, kv_start, 
         assert (sm[:, :dead] == np.float32(-1e30)).all() and (ss[:, :dead] == 0).all() and (so[:, :dead] == 0).all()
 
 
+# The interleaved worker exists with runs of 32 rows (64 at head_dim 64) and with runs of half that; which one a launch
+# takes follows from the full runs per run stream (four streams per workgroup = per tile of the call).  Per shape: many
+# tiles (at most one and a half full runs per stream: half runs) and two tiles (full runs), each with a window that starts
+# inside a run and a ragged end.
+RUN_LENGTH_CASES = [
+    (vf.KvDtype.F8, 32, 8, 128, 1501, 64, 0, 0.0),     # 24 tiles, 47 full runs over 96 streams: runs of 16 rows
+    (vf.KvDtype.F8, 32, 8, 128, 1501, 768, 333, 0.0),  # 2 tiles, 8 streams: runs of 32 rows
+    (vf.KvDtype.F8, 16, 4, 64, 1501, 64, 0, 20.0),     # head_dim 64: runs of 32 rows
+    (vf.KvDtype.F8, 16, 4, 64, 1501, 768, 333, 0.0),   # runs of 64 rows
+    (vf.KvDtype.F16, 32, 8, 128, 1501, 64, 0, 0.0),    # runs of 16 rows
+    (vf.KvDtype.F16, 32, 8, 128, 650, 384, 77, 0.0),   # 2 tiles, 21 full runs over 8 streams (between 1.5 and 4 per stream): 32 rows
+    (vf.KvDtype.F16, 32, 8, 128, 1501, 768, 0, 30.0),  # 47 full runs over 8 streams (4 and more per stream): 16 rows again
+    (vf.KvDtype.F16, 8, 4, 64, 1501, 768, 333, 0.0),   # F16 rows of 64: 32 rows at every length
+    (vf.KvDtype.F8, 16, 8, 256, 1501, 768, 333, 0.0),  # FP8 rows of 256: 16 rows at every length
+    (vf.KvDtype.F16, 16, 8, 256, 1501, 768, 333, 50.0),
+]
+
+
+@pytest.mark.parametrize("dtype,heads,hkv,d,seq,tile,kv_start,cap", RUN_LENGTH_CASES)
+def test_interleaved_worker_both_run_lengths(dtype, heads, hkv, d, seq, tile, kv_start, cap):
+    test_interleaved_split_reduce_matches_oracle(dtype, heads, hkv, d, seq, tile, kv_start, cap)
+
+
 @pytest.mark.parametrize("dtype,heads,hkv,d,seq,tile,kv_start,cap", CASES)
 def test_interleaved_split_reduce_matches_oracle(dtype, heads, hkv, d, seq, tile, kv_start, cap):
     # vfkv_flash_attn_split_interleaved: the partials are combs of rows rather than tiles, so only the merged
@@ -287,6 +310,9 @@ def test_config2_fp8_outliers_append_then_decode_two_layers():
     (vf.KvDtype.F8, 16, 8, 64, 1000, 0),
     (vf.KvDtype.F8, 16, 8, 64, 8192, 0),        # interleaved walk: the owner of the new row is not the last workgroup
     (vf.KvDtype.F8, 16, 8, 64, 5000, 700),      # the same under a sliding window
+    # the appending wavefront in the worker with full runs where the cases above take half runs (two to four full runs per stream)
+    (vf.KvDtype.F16, 32, 8, 128, 8192, 0),
+    (vf.KvDtype.F8, 16, 8, 64, 16384, 0),
 ])
 def test_kv_write_attention_in_one_call_matches_the_two_calls(dtype, heads, hkv, d, ctx, window):
     # step_kv_write + step_attention (executor/attention.rs:546-625) through the single entry point: cache bytes and

@@ -716,13 +716,12 @@ static hipError_t launch_split_il(const SplitArgs& a_in, uint32_t g, const RopeF
 static uint32_t il_full_run(uint32_t D) { return D == 64u ? 64u : 32u; }
 
 static bool il_half_runs(uint32_t dtype, uint32_t D, uint32_t span_rows, uint32_t n_tiles) {
-    static const bool off = [] { const char* e = getenv("VFKV_DECODE_HALF_RUNS"); return e && e[0] == '0'; }();   // for comparisons
+    static const bool off = [] { const char* e = getenv("VFKV_DECODE_HALF_RUNS"); return e && e[0] == '0'; }();   // for comparisons (the shapes that have both)
     if (off) return false;
     const uint32_t full = il_full_run(D), units = (span_rows + full - 1u) / full, S = (uint32_t)kMfmaWaves * n_tiles;
-    if (dtype == kF16 && D == 256u) return true;
     if (dtype == kF8 && D != 256u) return 2u * units <= 3u * S;
     if (dtype == kF16 && D == 128u) return 2u * units <= 3u * S || units >= 4u * S;
-    return true;
+    return true;                     // F16 rows of 64 and of 256 elements, FP8 rows of 256
 }
 
 // The shortest run the worker may take for this shape: what the caller sizes its workgroup count by.
@@ -860,8 +859,11 @@ hipError_t launch_split(const SplitLaunch& L, hipStream_t stream, bool* generic_
 #define VFKV_IL(DT, DD, FULL) \
     if (L.dtype == DT && L.head_dim == DD) \
         return half ? launch_split_il<DT, DD, FULL / 2>(a, g, L.rope, stream) : launch_split_il<DT, DD, FULL>(a, g, L.rope, stream);
-        VFKV_IL(kF8, 64u, 64) VFKV_IL(kF16, 64u, 64) VFKV_IL(kF8, 128u, 32) VFKV_IL(kF16, 128u, 32) VFKV_IL(kF8, 256u, 32)
+        VFKV_IL(kF8, 64u, 64) VFKV_IL(kF8, 128u, 32) VFKV_IL(kF16, 128u, 32)
 #undef VFKV_IL
+        // (these three take half runs at every length)
+        if (L.dtype == kF16 && L.head_dim == 64u) return launch_split_il<kF16, 64, 32>(a, g, L.rope, stream);
+        if (L.dtype == kF8 && L.head_dim == 256u) return launch_split_il<kF8, 256, 16>(a, g, L.rope, stream);
         if (L.dtype == kF16 && L.head_dim == 256u) return launch_split_il<kF16, 256, 16>(a, g, L.rope, stream);
     }
     if (aligned && out_aligned && slab_bytes < 0x7FFF0000ull && mfma_worker_enabled()) {

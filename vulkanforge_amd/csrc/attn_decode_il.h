@@ -10,6 +10,10 @@
 //     it rides along with the run in front of it as one unit of RUN + 16 rows (one memory round trip, 1.5 x the
 //     arithmetic) instead of costing one stream a whole extra round that the launch then waits for (8 193 keys, 128
 //     streams: 2 rounds and one row).
+//   * Runs of one tile.  RUN = 16 is the same worker with units of a single 16-row tile: the second product is then the
+//     16-deep matrix instruction (v_mfma_f32_16x16x16_f16) on the tile's own weights.  The launcher takes it where it measures
+//     faster: rows of 512 bytes (32 rows of K and V would be 32 KiB in flight per wavefront, twice what the memory system
+//     rewards) and launches whose run streams hold a run or two, where a smaller unit shortens the latency chain.
 //   * The append of the decode token (step_kv_write, executor/attention.rs:546).  The new row is the last row of the span,
 //     i.e. part of stream 0's first unit.  That wavefront converts the new K / V row itself, puts the converted bytes into
 //     the registers its loads of the unit have filled (whatever those loads found at that row), and stores the same bytes

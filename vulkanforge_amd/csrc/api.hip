@@ -686,11 +686,13 @@ static int decode_attention_impl(vfkv_cache* c, uint32_t layer, uint32_t kv_laye
     // The interleaved worker deals the runs of the span to its workgroups whatever the tile length says: the workgroup count
     // is chosen directly (one per CU, none without a run), and the launch covers the rows from the 64-row boundary at or
     // below kv_start.
-    if (n_tiles > 1u && forced_tile() == 0u && vfkv::split_interleaves(L)) {
+    const uint32_t streams = n_tiles > 1u && forced_tile() == 0u ? vfkv::split_run_streams(L) : 0u;
+    if (streams != 0u) {
         const uint32_t run_rows = vfkv::split_run_rows(c->dtype, hd), nz = (n_heads / kvh + 7u) / 8u;
         const uint32_t runs = (seq_len - kv_start / 64u * 64u + run_rows - 1u) / run_rows;
         uint32_t wgs = device_cus() / (kvh * nz);
-        if (wgs > (runs + 3u) / 4u) wgs = (runs + 3u) / 4u;             // four run streams per workgroup
+        if (wgs > (runs + streams - 1u) / streams) wgs = (runs + streams - 1u) / streams;   // none without a run
+        if (wgs > (seq_len + 63u) / 64u) wgs = (seq_len + 63u) / 64u;   // what a workspace sized for this length holds (head_dim 512: two streams per workgroup)
         if (!static_ws && wgs > ws->max_tiles) wgs = ws->max_tiles;
         if (wgs < 1u) wgs = 1u;
         tile = 64u; first = kv_start / 64u; n_tiles = wgs;

@@ -727,8 +727,7 @@ static bool il_half_runs(uint32_t dtype, uint32_t D, uint32_t span_rows, uint32_
 // The shortest run the worker may take for this shape: what the caller sizes its workgroup count by.
 uint32_t split_run_rows(uint32_t dtype, uint32_t D) {
     if ((dtype != kF8 && dtype != kF16) || (D != 64u && D != 128u && D != 256u && D != 512u)) return 0u;
-    if (D == 512u) return 32u;
-    return il_full_run(D) / 2u;
+    return il_full_run(D) / 2u;      // (head_dim 512: 16 rows as well)
 }
 
 template <int D>
@@ -755,6 +754,17 @@ static bool mfma_worker_shape(uint32_t dtype, uint32_t D) {
 static bool mfma_worker_enabled() {
     static const bool on = [] { const char* e = getenv("VFKV_DECODE_WORKER"); return !(e && e[0] == 'v'); }();
     return on;
+}
+
+// Run streams per workgroup of a launch that deals the runs of the whole span to its workgroups whatever the tile length
+// says (0: the launch keeps partial j = tile j): four for the interleaved worker, two at head_dim 512, where two wavefronts
+// share a run.
+uint32_t split_run_streams(const SplitLaunch& L) {
+    if (split_interleaves(L)) return (uint32_t)kMfmaWaves;
+    if (!L.interleave || L.n_kv_heads == 0u || L.head_dim != 512u || (L.dtype != kF8 && L.dtype != kF16)) return 0u;
+    const bool aligned = ((((uintptr_t)L.k) | ((uintptr_t)L.v) | ((uintptr_t)L.q) | ((uintptr_t)L.scratch_out) | ((uintptr_t)L.o_direct)) & 15u) == 0u;
+    const uint64_t slab_bytes = (uint64_t)L.seq_len * L.n_kv_heads * L.head_dim * elem_size(L.dtype);
+    return aligned && slab_bytes < 0x7FFF0000ull && mfma_worker_enabled() ? (uint32_t)kMfmaWaves / 2u : 0u;
 }
 
 template <int DT, int D, int GT>
@@ -873,8 +883,9 @@ hipError_t launch_split(const SplitLaunch& L, hipStream_t stream, bool* generic_
         if (L.dtype == kF16 && L.head_dim == 128u) return launch_split_mfma<kF16, 128, 32, 1>(a, g, stream);
         if (L.dtype == kF8 && L.head_dim == 256u) return launch_split_mfma<kF8, 256, 32, 1>(a, g, stream);
         if (L.dtype == kF16 && L.head_dim == 256u) return launch_split_mfma<kF16, 256, 32, 1>(a, g, stream);
-        if (L.dtype == kF8 && L.head_dim == 512u) return launch_split_mfma<kF8, 512, 32, 1, 2>(a, g, stream);
-        if (L.dtype == kF16 && L.head_dim == 512u) return launch_split_mfma<kF16, 512, 32, 1, 2>(a, g, stream);
+        // (runs of 16 rows: with 32 a wavefront has 48 KiB of F16 rows in flight; 9-10 % per layer at every length, FP8 and F16)
+        if (L.dtype == kF8 && L.head_dim == 512u) return launch_split_mfma<kF8, 512, 16, 1, 2>(a, g, stream);
+        if (L.dtype == kF16 && L.head_dim == 512u) return launch_split_mfma<kF16, 512, 16, 1, 2>(a, g, stream);
     }
     if (aligned && out_aligned && slab_bytes < 0x7FFF0000ull && mfma_worker_enabled() && f32_mfma_shape(L.dtype, L.head_dim)) {
         if (L.head_dim == 64u) return launch_split_f32<64>(a, g, stream);

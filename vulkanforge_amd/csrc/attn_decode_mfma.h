@@ -41,6 +41,7 @@ __global__ __launch_bounds__(NW * 64) void split_mfma_kernel(SplitArgs a, uint32
     constexpr int NP = NW / NH;                  // run streams of the workgroup
     constexpr int RT = RUN / 16;                 // 16-row tiles per run
     constexpr int PKS = RUN / 32;                // k-steps (32 rows) of the second product
+    constexpr bool HALF = RUN == 16;             // runs of one tile: the second product is the 16-deep matrix instruction
     constexpr int KS = D / 32;                   // k-steps of the first product
     constexpr int DTILES = DV / 16;
     constexpr int SEG = D / 4, SEGB = SEG * ES;  // a lane group's quarter of a K row
@@ -55,11 +56,12 @@ __global__ __launch_bounds__(NW * 64) void split_mfma_kernel(SplitArgs a, uint32
     constexpr int VCHUNK_ROW = DV * ES / 16;     // 16-byte chunks per V row (this wavefront's columns)
     constexpr int VLD = RUN * VCHUNK_ROW / 64;   // V loads per lane per run
     constexpr int VROWS = 64 / VCHUNK_ROW;       // rows covered by one V load of the wavefront
-    static_assert(D % 32 == 0 && SEGB % 16 == 0 && RUN % 32 == 0 && VCHUNK_ROW <= 64 && VLD >= 1, "unsupported shape");
-    static_assert(NW * RUN * VPITCH * 2 >= NW * (DV / 16) * 64 * 16, "merge buffer must fit in the V staging area");
+    static_assert(D % 32 == 0 && SEGB % 16 == 0 && (RUN % 32 == 0 || HALF) && VCHUNK_ROW <= 64 && VLD >= 1, "unsupported shape");
+    constexpr int MERGE_ROWS = ((DV / 16) * 64 * 16 + VPITCH * 2 - 1) / (VPITCH * 2);    // rows of the staging area the merge needs
+    constexpr int LROWS = RUN > MERGE_ROWS ? RUN : MERGE_ROWS;
     static_assert(NW % NH == 0, "whole run streams");
 
-    __shared__ __attribute__((aligned(16))) _Float16 vlds[NW][RUN * VPITCH];
+    __shared__ __attribute__((aligned(16))) _Float16 vlds[NW][LROWS * VPITCH];
     __shared__ float lds_m[NW][8], lds_l[NW][8];
     __shared__ __attribute__((aligned(16))) _Float16 qlds[16][D + 8];   // rows 0-7: f16(q) per head, rows 8-15: remainders
 
@@ -255,7 +257,8 @@ __global__ __launch_bounds__(NW * 64) void split_mfma_kernel(SplitArgs a, uint32
             }
             // ---------------- softmax: this lane owns rows rb + t*16 + kg*4 + i of column n16 ----------------
             const bool interior = rb >= lo && rb + RUN <= tile_end;      // wavefront-uniform
-            u32x4 pbits[PKS];
+            u32x4 pbits[PKS > 0 ? PKS : 1];
+            uint32_t pext[2] = {0u, 0u};
             auto softmax = [&](auto masked_tag) {
                 constexpr bool MASKED = decltype(masked_tag)::value;
                 constexpr bool FOLD = !MASKED && !CAP;                   // scores stay unscaled until the exponent
@@ -302,11 +305,12 @@ __global__ __launch_bounds__(NW * 64) void split_mfma_kernel(SplitArgs a, uint32
                         l_run += pp[0] + pp[1];
                         const uint32_t ph = __builtin_bit_cast(uint32_t, __builtin_convertvector(pp, half2_t));
                         const uint32_t pl = pack_f16_remainder(pp[0], pp[1], ph);
-                        pbits[t / 2][(t % 2) * 2 + i2] = is_lo ? pl : ph;
+                        if (HALF) pext[i2] = is_lo ? pl : ph;
+                        else pbits[t / 2][(t % 2) * 2 + i2] = is_lo ? pl : ph;
                     }
             };
             if (interior) softmax(std::false_type{}); else softmax(std::true_type{});
-            half8_t pb[PKS];
+            half8_t pb[PKS > 0 ? PKS : 1];
 #pragma unroll
             for (int ks = 0; ks < PKS; ++ks) pb[ks] = __builtin_bit_cast(half8_t, pbits[ks]);
             // ---------------- V run -> f16 row-major in LDS ----------------
@@ -343,6 +347,15 @@ __global__ __launch_bounds__(NW * 64) void split_mfma_kernel(SplitArgs a, uint32
                     va[0] = v0[0]; va[1] = v0[1]; va[2] = v0[2]; va[3] = v0[3]; va[4] = v1[0]; va[5] = v1[1]; va[6] = v1[2]; va[7] = v1[3];
                     oacc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(va, pb[ks], oacc[dt], 0, 0, 0);
                 }
+            if (HALF) {                    // one tile of 16 rows: the 16-deep product on the tile's own weights
+#pragma unroll
+                for (int dt = 0; dt < DTILES; ++dt) {
+                    const _Float16* p0 = vb + (kg * 4 + n16 / 4) * VPITCH + dt * 16 + 4 * (n16 % 4);
+                    const half4_t v0 = lds_read_tr16(p0);
+                    const u32x2 pw = u32x2{pext[0], pext[1]};
+                    oacc[dt] = __builtin_amdgcn_mfma_f32_16x16x16f16(v0, __builtin_bit_cast(half4_t, pw), oacc[dt], 0, 0, 0);
+                }
+            }
           }
         }
     }

@@ -261,6 +261,16 @@ __device__ __forceinline__ void split_mfma_il_body(const SplitArgs& a, uint32_t 
         }
         __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");     // (the row is read back by lanes of this wavefront only)
     }
+    // the pieces of the row that this lane's K / V registers hold, fetched now: the LDS round trip runs while the unit's rows
+    // are still on their way, and the patch inside the first unit is a select between registers
+    u32x4 knw[KLD], vnw = u32x4{0u, 0u, 0u, 0u};
+#pragma unroll
+    for (int x = 0; x < KLD; ++x) knw[x] = u32x4{0u, 0u, 0u, 0u};
+    if (appends) {
+#pragma unroll
+        for (int x = 0; x < KLD; ++x) knw[x] = *reinterpret_cast<const u32x4*>(&newrow[0][(KIL ? x * 4 + kg : kg * KLD + x) * 16]);
+        vnw = *reinterpret_cast<const u32x4*>(&newrow[1][vcol * 16]);
+    }
 
     float4_t oacc[DTILES];
 #pragma unroll
@@ -280,8 +290,7 @@ __device__ __forceinline__ void split_mfma_il_body(const SplitArgs& a, uint32_t 
 #pragma unroll
                     for (int x = 0; x < KLD; ++x) {
                         const u32x4 old = kraw[t][x];
-                        const u32x4 nw = *reinterpret_cast<const u32x4*>(&newrow[0][(KIL ? x * 4 + kg : kg * KLD + x) * 16]);
-                        kraw[t][x] = k_mine ? nw : old;
+                        kraw[t][x] = k_mine ? knw[x] : old;
                     }
                 }
         }
@@ -372,8 +381,7 @@ __device__ __forceinline__ void split_mfma_il_body(const SplitArgs& a, uint32_t 
             for (int c = 0; c < XT * VLT; ++c)
                 if ((uint32_t)c == cv) {
                     const u32x4 old = vraw[c];
-                    const u32x4 nw = *reinterpret_cast<const u32x4*>(&newrow[1][vcol * 16]);
-                    vraw[c] = v_mine ? nw : old;
+                    vraw[c] = v_mine ? vnw : old;
                 }
         }
         auto stage_v = [&](int c) {

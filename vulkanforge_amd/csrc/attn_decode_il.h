@@ -15,9 +15,10 @@
 //     faster: rows of 512 bytes (32 rows of K and V would be 32 KiB in flight per wavefront, twice what the memory system
 //     rewards) and launches whose run streams hold a run or two, where a smaller unit shortens the latency chain.
 //   * The append of the decode token (step_kv_write, executor/attention.rs:546).  The new row is the last row of the span,
-//     i.e. part of stream 0's first unit.  That wavefront converts the new K / V row itself, puts the converted bytes into
-//     the registers its loads of the unit have filled (whatever those loads found at that row), and stores the same bytes
-//     to the cache.  Nothing waits for the stores: no other wavefront of the launch reads that row.
+//     i.e. part of stream 0's first unit.  That wavefront converts the new K / V row itself, puts the converted K values
+//     into the first product's operand and the converted V values over the row's place in its staged copy of the unit
+//     (whatever the loads found at that row), and stores the same bytes to the cache.  Nothing waits for the stores: no
+//     other wavefront of the launch reads that row.
 //   * ROPE: the decode token's Q-norm / RoPE, K-norm / RoPE (step_q_norm_rope, step_k_norm_rope,
 //     executor/attention.rs:360-530) in the same launch.  Every workgroup normalises and rotates its (up to 8) query
 //     heads while its first K rows are in flight (the cos / sin table of the position is computed once per workgroup);
@@ -69,7 +70,7 @@ __device__ __forceinline__ void split_mfma_il_body(const SplitArgs& a, uint32_t 
     __shared__ __attribute__((aligned(16))) _Float16 qlds[16][D + 8];   // rows 0-7: f16(q) per head, rows 8-15: remainders
     __shared__ __attribute__((aligned(16))) float rot[ROPE ? 9 : 1][ROPE ? D : 4];   // ROPE: rotated query heads, then the K row
     __shared__ float cs_lds[ROPE ? D / 2 : 1], sn_lds[ROPE ? D / 2 : 1];
-    __shared__ __attribute__((aligned(16))) uint8_t newrow[2][D * ES];   // the decode token's K and V row in the cache's format (stream 0's wavefront)
+    __shared__ __attribute__((aligned(16))) uint8_t newrow[D * ES];      // the decode token's K row in the cache's format (stream 0's wavefront)
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -135,12 +136,11 @@ __device__ __forceinline__ void split_mfma_il_body(const SplitArgs& a, uint32_t 
 
     // ---- the new row of the decode token, in the wavefront that reads it (stream 0: the last row lies in its first unit).
     // Without ROPE its f32 values come straight from global memory: requested here (four elements per lane), converted after
-    // the queries have arrived (loads return in order), parked in LDS in the cache's format, and fetched from there by the
-    // lanes whose K / V registers hold pieces of that row.
+    // the queries have arrived (loads return in order); the K row is parked in LDS in the cache's format and fetched from
+    // there by the lanes whose K registers hold pieces of that row, the V row goes over the staged copy of its place.
     const bool appends = a.k_new != nullptr && active && sidx == 0u;            // wavefront-uniform
     const uint32_t rn = appends ? a.append_pos - cur_rb : 0u;                   // the row's index inside the unit
     const bool k_mine = appends && (uint32_t)n16 == (rn & 15u);                 // lanes whose K registers hold a piece of the row
-    const bool v_mine = appends && (uint32_t)vrow == rn % VROWS;                // lanes whose V registers (load rn / VROWS) do
     const bool row_lane = appends && lane * 4 < D;                              // lanes that convert four elements of the row
     float4 knew4 = make_float4(0.f, 0.f, 0.f, 0.f), vnew4 = make_float4(0.f, 0.f, 0.f, 0.f);
     if (row_lane) {
@@ -244,32 +244,29 @@ __device__ __forceinline__ void split_mfma_il_body(const SplitArgs& a, uint32_t 
     // stores count in the same in-order counter as the loads, so issued now, every later wait for rows would also wait for
     // their acknowledgement) and as a whole in LDS for the lanes that patch their registers inside the first unit.
     uint32_t kw0 = 0u, kw1 = 0u, vw0 = 0u, vw1 = 0u;
-    const uint32_t tk = rn >> 4, cv = rn / VROWS;               // the tile / the V load that hold the row (wavefront-uniform)
+    const uint32_t tk = rn >> 4;                                // the tile that holds the row (wavefront-uniform)
     if (appends) {
         if (row_lane) {
             if (DT == kF8) {
                 kw0 = pack4_e4m3(knew4.x, knew4.y, knew4.z, knew4.w);
                 vw0 = pack4_e4m3(vnew4.x, vnew4.y, vnew4.z, vnew4.w);
-                reinterpret_cast<uint32_t*>(&newrow[0][0])[lane] = kw0;
-                reinterpret_cast<uint32_t*>(&newrow[1][0])[lane] = vw0;
+                reinterpret_cast<uint32_t*>(&newrow[0])[lane] = kw0;
             } else {
                 kw0 = f32_to_h16_bits(knew4.x) | (f32_to_h16_bits(knew4.y) << 16); kw1 = f32_to_h16_bits(knew4.z) | (f32_to_h16_bits(knew4.w) << 16);
                 vw0 = f32_to_h16_bits(vnew4.x) | (f32_to_h16_bits(vnew4.y) << 16); vw1 = f32_to_h16_bits(vnew4.z) | (f32_to_h16_bits(vnew4.w) << 16);
-                reinterpret_cast<u32x2*>(&newrow[0][0])[lane] = u32x2{kw0, kw1};
-                reinterpret_cast<u32x2*>(&newrow[1][0])[lane] = u32x2{vw0, vw1};
+                reinterpret_cast<u32x2*>(&newrow[0])[lane] = u32x2{kw0, kw1};
             }
         }
         __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");     // (the row is read back by lanes of this wavefront only)
     }
-    // the pieces of the row that this lane's K / V registers hold, fetched now: the LDS round trip runs while the unit's rows
+    // the pieces of the K row that this lane's K registers hold, fetched now: the LDS round trip runs while the unit's rows
     // are still on their way, and the patch inside the first unit is a select between registers
-    u32x4 knw[KLD], vnw = u32x4{0u, 0u, 0u, 0u};
+    u32x4 knw[KLD];
 #pragma unroll
     for (int x = 0; x < KLD; ++x) knw[x] = u32x4{0u, 0u, 0u, 0u};
     if (appends) {
 #pragma unroll
-        for (int x = 0; x < KLD; ++x) knw[x] = *reinterpret_cast<const u32x4*>(&newrow[0][(KIL ? x * 4 + kg : kg * KLD + x) * 16]);
-        vnw = *reinterpret_cast<const u32x4*>(&newrow[1][vcol * 16]);
+        for (int x = 0; x < KLD; ++x) knw[x] = *reinterpret_cast<const u32x4*>(&newrow[(KIL ? x * 4 + kg : kg * KLD + x) * 16]);
     }
 
     float4_t oacc[DTILES];
@@ -283,32 +280,33 @@ __device__ __forceinline__ void split_mfma_il_body(const SplitArgs& a, uint32_t 
     // the end of the slab return zeros without traffic).  One body for both forms, so that the loop has a single shape.
     auto process = [&](uint32_t rb, uint32_t noff, bool extra, bool patch) {
         constexpr int PKS = RUN / 32;                        // k-steps of 32 rows of the second product
-        if (patch) {                                         // the new row's pieces replace what the loads found there
-#pragma unroll
-            for (int t = 0; t < XT; ++t)
-                if ((uint32_t)t == tk) {
-#pragma unroll
-                    for (int x = 0; x < KLD; ++x) {
-                        const u32x4 old = kraw[t][x];
-                        kraw[t][x] = k_mine ? knw[x] : old;
-                    }
-                }
-        }
         float4_t s[XT];
+        // k-step c of a row's pieces as the first product's A operand
+        auto k_operand = [&](const u32x4 (&raw)[KLD], int c) -> half8_t {
+            half8_t r;
+            if (DT == kF8) {
+                const uint32_t w0 = raw[c / 2][(c % 2) * 2], w1 = raw[c / 2][(c % 2) * 2 + 1];
+                half2_t p0, p1, p2, p3;
+                e4m3x4_to_h2(w0, p0, p1);
+                e4m3x4_to_h2(w1, p2, p3);
+                r[0] = p0[0]; r[1] = p0[1]; r[2] = p1[0]; r[3] = p1[1];
+                r[4] = p2[0]; r[5] = p2[1]; r[6] = p3[0]; r[7] = p3[1];
+            } else {
+                r = __builtin_bit_cast(half8_t, raw[c % KLD]);
+            }
+            return r;
+        };
         auto score_tile = [&](int t) {
             half8_t ka[KS];
 #pragma unroll
-            for (int c = 0; c < KS; ++c) {
-                if (DT == kF8) {
-                    const uint32_t w0 = kraw[t][c / 2][(c % 2) * 2], w1 = kraw[t][c / 2][(c % 2) * 2 + 1];
-                    half2_t p0, p1, p2, p3;
-                    e4m3x4_to_h2(w0, p0, p1);
-                    e4m3x4_to_h2(w1, p2, p3);
-                    ka[c][0] = p0[0]; ka[c][1] = p0[1]; ka[c][2] = p1[0]; ka[c][3] = p1[1];
-                    ka[c][4] = p2[0]; ka[c][5] = p2[1]; ka[c][6] = p3[0]; ka[c][7] = p3[1];
-                } else {
-                    const u32x4 wv = kraw[t][c % KLD];
-                    ka[c] = __builtin_bit_cast(half8_t, wv);
+            for (int c = 0; c < KS; ++c) ka[c] = k_operand(kraw[t], c);
+            // The new row replaces what the loads found at its place, in the operand rather than in the registers the loads
+            // fill: a branch that reads load destinations makes every later wait of the unit a full one.
+            if (patch && (uint32_t)t == tk) {                // wavefront-uniform
+#pragma unroll
+                for (int c = 0; c < KS; ++c) {
+                    const half8_t kn = k_operand(knw, c);
+                    ka[c] = k_mine ? kn : ka[c];
                 }
             }
             if (t < RT) issue_k(t, noff);
@@ -376,14 +374,6 @@ __device__ __forceinline__ void split_mfma_il_body(const SplitArgs& a, uint32_t 
         };
         if (interior) softmax(std::false_type{}); else softmax(std::true_type{});
         // ---------------- V rows -> f16 row-major in LDS ----------------
-        if (patch) {
-#pragma unroll
-            for (int c = 0; c < XT * VLT; ++c)
-                if ((uint32_t)c == cv) {
-                    const u32x4 old = vraw[c];
-                    vraw[c] = v_mine ? vnw : old;
-                }
-        }
         auto stage_v = [&](int c) {
             _Float16* dst = vb + (c * VROWS + vrow) * VPITCH + vcol * (16 / ES);
             if (DT == kF8) {
@@ -408,6 +398,17 @@ __device__ __forceinline__ void split_mfma_il_body(const SplitArgs& a, uint32_t 
         if (LONG && extra) {
 #pragma unroll
             for (int c = RT * VLT; c < XT * VLT; ++c) stage_v(c);
+        }
+        if (patch && row_lane) {           // the new V row over the staged copy of its place (this wavefront's LDS accesses run in order)
+            uint32_t h0w, h1w;
+            if (DT == kF8) {
+                half2_t lo2, hi2;
+                e4m3x4_to_h2(vw0, lo2, hi2);
+                h0w = __builtin_bit_cast(uint32_t, lo2); h1w = __builtin_bit_cast(uint32_t, hi2);
+            } else {
+                h0w = vw0; h1w = vw1;
+            }
+            *reinterpret_cast<u32x2*>(vb + rn * VPITCH + lane * 4) = u32x2{h0w, h1w};
         }
         // ---------------- O^T += V^T P ----------------
 #pragma unroll

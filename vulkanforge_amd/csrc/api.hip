@@ -686,9 +686,10 @@ static int decode_attention_impl(vfkv_cache* c, uint32_t layer, uint32_t kv_laye
     // The interleaved worker deals the runs of the span to its workgroups whatever the tile length says: the workgroup count
     // is chosen directly (one per CU, none without a run), and the launch covers the rows from the 64-row boundary at or
     // below kv_start.
-    const uint32_t streams = n_tiles > 1u && forced_tile() == 0u ? vfkv::split_run_streams(L) : 0u;
+    uint32_t heads_per_wg = 8u;
+    const uint32_t streams = n_tiles > 1u && forced_tile() == 0u ? vfkv::split_run_streams(L, &heads_per_wg) : 0u;
     if (streams != 0u) {
-        const uint32_t run_rows = vfkv::split_run_rows(c->dtype, hd), nz = (n_heads / kvh + 7u) / 8u;
+        const uint32_t run_rows = vfkv::split_run_rows(c->dtype, hd), nz = (n_heads / kvh + heads_per_wg - 1u) / heads_per_wg;
         const uint32_t runs = (seq_len - kv_start / 64u * 64u + run_rows - 1u) / run_rows;
         uint32_t wgs = device_cus() / (kvh * nz);
         if (wgs > (runs + streams - 1u) / streams) wgs = (runs + streams - 1u) / streams;   // none without a run

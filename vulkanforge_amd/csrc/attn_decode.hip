@@ -726,6 +726,7 @@ static bool il_half_runs(uint32_t dtype, uint32_t D, uint32_t span_rows, uint32_
 
 // The shortest run the worker may take for this shape: what the caller sizes its workgroup count by.
 uint32_t split_run_rows(uint32_t dtype, uint32_t D) {
+    if (dtype == kF32 && (D == 64u || D == 128u || D == 256u)) return 16u;      // the F32 worker: one tile per run
     if ((dtype != kF8 && dtype != kF16) || (D != 64u && D != 128u && D != 256u && D != 512u)) return 0u;
     return il_full_run(D) / 2u;      // (head_dim 512: 16 rows as well)
 }
@@ -757,14 +758,18 @@ static bool mfma_worker_enabled() {
 }
 
 // Run streams per workgroup of a launch that deals the runs of the whole span to its workgroups whatever the tile length
-// says (0: the launch keeps partial j = tile j): four for the interleaved worker, two at head_dim 512, where two wavefronts
-// share a run.
-uint32_t split_run_streams(const SplitLaunch& L) {
+// says (0: the launch keeps partial j = tile j): four for the interleaved worker and the F32 worker, two at head_dim 512,
+// where two wavefronts share a run.  *heads_per_wg: query heads of a GQA group that one workgroup serves.
+uint32_t split_run_streams(const SplitLaunch& L, uint32_t* heads_per_wg) {
+    if (heads_per_wg) *heads_per_wg = 8u;
     if (split_interleaves(L)) return (uint32_t)kMfmaWaves;
-    if (!L.interleave || L.n_kv_heads == 0u || L.head_dim != 512u || (L.dtype != kF8 && L.dtype != kF16)) return 0u;
+    if (!L.interleave || L.n_kv_heads == 0u) return 0u;
     const bool aligned = ((((uintptr_t)L.k) | ((uintptr_t)L.v) | ((uintptr_t)L.q) | ((uintptr_t)L.scratch_out) | ((uintptr_t)L.o_direct)) & 15u) == 0u;
     const uint64_t slab_bytes = (uint64_t)L.seq_len * L.n_kv_heads * L.head_dim * elem_size(L.dtype);
-    return aligned && slab_bytes < 0x7FFF0000ull && mfma_worker_enabled() ? (uint32_t)kMfmaWaves / 2u : 0u;
+    if (!aligned || slab_bytes >= 0x7FFF0000ull || !mfma_worker_enabled()) return 0u;
+    if (L.head_dim == 512u && (L.dtype == kF8 || L.dtype == kF16)) return (uint32_t)kMfmaWaves / 2u;
+    if (f32_mfma_shape(L.dtype, L.head_dim)) { if (heads_per_wg) *heads_per_wg = 16u; return (uint32_t)kMfmaWaves; }
+    return 0u;
 }
 
 template <int DT, int D, int GT>

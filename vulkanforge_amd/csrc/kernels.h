@@ -98,7 +98,9 @@ bool split_interleaves(const SplitLaunch& a);
 bool split_folds_rope(const SplitLaunch& a);
 // Rows per run of the matrix-core worker for this shape (0: the shape is not the matrix-core worker's).
 uint32_t split_run_rows(uint32_t dtype, uint32_t head_dim);
-uint32_t split_run_streams(const SplitLaunch& a);   // run streams per workgroup when the launch deals runs, not tiles (else 0)
+// Run streams per workgroup when the launch deals the runs of the span to its workgroups, not tiles (else 0), and how many
+// query heads of a GQA group one workgroup serves.
+uint32_t split_run_streams(const SplitLaunch& a, uint32_t* heads_per_wg);
 // Smallest tile granule (keys) the split kernel for this shape works in; 0 if unsupported.
 uint32_t split_tile_granule(uint32_t dtype, uint32_t head_dim);
 

@@ -62,6 +62,7 @@ __global__ __launch_bounds__(NW * 64) void split_mfma_f32_kernel(SplitArgs a, ui
     const uint32_t lane_voff = kg * row_stride + head_b + n16 * 16;              // row l / 16 of a group of four, elements 4 (l % 16) .. + 3 of a block
     const float scale_l2 = a.scale * 1.44269504088896f;
     const float cap_l2 = a.softcap * 1.44269504088896f;
+    const float inv_cap_l2 = CAP ? 1.0f / cap_l2 : 0.f;
 
     const uint32_t first_run = (lo - tile_base) / RUN;
     const uint32_t n_runs = tile_end > tile_base ? (tile_end - tile_base + RUN - 1) / RUN : 0;
@@ -144,7 +145,7 @@ __global__ __launch_bounds__(NW * 64) void split_mfma_f32_kernel(SplitArgs a, ui
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
                     float y = (s0[i] + s1[i]) * scale_l2;
-                    if (CAP) y = cap_l2 * tanhf(y / cap_l2);
+                    if (CAP) y = softcap_l2(y, cap_l2, inv_cap_l2);
                     if (MASKED) {
                         const uint32_t row = rb + kg * 4 + i;
                         y = (row >= lo && row < tile_end) ? y : kMasked;

@@ -95,6 +95,7 @@ __device__ __forceinline__ void split_mfma_il_body(const SplitArgs& a, uint32_t 
     const uint32_t lane_voff = vrow * row_stride + head_b + vcol * 16;
     const float scale_l2 = a.scale * 1.44269504088896f;
     const float cap_l2 = a.softcap * 1.44269504088896f;
+    const float inv_cap_l2 = CAP ? 1.0f / cap_l2 : 0.f;
 
     // ---- the deal: units counted from the end of the span ----
     const uint32_t span = tile_end > tile_base ? tile_end - tile_base : 0u;
@@ -332,7 +333,7 @@ __device__ __forceinline__ void split_mfma_il_body(const SplitArgs& a, uint32_t 
                     float y = s[t][i];
                     y += dpp_f<kDppRor8>(y);                         // f16(q) part + remainder part
                     if (!FOLD) y *= scale_l2;
-                    if (CAP) y = cap_l2 * tanhf(y / cap_l2);
+                    if (CAP) y = softcap_l2(y, cap_l2, inv_cap_l2);
                     if (MASKED) {
                         const uint32_t row = rb + t * 16 + kg * 4 + i;
                         y = (row >= lo && row < tile_end && (t < RT || extra)) ? y : kMasked;

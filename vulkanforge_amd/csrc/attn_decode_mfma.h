@@ -95,6 +95,7 @@ __global__ __launch_bounds__(NW * 64) void split_mfma_kernel(SplitArgs a, uint32
     const uint32_t lane_voff = vrow * row_stride + head_b + ds * DV * ES + vcol * 16;
     const float scale_l2 = a.scale * 1.44269504088896f;
     const float cap_l2 = a.softcap * 1.44269504088896f;
+    const float inv_cap_l2 = CAP ? 1.0f / cap_l2 : 0.f;
 
     // runs of this wavefront: w, w + NW, ... counted from the first run that reaches the window
     const uint32_t first_run = (lo - tile_base) / RUN;
@@ -271,7 +272,7 @@ __global__ __launch_bounds__(NW * 64) void split_mfma_kernel(SplitArgs a, uint32
                         float y = s[t][i];
                         y += dpp_f<kDppRor8>(y);                         // f16(q) part + remainder part
                         if (!FOLD) y *= scale_l2;                        // FOLD: the scale rides in the exponent's FMA
-                        if (CAP) y = cap_l2 * tanhf(y / cap_l2);
+                        if (CAP) y = softcap_l2(y, cap_l2, inv_cap_l2);
                         if (MASKED) {
                             const uint32_t row = rb + t * 16 + kg * 4 + i;
                             y = (row >= lo && row < tile_end) ? y : kMasked;

@@ -882,12 +882,16 @@ hipError_t launch_split(const SplitLaunch& L, hipStream_t stream, bool* generic_
         if (L.dtype == kF16 && L.head_dim == 256u) return launch_split_il<kF16, 256, 16>(a, g, L.rope, stream);
     }
     if (aligned && out_aligned && slab_bytes < 0x7FFF0000ull && mfma_worker_enabled()) {
-        if (L.dtype == kF8 && L.head_dim == 64u) return launch_split_mfma<kF8, 64, 64, 1>(a, g, stream);
-        if (L.dtype == kF8 && L.head_dim == 128u) return launch_split_mfma<kF8, 128, 32, 1>(a, g, stream);
-        if (L.dtype == kF16 && L.head_dim == 64u) return launch_split_mfma<kF16, 64, 64, 1>(a, g, stream);
-        if (L.dtype == kF16 && L.head_dim == 128u) return launch_split_mfma<kF16, 128, 32, 1>(a, g, stream);
-        if (L.dtype == kF8 && L.head_dim == 256u) return launch_split_mfma<kF8, 256, 32, 1>(a, g, stream);
-        if (L.dtype == kF16 && L.head_dim == 256u) return launch_split_mfma<kF16, 256, 32, 1>(a, g, stream);
+        // Tiles with fewer full runs than the workgroup has run streams (the reference's 64-key tiles: two runs of 32 rows for
+        // four wavefronts) take runs of half the rows, so that every wavefront has one; a launch that deals the runs of the
+        // whole span (interleave) keeps full runs.
+        const bool short_tiles = !a.interleave && a.tile < (uint32_t)kMfmaWaves * il_full_run(L.head_dim);
+#define VFKV_TM(DT, DD, FULL) \
+    if (L.dtype == DT && L.head_dim == DD) \
+        return short_tiles ? launch_split_mfma<DT, DD, FULL / 2, 1>(a, g, stream) : launch_split_mfma<DT, DD, FULL, 1>(a, g, stream);
+        VFKV_TM(kF8, 64u, 64) VFKV_TM(kF16, 64u, 64) VFKV_TM(kF8, 128u, 32) VFKV_TM(kF16, 128u, 32) VFKV_TM(kF8, 256u, 32)
+#undef VFKV_TM
+        if (L.dtype == kF16 && L.head_dim == 256u) return launch_split_mfma<kF16, 256, 16, 1>(a, g, stream);      // (32 rows of 512 bytes: 32 KiB per wavefront in flight)
         // (runs of 16 rows: with 32 a wavefront has 48 KiB of F16 rows in flight; 9-10 % per layer at every length, FP8 and F16)
         if (L.dtype == kF8 && L.head_dim == 512u) return launch_split_mfma<kF8, 512, 16, 1, 2>(a, g, stream);
         if (L.dtype == kF16 && L.head_dim == 512u) return launch_split_mfma<kF16, 512, 16, 1, 2>(a, g, stream);

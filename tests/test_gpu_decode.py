@@ -75,6 +75,11 @@ CASES = [
     (vf.KvDtype.F16, 8, 4, 512, 200, 64, 0, 0.0),
     (vf.KvDtype.F16, 8, 2, 512, 1900, 192, 700, 40.0),   # head_dim 512 over a 2-byte cache: window, soft-cap
     (vf.KvDtype.F16, 12, 4, 64, 1000, 512, 0, 0.0),
+    # tiles with fewer full runs than the workgroup has run streams (the reference's 64-key tiles): runs of half the rows
+    (vf.KvDtype.F8, 16, 8, 256, 700, 64, 100, 0.0),
+    (vf.KvDtype.F16, 32, 8, 128, 900, 64, 0, 0.0),
+    (vf.KvDtype.F8, 32, 8, 128, 900, 96, 50, 30.0),      # 96-key tiles: three full runs, or six of half the rows
+    (vf.KvDtype.F8, 16, 8, 64, 900, 128, 0, 0.0),        # head_dim 64: two full runs of 64 rows per tile
     (vf.KvDtype.F32, 32, 8, 128, 700, 128, 0, 0.0),
     (vf.KvDtype.F32, 8, 2, 256, 300, 64, 50, 0.0),
     (vf.KvDtype.F32, 4, 2, 64, 300, 64, 0, 10.0),

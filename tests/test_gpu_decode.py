@@ -124,8 +124,8 @@ RUN_LENGTH_CASES = [
     (vf.KvDtype.F8, 16, 4, 64, 1501, 64, 0, 20.0),     # head_dim 64: runs of 32 rows
     (vf.KvDtype.F8, 16, 4, 64, 1501, 768, 333, 0.0),   # runs of 64 rows
     (vf.KvDtype.F16, 32, 8, 128, 1501, 64, 0, 0.0),    # runs of 16 rows
-    (vf.KvDtype.F16, 32, 8, 128, 650, 384, 77, 0.0),   # 2 tiles, 21 full runs over 8 streams (between 1.5 and 4 per stream): 32 rows
-    (vf.KvDtype.F16, 32, 8, 128, 1501, 768, 0, 30.0),  # 47 full runs over 8 streams (4 and more per stream): 16 rows again
+    (vf.KvDtype.F16, 32, 8, 128, 650, 384, 77, 0.0),   # 2 tiles, 21 full runs over 8 streams (more than 1.5 per stream): 32 rows
+    (vf.KvDtype.F16, 32, 8, 128, 1501, 768, 0, 30.0),  # 47 full runs over 8 streams, with the soft-cap: 32 rows
     (vf.KvDtype.F16, 8, 4, 64, 1501, 768, 333, 0.0),   # F16 rows of 64: 32 rows at every length
     (vf.KvDtype.F8, 16, 8, 256, 1501, 768, 333, 0.0),  # FP8 rows of 256: 16 rows at every length
     (vf.KvDtype.F16, 16, 8, 256, 1501, 768, 333, 50.0),

@@ -712,15 +712,15 @@ static hipError_t launch_split_il(const SplitArgs& a_in, uint32_t g, const RopeF
 //     4-12 % per layer: the launch is a latency chain there and a smaller unit shortens it;
 //   * 32 KiB in flight per wavefront is too much at every length (F16 256: 13.8 -> 11.7 us at 4 096 keys, 28.9 -> 26.9 at 16 384);
 //   * the 8 KiB shapes lose with half runs from two full runs per stream on (FP8 128: 8.8 -> 9.3 us at 8 192 keys, 10.0 -> 11.2
-//     at 12 288, 16.4 -> 18.6 at 32 768), the 16 KiB shapes are level or 1-4 % ahead there (F16 128 at 32 768: 26.6 -> 25.7).
+//     at 12 288, 16.4 -> 18.6 at 32 768), and so do F16 rows of 128 (15.6 -> 16.0 us at 16 384 keys, 25.9 -> 26.8 at 32 768,
+//     47.2 -> 48.5 at 65 536); F16 rows of 64 and FP8 rows of 256 are level there.
 static uint32_t il_full_run(uint32_t D) { return D == 64u ? 64u : 32u; }
 
 static bool il_half_runs(uint32_t dtype, uint32_t D, uint32_t span_rows, uint32_t n_tiles) {
     static const bool off = [] { const char* e = getenv("VFKV_DECODE_HALF_RUNS"); return e && e[0] == '0'; }();   // for comparisons (the shapes that have both)
     if (off) return false;
     const uint32_t full = il_full_run(D), units = (span_rows + full - 1u) / full, S = (uint32_t)kMfmaWaves * n_tiles;
-    if (dtype == kF8 && D != 256u) return 2u * units <= 3u * S;
-    if (dtype == kF16 && D == 128u) return 2u * units <= 3u * S || units >= 4u * S;
+    if ((dtype == kF8 && D != 256u) || (dtype == kF16 && D == 128u)) return 2u * units <= 3u * S;
     return true;                     // F16 rows of 64 and of 256 elements, FP8 rows of 256
 }
 

@@ -92,9 +92,10 @@ MFMA_DTYPE = "f16 mfma on value + remainder operand pairs, f32 accumulate"   # w
 
 
 def mfma_decode_worker(dtype_label, head_dim):
-    """Mirrors the library's choice: FP8 / F16 caches at head_dim 64 / 128 / 256 / 512 run on the matrix-core worker."""
+    """Mirrors the library's choice: FP8 / F16 caches at head_dim 64 / 128 / 256 / 512 run on the matrix-core worker, and so
+    do the multiples of 16 between 64 and 256 (on the next wider worker, tail masked off)."""
     return (os.environ.get("VFKV_DECODE_WORKER", "m")[:1] != "v" and dtype_label in ("FP8", "FP16")
-            and head_dim in (64, 128, 256, 512))
+            and (head_dim in (64, 128, 256, 512) or (64 < head_dim < 256 and head_dim % 16 == 0)))
 
 
 def parse_args():
@@ -402,7 +403,7 @@ def bench_decode(args, wl):
 
     mfma_worker = mfma_decode_worker(wl.dtype.label(), D)
     f32_mfma = wl.dtype.label() == "FP32" and D in (64, 128, 256) and os.environ.get("VFKV_DECODE_WORKER", "m")[:1] != "v"
-    il_worker = mfma_worker and D != 512 and os.environ.get("VFKV_DECODE_IL", "1")[:1] != "0"   # (mirrors split_interleaves() of the library)
+    il_worker = mfma_worker and D in (64, 128, 256) and os.environ.get("VFKV_DECODE_IL", "1")[:1] != "0"   # (mirrors split_interleaves() of the library)
     worker_name = (("split_mfma_il_rope_kernel" if wl.rope else "split_mfma_il_kernel") if il_worker else "split_mfma_kernel" if mfma_worker
                    else "split_mfma_f32_kernel" if f32_mfma else "split_kernel")
     traffic, traffic_source = profiled_traffic(wl.name) if mfma_worker else (None, None)   # the profiles cover the default worker

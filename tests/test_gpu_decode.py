@@ -83,11 +83,22 @@ CASES = [
     (vf.KvDtype.F32, 32, 8, 128, 700, 128, 0, 0.0),
     (vf.KvDtype.F32, 8, 2, 256, 300, 64, 50, 0.0),
     (vf.KvDtype.F32, 4, 2, 64, 300, 64, 0, 10.0),
-    # shapes only the generic worker covers
-    (vf.KvDtype.F32, 4, 2, 512, 200, 64, 0, 0.0),
+    # head widths between the tiled ones (FP8 / F16): the next wider matrix-core worker with its tail masked off
     (vf.KvDtype.F16, 6, 2, 80, 333, 64, 10, 0.0),
     (vf.KvDtype.F8, 4, 4, 96, 333, 128, 0, 0.0),
+    (vf.KvDtype.F8, 32, 32, 96, 1500, 256, 0, 0.0),      # Phi-3-mini geometry (G = 1)
+    (vf.KvDtype.F16, 32, 32, 96, 777, 64, 100, 0.0),     # 64-key tiles (runs of 16 rows), window inside a tile
+    (vf.KvDtype.F16, 32, 32, 80, 1200, 320, 0, 30.0),    # Phi-2 geometry, soft-cap
+    (vf.KvDtype.F8, 16, 4, 112, 900, 128, 50, 0.0),
+    (vf.KvDtype.F8, 24, 2, 96, 800, 512, 0, 0.0),        # G = 12: slices of 8 and 4 heads
+    (vf.KvDtype.F8, 8, 2, 160, 700, 64, 0, 0.0),         # on the worker for 256
+    (vf.KvDtype.F16, 16, 8, 192, 1300, 256, 300, 50.0),
+    (vf.KvDtype.F16, 8, 4, 224, 500, 128, 0, 0.0),
+    # shapes only the generic worker covers
+    (vf.KvDtype.F32, 4, 2, 512, 200, 64, 0, 0.0),
     (vf.KvDtype.F32, 3, 1, 50, 100, 64, 0, 0.0),
+    (vf.KvDtype.F32, 4, 2, 96, 300, 64, 0, 0.0),
+    (vf.KvDtype.F16, 4, 2, 40, 200, 64, 0, 0.0),
 ]
 
 
@@ -318,6 +329,10 @@ def test_config2_fp8_outliers_append_then_decode_two_layers():
     # the appending wavefront in the worker with full runs where the cases above take half runs (two to four full runs per stream)
     (vf.KvDtype.F16, 32, 8, 128, 8192, 0),
     (vf.KvDtype.F8, 16, 8, 64, 16384, 0),
+    # head widths served by the next wider worker with its tail masked off: the row is written with its real stride
+    (vf.KvDtype.F8, 32, 32, 96, 3000, 0),
+    (vf.KvDtype.F16, 8, 4, 192, 2000, 500),
+    (vf.KvDtype.F16, 32, 32, 80, 100, 0),       # one tile: the worker also writes the output
 ])
 def test_kv_write_attention_in_one_call_matches_the_two_calls(dtype, heads, hkv, d, ctx, window):
     # step_kv_write + step_attention (executor/attention.rs:546-625) through the single entry point: cache bytes and
@@ -487,11 +502,11 @@ def test_caller_owned_buffers_give_the_same_output_at_any_relative_alignment(dty
 
 
 def test_shapes_on_the_generic_fallback_leave_a_note():
-    # head_dim 80 has no tiled kernel: the result is still right, and vfkv_last_note says that the call was a slow one;
-    # a shape on the tiled kernels clears it
+    # head_dim 72 has no tiled kernel (80 runs on the worker for 128 with its tail masked off): the result is still right,
+    # and vfkv_last_note says that the call was a slow one; a shape on the tiled kernels clears it
     L = vf._ffi.lib()
     r = rng(80)
-    for d, slow in ((80, True), (128, False)):
+    for d, slow in ((72, True), (80, False), (128, False)):
         heads, hkv, seq = 8, 2, 300
         q = fp16_normal(r, (heads, d))
         k, v = encode_np(fp16_normal(r, (seq, hkv, d)), vf.KvDtype.F16), encode_np(fp16_normal(r, (seq, hkv, d)), vf.KvDtype.F16)

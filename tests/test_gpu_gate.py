@@ -70,7 +70,10 @@ DECODE_CASES = (
     (vf.KvDtype.F16, 16, 8, 256, 3000, 1024, True),
     (vf.KvDtype.F8, 16, 4, 128, 100, 0, True),         # one tile: the worker writes o, the gate runs as its own launch
     (vf.KvDtype.F32, 8, 2, 64, 700, 0, True),          # vector-ALU worker, separate append
-    (vf.KvDtype.F8, 6, 2, 80, 300, 0, False),          # generic kernels: the merge cannot take the gate
+    (vf.KvDtype.F8, 6, 2, 80, 300, 0, False),          # head_dim 80: the ragged form of the merge applies the gate
+    (vf.KvDtype.F16, 32, 32, 96, 2500, 0, True),       # Phi-3 geometry with a gate
+    (vf.KvDtype.F32, 6, 2, 72, 300, 0, False),         # generic worker; the ragged merge still takes the gate
+    (vf.KvDtype.F32, 2, 1, 72, 9000, 0, False),        # generic kernels with more than 64 partials: the merge cannot take the gate
     (vf.KvDtype.F16, 8, 1, 256, 12000, 0, True),       # one KV head, 188 tiles: the four-wavefront merge applies the gate
 )
 

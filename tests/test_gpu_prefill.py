@@ -75,6 +75,15 @@ CASES = [
     (vf.KvDtype.F8, 12, 4, 96, 33, 200, 0, 0.0),      # head_dim 96: 4-byte loads of the 24-byte row quarters
     (vf.KvDtype.F16, 6, 6, 96, 17, 50, 10, 0.0),
     (vf.KvDtype.F32, 8, 4, 96, 21, 80, 0, 0.0),
+    # the other head widths between the tiled ones, on the same f32 matrix-core kernel
+    (vf.KvDtype.F16, 32, 32, 80, 40, 300, 0, 0.0),    # Phi-2 geometry (G = 1)
+    (vf.KvDtype.F8, 8, 2, 80, 19, 100, 30, 20.0),
+    (vf.KvDtype.F32, 6, 2, 112, 33, 150, 0, 0.0),
+    (vf.KvDtype.F8, 16, 4, 112, 25, 90, 0, 0.0),
+    (vf.KvDtype.F16, 8, 2, 160, 21, 200, 50, 0.0),
+    (vf.KvDtype.F8, 12, 4, 192, 35, 120, 0, 30.0),
+    (vf.KvDtype.F16, 4, 4, 224, 18, 70, 0, 0.0),
+    (vf.KvDtype.F32, 4, 2, 192, 17, 60, 0, 0.0),
     (vf.KvDtype.F8, 16, 8, 256, 48, 700, 0, 50.0),    # head_dim 256, G = 2: three key splits, soft-cap
     (vf.KvDtype.F16, 8, 2, 256, 35, 260, 100, 0.0),   # head_dim 256, G = 4 on a 2-byte cache, window
     (vf.KvDtype.F8, 32, 4, 256, 18, 130, 0, 0.0),     # head_dim 256, G = 8: the group is spread over workgroups so that the Q planes fit

@@ -628,7 +628,8 @@ uint32_t vfkv_decode_tile_for(uint32_t span, uint32_t n_heads, uint32_t n_kv_hea
     // The matrix-core worker (1- and 2-byte caches, head_dim 64 / 128) runs best with one workgroup per CU and
     // serves up to 8 heads of a group per workgroup; the vector-ALU worker wants two and serves up to 4.
     const bool mfma = (kv_dtype == VFKV_F8E4M3 || kv_dtype == VFKV_F16) &&
-                      (head_dim == 64u || head_dim == 128u || head_dim == 256u || head_dim == 512u);
+                      (head_dim == 64u || head_dim == 128u || head_dim == 256u || head_dim == 512u ||
+                       vfkv::split_padded_dim(kv_dtype, head_dim) != 0u);
     if (mfma) {
         // short spans: one tile, so the worker writes the output itself and no merge launch follows.  The tile's runs of 32
         // keys are walked by the workgroup's four run streams (two at head_dim 512) one after the other, and a further round

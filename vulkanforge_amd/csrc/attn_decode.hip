@@ -1,8 +1,10 @@
 // Split-K decode attention for gfx950: worker (flash_attn_split.comp:82-162) and log-sum-exp
 // merge (flash_attn_reduce.comp:35-81), re-designed around the HBM stream.
 //
-//   split_mfma_kernel    (attn_decode_mfma.h) matrix-core worker: FP8 / F16 caches, head_dim 64 / 128 / 256 / 512 -- the
-//                        kernel every benchmark configuration runs on
+//   split_mfma_kernel    (attn_decode_mfma.h) matrix-core worker: FP8 / F16 caches, head_dim 64 / 128 / 256 / 512, and the
+//                        multiples of 16 in between on the next wider instantiation with its tail masked off
+//   split_mfma_il_kernel (attn_decode_il.h) the same arithmetic with the runs of the whole span dealt to the workgroups:
+//                        head_dim 64 / 128 / 256, the kernel every benchmark configuration runs on
 //   split_kernel         vector-ALU worker described below: F32 caches (and every shape under VFKV_DECODE_WORKER=valu)
 //   split_generic_kernel one wavefront per (head, tile), any dtype, head_dim <= 512
 //   reduce_direct_kernel merge of up to 64 partials per head without LDS; reduce_kernel / reduce_generic_kernel beyond
@@ -544,12 +546,14 @@ __global__ __launch_bounds__(kReduceThreads) void reduce_kernel(const float* __r
 // dimension of all partial outputs before the first reduction, so the kernel costs one memory round trip.
 // GATED: the output element is multiplied by sigmoid(gate) in the same store (the reference's separate sigmoid_mul dispatch,
 // executor/attention.rs:632-680); the gate value is requested with the partials.
-template <int MAXT, bool GATED>
+// RAGGED: head_dim is no multiple of 64; the lanes past the last output dimension follow it and store nothing.
+template <int MAXT, bool GATED, bool RAGGED = false>
 __global__ __launch_bounds__(kWave) void reduce_direct_kernel(const float* __restrict__ so, const float* __restrict__ sm,
                                                               const float* __restrict__ ss, float* __restrict__ o,
                                                               uint32_t D, uint32_t n_tiles, GateArgs gate) {
     const uint32_t h = blockIdx.y, lane = threadIdx.x;
-    const uint32_t d = blockIdx.x * kWave + lane;
+    const uint32_t d_lane = blockIdx.x * kWave + lane;
+    const uint32_t d = RAGGED && d_lane >= D ? D - 1u : d_lane;
     const float* ho = so + (size_t)h * n_tiles * D + d;
     float x[MAXT];
 #pragma unroll
@@ -569,7 +573,7 @@ __global__ __launch_bounds__(kWave) void reduce_direct_kernel(const float* __res
     for (int j = 0; j < MAXT; ++j)
         acc = fmaf(__builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, wj), j)), x[j], acc);
     const float r = acc * (1.0f / L);
-    o[(size_t)h * D + d] = GATED ? sigmoid_gate(r, gv) : r;
+    if (!RAGGED || d_lane < D) o[(size_t)h * D + d] = GATED ? sigmoid_gate(r, gv) : r;
 }
 
 // 65 to 2 048 tiles (few KV heads over long contexts: one tile per compute unit then means many per head; the reference's
@@ -663,15 +667,16 @@ constexpr int kSplitWaves = 4;
 // were each measured slower on the 32 k and 8 k FP8 workloads.
 constexpr int kMfmaWaves = 4;
 
-template <int DT, int D, int RUN, int PF, int NH = 1>
-static hipError_t launch_split_mfma(const SplitArgs& a, uint32_t g, hipStream_t stream) {
+template <int DT, int D, int RUN, int PF, int NH = 1, bool PAD = false>
+static hipError_t launch_split_mfma(const SplitArgs& a, uint32_t g, hipStream_t stream, uint32_t head_dim = (uint32_t)D) {
     constexpr int NW = kMfmaWaves;
     const uint32_t gt = g < 8u ? g : 8u;
     dim3 grid(a.n_kv_heads, a.n_tiles, (g + gt - 1u) / gt);
+    if (PAD && (head_dim >= (uint32_t)D || head_dim % 16u != 0u)) return hipErrorInvalidValue;
     if (a.softcap > 0.f)
-        hipLaunchKernelGGL((split_mfma_kernel<DT, D, RUN, PF, NW, true, NH>), grid, dim3(NW * kWave), 0, stream, a, gt);
+        hipLaunchKernelGGL((split_mfma_kernel<DT, D, RUN, PF, NW, true, NH, PAD>), grid, dim3(NW * kWave), 0, stream, a, gt, head_dim);
     else
-        hipLaunchKernelGGL((split_mfma_kernel<DT, D, RUN, PF, NW, false, NH>), grid, dim3(NW * kWave), 0, stream, a, gt);
+        hipLaunchKernelGGL((split_mfma_kernel<DT, D, RUN, PF, NW, false, NH, PAD>), grid, dim3(NW * kWave), 0, stream, a, gt, head_dim);
     return hipGetLastError();
 }
 
@@ -727,6 +732,7 @@ static bool il_half_runs(uint32_t dtype, uint32_t D, uint32_t span_rows, uint32_
 // The shortest run the worker may take for this shape: what the caller sizes its workgroup count by.
 uint32_t split_run_rows(uint32_t dtype, uint32_t D) {
     if (dtype == kF32 && (D == 64u || D == 128u || D == 256u)) return 16u;      // the F32 worker: one tile per run
+    if (const uint32_t dp = split_padded_dim(dtype, D)) return dp == 256u && dtype == kF16 ? 16u : 32u;   // as launch_split deals them
     if ((dtype != kF8 && dtype != kF16) || (D != 64u && D != 128u && D != 256u && D != 512u)) return 0u;
     return il_full_run(D) / 2u;      // (head_dim 512: 16 rows as well)
 }
@@ -746,9 +752,16 @@ static bool f32_mfma_shape(uint32_t dtype, uint32_t D) {
     return dtype == kF32 && (D == 64u || D == 128u || D == 256u);
 }
 
+// Head widths between the tiled ones (Phi-style 80 / 96, 112, 160, 192, 224) over FP8 / F16 rows: the width of the worker
+// that serves them with its tail masked off (split_mfma_kernel's PAD form), 0 for every other shape.
+uint32_t split_padded_dim(uint32_t dtype, uint32_t D) {
+    if ((dtype != kF8 && dtype != kF16) || D % 16u != 0u) return 0u;
+    return (D > 64u && D < 128u) ? 128u : (D > 128u && D < 256u) ? 256u : 0u;
+}
+
 // Shapes the matrix-core worker is built for (head_dim 512: two wavefronts per run, each half of the output columns).
 static bool mfma_worker_shape(uint32_t dtype, uint32_t D) {
-    return (dtype == kF8 || dtype == kF16) && (D == 64u || D == 128u || D == 256u || D == 512u);
+    return (dtype == kF8 || dtype == kF16) && (D == 64u || D == 128u || D == 256u || D == 512u || split_padded_dim(dtype, D) != 0u);
 }
 
 // VFKV_DECODE_WORKER=valu keeps the vector-ALU worker for every shape (for comparisons).
@@ -769,6 +782,7 @@ uint32_t split_run_streams(const SplitLaunch& L, uint32_t* heads_per_wg) {
     if (!aligned || slab_bytes >= 0x7FFF0000ull || !mfma_worker_enabled()) return 0u;
     if (L.head_dim == 512u && (L.dtype == kF8 || L.dtype == kF16)) return (uint32_t)kMfmaWaves / 2u;
     if (f32_mfma_shape(L.dtype, L.head_dim)) { if (heads_per_wg) *heads_per_wg = 16u; return (uint32_t)kMfmaWaves; }
+    if (split_padded_dim(L.dtype, L.head_dim) != 0u) return (uint32_t)kMfmaWaves;
     return 0u;
 }
 
@@ -895,6 +909,15 @@ hipError_t launch_split(const SplitLaunch& L, hipStream_t stream, bool* generic_
         // (runs of 16 rows: with 32 a wavefront has 48 KiB of F16 rows in flight; 9-10 % per layer at every length, FP8 and F16)
         if (L.dtype == kF8 && L.head_dim == 512u) return launch_split_mfma<kF8, 512, 16, 1, 2>(a, g, stream);
         if (L.dtype == kF16 && L.head_dim == 512u) return launch_split_mfma<kF16, 512, 16, 1, 2>(a, g, stream);
+        // head widths between the tiled ones: the next wider worker with its tail masked off
+        if (const uint32_t dp = split_padded_dim(L.dtype, L.head_dim)) {
+            const bool short_pad = !a.interleave && a.tile < (uint32_t)kMfmaWaves * 32u;
+#define VFKV_TP(DT, DD, FULL) \
+    if (L.dtype == DT && dp == DD) \
+        return short_pad ? launch_split_mfma<DT, DD, 16, 1, 1, true>(a, g, stream, L.head_dim) : launch_split_mfma<DT, DD, FULL, 1, 1, true>(a, g, stream, L.head_dim);
+            VFKV_TP(kF8, 128u, 32) VFKV_TP(kF16, 128u, 32) VFKV_TP(kF8, 256u, 32) VFKV_TP(kF16, 256u, 16)
+#undef VFKV_TP
+        }
     }
     if (aligned && out_aligned && slab_bytes < 0x7FFF0000ull && mfma_worker_enabled() && f32_mfma_shape(L.dtype, L.head_dim)) {
         if (L.head_dim == 64u) return launch_split_f32<64>(a, g, stream);
@@ -933,6 +956,17 @@ hipError_t launch_reduce(const float* so, const float* sm, const float* ss, floa
         } else {
             if (n_tiles <= 32u) hipLaunchKernelGGL((reduce_direct_kernel<32, false>), grid, dim3(kWave), 0, stream, so, sm, ss, o, D, n_tiles, g);
             else hipLaunchKernelGGL((reduce_direct_kernel<64, false>), grid, dim3(kWave), 0, stream, so, sm, ss, o, D, n_tiles, g);
+        }
+    } else if (n_tiles <= 64u) {                       // head sizes that are no multiple of 64
+        const dim3 grid((D + kWave - 1u) / kWave, n_heads);
+        const GateArgs g = gated ? *gate : GateArgs();
+        if (gated) {
+            if (n_tiles <= 32u) hipLaunchKernelGGL((reduce_direct_kernel<32, true, true>), grid, dim3(kWave), 0, stream, so, sm, ss, o, D, n_tiles, g);
+            else hipLaunchKernelGGL((reduce_direct_kernel<64, true, true>), grid, dim3(kWave), 0, stream, so, sm, ss, o, D, n_tiles, g);
+            if (gate_applied) *gate_applied = true;
+        } else {
+            if (n_tiles <= 32u) hipLaunchKernelGGL((reduce_direct_kernel<32, false, true>), grid, dim3(kWave), 0, stream, so, sm, ss, o, D, n_tiles, g);
+            else hipLaunchKernelGGL((reduce_direct_kernel<64, false, true>), grid, dim3(kWave), 0, stream, so, sm, ss, o, D, n_tiles, g);
         }
     } else if (n_tiles <= 2048u && D % (uint32_t)kWave == 0u) {
         const dim3 grid(D / kWave, n_heads);

@@ -34,8 +34,14 @@ namespace vfkv {
 // NH > 1 (head_dim 512): NH wavefronts walk the same runs.  Each computes the scores over the whole head_dim and stages,
 // accumulates, merges and stores its own slice of D / NH output columns (the accumulators of a 512-wide head do not fit
 // one wavefront); the workgroup then walks NW / NH runs at a time.
-template <int DT, int D, int RUN, int PF, int NW, bool CAP, int NH = 1>
-__global__ __launch_bounds__(NW * 64) void split_mfma_kernel(SplitArgs a, uint32_t gt) {
+//
+// PAD (NH == 1): the heads of the cache are `head_dim` < D elements wide (a multiple of 16: 80 / 96 / 112 on the kernel for
+// 128, 160 / 192 / 224 on the one for 256).  The kernel works on rows of D elements whose tail does not exist: the query
+// planes hold zeros there, the lanes whose 16-byte piece of a K or V row would lie past the head read the head's first
+// piece again (finite cache values that meet query zeros, or output columns nobody stores), and the d-tiles past head_dim
+// are neither multiplied nor stored.  Rows, queries, partials and the appended row keep their real stride of head_dim.
+template <int DT, int D, int RUN, int PF, int NW, bool CAP, int NH = 1, bool PAD = false>
+__global__ __launch_bounds__(NW * 64) void split_mfma_kernel(SplitArgs a, uint32_t gt, uint32_t head_dim) {
     constexpr int ES = DT == kF16 ? 2 : 1;
     constexpr int DV = D / NH;                   // output columns of a wavefront
     constexpr int NP = NW / NH;                  // run streams of the workgroup
@@ -60,6 +66,8 @@ __global__ __launch_bounds__(NW * 64) void split_mfma_kernel(SplitArgs a, uint32
     constexpr int MERGE_ROWS = ((DV / 16) * 64 * 16 + VPITCH * 2 - 1) / (VPITCH * 2);    // rows of the staging area the merge needs
     constexpr int LROWS = RUN > MERGE_ROWS ? RUN : MERGE_ROWS;
     static_assert(NW % NH == 0, "whole run streams");
+    static_assert(!PAD || NH == 1, "padded heads: one wavefront per run");
+    const uint32_t dr = PAD ? head_dim : (uint32_t)D;                   // elements per head as the cache holds them
 
     __shared__ __attribute__((aligned(16))) _Float16 vlds[NW][LROWS * VPITCH];
     __shared__ float lds_m[NW][8], lds_l[NW][8];
@@ -71,7 +79,11 @@ __global__ __launch_bounds__(NW * 64) void split_mfma_kernel(SplitArgs a, uint32
     const int n16 = lane & 15, kg = lane >> 4;
     const int col = n16 & 7;
     const bool is_lo = n16 >= 8;
-    const uint32_t kvh = blockIdx.x, jl = blockIdx.y;     // KV head fastest: the workgroups of one tile start together
+    // KV head fastest: the workgroups of one tile start together.  PAD: a head's slice of a row is not a whole number of
+    // 128-byte lines, so neighbouring KV heads share lines; consecutive workgroups go to different XCDs (each with its own
+    // L2), so the heads are dealt such that every XCD gets a block of neighbours.
+    const uint32_t jl = blockIdx.y;
+    const uint32_t kvh = (PAD && (a.n_kv_heads & 7u) == 0u) ? (blockIdx.x & 7u) * (a.n_kv_heads >> 3) + (blockIdx.x >> 3) : blockIdx.x;
     const uint32_t g_all = a.group;                        // n_heads / n_kv_heads, divided on the host
     const uint32_t hz = blockIdx.z * gt;
     const uint32_t gcount = g_all - hz < gt ? g_all - hz : gt;
@@ -86,13 +98,19 @@ __global__ __launch_bounds__(NW * 64) void split_mfma_kernel(SplitArgs a, uint32
     uint32_t tile_end = tile_base + a.tile; if (il || tile_end > a.seq_len) tile_end = a.seq_len;
     const uint32_t lo = tile_base > a.kv_start ? tile_base : a.kv_start;
 
-    const uint32_t row_stride = a.n_kv_heads * D * ES;
+    const uint32_t row_stride = a.n_kv_heads * dr * ES;
     const __amdgpu_buffer_rsrc_t krsrc = __builtin_amdgcn_make_buffer_rsrc((void*)a.k, 0, a.seq_len * row_stride, 0x00020000);
     const __amdgpu_buffer_rsrc_t vrsrc = __builtin_amdgcn_make_buffer_rsrc((void*)a.v, 0, a.seq_len * row_stride, 0x00020000);
-    const uint32_t head_b = kvh * D * ES;
+    const uint32_t head_b = kvh * dr * ES;
     const uint32_t lane_koff = n16 * row_stride + head_b + kg * (KIL ? 16 : SEGB);
     const int vrow = lane / VCHUNK_ROW, vcol = lane % VCHUNK_ROW;
-    const uint32_t lane_voff = vrow * row_stride + head_b + ds * DV * ES + vcol * 16;
+    const uint32_t lane_voff = vrow * row_stride + head_b + ds * DV * ES + (PAD && (uint32_t)vcol * 16u >= dr * ES ? 0 : vcol * 16);
+    uint32_t kpiece[KLD];                        // PAD: byte offset of piece x in the head's row (0 where the piece does not exist)
+#pragma unroll
+    for (int x = 0; x < KLD; ++x) {
+        const uint32_t bo = (uint32_t)(kg * (KIL ? 16 : SEGB) + x * (KIL ? 64 : 16));
+        kpiece[x] = bo < dr * ES ? bo : 0u;
+    }
     const float scale_l2 = a.scale * 1.44269504088896f;
     const float cap_l2 = a.softcap * 1.44269504088896f;
     const float inv_cap_l2 = CAP ? 1.0f / cap_l2 : 0.f;
@@ -109,11 +127,17 @@ __global__ __launch_bounds__(NW * 64) void split_mfma_kernel(SplitArgs a, uint32
     auto issue_k = [&](int b, int t, uint32_t off) {
 #pragma unroll
         for (int x = 0; x < KLD; ++x)
-            kraw[b][t][x] = __builtin_amdgcn_raw_buffer_load_b128(krsrc, lane_koff + x * (KIL ? 64 : 16), off + (uint32_t)(t * 16) * row_stride, 0);
+            kraw[b][t][x] = __builtin_amdgcn_raw_buffer_load_b128(krsrc, PAD ? n16 * row_stride + head_b + kpiece[x] : lane_koff + x * (KIL ? 64 : 16),
+                                                                  off + (uint32_t)(t * 16) * row_stride, 0);
     };
     auto issue_v = [&](int b, int c, uint32_t off) {
         vraw[b][c] = __builtin_amdgcn_raw_buffer_load_b128(vrsrc, lane_voff, off + (uint32_t)(c * VROWS) * row_stride, 0);
     };
+
+    if (PAD) {                                                      // the query planes' tails stay zero (nothing is in flight yet: the barrier is cheap here)
+        for (int i = tid; i < 16 * (D + 8) / 8; i += NW * 64) reinterpret_cast<u32x4*>(&qlds[0][0])[i] = u32x4{0u, 0u, 0u, 0u};
+        __syncthreads();
+    }
 
     // ---- optional fused append (step_kv_write, executor/attention.rs:546): the workgroup whose tile holds the new
     // position converts and stores this KV head's slice of the new K and V rows before anything reads them.  The
@@ -125,9 +149,9 @@ __global__ __launch_bounds__(NW * 64) void split_mfma_kernel(SplitArgs a, uint32
                           : (a.append_pos >= tile_base && a.append_pos < tile_end);
     if (owns_new_row) {
         constexpr int EPW = 4 / ES;                              // elements per 32-bit word of the cache
-        if (tid < D / EPW) {
-            const size_t src = (size_t)kvh * D + (size_t)tid * EPW;
-            const size_t dst = ((size_t)a.append_pos * a.n_kv_heads + kvh) * D * ES + (size_t)tid * 4;
+        if ((uint32_t)tid < dr / EPW) {
+            const size_t src = (size_t)kvh * dr + (size_t)tid * EPW;
+            const size_t dst = ((size_t)a.append_pos * a.n_kv_heads + kvh) * dr * ES + (size_t)tid * 4;
             uint32_t kw, vw;
             if (DT == kF8) {
                 const float4 kf = *reinterpret_cast<const float4*>(a.k_new + src);
@@ -173,12 +197,12 @@ __global__ __launch_bounds__(NW * 64) void split_mfma_kernel(SplitArgs a, uint32
     // remainder planes in LDS; lane (column n16, group kg) then holds q[kg*SEG + c*8 + j], j < 8, per k-step c.
     // The query load sits between the K and the V requests: loads return in order, so the wait for it covers K only.
     constexpr int QLD = (8 * D / 4 + NW * 64 - 1) / (NW * 64);      // 16-byte query loads per thread (<= 8 heads)
-    const int nq4 = (int)gcount * D / 4;
+    const int nq4 = (int)(gcount * dr) / 4;
     float4 qf[QLD];
 #pragma unroll
     for (int i = 0; i < QLD; ++i) {
         const int idx = tid + i * NW * 64;
-        qf[i] = *reinterpret_cast<const float4*>(a.q + (size_t)h0 * D + (idx < nq4 ? idx : 0) * 4);
+        qf[i] = *reinterpret_cast<const float4*>(a.q + (size_t)h0 * dr + (idx < nq4 ? idx : 0) * 4);
     }
 #pragma unroll
     for (int c = 0; c < VLD; ++c) issue_v(0, c, off0);
@@ -196,7 +220,7 @@ __global__ __launch_bounds__(NW * 64) void split_mfma_kernel(SplitArgs a, uint32
             const int idx = tid + i * NW * 64;
             if (idx >= nq4) continue;
             const float4 f = qf[i];
-            const int g = (idx * 4) / D, d = (idx * 4) % D;
+            const int g = PAD ? (int)((uint32_t)(idx * 4) / dr) : (idx * 4) / D, d = PAD ? idx * 4 - g * (int)dr : (idx * 4) % D;
             const float v4[4] = {f.x, f.y, f.z, f.w};
             _Float16 hv[4], lv[4];
 #pragma unroll
@@ -340,6 +364,7 @@ __global__ __launch_bounds__(NW * 64) void split_mfma_kernel(SplitArgs a, uint32
             for (int ks = 0; ks < PKS; ++ks)
 #pragma unroll
                 for (int dt = 0; dt < DTILES; ++dt) {
+                    if (PAD && (uint32_t)dt * 16u >= dr) continue;     // wavefront-uniform
                     // supplier lane s of a 16-lane group points at V[row = ks*32 + 4*kg + s/4 (+16)][d = dt*16 + 4*(s%4)]
                     const _Float16* p0 = vb + (ks * 32 + kg * 4 + n16 / 4) * VPITCH + dt * 16 + 4 * (n16 % 4);
                     const half4_t v0 = lds_read_tr16(p0);
@@ -351,6 +376,7 @@ __global__ __launch_bounds__(NW * 64) void split_mfma_kernel(SplitArgs a, uint32
             if (HALF) {                    // one tile of 16 rows: the 16-deep product on the tile's own weights
 #pragma unroll
                 for (int dt = 0; dt < DTILES; ++dt) {
+                    if (PAD && (uint32_t)dt * 16u >= dr) continue;
                     const _Float16* p0 = vb + (kg * 4 + n16 / 4) * VPITCH + dt * 16 + 4 * (n16 % 4);
                     const half4_t v0 = lds_read_tr16(p0);
                     const u32x2 pw = u32x2{pext[0], pext[1]};
@@ -403,7 +429,7 @@ __global__ __launch_bounds__(NW * 64) void split_mfma_kernel(SplitArgs a, uint32
     // forward/runs.rs:776-821): the merge is a plain normalisation, done here, and no merge launch follows
     const bool direct = a.o_direct != nullptr;
     const float inv_l = direct ? __builtin_amdgcn_rcpf(l) : 1.0f;
-    float* const obase = (direct ? a.o_direct + (size_t)(h0 + col) * D : a.so + pidx * D) + ds * DV;
+    float* const obase = (direct ? a.o_direct + (size_t)(h0 + col) * dr : a.so + pidx * dr) + ds * DV;
 #pragma unroll
     for (int t = 0; t < MT; ++t) {
         float4_t o = fw[0] * part[t][0];
@@ -413,7 +439,7 @@ __global__ __launch_bounds__(NW * 64) void split_mfma_kernel(SplitArgs a, uint32
             const float r = inv_l * (2.0f - l * inv_l);
             o *= r;
         }
-        if (writer) *reinterpret_cast<float4_t*>(obase + (t * NP + wp) * 16 + kg * 4) = o;
+        if (writer && (!PAD || (uint32_t)(t * NP + wp) * 16u < dr)) *reinterpret_cast<float4_t*>(obase + (t * NP + wp) * 16 + kg * 4) = o;
     }
     if (writer && w == 0 && kg == 0 && a.o_direct == nullptr) {
         a.sm[pidx] = M > -1e29f ? M * 0.693147180559945f : kMasked;

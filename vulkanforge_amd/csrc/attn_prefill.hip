@@ -2,8 +2,8 @@
 //
 // batch_mfma2_kernel   (attn_prefill_mfma2.h) f16 matrix-core tiles, private K / V tiles per wavefront: FP8 / F16 caches,
 //                      head_dim 64 / 128 / 256 / 512, any GQA group.
-// batch_mfma_f32_kernel (attn_prefill_f32.h) f32 matrix-core tiles: F32 caches (head_dim 64 / 96 / 128 / 256 / 512), FP8 / F16 caches at
-//                      head_dim 96.
+// batch_mfma_f32_kernel (attn_prefill_f32.h) f32 matrix-core tiles: F32 caches (head_dim 64 / 128 / 256 / 512), and every cache
+//                      type at the head widths between the tiled ones (80, 96, 112, 160, 192, 224).
 // batch_generic_kernel one wavefront per (query, head); covers every dtype and head_dim <= 512.
 #include "device_utils.h"
 #include "kernels.h"
@@ -285,6 +285,12 @@ static hipError_t launch_batch_kernels(const BatchLaunch& L, hipStream_t stream,
     }
         VFKV_PF32(kF32, 64, 1) VFKV_PF32(kF32, 128, 1) VFKV_PF32(kF32, 256, 1) VFKV_PF32(kF32, 96, 1)
         VFKV_PF32(kF16, 96, 1) VFKV_PF32(kF8, 96, 1) VFKV_PF32(kF32, 512, 2)
+        // the other head widths between the tiled ones (multiples of 16 up to 224), every cache type
+        VFKV_PF32(kF32, 80, 1) VFKV_PF32(kF16, 80, 1) VFKV_PF32(kF8, 80, 1)
+        VFKV_PF32(kF32, 112, 1) VFKV_PF32(kF16, 112, 1) VFKV_PF32(kF8, 112, 1)
+        VFKV_PF32(kF32, 160, 1) VFKV_PF32(kF16, 160, 1) VFKV_PF32(kF8, 160, 1)
+        VFKV_PF32(kF32, 192, 1) VFKV_PF32(kF16, 192, 1) VFKV_PF32(kF8, 192, 1)
+        VFKV_PF32(kF32, 224, 1) VFKV_PF32(kF16, 224, 1) VFKV_PF32(kF8, 224, 1)
 #undef VFKV_PF32
     }
     if (generic_used) *generic_used = true;

@@ -96,6 +96,9 @@ hipError_t launch_sigmoid_mul(float* data, uint32_t ne, const GateArgs& gate, hi
 // fold L.rope (which needs k_new / v_new as well).
 bool split_interleaves(const SplitLaunch& a);
 bool split_folds_rope(const SplitLaunch& a);
+// Width of the matrix-core worker that serves this head width with its tail masked off (FP8 / F16 rows of 80 / 96 / 112 ->
+// 128, 160 / 192 / 224 -> 256); 0 for every other shape.
+uint32_t split_padded_dim(uint32_t dtype, uint32_t head_dim);
 // Rows per run of the matrix-core worker for this shape (0: the shape is not the matrix-core worker's).
 uint32_t split_run_rows(uint32_t dtype, uint32_t head_dim);
 // Run streams per workgroup when the launch deals the runs of the span to its workgroups, not tiles (else 0), and how many

@@ -80,6 +80,9 @@ DECODE = {
     # the configuration-2 geometry over an F32 cache (the reference's VULKANFORGE_FP16_KV=0 mode; not a reference configuration):
     # the same bytes per layer as the headline workload
     "decode_f32_8k_32layers": DecodeWorkload("decode_f32_8k_32layers", 32, 32, 8, 128, 8193, KvDtype.F32, True),
+    # Phi-3-mini geometry (32 heads, no grouping, head_dim 96, F16 cache; not a reference configuration): a head width between
+    # the tiled ones, served by the worker for 128 with its tail masked off
+    "decode_f16_hd96_4k_32layers": DecodeWorkload("decode_f16_hd96_4k_32layers", 32, 32, 32, 96, 4097, KvDtype.F16, True),
     "decode_f16_hd256_sliding_12layers": DecodeWorkload("decode_f16_hd256_sliding_12layers", 12, 16, 8, 256, 16384,
                                                         KvDtype.F16, False, softcap=50.0, window=4096,
                                                         sliding_pattern=5),

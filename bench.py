@@ -49,7 +49,7 @@ PROFILED_TRAFFIC = {
 
 def prefill_kernel_name(kv_label, head_dim, group):
     """The kernel attn_prefill.hip launches for a shape with 16-byte aligned buffers."""
-    if kv_label == "FP32" or head_dim == 96:
+    if kv_label == "FP32":
         return "batch_mfma_f32_kernel"
     if kv_label == "FP8" and head_dim == 128 and group >= 2:
         return "batch_dma_kernel"       # two heads per wavefront over FP8 rows: V loaded straight into LDS

@@ -123,7 +123,9 @@ def test_decode_attention_gated_is_attention_then_gate(dtype, heads, hkv, d, n, 
     (vf.KvDtype.F8, 8, 2, 512, 21, 100),        # two wavefronts share a head, each gates its own output columns
     (vf.KvDtype.F16, 4, 4, 64, 1, 0),
     (vf.KvDtype.F32, 4, 2, 128, 20, 10),        # kernels without a gated store: the gate follows as its own launch
-    (vf.KvDtype.F8, 6, 2, 96, 20, 10),
+    (vf.KvDtype.F8, 6, 2, 96, 20, 10),          # heads of 96 elements on the kernel for 128: the gate keeps its real stride
+    (vf.KvDtype.F16, 32, 32, 80, 40, 100),      # one head per wavefront
+    (vf.KvDtype.F16, 8, 4, 192, 18, 30),
     (vf.KvDtype.F8, 128, 32, 128, 125, 200),    # 256 workgroups: two head pairs x four key splits, every wavefront gates the tiles it stores
 ))
 def test_prefill_attention_gated_is_attention_then_gate(dtype, heads, hkv, d, m, base):

@@ -304,6 +304,8 @@ def test_scores_that_drift_past_the_running_maximum(dtype, shape):
     (vf.KvDtype.F16, 28, 4, 128, 50, 1500, 0, 0.0),      # G = 7
     (vf.KvDtype.F8, 32, 8, 128, 512, 4096, 0, 0.0),      # a full chunk: plenty of workgroups, the plain path is taken
     (vf.KvDtype.F32, 8, 2, 128, 16, 2000, 0, 0.0),       # F32 cache: no key chunks, same result
+    (vf.KvDtype.F16, 32, 32, 96, 24, 5000, 0, 0.0),      # heads of 96 elements on the kernel for 128: partials with their real stride
+    (vf.KvDtype.F8, 8, 2, 192, 16, 3000, 1000, 20.0),    # heads of 192 on the kernel for 256, window, soft-cap
 ))
 def test_prefill_with_workspace_matches_plain_call_and_oracle(dtype, heads, hkv, d, m, base, window, cap):
     # vfkv_prefill_attention_ws cuts the keys into chunks over workgroups and merges the partials

@@ -2,8 +2,8 @@
 //
 // batch_mfma2_kernel   (attn_prefill_mfma2.h) f16 matrix-core tiles, private K / V tiles per wavefront: FP8 / F16 caches,
 //                      head_dim 64 / 128 / 256 / 512, any GQA group.
-// batch_mfma_f32_kernel (attn_prefill_f32.h) f32 matrix-core tiles: F32 caches (head_dim 64 / 128 / 256 / 512), and every cache
-//                      type at the head widths between the tiled ones (80, 96, 112, 160, 192, 224).
+// batch_mfma_f32_kernel (attn_prefill_f32.h) f32 matrix-core tiles: F32 caches (head_dim 64 / 128 / 256 / 512 and the multiples of
+//                      16 in between); FP8 / F16 caches of those in-between widths run on batch_mfma2_kernel's padded form.
 // batch_generic_kernel one wavefront per (query, head); covers every dtype and head_dim <= 512.
 #include "device_utils.h"
 #include "kernels.h"
@@ -116,12 +116,16 @@ static hipError_t launch_batch_kernels(const BatchLaunch& L, hipStream_t stream,
     const uint32_t g = L.n_heads / L.n_kv_heads;
     const uint64_t slab_bytes = (uint64_t)L.n_kv * L.n_kv_heads * L.head_dim * elem_size(L.dtype);
     const bool aligned = ((((uintptr_t)L.k) | ((uintptr_t)L.v) | ((uintptr_t)L.q) | ((uintptr_t)L.o)) & 15u) == 0u;
+    // Head widths between the tiled ones (80 / 96 / 112, 160 / 192 / 224) run on the next wider instantiation of the f16
+    // kernel with its tail masked off (PAD): hd is the width of the kernel, L.head_dim what the buffers hold.
+    const uint32_t dpad = split_padded_dim(L.dtype, L.head_dim);
+    const uint32_t hd = dpad != 0u ? dpad : L.head_dim;
     const bool mfma_ok = (L.dtype == kF8 || L.dtype == kF16) && aligned && slab_bytes < 0x7FFF0000ull &&
-                         (L.head_dim == 64u || L.head_dim == 128u || L.head_dim == 256u || L.head_dim == 512u);
+                         (hd == 64u || hd == 128u || hd == 256u || hd == 512u);
     // f16 matrix-core kernel: NCB heads per wavefront, private tiles per wavefront, no barrier in the loop
     if (mfma_ok) {
         // head_dim 512: one head per wavefront, and two wavefronts share a head (each owns half of the output columns)
-        const uint32_t nh = L.head_dim == 512u ? 2u : 1u;
+        const uint32_t nh = hd == 512u ? 2u : 1u;
         // Heads per wavefront.  Two where the registers allow it (a K / V tile is then converted once for both); odd groups
         // of three and more heads round up, the spare slot computes on zeros and stores nothing.  Where the rows are wide
         // (F16 at head_dim 128, everything at head_dim 256) the traffic between L2 and the CUs is what binds: four / two heads
@@ -132,22 +136,22 @@ static hipError_t launch_batch_kernels(const BatchLaunch& L, hipStream_t stream,
             // head_dim 512: a second head per wavefront only for FP8 rows (F16 rows leave no registers for it) and only while
             // head pairs still give every compute unit a workgroup
             if (nh == 2u) ncb = (L.dtype == kF8 && (uint64_t)((L.m + 15u) / 16u) * L.n_kv_heads * ((g + 1u) / 2u) >= 256u) ? 2u : 1u;
-            else if (L.head_dim == 128u && L.dtype == kF16 && g >= 3u) ncb = 4u;
+            else if (hd == 128u && L.dtype == kF16 && g >= 3u && dpad == 0u) ncb = 4u;   // (the padded form of it crashes the compiler's AGPR rewriting pass)
             else ncb = 2u;
         }
-        const uint32_t dv = L.head_dim / nh;
+        const uint32_t dv = hd / nh;
         const uint32_t hp_group = (g + ncb - 1u) / ncb * nh;     // (head slice, output slice) units of a whole GQA group
         // wavefronts per workgroup the registers allow: one head per wavefront at head_dim <= 128 needs few (three wavefronts
         // per SIMD), 512 accumulator columns per wavefront need the whole register file of a SIMD (one wavefront per SIMD)
-        const uint32_t reg_waves = (ncb == 1u && L.head_dim <= 128u) ? (uint32_t)kPrefillOneHeadWaves
-                                 : (ncb * L.head_dim >= 512u || (L.dtype == kF16 && L.head_dim == 256u)) ? 4u : 8u;   // (always 4 at head_dim 512)
+        const uint32_t reg_waves = (ncb == 1u && hd <= 128u) ? (uint32_t)kPrefillOneHeadWaves
+                                 : (ncb * hd >= 512u || (L.dtype == kF16 && hd == 256u)) ? 4u : 8u;   // (always 4 at head_dim 512)
         // FP8 rows of 128 elements, two heads per wavefront: three raw V tiles per wavefront (filled by loads that write LDS)
         // instead of one f16 copy
-        const bool vdma = L.dtype == kF8 && L.head_dim == 128u && ncb == 2u;
+        const bool vdma = L.dtype == kF8 && L.head_dim == 128u && ncb == 2u;      // (not the padded widths)
         // the private V tiles and the two Q planes have to fit in 160 KiB of LDS
         auto waves_for = [&](uint32_t slices) -> uint32_t {
-            const size_t qbytes = (size_t)2 * (slices / nh) * ncb * 16 * (L.head_dim + 8) * sizeof(_Float16) +
-                                  (vdma ? (size_t)slices * ncb * 16 * (L.head_dim + 16) : 0u);   // (that kernel: a third plane of one byte per element)
+            const size_t qbytes = (size_t)2 * (slices / nh) * ncb * 16 * (hd + 8) * sizeof(_Float16) +
+                                  (vdma ? (size_t)slices * ncb * 16 * (hd + 16) : 0u);   // (that kernel: a third plane of one byte per element)
             // private V tile, and with two wavefronts per head the two buffers through which they swap score halves
             const size_t per_wave = (vdma ? (size_t)3 * 32 * 128 : (size_t)32 * (dv + 16) * sizeof(_Float16)) +
                                     (nh == 2u ? (size_t)2 * ncb * 64 * 16 : 0u);   // (unused by the two-heads FP8 form)
@@ -209,8 +213,8 @@ static hipError_t launch_batch_kernels(const BatchLaunch& L, hipStream_t stream,
             // query blocks of a head share one XCD's L2 and its K / V rows come from memory once, not once per XCD
             const dim3 grid(L.n_kv_heads, (L.m + 15u) / 16u, nz * nk), block(nwaves * kWave);
             const size_t vbytes = (size_t)nwaves * (vdma ? (size_t)3 * 32 * 128 : (size_t)32 * (dv + 16) * sizeof(_Float16)) +
-                                  (size_t)2 * (hp / nh) * ncb * 16 * (L.head_dim + 8) * sizeof(_Float16) +
-                                  (vdma ? (size_t)hp * ncb * 16 * (L.head_dim + 16) : 0u) +
+                                  (size_t)2 * (hp / nh) * ncb * 16 * (hd + 8) * sizeof(_Float16) +
+                                  (vdma ? (size_t)hp * ncb * 16 * (hd + 16) : 0u) +
                                   (nh == 2u ? (size_t)2 * nwaves * ncb * 64 * 16 : 0u);
             // merge area: the general kernel keeps the records of all splits but the first; the V-through-LDS kernel the
             // output tiles and (m, l) of every wavefront
@@ -224,6 +228,11 @@ static hipError_t launch_batch_kernels(const BatchLaunch& L, hipStream_t stream,
     if (L.dtype == DT && L.head_dim == DD && ncb == NCBV) {                                                 \
         if (cap) hipLaunchKernelGGL((batch_mfma2_kernel<DT, DD, NCBV, PFDV, true>), grid, block, lds, stream, a, (int)hp, (int)ns);  \
         else hipLaunchKernelGGL((batch_mfma2_kernel<DT, DD, NCBV, PFDV, false>), grid, block, lds, stream, a, (int)hp, (int)ns);      \
+    } else
+#define VFKV_P2PAD(DT, DD, NCBV, PFDV)                                                                      \
+    if (L.dtype == DT && dpad == DD && ncb == NCBV) {                                                       \
+        if (cap) hipLaunchKernelGGL((batch_mfma2_kernel<DT, DD, NCBV, PFDV, true, 1, false, true>), grid, block, lds, stream, a, (int)hp, (int)ns);  \
+        else hipLaunchKernelGGL((batch_mfma2_kernel<DT, DD, NCBV, PFDV, false, 1, false, true>), grid, block, lds, stream, a, (int)hp, (int)ns);      \
     } else
             // FP8 rows of 128 elements, two heads per wavefront: the kernel that loads V straight into LDS.  Its options --
             // f16_weights: one product with the weights instead of value + remainder; fp8_scores: the first product on the
@@ -250,6 +259,8 @@ static hipError_t launch_batch_kernels(const BatchLaunch& L, hipStream_t stream,
             VFKV_P2(kF16, 64, 2, 2) VFKV_P2(kF16, 64, 1, 2) VFKV_P2(kF16, 128, 1, 1) VFKV_P2(kF16, 128, 2, 1)
             VFKV_P2(kF8, 256, 1, 1) VFKV_P2(kF16, 256, 1, 1)
             VFKV_P2(kF16, 128, 4, 1) VFKV_P2(kF8, 256, 2, 1) VFKV_P2(kF16, 256, 2, 1)
+            VFKV_P2PAD(kF8, 128, 1, 2) VFKV_P2PAD(kF8, 128, 2, 2) VFKV_P2PAD(kF16, 128, 1, 1) VFKV_P2PAD(kF16, 128, 2, 1)
+            VFKV_P2PAD(kF8, 256, 1, 1) VFKV_P2PAD(kF8, 256, 2, 1) VFKV_P2PAD(kF16, 256, 1, 1) VFKV_P2PAD(kF16, 256, 2, 1)
             if (L.head_dim == 512u && L.dtype == kF8 && ncb == 2u) {
                 if (cap) hipLaunchKernelGGL((batch_mfma2_kernel<kF8, 512, 2, 1, true, 2>), grid, block, lds, stream, a, (int)hp, (int)ns);
                 else hipLaunchKernelGGL((batch_mfma2_kernel<kF8, 512, 2, 1, false, 2>), grid, block, lds, stream, a, (int)hp, (int)ns);
@@ -262,6 +273,7 @@ static hipError_t launch_batch_kernels(const BatchLaunch& L, hipStream_t stream,
             } else
             { launched = false; }
 #undef VFKV_P2
+#undef VFKV_P2PAD
             if (launched) {
                 hipError_t e = hipGetLastError();
                 if (e == hipSuccess && nk > 1u)
@@ -285,12 +297,8 @@ static hipError_t launch_batch_kernels(const BatchLaunch& L, hipStream_t stream,
     }
         VFKV_PF32(kF32, 64, 1) VFKV_PF32(kF32, 128, 1) VFKV_PF32(kF32, 256, 1) VFKV_PF32(kF32, 96, 1)
         VFKV_PF32(kF16, 96, 1) VFKV_PF32(kF8, 96, 1) VFKV_PF32(kF32, 512, 2)
-        // the other head widths between the tiled ones (multiples of 16 up to 224), every cache type
-        VFKV_PF32(kF32, 80, 1) VFKV_PF32(kF16, 80, 1) VFKV_PF32(kF8, 80, 1)
-        VFKV_PF32(kF32, 112, 1) VFKV_PF32(kF16, 112, 1) VFKV_PF32(kF8, 112, 1)
-        VFKV_PF32(kF32, 160, 1) VFKV_PF32(kF16, 160, 1) VFKV_PF32(kF8, 160, 1)
-        VFKV_PF32(kF32, 192, 1) VFKV_PF32(kF16, 192, 1) VFKV_PF32(kF8, 192, 1)
-        VFKV_PF32(kF32, 224, 1) VFKV_PF32(kF16, 224, 1) VFKV_PF32(kF8, 224, 1)
+        // the other head widths between the tiled ones over F32 caches (FP8 / F16 caches take the f16 kernel's padded form)
+        VFKV_PF32(kF32, 80, 1) VFKV_PF32(kF32, 112, 1) VFKV_PF32(kF32, 160, 1) VFKV_PF32(kF32, 192, 1) VFKV_PF32(kF32, 224, 1)
 #undef VFKV_PF32
     }
     if (generic_used) *generic_used = true;

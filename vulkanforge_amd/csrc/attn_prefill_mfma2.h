@@ -32,7 +32,13 @@ constexpr int kPrefillOneHeadWaves = 12;
 // workgroup barrier per tile, and each then
 // accumulates, merges and stores its own slice of D / NH output elements: the accumulators of a 512-wide head do not fit
 // one wavefront.  HP then counts (head, slice) units.
-template <int DT, int D, int NCB, int PFD, bool CAP, int NH = 1, bool F16W = false>
+//
+// PAD (NH == 1): the heads are a.head_dim < D elements wide (a multiple of 16: 80 / 96 / 112 on the kernel for 128, 160 /
+// 192 / 224 on the one for 256).  The kernel works on rows of D elements whose tail does not exist: the query planes hold
+// zeros there, a lane whose 16-byte piece of a K or V row would lie past the head reads the head's first piece again
+// (finite values that meet query zeros, or output columns nobody stores), and the d-tiles past head_dim are neither
+// multiplied nor stored.  Rows, queries, outputs, partials and the gate keep their real stride of head_dim.
+template <int DT, int D, int NCB, int PFD, bool CAP, int NH = 1, bool F16W = false, bool PAD = false>
 __global__ __launch_bounds__((NCB == 1 && D <= 128) ? kPrefillOneHeadWaves * 64 : (NCB * D >= 512 || (DT == kF16 && D == 256)) ? 256 : 512) void batch_mfma2_kernel(BatchArgs a, int HP, int NS) {
     constexpr int DV = D / NH;                   // output elements (V columns) of this wavefront
     constexpr int ES = DT == kF16 ? 2 : 1;
@@ -54,6 +60,8 @@ __global__ __launch_bounds__((NCB == 1 && D <= 128) ? kPrefillOneHeadWaves * 64 
     constexpr int NKT = XCH ? 1 : 2;             // 16-key halves of a tile this wavefront loads and scores
     static_assert(NH == 1 || NH == 2, "one or two wavefronts per head");
     static_assert(D % 32 == 0 && SEGB % 16 == 0 && VLD >= 1, "unsupported head_dim");
+    static_assert(!PAD || NH == 1, "padded heads: one wavefront per head");
+    const uint32_t dr = PAD ? a.head_dim : (uint32_t)D;                 // elements per head as the buffers hold them
 
     extern __shared__ __attribute__((aligned(16))) _Float16 lds[];      // [waves][KT][VPITCH] V tiles | [GP][16][D + 8] f16(q) | [GP][16][D + 8] remainders
     __shared__ int lds_haslo;
@@ -68,7 +76,7 @@ __global__ __launch_bounds__((NCB == 1 && D <= 128) ? kPrefillOneHeadWaves * 64 
     const uint32_t q0 = (gridDim.y - 1u - blockIdx.y) * 16;   // later query blocks see more keys: longest workgroups first
     const uint32_t qi = q0 + n16;                               // this lane's query (column of S^T)
     const bool q_ok = qi < a.m;
-    const uint32_t row_stride = a.n_kv_heads * D * ES;
+    const uint32_t row_stride = a.n_kv_heads * dr * ES;
     const uint32_t kc = blockIdx.z % a.nk;                      // key chunk of this workgroup (a.nk == 1: all keys)
     const int gz = (blockIdx.z / a.nk) * (HP / NH) * NCB;       // first head (inside the group) of this workgroup
     const int g0 = (hp / NH) * NCB;                             // first head slot (inside the workgroup) of this wavefront
@@ -99,10 +107,16 @@ __global__ __launch_bounds__((NCB == 1 && D <= 128) ? kPrefillOneHeadWaves * 64 
 
     const __amdgpu_buffer_rsrc_t krsrc = __builtin_amdgcn_make_buffer_rsrc((void*)a.k, 0, a.n_kv * row_stride, 0x00020000);
     const __amdgpu_buffer_rsrc_t vrsrc = __builtin_amdgcn_make_buffer_rsrc((void*)a.v, 0, a.n_kv * row_stride, 0x00020000);
-    const uint32_t head_b = kvh * D * ES;
+    const uint32_t head_b = kvh * dr * ES;
     const uint32_t lane_koff = n16 * row_stride + head_b + kg * SEGB;
     const int vrow = lane / VCHUNK_ROW, vcol = lane % VCHUNK_ROW;
-    const uint32_t lane_voff = vrow * row_stride + head_b + dslice * DV * ES + vcol * 16;
+    const uint32_t lane_voff = vrow * row_stride + head_b + dslice * DV * ES + (PAD && (uint32_t)vcol * 16u >= dr * ES ? 0 : vcol * 16);
+    uint32_t kpiece[KLD];                        // PAD: offset of the lane's piece x (the head's first piece where x does not exist)
+#pragma unroll
+    for (int x = 0; x < KLD; ++x) {
+        const uint32_t bo = (uint32_t)(kg * SEGB + x * 16);
+        kpiece[x] = n16 * row_stride + head_b + (bo < dr * ES ? bo : 0u);
+    }
 
     const uint32_t kt_own = XCH ? (uint32_t)dslice : 0u;         // XCH: the half this wavefront scores
     u32x4 kraw[PFD][NKT][KLD];
@@ -112,7 +126,7 @@ __global__ __launch_bounds__((NCB == 1 && D <= 128) ? kPrefillOneHeadWaves * 64 
         for (int kt = 0; kt < NKT; ++kt)
 #pragma unroll
             for (int x = 0; x < KLD; ++x)
-                kraw[slot][kt][x] = __builtin_amdgcn_raw_buffer_load_b128(krsrc, lane_koff + x * 16, toff + ((uint32_t)kt + kt_own) * 16u * row_stride, 0);
+                kraw[slot][kt][x] = __builtin_amdgcn_raw_buffer_load_b128(krsrc, PAD ? kpiece[x] : lane_koff + x * 16, toff + ((uint32_t)kt + kt_own) * 16u * row_stride, 0);
 #pragma unroll
         for (int c = 0; c < VLD; ++c)
             vraw[slot][c] = __builtin_amdgcn_raw_buffer_load_b128(vrsrc, lane_voff, toff + (uint32_t)(c * VROWS) * row_stride, 0);
@@ -139,7 +153,12 @@ __global__ __launch_bounds__((NCB == 1 && D <= 128) ? kPrefillOneHeadWaves * 64 
         for (int i = 0; i < QLD; ++i) {
             const int idx = base + tid + i * nthreads;
             const int qq = idx / (GP * (D / 4)), rem = idx - qq * (GP * (D / 4));
-            const bool ok = idx < q4_total && q0 + qq < a.m && rem < (G - gz) * (D / 4);      // head slots past G read nothing
+            bool ok = idx < q4_total && q0 + qq < a.m && rem < (G - gz) * (D / 4);      // head slots past G read nothing
+            if (PAD) {                                          // the heads are dr floats apart; the tail of a slot reads nothing
+                const int gq = rem / (D / 4), d4 = rem - gq * (D / 4);
+                ok = ok && (uint32_t)d4 * 4u < dr;
+                qf[i] = *reinterpret_cast<const float4*>(a.q + ((size_t)(ok ? q0 + qq : 0) * a.n_heads + kvh * G + gz + (ok ? gq : 0)) * dr + (ok ? d4 * 4 : 0));
+            } else
             qf[i] = *reinterpret_cast<const float4*>(a.q + ((size_t)(ok ? q0 + qq : 0) * a.n_heads + kvh * G + gz) * D + (ok ? rem * 4 : 0));
             if (!ok) qf[i] = make_float4(0.f, 0.f, 0.f, 0.f);
         }
@@ -228,7 +247,7 @@ __global__ __launch_bounds__((NCB == 1 && D <= 128) ? kPrefillOneHeadWaves * 64 
             }
 #pragma unroll
             for (int xx = 0; xx < KLD; ++xx)
-                kraw[sl][kt][xx] = __builtin_amdgcn_raw_buffer_load_b128(krsrc, lane_koff + xx * 16, noff + ((uint32_t)kt + kt_own) * 16u * row_stride, 0);
+                kraw[sl][kt][xx] = __builtin_amdgcn_raw_buffer_load_b128(krsrc, PAD ? kpiece[xx] : lane_koff + xx * 16, noff + ((uint32_t)kt + kt_own) * 16u * row_stride, 0);
 #pragma unroll
             for (int cb = 0; cb < NCB; ++cb) {
                 float4_t acc = float4_t{0.f, 0.f, 0.f, 0.f};
@@ -334,6 +353,7 @@ __global__ __launch_bounds__((NCB == 1 && D <= 128) ? kPrefillOneHeadWaves * 64 
             }
 #pragma unroll
         for (int dt = 0; dt < DTILES; ++dt) {
+            if (PAD && (uint32_t)dt * 16u >= dr) continue;          // wavefront-uniform
             // supplier lane s of a 16-lane group points at V[key = 4*kg + s/4 (+16)][d = dt*16 + 4*(s%4)]
             const _Float16* p0 = vb + (kg * 4 + n16 / 4) * VPITCH + dt * 16 + 4 * (n16 % 4);
             const half4_t v0 = lds_read_tr16(p0);
@@ -406,11 +426,12 @@ __global__ __launch_bounds__((NCB == 1 && D <= 128) ? kPrefillOneHeadWaves * 64 
 #pragma unroll
         for (int cb = 0; cb < NCB; ++cb) {
             if (gz + g0 + cb >= G) continue;
-            const uint32_t i0 = (qi * a.n_heads + kvh * G + gz + g0 + cb) * D;
+            const uint32_t i0 = (qi * a.n_heads + kvh * G + gz + g0 + cb) * dr;
             const uint32_t token = i0 / a.gchunk;
             const float* gp = a.gate + (size_t)token * a.gstride + a.goff + (i0 - token * a.gchunk) + dslice * DV + kg * 4;
 #pragma unroll
             for (int dt = 0; dt < DTILES; ++dt) {
+                if (PAD && (uint32_t)dt * 16u >= dr) continue;
                 const float4 gv = *reinterpret_cast<const float4*>(gp + dt * 16);
                 gfac[cb][dt] = float4_t{sigmoid_gate(1.0f, gv.x), sigmoid_gate(1.0f, gv.y), sigmoid_gate(1.0f, gv.z), sigmoid_gate(1.0f, gv.w)};
             }
@@ -459,10 +480,10 @@ __global__ __launch_bounds__((NCB == 1 && D <= 128) ? kPrefillOneHeadWaves * 64 
                 const uint32_t h = kvh * G + gz + g0 + cb;
                 const size_t pidx = ((size_t)qi * a.n_heads + h) * a.nk + kc;      // (key chunks: the partial of this chunk)
                 const float inv = a.so != nullptr ? 1.0f : 1.0f / lsum;
-                float* op = a.so != nullptr ? a.so + pidx * D + kg * 4 : a.o + ((size_t)qi * a.n_heads + h) * D + kg * 4;
+                float* op = a.so != nullptr ? a.so + pidx * dr + kg * 4 : a.o + ((size_t)qi * a.n_heads + h) * dr + kg * 4;
                 const float* gp = nullptr;
                 if (a.gate != nullptr) {
-                    const uint32_t i0 = (qi * a.n_heads + h) * D;
+                    const uint32_t i0 = (qi * a.n_heads + h) * dr;
                     const uint32_t token = i0 / a.gchunk;
                     gp = a.gate + (size_t)token * a.gstride + a.goff + (i0 - token * a.gchunk) + kg * 4;
                 }
@@ -470,6 +491,7 @@ __global__ __launch_bounds__((NCB == 1 && D <= 128) ? kPrefillOneHeadWaves * 64 
                 for (int j = 0; j < (DTILES + NSC - 1) / NSC; ++j) {   // lane (query n16) holds d = dt*16 + kg*4 + i
                     const int dt = sp + j * NSC;
                     if (DTILES % NSC != 0 && dt >= DTILES) break;
+                    if (PAD && (uint32_t)dt * 16u >= dr) break;
                     float4_t r = float4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
                     for (int s2 = 0; s2 < NSC; ++s2)
@@ -535,9 +557,10 @@ __global__ __launch_bounds__((NCB == 1 && D <= 128) ? kPrefillOneHeadWaves * 64 
                 // key chunks: the unnormalised partial of this chunk in the layout of the decode merge ([row][chunk][D], the
                 // maximum in natural-log units); a query that sees no key of the chunk leaves (0, "minus infinity", 0)
                 const size_t pidx = ((size_t)qi * a.n_heads + h) * a.nk + kc;
-                float* op = a.so + pidx * D + dslice * DV + kg * 4;
+                float* op = a.so + pidx * dr + dslice * DV + kg * 4;
 #pragma unroll
                 for (int dt = 0; dt < DTILES; ++dt) {
+                    if (PAD && (uint32_t)dt * 16u >= dr) continue;
                     const float4_t r = oacc[cb][dt];
                     *reinterpret_cast<float4*>(op + dt * 16) = make_float4(r[0], r[1], r[2], r[3]);
                 }
@@ -548,10 +571,11 @@ __global__ __launch_bounds__((NCB == 1 && D <= 128) ? kPrefillOneHeadWaves * 64 
                 continue;
             }
             const float inv = 1.0f / l_run[cb];
-            float* op = a.o + ((size_t)qi * a.n_heads + h) * D + dslice * DV + kg * 4;   // lane (query n16) holds d = dslice*DV + dt*16 + kg*4 + i
+            float* op = a.o + ((size_t)qi * a.n_heads + h) * dr + dslice * DV + kg * 4;   // lane (query n16) holds d = dslice*DV + dt*16 + kg*4 + i
             if (a.gate != nullptr) {
 #pragma unroll
                 for (int dt = 0; dt < DTILES; ++dt) {
+                    if (PAD && (uint32_t)dt * 16u >= dr) continue;
                     const float4_t r = oacc[cb][dt] * inv * gfac[cb][dt];
                     *reinterpret_cast<float4*>(op + dt * 16) = make_float4(r[0], r[1], r[2], r[3]);
                 }
@@ -559,6 +583,7 @@ __global__ __launch_bounds__((NCB == 1 && D <= 128) ? kPrefillOneHeadWaves * 64 
             }
 #pragma unroll
             for (int dt = 0; dt < DTILES; ++dt) {
+                if (PAD && (uint32_t)dt * 16u >= dr) continue;
                 const float4_t r = oacc[cb][dt] * inv;
                 *reinterpret_cast<float4*>(op + dt * 16) = make_float4(r[0], r[1], r[2], r[3]);
             }

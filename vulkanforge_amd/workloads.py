@@ -98,6 +98,9 @@ PREFILL = {
                                                            512, KvDtype.F16),
     "prefill_fp8_hd256_512x4608_12layers": PrefillWorkload("prefill_fp8_hd256_512x4608_12layers", 12, 16, 8, 256, 4096,
                                                            512, KvDtype.F8),
+    # Phi-3-mini geometry (head_dim 96, F16 cache; not a reference configuration): the padded form of the f16 kernel
+    "prefill_f16_hd96_512x4608_32layers": PrefillWorkload("prefill_f16_hd96_512x4608_32layers", 32, 32, 32, 96, 4096, 512,
+                                                          KvDtype.F16),
     # the suffix of a request that reuses its prefix: 64 new tokens over 16 k resident rows, with and without the workspace
     "prefill_fp8_suffix64_over_16k_32layers": PrefillWorkload("prefill_fp8_suffix64_over_16k_32layers", 32, 32, 8, 128,
                                                               16384, 64, KvDtype.F8, workspace=True),

@@ -84,6 +84,11 @@ CASES = [
     (vf.KvDtype.F8, 12, 4, 192, 35, 120, 0, 30.0),
     (vf.KvDtype.F16, 4, 4, 224, 18, 70, 0, 0.0),
     (vf.KvDtype.F32, 4, 2, 192, 17, 60, 0, 0.0),
+    # more than eight KV heads over FP8 rows: the workgroups are renumbered so that an XCD takes one KV head at a time
+    (vf.KvDtype.F8, 16, 16, 128, 50, 300, 0, 0.0),    # G = 1, ragged last query block
+    (vf.KvDtype.F8, 32, 16, 64, 70, 200, 100, 0.0),   # G = 2 at head_dim 64, window
+    (vf.KvDtype.F8, 32, 32, 96, 40, 300, 0, 0.0),     # Phi-3 geometry over an FP8 cache
+    (vf.KvDtype.F8, 48, 24, 256, 20, 100, 0, 30.0),   # 24 KV heads, head_dim 256, soft-cap
     (vf.KvDtype.F8, 16, 8, 256, 48, 700, 0, 50.0),    # head_dim 256, G = 2: three key splits, soft-cap
     (vf.KvDtype.F16, 8, 2, 256, 35, 260, 100, 0.0),   # head_dim 256, G = 4 on a 2-byte cache, window
     (vf.KvDtype.F8, 32, 4, 256, 18, 130, 0, 0.0),     # head_dim 256, G = 8: the group is spread over workgroups so that the Q planes fit

@@ -32,6 +32,7 @@ struct BatchArgs {
     uint32_t gchunk, gstride, goff;
     uint32_t q_f16;          // f16 matrix-core kernels: use f16(q) alone, whatever the queries hold
     uint32_t merge_all;      // batch_mfma2_kernel: the LDS area holds the (o, m, l) of every wavefront, and every wavefront merges a share
+    uint32_t xcd_heads;      // batch_mfma2_kernel: deal the (KV head, query block) pairs so that an XCD works on one KV head at a time
 };
 
 }  // namespace vfkv
@@ -113,6 +114,7 @@ static hipError_t launch_batch_kernels(const BatchLaunch& L, hipStream_t stream,
     a.gate = nullptr; a.gchunk = 1u; a.gstride = 0u; a.goff = 0u;
     a.q_f16 = L.f16_queries ? 1u : 0u;
     a.merge_all = 0u;
+    a.xcd_heads = 0u;
     const uint32_t g = L.n_heads / L.n_kv_heads;
     const uint64_t slab_bytes = (uint64_t)L.n_kv * L.n_kv_heads * L.head_dim * elem_size(L.dtype);
     const bool aligned = ((((uintptr_t)L.k) | ((uintptr_t)L.v) | ((uintptr_t)L.q) | ((uintptr_t)L.o)) & 15u) == 0u;
@@ -211,6 +213,12 @@ static hipError_t launch_batch_kernels(const BatchLaunch& L, hipStream_t stream,
             if (gate_in_store) { a.gate = L.gate->gate; a.gchunk = L.gate->chunk; a.gstride = L.gate->stride; a.goff = L.gate->gate_offset; }
             // the KV head is the fastest grid index: consecutive workgroups go to consecutive XCDs, so with eight KV heads all
             // query blocks of a head share one XCD's L2 and its K / V rows come from memory once, not once per XCD
+            // With more than eight KV heads that order gives every XCD several heads at once, whose K / V rows then compete
+            // for its L2 (32 KV heads of 2.4 MB each: 320 MB fetched per launch for 57 MB of rows); the kernel then renumbers
+            // its workgroups so that an XCD takes all query blocks of one head before the next head.  512 queries over 4 608
+            // keys, 32 / 32 heads: FP8 rows of 96 / 128 elements 141.7 -> 129.1 / 119.0 -> 117.9 us; F16 rows did not gain
+            // (96: 190.9 -> 191.7, 128: 199.5 -> 211.4 us) and keep the plain order.
+            a.xcd_heads = (L.dtype == kF8 && L.n_kv_heads > 8u && L.n_kv_heads % 8u == 0u) ? 1u : 0u;
             const dim3 grid(L.n_kv_heads, (L.m + 15u) / 16u, nz * nk), block(nwaves * kWave);
             const size_t vbytes = (size_t)nwaves * (vdma ? (size_t)3 * 32 * 128 : (size_t)32 * (dv + 16) * sizeof(_Float16)) +
                                   (size_t)2 * (hp / nh) * ncb * 16 * (hd + 8) * sizeof(_Float16) +

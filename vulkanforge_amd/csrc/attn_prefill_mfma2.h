@@ -72,8 +72,16 @@ __global__ __launch_bounds__((NCB == 1 && D <= 128) ? kPrefillOneHeadWaves * 64 
     const int hp = w % HP, sp = w / HP;
     const int n16 = lane & 15, kg = lane >> 4;
     const int G = a.n_heads / a.n_kv_heads;
-    const uint32_t kvh = blockIdx.x;
-    const uint32_t q0 = (gridDim.y - 1u - blockIdx.y) * 16;   // later query blocks see more keys: longest workgroups first
+    // Workgroups are dispatched to the XCDs round-robin in the order of their linear index.  a.xcd_heads (more than eight KV
+    // heads, a multiple of eight): XCD x takes the query blocks of KV head x, then those of head x + 8, and so on, so that
+    // the rows of one head at a time occupy its L2.
+    uint32_t kvh = blockIdx.x, qblk = blockIdx.y;
+    if (a.xcd_heads != 0u) {
+        const uint32_t id = blockIdx.x + gridDim.x * blockIdx.y, t = id >> 3;
+        kvh = (id & 7u) + 8u * (t / gridDim.y);
+        qblk = t % gridDim.y;
+    }
+    const uint32_t q0 = (gridDim.y - 1u - qblk) * 16;         // later query blocks see more keys: longest workgroups first
     const uint32_t qi = q0 + n16;                               // this lane's query (column of S^T)
     const bool q_ok = qi < a.m;
     const uint32_t row_stride = a.n_kv_heads * dr * ES;

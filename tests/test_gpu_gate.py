@@ -126,6 +126,7 @@ def test_decode_attention_gated_is_attention_then_gate(dtype, heads, hkv, d, n, 
     (vf.KvDtype.F8, 6, 2, 96, 20, 10),          # heads of 96 elements on the kernel for 128: the gate keeps its real stride
     (vf.KvDtype.F16, 32, 32, 80, 40, 100),      # one head per wavefront
     (vf.KvDtype.F16, 8, 4, 192, 18, 30),
+    (vf.KvDtype.F8, 8, 8, 128, 45, 100),        # groups of one head: each of a wavefront's two query blocks gates its own rows
     (vf.KvDtype.F8, 128, 32, 128, 125, 200),    # 256 workgroups: two head pairs x four key splits, every wavefront gates the tiles it stores
 ))
 def test_prefill_attention_gated_is_attention_then_gate(dtype, heads, hkv, d, m, base):

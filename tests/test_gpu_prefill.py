@@ -84,6 +84,14 @@ CASES = [
     (vf.KvDtype.F8, 12, 4, 192, 35, 120, 0, 30.0),
     (vf.KvDtype.F16, 4, 4, 224, 18, 70, 0, 0.0),
     (vf.KvDtype.F32, 4, 2, 192, 17, 60, 0, 0.0),
+    # groups of one head: two blocks of 16 queries of the same head per wavefront, 32 queries per workgroup
+    (vf.KvDtype.F16, 8, 8, 128, 47, 300, 0, 0.0),     # ragged: the last workgroup has 15 queries, all in its first block
+    (vf.KvDtype.F16, 8, 8, 128, 49, 0, 0, 0.0),       # from position 0; the last workgroup's second block holds one query
+    (vf.KvDtype.F8, 4, 4, 64, 100, 250, 200, 30.0),   # window that starts inside a tile, soft-cap
+    (vf.KvDtype.F8, 16, 16, 256, 33, 500, 0, 0.0),
+    (vf.KvDtype.F16, 4, 4, 256, 64, 300, 100, 0.0),   # window that starts past a tile boundary
+    (vf.KvDtype.F8, 2, 2, 128, 17, 1000, 0, 0.0),     # one query in the second block
+    (vf.KvDtype.F16, 3, 3, 64, 16, 40, 0, 0.0),       # 16 queries: one block, the one-head-per-wavefront form stays
     # more than eight KV heads over FP8 rows: the workgroups are renumbered so that an XCD takes one KV head at a time
     (vf.KvDtype.F8, 16, 16, 128, 50, 300, 0, 0.0),    # G = 1, ragged last query block
     (vf.KvDtype.F8, 32, 16, 64, 70, 200, 100, 0.0),   # G = 2 at head_dim 64, window
@@ -311,6 +319,7 @@ def test_scores_that_drift_past_the_running_maximum(dtype, shape):
     (vf.KvDtype.F32, 8, 2, 128, 16, 2000, 0, 0.0),       # F32 cache: no key chunks, same result
     (vf.KvDtype.F16, 32, 32, 96, 24, 5000, 0, 0.0),      # heads of 96 elements on the kernel for 128: partials with their real stride
     (vf.KvDtype.F8, 8, 2, 192, 16, 3000, 1000, 20.0),    # heads of 192 on the kernel for 256, window, soft-cap
+    (vf.KvDtype.F8, 8, 8, 128, 40, 6000, 0, 0.0),        # groups of one head: two query blocks per wavefront, partials per query
 ))
 def test_prefill_with_workspace_matches_plain_call_and_oracle(dtype, heads, hkv, d, m, base, window, cap):
     # vfkv_prefill_attention_ws cuts the keys into chunks over workgroups and merges the partials

@@ -134,6 +134,10 @@ static hipError_t launch_batch_kernels(const BatchLaunch& L, hipStream_t stream,
         // per wavefront in workgroups of four wavefronts (one per SIMD, up to 512 registers), so that a K / V tile is loaded
         // by one wavefront of the workgroup only.
         uint32_t ncb = 1u;
+        // Groups of one head (no grouping): two blocks of 16 queries of the same head per wavefront instead of two heads, so
+        // that a K / V tile is still widened and staged once for two column blocks; a workgroup then covers 32 queries.
+        const bool qb2 = g == 1u && nh == 1u && L.m > 16u;
+        if (qb2) ncb = 2u;
         if (g >= 2u) {
             // head_dim 512: a second head per wavefront only for FP8 rows (F16 rows leave no registers for it) and only while
             // head pairs still give every compute unit a workgroup
@@ -142,14 +146,15 @@ static hipError_t launch_batch_kernels(const BatchLaunch& L, hipStream_t stream,
             else ncb = 2u;
         }
         const uint32_t dv = hd / nh;
-        const uint32_t hp_group = (g + ncb - 1u) / ncb * nh;     // (head slice, output slice) units of a whole GQA group
+        const uint32_t hp_group = qb2 ? 1u : (g + ncb - 1u) / ncb * nh;     // (head slice, output slice) units of a whole GQA group
+        const uint32_t qblocks = qb2 ? (L.m + 31u) / 32u : (L.m + 15u) / 16u;   // query blocks = workgroups per (KV head, head slice)
         // wavefronts per workgroup the registers allow: one head per wavefront at head_dim <= 128 needs few (three wavefronts
         // per SIMD), 512 accumulator columns per wavefront need the whole register file of a SIMD (one wavefront per SIMD)
         const uint32_t reg_waves = (ncb == 1u && hd <= 128u) ? (uint32_t)kPrefillOneHeadWaves
                                  : (ncb * hd >= 512u || (L.dtype == kF16 && hd == 256u)) ? 4u : 8u;   // (always 4 at head_dim 512)
         // FP8 rows of 128 elements, two heads per wavefront: three raw V tiles per wavefront (filled by loads that write LDS)
         // instead of one f16 copy
-        const bool vdma = L.dtype == kF8 && L.head_dim == 128u && ncb == 2u;      // (not the padded widths)
+        const bool vdma = L.dtype == kF8 && L.head_dim == 128u && ncb == 2u && !qb2;      // (not the padded widths)
         // the private V tiles and the two Q planes have to fit in 160 KiB of LDS
         auto waves_for = [&](uint32_t slices) -> uint32_t {
             const size_t qbytes = (size_t)2 * (slices / nh) * ncb * 16 * (hd + 8) * sizeof(_Float16) +
@@ -165,7 +170,7 @@ static hipError_t launch_batch_kernels(const BatchLaunch& L, hipStream_t stream,
         // several workgroups (each then splits the keys further: same work per workgroup, more of them).
         uint32_t hp = hp_group;
         {
-            const uint64_t wgs = (uint64_t)((L.m + 15u) / 16u) * L.n_kv_heads;
+            const uint64_t wgs = (uint64_t)qblocks * L.n_kv_heads;
             if (wgs < 256u) {
                 uint32_t want = (uint32_t)((256u + wgs - 1u) / wgs);
                 if (want > hp_group / nh) want = hp_group / nh;
@@ -179,7 +184,7 @@ static hipError_t launch_batch_kernels(const BatchLaunch& L, hipStream_t stream,
         }
         const uint32_t nz = (hp_group + hp - 1u) / hp;
         const uint32_t max_waves = waves_for(hp);
-        if (max_waves >= hp && nz <= 65535u && (L.m + 15u) / 16u <= 65535u) {
+        if (max_waves >= hp && nz <= 65535u && qblocks <= 65535u) {
             uint32_t ns = max_waves / hp;                     // key splits: fill the workgroup
             if (vdma) while (ns & (ns - 1u)) --ns;            // (that kernel's merge deals the 8 output tiles of a head to the splits)
             const uint32_t nwaves = hp * ns;
@@ -188,7 +193,7 @@ static hipError_t launch_batch_kernels(const BatchLaunch& L, hipStream_t stream,
             // partial per (query, head, chunk), and the decode merge kernel combines them.
             uint32_t nk = 1u;
             if (L.scratch_out != nullptr && L.n_heads != 0u) {
-                const uint64_t wgs = (uint64_t)((L.m + 15u) / 16u) * L.n_kv_heads * nz;
+                const uint64_t wgs = (uint64_t)qblocks * L.n_kv_heads * nz;
                 const uint32_t t0 = (L.kv_start / 32u) * 32u;
                 const uint32_t kend = L.q_start + L.m < L.n_kv ? L.q_start + L.m : L.n_kv;
                 const uint32_t span = kend > t0 ? kend - t0 : 0u;
@@ -219,7 +224,7 @@ static hipError_t launch_batch_kernels(const BatchLaunch& L, hipStream_t stream,
             // keys, 32 / 32 heads: FP8 rows of 96 / 128 elements 141.7 -> 129.1 / 119.0 -> 117.9 us; F16 rows did not gain
             // (96: 190.9 -> 191.7, 128: 199.5 -> 211.4 us) and keep the plain order.
             a.xcd_heads = (L.dtype == kF8 && L.n_kv_heads > 8u && L.n_kv_heads % 8u == 0u) ? 1u : 0u;
-            const dim3 grid(L.n_kv_heads, (L.m + 15u) / 16u, nz * nk), block(nwaves * kWave);
+            const dim3 grid(L.n_kv_heads, qblocks, nz * nk), block(nwaves * kWave);
             const size_t vbytes = (size_t)nwaves * (vdma ? (size_t)3 * 32 * 128 : (size_t)32 * (dv + 16) * sizeof(_Float16)) +
                                   (size_t)2 * (hp / nh) * ncb * 16 * (hd + 8) * sizeof(_Float16) +
                                   (vdma ? (size_t)hp * ncb * 16 * (hd + 16) : 0u) +
@@ -259,7 +264,17 @@ static hipError_t launch_batch_kernels(const BatchLaunch& L, hipStream_t stream,
             else if (vdma && L.f16_weights) VFKV_PDMA(true, false)
             else if (vdma) VFKV_PDMA(false, false)
 #undef VFKV_PDMA
-            else if (L.f16_weights && L.dtype == kF16 && L.head_dim == 128u && ncb == 4u) {
+            else
+#define VFKV_P2QB(DT, DD, PFDV, PADV)                                                                       \
+    if (qb2 && L.dtype == DT && hd == DD && (dpad != 0u) == PADV) {                                         \
+        if (cap) hipLaunchKernelGGL((batch_mfma2_kernel<DT, DD, 2, PFDV, true, 1, false, PADV, true>), grid, block, lds, stream, a, (int)hp, (int)ns);  \
+        else hipLaunchKernelGGL((batch_mfma2_kernel<DT, DD, 2, PFDV, false, 1, false, PADV, true>), grid, block, lds, stream, a, (int)hp, (int)ns);      \
+    } else
+            VFKV_P2QB(kF8, 64, 2, false) VFKV_P2QB(kF16, 64, 2, false) VFKV_P2QB(kF8, 128, 2, false) VFKV_P2QB(kF16, 128, 1, false)
+            VFKV_P2QB(kF8, 256, 1, false) VFKV_P2QB(kF16, 256, 1, false)
+            VFKV_P2QB(kF8, 128, 2, true) VFKV_P2QB(kF16, 128, 1, true) VFKV_P2QB(kF8, 256, 1, true) VFKV_P2QB(kF16, 256, 1, true)
+#undef VFKV_P2QB
+            if (L.f16_weights && L.dtype == kF16 && L.head_dim == 128u && ncb == 4u) {
                 if (cap) hipLaunchKernelGGL((batch_mfma2_kernel<kF16, 128, 4, 1, true, 1, true>), grid, block, lds, stream, a, (int)hp, (int)ns);
                 else hipLaunchKernelGGL((batch_mfma2_kernel<kF16, 128, 4, 1, false, 1, true>), grid, block, lds, stream, a, (int)hp, (int)ns);
             } else

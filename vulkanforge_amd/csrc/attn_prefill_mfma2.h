@@ -38,7 +38,11 @@ constexpr int kPrefillOneHeadWaves = 12;
 // zeros there, a lane whose 16-byte piece of a K or V row would lie past the head reads the head's first piece again
 // (finite values that meet query zeros, or output columns nobody stores), and the d-tiles past head_dim are neither
 // multiplied nor stored.  Rows, queries, outputs, partials and the gate keep their real stride of head_dim.
-template <int DT, int D, int NCB, int PFD, bool CAP, int NH = 1, bool F16W = false, bool PAD = false>
+//
+// QB2 (NCB == 2, NH == 1; groups of one head): the two column blocks of a wavefront are two blocks of 16 queries of the SAME
+// head instead of two heads, so a workgroup covers 32 consecutive queries and a K / V tile is still widened and staged once
+// for two column blocks.  Head slot s of the workgroup's query planes then holds queries q0 + 16 (s % 2) .. of head s / 2.
+template <int DT, int D, int NCB, int PFD, bool CAP, int NH = 1, bool F16W = false, bool PAD = false, bool QB2 = false>
 __global__ __launch_bounds__((NCB == 1 && D <= 128) ? kPrefillOneHeadWaves * 64 : (NCB * D >= 512 || (DT == kF16 && D == 256)) ? 256 : 512) void batch_mfma2_kernel(BatchArgs a, int HP, int NS) {
     constexpr int DV = D / NH;                   // output elements (V columns) of this wavefront
     constexpr int ES = DT == kF16 ? 2 : 1;
@@ -61,6 +65,8 @@ __global__ __launch_bounds__((NCB == 1 && D <= 128) ? kPrefillOneHeadWaves * 64 
     static_assert(NH == 1 || NH == 2, "one or two wavefronts per head");
     static_assert(D % 32 == 0 && SEGB % 16 == 0 && VLD >= 1, "unsupported head_dim");
     static_assert(!PAD || NH == 1, "padded heads: one wavefront per head");
+    static_assert(!QB2 || (NCB == 2 && NH == 1), "two query blocks per wavefront");
+    constexpr int QW = QB2 ? 32 : 16;            // queries of a workgroup
     const uint32_t dr = PAD ? a.head_dim : (uint32_t)D;                 // elements per head as the buffers hold them
 
     extern __shared__ __attribute__((aligned(16))) _Float16 lds[];      // [waves][KT][VPITCH] V tiles | [GP][16][D + 8] f16(q) | [GP][16][D + 8] remainders
@@ -81,13 +87,17 @@ __global__ __launch_bounds__((NCB == 1 && D <= 128) ? kPrefillOneHeadWaves * 64 
         kvh = (id & 7u) + 8u * (t / gridDim.y);
         qblk = t % gridDim.y;
     }
-    const uint32_t q0 = (gridDim.y - 1u - qblk) * 16;         // later query blocks see more keys: longest workgroups first
-    const uint32_t qi = q0 + n16;                               // this lane's query (column of S^T)
+    const uint32_t q0 = (gridDim.y - 1u - qblk) * QW;         // later query blocks see more keys: longest workgroups first
+    const uint32_t qi = q0 + n16;                               // this lane's query (column of S^T; QB2: of column block 0)
     const bool q_ok = qi < a.m;
+    auto qi_of = [&](int cb) -> uint32_t { return QB2 ? qi + (uint32_t)cb * 16u : qi; };
+    auto qok_of = [&](int cb) -> bool { return QB2 ? qi + (uint32_t)cb * 16u < a.m : q_ok; };
     const uint32_t row_stride = a.n_kv_heads * dr * ES;
     const uint32_t kc = blockIdx.z % a.nk;                      // key chunk of this workgroup (a.nk == 1: all keys)
-    const int gz = (blockIdx.z / a.nk) * (HP / NH) * NCB;       // first head (inside the group) of this workgroup
-    const int g0 = (hp / NH) * NCB;                             // first head slot (inside the workgroup) of this wavefront
+    const int gz = (blockIdx.z / a.nk) * (HP / NH) * (QB2 ? 1 : NCB);   // first head (inside the group) of this workgroup
+    const int g0 = (hp / NH) * (QB2 ? 1 : NCB);                 // first head (inside the workgroup) of this wavefront
+    const int s0 = (hp / NH) * NCB;                             // its first head slot in the query planes
+    auto head_of = [&](int cb) -> int { return gz + g0 + (QB2 ? 0 : cb); };   // head (inside the group) of column block cb
     const int dslice = hp % NH;                                 // which D / NH output elements this wavefront owns
 
     _Float16* const vb = lds + (size_t)w * KT * VPITCH;
@@ -98,9 +108,11 @@ __global__ __launch_bounds__((NCB == 1 && D <= 128) ? kPrefillOneHeadWaves * 64 
     float4_t* const xbuf = reinterpret_cast<float4_t*>(qlo_lds + (size_t)GP * 16 * QPITCH);   // XCH: [2][waves][NCB][64] score halves
 
     // ---- key range ----
-    uint32_t kmax = a.q_start + q0 + 16;                        // one past the last key any of the 16 queries sees
+    uint32_t kmax = a.q_start + q0 + QW;                        // one past the last key any of the workgroup's queries sees
     if (kmax > a.n_kv) kmax = a.n_kv;
     const uint32_t my_len = q_ok ? (a.q_start + qi + 1 < a.n_kv ? a.q_start + qi + 1 : a.n_kv) : 0;   // causal_len of this lane's query
+    const uint32_t my_len1 = (QB2 && qok_of(1)) ? (a.q_start + qi + 17 < a.n_kv ? a.q_start + qi + 17 : a.n_kv) : 0;   // QB2: of its query in column block 1
+    auto len_of = [&](int cb) -> uint32_t { return (QB2 && cb == 1) ? my_len1 : my_len; };
     uint32_t full_len = a.q_start + q0 + 1;                     // keys every query of the block sees
     if (full_len > a.n_kv) full_len = a.n_kv;
     uint32_t t_first = (a.kv_start / KT) * KT;
@@ -162,10 +174,13 @@ __global__ __launch_bounds__((NCB == 1 && D <= 128) ? kPrefillOneHeadWaves * 64 
             const int idx = base + tid + i * nthreads;
             const int qq = idx / (GP * (D / 4)), rem = idx - qq * (GP * (D / 4));
             bool ok = idx < q4_total && q0 + qq < a.m && rem < (G - gz) * (D / 4);      // head slots past G read nothing
-            if (PAD) {                                          // the heads are dr floats apart; the tail of a slot reads nothing
-                const int gq = rem / (D / 4), d4 = rem - gq * (D / 4);
-                ok = ok && (uint32_t)d4 * 4u < dr;
-                qf[i] = *reinterpret_cast<const float4*>(a.q + ((size_t)(ok ? q0 + qq : 0) * a.n_heads + kvh * G + gz + (ok ? gq : 0)) * dr + (ok ? d4 * 4 : 0));
+            if (PAD || QB2) {                                   // slot by slot: the heads are dr floats apart (the tail of a slot reads
+                                                                // nothing); QB2: slot s holds queries q0 + 16 (s % 2) + qq of head s / 2
+                const int sl = rem / (D / 4), d4 = rem - sl * (D / 4);
+                const int gq = QB2 ? sl / 2 : sl;
+                const uint32_t qrow = q0 + (uint32_t)qq + (QB2 ? (uint32_t)(sl & 1) * 16u : 0u);
+                ok = idx < q4_total && qrow < a.m && gq < G - gz && (uint32_t)d4 * 4u < dr;
+                qf[i] = *reinterpret_cast<const float4*>(a.q + ((size_t)(ok ? qrow : 0) * a.n_heads + kvh * G + gz + (ok ? gq : 0)) * dr + (ok ? d4 * 4 : 0));
             } else
             qf[i] = *reinterpret_cast<const float4*>(a.q + ((size_t)(ok ? q0 + qq : 0) * a.n_heads + kvh * G + gz) * D + (ok ? rem * 4 : 0));
             if (!ok) qf[i] = make_float4(0.f, 0.f, 0.f, 0.f);
@@ -234,7 +249,7 @@ __global__ __launch_bounds__((NCB == 1 && D <= 128) ? kPrefillOneHeadWaves * 64 
         for (int cb = 0; cb < NCB; ++cb)
 #pragma unroll
             for (int c = 0; c < KS; ++c)
-                qhi[cb][c] = *reinterpret_cast<const half8_t*>(qhi_lds + ((size_t)(g0 + cb) * 16 + n16) * QPITCH + kg * SEG + c * 8);
+                qhi[cb][c] = *reinterpret_cast<const half8_t*>(qhi_lds + ((size_t)(s0 + cb) * 16 + n16) * QPITCH + kg * SEG + c * 8);
         float4_t sown[NCB];                                     // XCH: this wavefront's half of the scores
 #pragma unroll
         for (int kt = 0; kt < NKT; ++kt) {
@@ -266,7 +281,7 @@ __global__ __launch_bounds__((NCB == 1 && D <= 128) ? kPrefillOneHeadWaves * 64 
             if (has_lo) {
 #pragma unroll
                 for (int cb = 0; cb < NCB; ++cb) {
-                    const _Float16* lo_row = qlo_lds + ((size_t)(g0 + cb) * 16 + n16) * QPITCH + kg * SEG;
+                    const _Float16* lo_row = qlo_lds + ((size_t)(s0 + cb) * 16 + n16) * QPITCH + kg * SEG;
                     float4_t acc = XCH ? sown[cb] : s[cb][kt];
 #pragma unroll
                     for (int c = 0; c < KS; ++c) {
@@ -312,7 +327,7 @@ __global__ __launch_bounds__((NCB == 1 && D <= 128) ? kPrefillOneHeadWaves * 64 
                     if (CAP) y = cap_l2 * tanhf(y / cap_l2);
                     if (MASKED) {
                         const uint32_t t = tcur + kt * 16 + kg * 4 + i;
-                        y = (t < my_len && t >= a.kv_start && t < kmax) ? y : kMasked;    // (t >= kmax: padding tiles of a key chunk)
+                        y = (t < len_of(cb) && t >= a.kv_start && t < kmax) ? y : kMasked;    // (t >= kmax: padding tiles of a key chunk)
                     }
                     x[cb][kt * 4 + i] = y;
                     tmax[cb] = fmaxf(tmax[cb], y);
@@ -433,8 +448,9 @@ __global__ __launch_bounds__((NCB == 1 && D <= 128) ? kPrefillOneHeadWaves * 64 
     if (a.gate != nullptr && sp == 0 && q_ok) {
 #pragma unroll
         for (int cb = 0; cb < NCB; ++cb) {
-            if (gz + g0 + cb >= G) continue;
-            const uint32_t i0 = (qi * a.n_heads + kvh * G + gz + g0 + cb) * dr;
+            if (head_of(cb) >= G) continue;
+            if (QB2 && !qok_of(cb)) continue;
+            const uint32_t i0 = (qi_of(cb) * a.n_heads + kvh * G + head_of(cb)) * dr;
             const uint32_t token = i0 / a.gchunk;
             const float* gp = a.gate + (size_t)token * a.gstride + a.goff + (i0 - token * a.gchunk) + dslice * DV + kg * 4;
 #pragma unroll
@@ -472,7 +488,8 @@ __global__ __launch_bounds__((NCB == 1 && D <= 128) ? kPrefillOneHeadWaves * 64 
             constexpr int NSC = decltype(ns_tag)::value;
 #pragma unroll
             for (int cb = 0; cb < NCB; ++cb) {
-                if (gz + g0 + cb >= G) continue;                // padding slot of an odd group
+                if (head_of(cb) >= G) continue;                 // padding slot of an odd group
+                if (QB2 && !qok_of(cb)) continue;
                 float f[NSC], lv[NSC];
 #pragma unroll
                 for (int s2 = 0; s2 < NSC; ++s2) {
@@ -485,13 +502,13 @@ __global__ __launch_bounds__((NCB == 1 && D <= 128) ? kPrefillOneHeadWaves * 64 
                 float lsum = 0.f;
 #pragma unroll
                 for (int s2 = 0; s2 < NSC; ++s2) { f[s2] = __builtin_amdgcn_exp2f(f[s2] - mm); lsum += lv[s2] * f[s2]; }
-                const uint32_t h = kvh * G + gz + g0 + cb;
-                const size_t pidx = ((size_t)qi * a.n_heads + h) * a.nk + kc;      // (key chunks: the partial of this chunk)
+                const uint32_t h = kvh * G + head_of(cb), qc = qi_of(cb);
+                const size_t pidx = ((size_t)qc * a.n_heads + h) * a.nk + kc;      // (key chunks: the partial of this chunk)
                 const float inv = a.so != nullptr ? 1.0f : 1.0f / lsum;
-                float* op = a.so != nullptr ? a.so + pidx * dr + kg * 4 : a.o + ((size_t)qi * a.n_heads + h) * dr + kg * 4;
+                float* op = a.so != nullptr ? a.so + pidx * dr + kg * 4 : a.o + ((size_t)qc * a.n_heads + h) * dr + kg * 4;
                 const float* gp = nullptr;
                 if (a.gate != nullptr) {
-                    const uint32_t i0 = (qi * a.n_heads + h) * dr;
+                    const uint32_t i0 = (qc * a.n_heads + h) * dr;
                     const uint32_t token = i0 / a.gchunk;
                     gp = a.gate + (size_t)token * a.gstride + a.goff + (i0 - token * a.gchunk) + kg * 4;
                 }
@@ -559,12 +576,13 @@ __global__ __launch_bounds__((NCB == 1 && D <= 128) ? kPrefillOneHeadWaves * 64 
     if (q_ok) {
 #pragma unroll
         for (int cb = 0; cb < NCB; ++cb) {
-            if (gz + g0 + cb >= G) continue;                                  // padding slot of an odd group
-            const uint32_t h = kvh * G + gz + g0 + cb;
+            if (head_of(cb) >= G) continue;                                   // padding slot of an odd group
+            if (QB2 && !qok_of(cb)) continue;
+            const uint32_t h = kvh * G + head_of(cb), qc = qi_of(cb);
             if (a.so != nullptr) {
                 // key chunks: the unnormalised partial of this chunk in the layout of the decode merge ([row][chunk][D], the
                 // maximum in natural-log units); a query that sees no key of the chunk leaves (0, "minus infinity", 0)
-                const size_t pidx = ((size_t)qi * a.n_heads + h) * a.nk + kc;
+                const size_t pidx = ((size_t)qc * a.n_heads + h) * a.nk + kc;
                 float* op = a.so + pidx * dr + dslice * DV + kg * 4;
 #pragma unroll
                 for (int dt = 0; dt < DTILES; ++dt) {
@@ -579,7 +597,7 @@ __global__ __launch_bounds__((NCB == 1 && D <= 128) ? kPrefillOneHeadWaves * 64 
                 continue;
             }
             const float inv = 1.0f / l_run[cb];
-            float* op = a.o + ((size_t)qi * a.n_heads + h) * dr + dslice * DV + kg * 4;   // lane (query n16) holds d = dslice*DV + dt*16 + kg*4 + i
+            float* op = a.o + ((size_t)qc * a.n_heads + h) * dr + dslice * DV + kg * 4;   // lane (query n16) holds d = dslice*DV + dt*16 + kg*4 + i
             if (a.gate != nullptr) {
 #pragma unroll
                 for (int dt = 0; dt < DTILES; ++dt) {

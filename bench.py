@@ -43,7 +43,7 @@ PROFILED_TRAFFIC = {
         "sources": ('attn_decode.hip', 'attn_decode_il.h', 'rope_device.h', 'device_utils.h'), "sha256_16": "b6d6b44e802c4527"},
     "prefill_fp8_512x4608_32layers": {
         "bytes": (19411 + 10240) * 1024, "profile": "profiles/prefill_fp8_512x4608_batch_dma_kernel.md",
-        "sources": ('attn_prefill.hip', 'attn_prefill_dma.h', 'device_utils.h'), "sha256_16": "bd15257c8b685b4f"},
+        "sources": ('attn_prefill.hip', 'attn_prefill_dma.h', 'device_utils.h'), "sha256_16": "02724788657c85e4"},
 }
 
 

@@ -402,7 +402,7 @@ def bench_decode(args, wl):
         floors = {"stream_floor_us": stream_us, "pattern_floor_us": pattern_us, "empty_launch_us": empty_us}
 
     mfma_worker = mfma_decode_worker(wl.dtype.label(), D)
-    f32_mfma = wl.dtype.label() == "FP32" and D in (64, 128, 256) and os.environ.get("VFKV_DECODE_WORKER", "m")[:1] != "v"
+    f32_mfma = wl.dtype.label() == "FP32" and (D in (64, 128, 256) or (64 < D < 256 and D % 16 == 0)) and os.environ.get("VFKV_DECODE_WORKER", "m")[:1] != "v"
     il_worker = mfma_worker and D in (64, 128, 256) and os.environ.get("VFKV_DECODE_IL", "1")[:1] != "0"   # (mirrors split_interleaves() of the library)
     worker_name = (("split_mfma_il_rope_kernel" if wl.rope else "split_mfma_il_kernel") if il_worker else "split_mfma_kernel" if mfma_worker
                    else "split_mfma_f32_kernel" if f32_mfma else "split_kernel")

@@ -58,8 +58,8 @@ const char* vfkv_status_string(int status);
 const char* vfkv_last_error(void);
 /* Advisory left by the last attention call of this thread ("" when there is none; never an error and never mixed into
  * vfkv_last_error): set when the shape fell to the generic fallback kernels (head_dim other than 64, 128, 256, 512 or a
- * multiple of 16 between 64 and 256 -- over F32 caches decode has tiled kernels for 64 / 128 / 256 only --, pointers not
- * 16-byte aligned, or a layer slab of 2 GiB or more), which are 50-100x slower than the tiled kernels. */
+ * multiple of 16 between 64 and 256 -- over F32 caches decode has no tiled kernel for 512 --, pointers not 16-byte aligned,
+ * or a layer slab of 2 GiB or more), which are 50-100x slower than the tiled kernels. */
 const char* vfkv_last_note(void);
 uint32_t vfkv_abi_version(void);
 /* Number of visible HIP devices (0 when there is none or the runtime cannot initialise). */

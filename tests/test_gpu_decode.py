@@ -94,10 +94,16 @@ CASES = [
     (vf.KvDtype.F8, 8, 2, 160, 700, 64, 0, 0.0),         # on the worker for 256
     (vf.KvDtype.F16, 16, 8, 192, 1300, 256, 300, 50.0),
     (vf.KvDtype.F16, 8, 4, 224, 500, 128, 0, 0.0),
+    (vf.KvDtype.F32, 4, 2, 96, 300, 64, 0, 0.0),         # F32 caches: the padded form of the f32 matrix-core worker
+    (vf.KvDtype.F32, 32, 32, 80, 1100, 256, 100, 20.0),
+    (vf.KvDtype.F32, 20, 1, 112, 700, 128, 0, 0.0),      # G = 20: slices of 16 and 4 heads
+    (vf.KvDtype.F32, 8, 4, 192, 900, 512, 333, 0.0),
+    (vf.KvDtype.F32, 6, 2, 160, 400, 64, 0, 50.0),
+    (vf.KvDtype.F32, 4, 4, 224, 200, 64, 0, 0.0),
     # shapes only the generic worker covers
     (vf.KvDtype.F32, 4, 2, 512, 200, 64, 0, 0.0),
     (vf.KvDtype.F32, 3, 1, 50, 100, 64, 0, 0.0),
-    (vf.KvDtype.F32, 4, 2, 96, 300, 64, 0, 0.0),
+    (vf.KvDtype.F16, 4, 2, 72, 300, 64, 0, 0.0),
     (vf.KvDtype.F16, 4, 2, 40, 200, 64, 0, 0.0),
 ]
 

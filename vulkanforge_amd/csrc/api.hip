@@ -641,7 +641,8 @@ uint32_t vfkv_decode_tile_for(uint32_t span, uint32_t n_heads, uint32_t n_kv_hea
     }
     // F32 caches on the f32 matrix instruction: one workgroup per CU as well, up to 16 heads of a group per workgroup
     static const bool valu_forced = [] { const char* e = getenv("VFKV_DECODE_WORKER"); return e && e[0] == 'v'; }();
-    if (kv_dtype == VFKV_F32 && !valu_forced && (head_dim == 64u || head_dim == 128u || head_dim == 256u)) {
+    if (kv_dtype == VFKV_F32 && !valu_forced &&
+        (head_dim == 64u || head_dim == 128u || head_dim == 256u || vfkv::split_padded_dim(kv_dtype, head_dim) != 0u)) {
         static const bool forced = getenv("VFKV_DECODE_TILE") != nullptr;
         if (span <= 256u && !forced) return 256u;
         return choose_tile(span, n_kv_heads, (g + 15u) / 16u, device_cus());

@@ -708,6 +708,18 @@ static hipError_t launch_split_il(const SplitArgs& a_in, uint32_t g, const RopeF
     return hipGetLastError();
 }
 
+// Head widths between the tiled ones (Phi-style 80 / 96, 112, 160, 192, 224): the width of the worker that serves them with
+// its tail masked off (the PAD forms of split_mfma_kernel and split_mfma_f32_kernel), 0 for every other width.
+uint32_t split_padded_dim(uint32_t dtype, uint32_t D) {
+    if (dtype > kF8 || D % 16u != 0u) return 0u;
+    return (D > 64u && D < 128u) ? 128u : (D > 128u && D < 256u) ? 256u : 0u;
+}
+
+// F32 caches on the f32 matrix instruction (attn_decode_f32.h)
+static bool f32_mfma_shape(uint32_t dtype, uint32_t D) {
+    return dtype == kF32 && (D == 64u || D == 128u || D == 256u || split_padded_dim(dtype, D) != 0u);
+}
+
 // Rows per run of the interleaved worker.  The full run is 32 rows (64 at head_dim 64): 8 KiB of K and V per wavefront in
 // flight over FP8 rows of 64 / 128 elements, 16 KiB over F16 rows of 64 / 128 and FP8 rows of 256, 32 KiB over F16 rows of 256.
 // Every shape also has a worker with runs of half that, and a launch takes whichever measured faster for its shape and its
@@ -731,32 +743,21 @@ static bool il_half_runs(uint32_t dtype, uint32_t D, uint32_t span_rows, uint32_
 
 // The shortest run the worker may take for this shape: what the caller sizes its workgroup count by.
 uint32_t split_run_rows(uint32_t dtype, uint32_t D) {
-    if (dtype == kF32 && (D == 64u || D == 128u || D == 256u)) return 16u;      // the F32 worker: one tile per run
+    if (f32_mfma_shape(dtype, D)) return 16u;                                   // the F32 worker: one tile per run
     if (const uint32_t dp = split_padded_dim(dtype, D)) return dp == 256u && dtype == kF16 ? 16u : 32u;   // as launch_split deals them
     if ((dtype != kF8 && dtype != kF16) || (D != 64u && D != 128u && D != 256u && D != 512u)) return 0u;
     return il_full_run(D) / 2u;      // (head_dim 512: 16 rows as well)
 }
 
-template <int D>
-static hipError_t launch_split_f32(const SplitArgs& a, uint32_t g, hipStream_t stream) {
+template <int D, bool PAD = false>
+static hipError_t launch_split_f32(const SplitArgs& a, uint32_t g, hipStream_t stream, uint32_t head_dim = (uint32_t)D) {
     constexpr int NW = kMfmaWaves;
     const uint32_t gt = g < 16u ? g : 16u;          // up to 16 heads of a group share a workgroup's K / V stream
     dim3 grid(a.n_kv_heads, a.n_tiles, (g + gt - 1u) / gt);
-    if (a.softcap > 0.f) hipLaunchKernelGGL((split_mfma_f32_kernel<D, NW, true>), grid, dim3(NW * kWave), 0, stream, a, gt);
-    else hipLaunchKernelGGL((split_mfma_f32_kernel<D, NW, false>), grid, dim3(NW * kWave), 0, stream, a, gt);
+    if (PAD && (head_dim >= (uint32_t)D || head_dim % 16u != 0u)) return hipErrorInvalidValue;
+    if (a.softcap > 0.f) hipLaunchKernelGGL((split_mfma_f32_kernel<D, NW, true, PAD>), grid, dim3(NW * kWave), 0, stream, a, gt, head_dim);
+    else hipLaunchKernelGGL((split_mfma_f32_kernel<D, NW, false, PAD>), grid, dim3(NW * kWave), 0, stream, a, gt, head_dim);
     return hipGetLastError();
-}
-
-// F32 caches on the f32 matrix instruction (attn_decode_f32.h)
-static bool f32_mfma_shape(uint32_t dtype, uint32_t D) {
-    return dtype == kF32 && (D == 64u || D == 128u || D == 256u);
-}
-
-// Head widths between the tiled ones (Phi-style 80 / 96, 112, 160, 192, 224) over FP8 / F16 rows: the width of the worker
-// that serves them with its tail masked off (split_mfma_kernel's PAD form), 0 for every other shape.
-uint32_t split_padded_dim(uint32_t dtype, uint32_t D) {
-    if ((dtype != kF8 && dtype != kF16) || D % 16u != 0u) return 0u;
-    return (D > 64u && D < 128u) ? 128u : (D > 128u && D < 256u) ? 256u : 0u;
 }
 
 // Shapes the matrix-core worker is built for (head_dim 512: two wavefronts per run, each half of the output columns).
@@ -922,7 +923,9 @@ hipError_t launch_split(const SplitLaunch& L, hipStream_t stream, bool* generic_
     if (aligned && out_aligned && slab_bytes < 0x7FFF0000ull && mfma_worker_enabled() && f32_mfma_shape(L.dtype, L.head_dim)) {
         if (L.head_dim == 64u) return launch_split_f32<64>(a, g, stream);
         if (L.head_dim == 128u) return launch_split_f32<128>(a, g, stream);
-        return launch_split_f32<256>(a, g, stream);
+        if (L.head_dim == 256u) return launch_split_f32<256>(a, g, stream);
+        if (L.head_dim < 128u) return launch_split_f32<128, true>(a, g, stream, L.head_dim);
+        return launch_split_f32<256, true>(a, g, stream, L.head_dim);
     }
     if (fast_shape(L.dtype, L.head_dim) && aligned && slab_bytes < 0x7FFF0000ull) {
 #define VFKV_CASE(DT, DD) \

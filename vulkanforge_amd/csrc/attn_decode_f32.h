@@ -29,8 +29,12 @@
 
 namespace vfkv {
 
-template <int D, int NW, bool CAP>
-__global__ __launch_bounds__(NW * 64) void split_mfma_f32_kernel(SplitArgs a, uint32_t gt) {
+// PAD: the heads are `head_dim` < D elements wide (a multiple of 16).  The kernel works on rows of D elements whose tail
+// does not exist: a lane's query elements past head_dim are zeros, its 16-byte pieces of a K or V row past the head are
+// the head's first piece read again (finite values that meet the zeros, or output elements nobody stores), and output
+// elements past head_dim are not stored.  Rows, queries and partials keep their real stride of head_dim.
+template <int D, int NW, bool CAP, bool PAD = false>
+__global__ __launch_bounds__(NW * 64) void split_mfma_f32_kernel(SplitArgs a, uint32_t gt, uint32_t head_dim) {
     constexpr int RUN = 16;                      // rows per run: one MFMA tile
     constexpr int NC = D / 4;                    // MFMA steps of the first product = elements of a row per lane group
     constexpr int KV4 = NC / 4;                  // 16-byte loads per lane and run (K)
@@ -54,10 +58,11 @@ __global__ __launch_bounds__(NW * 64) void split_mfma_f32_kernel(SplitArgs a, ui
     uint32_t tile_end = tile_base + a.tile; if (il || tile_end > a.seq_len) tile_end = a.seq_len;
     const uint32_t lo = tile_base > a.kv_start ? tile_base : a.kv_start;
 
-    const uint32_t row_stride = a.n_kv_heads * D * 4u;
+    const uint32_t dr = PAD ? head_dim : (uint32_t)D;                           // elements per head as the cache holds them
+    const uint32_t row_stride = a.n_kv_heads * dr * 4u;
     const __amdgpu_buffer_rsrc_t krsrc = __builtin_amdgcn_make_buffer_rsrc((void*)a.k, 0, a.seq_len * row_stride, 0x00020000);
     const __amdgpu_buffer_rsrc_t vrsrc = __builtin_amdgcn_make_buffer_rsrc((void*)a.v, 0, a.seq_len * row_stride, 0x00020000);
-    const uint32_t head_b = kvh * D * 4u;
+    const uint32_t head_b = kvh * dr * 4u;
     const uint32_t lane_koff = n16 * row_stride + head_b + kg * 16;              // row l % 16, pieces kg, kg + 4, ...
     const uint32_t lane_voff = kg * row_stride + head_b + n16 * 16;              // row l / 16 of a group of four, elements 4 (l % 16) .. + 3 of a block
     const float scale_l2 = a.scale * 1.44269504088896f;
@@ -75,14 +80,18 @@ __global__ __launch_bounds__(NW * 64) void split_mfma_f32_kernel(SplitArgs a, ui
     u32x4 vraw[4][VB];
     auto issue_k = [&](uint32_t off) {
 #pragma unroll
-        for (int x = 0; x < KV4; ++x) kraw[x] = __builtin_amdgcn_raw_buffer_load_b128(krsrc, lane_koff + x * 64, off, 0);
+        for (int x = 0; x < KV4; ++x)
+            kraw[x] = __builtin_amdgcn_raw_buffer_load_b128(krsrc, (PAD && (uint32_t)(kg * 16 + x * 64) >= dr * 4u) ? n16 * row_stride + head_b
+                                                                                                                : lane_koff + x * 64, off, 0);
     };
     auto issue_v = [&](uint32_t off) {
 #pragma unroll
         for (int g4 = 0; g4 < 4; ++g4)
 #pragma unroll
             for (int b = 0; b < VB; ++b)
-                vraw[g4][b] = __builtin_amdgcn_raw_buffer_load_b128(vrsrc, lane_voff + b * 256, off + (uint32_t)(g4 * 4) * row_stride, 0);
+                vraw[g4][b] = __builtin_amdgcn_raw_buffer_load_b128(vrsrc, (PAD && (uint32_t)(n16 * 16 + b * 256) >= dr * 4u) ? kg * row_stride + head_b
+                                                                                                                          : lane_voff + b * 256,
+                                                                    off + (uint32_t)(g4 * 4) * row_stride, 0);
     };
     const uint32_t off0 = active ? run_off(r0) : kOOB;
     issue_k(off0);
@@ -91,10 +100,12 @@ __global__ __launch_bounds__(NW * 64) void split_mfma_f32_kernel(SplitArgs a, ui
     float qf[NC];
     {
         const bool col_ok = (uint32_t)n16 < gcount;
-        const float* qrow = a.q + (size_t)(h0 + (col_ok ? n16 : 0)) * D + kg * 4;
+        const float* qrow = a.q + (size_t)(h0 + (col_ok ? n16 : 0)) * dr + kg * 4;
 #pragma unroll
         for (int x = 0; x < KV4; ++x) {
-            const float4 v = *reinterpret_cast<const float4*>(qrow + x * 16);
+            const bool piece_ok = !PAD || (uint32_t)(kg * 4 + x * 16) < dr;
+            float4 v = *reinterpret_cast<const float4*>(qrow + (piece_ok ? x * 16 : -kg * 4));
+            if (!piece_ok) v = make_float4(0.f, 0.f, 0.f, 0.f);
             qf[4 * x] = col_ok ? v.x : 0.f; qf[4 * x + 1] = col_ok ? v.y : 0.f;
             qf[4 * x + 2] = col_ok ? v.z : 0.f; qf[4 * x + 3] = col_ok ? v.w : 0.f;
         }
@@ -218,7 +229,7 @@ __global__ __launch_bounds__(NW * 64) void split_mfma_f32_kernel(SplitArgs a, ui
     // forward/runs.rs:776-821): the merge is a plain normalisation, done here, and no merge launch follows
     const bool direct = a.o_direct != nullptr;
     const float inv_l = direct ? __builtin_amdgcn_rcpf(l) : 1.0f;
-    float* const obase = direct ? a.o_direct + (size_t)(h0 + n16) * D : a.so + pidx * D;
+    float* const obase = direct ? a.o_direct + (size_t)(h0 + n16) * dr : a.so + pidx * dr;
 #pragma unroll
     for (int t = 0; t < MT; ++t) {
         float4_t o = fw[0] * part[t][0];
@@ -232,7 +243,8 @@ __global__ __launch_bounds__(NW * 64) void split_mfma_f32_kernel(SplitArgs a, ui
             const int dt = t * NW + w;
             float* const dst = obase + (dt / 4) * 64 + (kg * 4) * 4 + (dt % 4);
 #pragma unroll
-            for (int i = 0; i < 4; ++i) dst[i * 4] = o[i];
+            for (int i = 0; i < 4; ++i)
+                if (!PAD || (uint32_t)((dt / 4) * 64 + (kg * 4 + i) * 4 + (dt % 4)) < dr) dst[i * 4] = o[i];
         }
     }
     if (writer && w == 0 && kg == 0 && !direct) {

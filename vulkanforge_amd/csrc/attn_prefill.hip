@@ -127,7 +127,10 @@ static hipError_t launch_batch_kernels(const BatchLaunch& L, hipStream_t stream,
     // f16 matrix-core kernel: NCB heads per wavefront, private tiles per wavefront, no barrier in the loop
     if (mfma_ok) {
         // head_dim 512: one head per wavefront, and two wavefronts share a head (each owns half of the output columns)
-        const uint32_t nh = hd == 512u ? 2u : 1u;
+        // (also FP8 rows of 256 elements without grouping: 8 / 8 / 256, 512 queries over 4 608 keys, 76.3 us with two query
+        // blocks per wavefront, 56.4 us with two wavefronts per head; every grouped shape and F16 rows measured slower so:
+        // 16 / 8 / 256 FP8 87 -> 100 us, F16 105 -> 120 us)
+        const uint32_t nh = hd == 512u ? 2u : (hd == 256u && dpad == 0u && L.dtype == kF8 && g == 1u) ? 2u : 1u;
         // Heads per wavefront.  Two where the registers allow it (a K / V tile is then converted once for both); odd groups
         // of three and more heads round up, the spare slot computes on zeros and stores nothing.  Where the rows are wide
         // (F16 at head_dim 128, everything at head_dim 256) the traffic between L2 and the CUs is what binds: four / two heads
@@ -150,7 +153,7 @@ static hipError_t launch_batch_kernels(const BatchLaunch& L, hipStream_t stream,
         const uint32_t qblocks = qb2 ? (L.m + 31u) / 32u : (L.m + 15u) / 16u;   // query blocks = workgroups per (KV head, head slice)
         // wavefronts per workgroup the registers allow: one head per wavefront at head_dim <= 128 needs few (three wavefronts
         // per SIMD), 512 accumulator columns per wavefront need the whole register file of a SIMD (one wavefront per SIMD)
-        const uint32_t reg_waves = (ncb == 1u && hd <= 128u) ? (uint32_t)kPrefillOneHeadWaves
+        const uint32_t reg_waves = (ncb == 1u && hd <= 128u) ? (uint32_t)kPrefillOneHeadWaves : (hd == 256u && nh == 2u) ? 8u
                                  : (ncb * hd >= 512u || (L.dtype == kF16 && hd == 256u)) ? 4u : 8u;   // (always 4 at head_dim 512)
         // FP8 rows of 128 elements, two heads per wavefront: three raw V tiles per wavefront (filled by loads that write LDS)
         // instead of one f16 copy
@@ -274,6 +277,10 @@ static hipError_t launch_batch_kernels(const BatchLaunch& L, hipStream_t stream,
             VFKV_P2QB(kF8, 256, 1, false) VFKV_P2QB(kF16, 256, 1, false)
             VFKV_P2QB(kF8, 128, 2, true) VFKV_P2QB(kF16, 128, 1, true) VFKV_P2QB(kF8, 256, 1, true) VFKV_P2QB(kF16, 256, 1, true)
 #undef VFKV_P2QB
+            if (hd == 256u && nh == 2u) {
+                if (cap) hipLaunchKernelGGL((batch_mfma2_kernel<kF8, 256, 1, 1, true, 2>), grid, block, lds, stream, a, (int)hp, (int)ns);
+                else hipLaunchKernelGGL((batch_mfma2_kernel<kF8, 256, 1, 1, false, 2>), grid, block, lds, stream, a, (int)hp, (int)ns);
+            } else
             if (L.f16_weights && L.dtype == kF16 && L.head_dim == 128u && ncb == 4u) {
                 if (cap) hipLaunchKernelGGL((batch_mfma2_kernel<kF16, 128, 4, 1, true, 1, true>), grid, block, lds, stream, a, (int)hp, (int)ns);
                 else hipLaunchKernelGGL((batch_mfma2_kernel<kF16, 128, 4, 1, false, 1, true>), grid, block, lds, stream, a, (int)hp, (int)ns);

@@ -43,7 +43,7 @@ constexpr int kPrefillOneHeadWaves = 12;
 // head instead of two heads, so a workgroup covers 32 consecutive queries and a K / V tile is still widened and staged once
 // for two column blocks.  Head slot s of the workgroup's query planes then holds queries q0 + 16 (s % 2) .. of head s / 2.
 template <int DT, int D, int NCB, int PFD, bool CAP, int NH = 1, bool F16W = false, bool PAD = false, bool QB2 = false>
-__global__ __launch_bounds__((NCB == 1 && D <= 128) ? kPrefillOneHeadWaves * 64 : (NCB * D >= 512 || (DT == kF16 && D == 256)) ? 256 : 512) void batch_mfma2_kernel(BatchArgs a, int HP, int NS) {
+__global__ __launch_bounds__((NCB == 1 && D <= 128) ? kPrefillOneHeadWaves * 64 : (D == 256 && NH == 2) ? 512 : (NCB * D >= 512 || (DT == kF16 && D == 256)) ? 256 : 512) void batch_mfma2_kernel(BatchArgs a, int HP, int NS) {
     constexpr int DV = D / NH;                   // output elements (V columns) of this wavefront
     constexpr int ES = DT == kF16 ? 2 : 1;
     constexpr int KT = 32;                       // keys per tile

@@ -100,6 +100,15 @@ CASES = [
     (vf.KvDtype.F32, 8, 4, 192, 900, 512, 333, 0.0),
     (vf.KvDtype.F32, 6, 2, 160, 400, 64, 0, 50.0),
     (vf.KvDtype.F32, 4, 4, 224, 200, 64, 0, 0.0),
+    # FP8 heads of 64 elements over long spans (131 072 / n_kv_heads visible rows and more): interleaved launches take two
+    # neighbouring KV heads as one row of 128 bytes (groups of up to four heads)
+    (vf.KvDtype.F8, 32, 8, 64, 17000, 1024, 0, 0.0),     # G = 4: the eight heads of a pair fill the worker's columns
+    (vf.KvDtype.F8, 24, 8, 64, 20000, 512, 3000, 30.0),  # G = 3, window, soft-cap
+    (vf.KvDtype.F8, 6, 6, 64, 16500, 2048, 0, 0.0),      # G = 1
+    (vf.KvDtype.F8, 20, 4, 64, 16400, 4096, 0, 0.0),     # G = 5: too many heads for a pair, separate heads
+    (vf.KvDtype.F8, 12, 3, 64, 16400, 4096, 0, 0.0),     # odd number of KV heads: separate heads
+    (vf.KvDtype.F8, 32, 32, 64, 4500, 512, 300, 0.0),    # 32 KV heads: pairs from 4 096 visible rows on
+    (vf.KvDtype.F8, 64, 16, 64, 8300, 1024, 0, 20.0),    # 16 KV heads: from 8 192 on
     # shapes only the generic worker covers
     (vf.KvDtype.F32, 4, 2, 512, 200, 64, 0, 0.0),
     (vf.KvDtype.F32, 3, 1, 50, 100, 64, 0, 0.0),
@@ -339,6 +348,10 @@ def test_config2_fp8_outliers_append_then_decode_two_layers():
     (vf.KvDtype.F8, 32, 32, 96, 3000, 0),
     (vf.KvDtype.F16, 8, 4, 192, 2000, 500),
     (vf.KvDtype.F16, 32, 32, 80, 100, 0),       # one tile: the worker also writes the output
+    # FP8 heads of 64 elements taken in pairs (8 KV heads: at least 16 384 visible rows): the pair's workgroup writes both heads' slices
+    (vf.KvDtype.F8, 32, 8, 64, 33000, 0),
+    (vf.KvDtype.F8, 24, 8, 64, 40000, 20000),
+    (vf.KvDtype.F8, 32, 8, 64, 20000, 3000),    # a window shorter than that: separate heads
 ])
 def test_kv_write_attention_in_one_call_matches_the_two_calls(dtype, heads, hkv, d, ctx, window):
     # step_kv_write + step_attention (executor/attention.rs:546-625) through the single entry point: cache bytes and

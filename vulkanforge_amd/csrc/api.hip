@@ -685,6 +685,7 @@ static int decode_attention_impl(vfkv_cache* c, uint32_t layer, uint32_t kv_laye
     L.scale = scale; L.softcap = softcap;
     // the partials stay inside the workspace, so they need not correspond to tiles
     L.interleave = true;
+    L.rope = rope;                      // (the choice of worker below depends on it)
     // The interleaved worker deals the runs of the span to its workgroups whatever the tile length says: the workgroup count
     // is chosen directly (one per CU, none without a run), and the launch covers the rows from the 64-row boundary at or
     // below kv_start.
@@ -693,7 +694,8 @@ static int decode_attention_impl(vfkv_cache* c, uint32_t layer, uint32_t kv_laye
     if (streams != 0u) {
         const uint32_t run_rows = vfkv::split_run_rows(c->dtype, hd), nz = (n_heads / kvh + heads_per_wg - 1u) / heads_per_wg;
         const uint32_t runs = (seq_len - kv_start / 64u * 64u + run_rows - 1u) / run_rows;
-        uint32_t wgs = device_cus() / (kvh * nz);
+        const uint32_t kvh_wg = vfkv::split_pairs_heads(L) ? kvh / 2u : kvh;      // KV heads (or pairs of them) that get workgroups
+        uint32_t wgs = device_cus() / (kvh_wg * nz);
         if (wgs > (runs + streams - 1u) / streams) wgs = (runs + streams - 1u) / streams;   // none without a run
         if (wgs > (seq_len + 63u) / 64u) wgs = (seq_len + 63u) / 64u;   // what a workspace sized for this length holds (head_dim 512: two streams per workgroup)
         if (!static_ws && wgs > ws->max_tiles) wgs = ws->max_tiles;

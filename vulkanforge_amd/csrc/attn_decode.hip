@@ -667,16 +667,17 @@ constexpr int kSplitWaves = 4;
 // were each measured slower on the 32 k and 8 k FP8 workloads.
 constexpr int kMfmaWaves = 4;
 
-template <int DT, int D, int RUN, int PF, int NH = 1, bool PAD = false>
+template <int DT, int D, int RUN, int PF, int NH = 1, bool PAD = false, bool PAIR = false>
 static hipError_t launch_split_mfma(const SplitArgs& a, uint32_t g, hipStream_t stream, uint32_t head_dim = (uint32_t)D) {
     constexpr int NW = kMfmaWaves;
     const uint32_t gt = g < 8u ? g : 8u;
     dim3 grid(a.n_kv_heads, a.n_tiles, (g + gt - 1u) / gt);
     if (PAD && (head_dim >= (uint32_t)D || head_dim % 16u != 0u)) return hipErrorInvalidValue;
+    if (PAIR && (g > 8u || g % 2u != 0u)) return hipErrorInvalidValue;
     if (a.softcap > 0.f)
-        hipLaunchKernelGGL((split_mfma_kernel<DT, D, RUN, PF, NW, true, NH, PAD>), grid, dim3(NW * kWave), 0, stream, a, gt, head_dim);
+        hipLaunchKernelGGL((split_mfma_kernel<DT, D, RUN, PF, NW, true, NH, PAD, PAIR>), grid, dim3(NW * kWave), 0, stream, a, gt, head_dim);
     else
-        hipLaunchKernelGGL((split_mfma_kernel<DT, D, RUN, PF, NW, false, NH, PAD>), grid, dim3(NW * kWave), 0, stream, a, gt, head_dim);
+        hipLaunchKernelGGL((split_mfma_kernel<DT, D, RUN, PF, NW, false, NH, PAD, PAIR>), grid, dim3(NW * kWave), 0, stream, a, gt, head_dim);
     return hipGetLastError();
 }
 
@@ -771,12 +772,31 @@ static bool mfma_worker_enabled() {
     return on;
 }
 
+// FP8 heads of 64 elements are half a 128-byte memory line each: taken as separate KV heads (whose workgroups may sit on
+// different XCDs) every line of the cache is fetched twice.  Over long spans a launch that deals runs takes two neighbouring
+// KV heads as one row of 128 bytes instead (split_mfma_kernel's PAIR form), when the pair's query heads fit one workgroup
+// (2 G <= 8).  Us per layer, worker + merge, separate heads -> pairs: 32 / 8 / 64 at 65 536 rows 23.1 -> 17.1, 32 768 rows
+// 14.1 -> 11.6, 16 384 rows 9.7 -> 9.4, 12 288 rows 8.4 -> 9.0; 16 / 16 / 64 at 16 384 rows 14.7 -> 11.6, 8 192 rows 9.5 -> 8.4,
+// 4 096 rows 7.2 -> 7.5; 32 / 32 / 64 at 8 192 rows 14.3 -> 11.1, 4 096 rows 9.7 -> 8.6, 2 048 rows level: pairs pay from about
+// 131 072 / n_kv_heads visible rows on.
+bool split_pairs_heads(const SplitLaunch& L) {
+    static const bool off = [] { const char* e = getenv("VFKV_DECODE_PAIRS"); return e && e[0] == '0'; }();   // for comparisons
+    if (off || !L.interleave || L.rope != nullptr || L.dtype != kF8 || L.head_dim != 64u || L.n_kv_heads == 0u || L.n_kv_heads % 2u != 0u)
+        return false;
+    const uint32_t g = L.n_heads / L.n_kv_heads;
+    const uint32_t min_rows = 131072u / L.n_kv_heads;      // 16 384 visible rows with 8 KV heads, 8 192 with 16, 4 096 with 32
+    if (g == 0u || g > 4u || L.n_heads % L.n_kv_heads != 0u || L.seq_len < L.kv_start + min_rows) return false;
+    const bool aligned = ((((uintptr_t)L.k) | ((uintptr_t)L.v) | ((uintptr_t)L.q) | ((uintptr_t)L.scratch_out) | ((uintptr_t)L.o_direct)) & 15u) == 0u;
+    const uint64_t slab_bytes = (uint64_t)L.seq_len * L.n_kv_heads * L.head_dim;
+    return aligned && slab_bytes < 0x7FFF0000ull && mfma_worker_enabled();
+}
+
 // Run streams per workgroup of a launch that deals the runs of the whole span to its workgroups whatever the tile length
 // says (0: the launch keeps partial j = tile j): four for the interleaved worker and the F32 worker, two at head_dim 512,
 // where two wavefronts share a run.  *heads_per_wg: query heads of a GQA group that one workgroup serves.
 uint32_t split_run_streams(const SplitLaunch& L, uint32_t* heads_per_wg) {
     if (heads_per_wg) *heads_per_wg = 8u;
-    if (split_interleaves(L)) return (uint32_t)kMfmaWaves;
+    if (split_pairs_heads(L) || split_interleaves(L)) return (uint32_t)kMfmaWaves;
     if (!L.interleave || L.n_kv_heads == 0u) return 0u;
     const bool aligned = ((((uintptr_t)L.k) | ((uintptr_t)L.v) | ((uintptr_t)L.q) | ((uintptr_t)L.scratch_out) | ((uintptr_t)L.o_direct)) & 15u) == 0u;
     const uint64_t slab_bytes = (uint64_t)L.seq_len * L.n_kv_heads * L.head_dim * elem_size(L.dtype);
@@ -823,6 +843,7 @@ bool split_appends(const SplitLaunch& L) {
     const uint32_t g = L.n_heads / L.n_kv_heads;
     const bool aligned = ((((uintptr_t)L.k) | ((uintptr_t)L.v) | ((uintptr_t)L.q) | ((uintptr_t)L.k_new) | ((uintptr_t)L.v_new) |
                            ((uintptr_t)L.scratch_out)) & 15u) == 0u;
+    if (split_pairs_heads(L)) return aligned && L.append_pos < L.seq_len && L.append_pos >= L.kv_start;   // (split_mfma_kernel, one head slice)
     if (split_interleaves(L)) return aligned && L.append_pos + 1u == L.seq_len && L.append_pos >= L.kv_start;
     const uint64_t slab_bytes = (uint64_t)L.seq_len * L.n_kv_heads * L.head_dim * elem_size(L.dtype);
     const bool mfma_shape = mfma_worker_shape(L.dtype, L.head_dim);
@@ -841,7 +862,7 @@ bool split_writes_output(const SplitLaunch& L) {
 
 bool split_interleaves(const SplitLaunch& L) {
     static const bool off = [] { const char* e = getenv("VFKV_DECODE_IL"); return e && e[0] == '0'; }();
-    if (off || !L.interleave || L.n_kv_heads == 0u || L.n_tiles == 0u) return false;
+    if (off || !L.interleave || L.n_kv_heads == 0u || L.n_tiles == 0u || split_pairs_heads(L)) return false;
     const bool aligned = ((((uintptr_t)L.k) | ((uintptr_t)L.v) | ((uintptr_t)L.q) | ((uintptr_t)L.scratch_out) | ((uintptr_t)L.o_direct)) & 15u) == 0u;
     const uint64_t slab_bytes = (uint64_t)L.seq_len * L.n_kv_heads * L.head_dim * elem_size(L.dtype);
     return aligned && slab_bytes < 0x7FFF0000ull && mfma_worker_enabled() && (L.dtype == kF8 || L.dtype == kF16) &&
@@ -883,6 +904,11 @@ hipError_t launch_split(const SplitLaunch& L, hipStream_t stream, bool* generic_
     // the matrix-core worker also stores its partials (or the output) 16 bytes at a time
     const bool out_aligned = ((((uintptr_t)L.scratch_out) | ((uintptr_t)L.o_direct)) & 15u) == 0u;
     if (L.rope != nullptr && !split_folds_rope(L)) return hipErrorInvalidValue;      // the caller rotates in a launch of its own then
+    if (split_pairs_heads(L) && out_aligned) {     // two 64-wide FP8 heads as one row of 128: half as many KV heads, twice the group
+        SplitArgs ap = a;
+        ap.n_kv_heads = a.n_kv_heads / 2u; ap.group = a.group * 2u;
+        return launch_split_mfma<kF8, 128, 32, 1, 1, false, true>(ap, ap.group, stream);
+    }
     if (split_interleaves(L) && out_aligned) {
         const uint32_t base_row = a.tile_first * a.tile;
         const bool half = il_half_runs(L.dtype, L.head_dim, a.seq_len > base_row ? a.seq_len - base_row : 0u, a.n_tiles);

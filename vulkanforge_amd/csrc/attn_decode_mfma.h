@@ -40,7 +40,14 @@ namespace vfkv {
 // planes hold zeros there, the lanes whose 16-byte piece of a K or V row would lie past the head read the head's first
 // piece again (finite cache values that meet query zeros, or output columns nobody stores), and the d-tiles past head_dim
 // are neither multiplied nor stored.  Rows, queries, partials and the appended row keep their real stride of head_dim.
-template <int DT, int D, int RUN, int PF, int NW, bool CAP, int NH = 1, bool PAD = false>
+//
+// PAIR (D == 128, NH == 1): the cache holds heads of 64 elements, and the kernel takes two neighbouring KV heads as one row
+// of 128 (over FP8 rows a head's 64 bytes are half a memory line: as separate heads, possibly on different XCDs, every line
+// is fetched twice).  a.n_kv_heads counts the pairs and a.group the query heads of a pair (2 G <= 8, those of the first KV
+// head first, as the model numbers them).  A query occupies its own KV head's half of the 128-wide plane row and zeros the
+// other half, so its scores only see its own K; of its output row only its own V half is stored.  The cache side
+// (rows, the appended row) is exactly that of a head_dim 128 cache with half as many heads.
+template <int DT, int D, int RUN, int PF, int NW, bool CAP, int NH = 1, bool PAD = false, bool PAIR = false>
 __global__ __launch_bounds__(NW * 64) void split_mfma_kernel(SplitArgs a, uint32_t gt, uint32_t head_dim) {
     constexpr int ES = DT == kF16 ? 2 : 1;
     constexpr int DV = D / NH;                   // output columns of a wavefront
@@ -67,6 +74,8 @@ __global__ __launch_bounds__(NW * 64) void split_mfma_kernel(SplitArgs a, uint32
     constexpr int LROWS = RUN > MERGE_ROWS ? RUN : MERGE_ROWS;
     static_assert(NW % NH == 0, "whole run streams");
     static_assert(!PAD || NH == 1, "padded heads: one wavefront per run");
+    static_assert(!PAIR || (D == 128 && NH == 1 && !PAD), "pairs of 64-wide heads");
+    constexpr int QD = PAIR ? 64 : D;                                   // elements of a query / output row (PAD: dr)
     const uint32_t dr = PAD ? head_dim : (uint32_t)D;                   // elements per head as the cache holds them
 
     __shared__ __attribute__((aligned(16))) _Float16 vlds[NW][LROWS * VPITCH];
@@ -134,7 +143,7 @@ __global__ __launch_bounds__(NW * 64) void split_mfma_kernel(SplitArgs a, uint32
         vraw[b][c] = __builtin_amdgcn_raw_buffer_load_b128(vrsrc, lane_voff, off + (uint32_t)(c * VROWS) * row_stride, 0);
     };
 
-    if (PAD) {                                                      // the query planes' tails stay zero (nothing is in flight yet: the barrier is cheap here)
+    if (PAD || PAIR) {                                              // the query planes' tails stay zero (nothing is in flight yet: the barrier is cheap here)
         for (int i = tid; i < 16 * (D + 8) / 8; i += NW * 64) reinterpret_cast<u32x4*>(&qlds[0][0])[i] = u32x4{0u, 0u, 0u, 0u};
         __syncthreads();
     }
@@ -197,12 +206,12 @@ __global__ __launch_bounds__(NW * 64) void split_mfma_kernel(SplitArgs a, uint32
     // remainder planes in LDS; lane (column n16, group kg) then holds q[kg*SEG + c*8 + j], j < 8, per k-step c.
     // The query load sits between the K and the V requests: loads return in order, so the wait for it covers K only.
     constexpr int QLD = (8 * D / 4 + NW * 64 - 1) / (NW * 64);      // 16-byte query loads per thread (<= 8 heads)
-    const int nq4 = (int)(gcount * dr) / 4;
+    const int nq4 = PAIR ? (int)gcount * (QD / 4) : (int)(gcount * dr) / 4;
     float4 qf[QLD];
 #pragma unroll
     for (int i = 0; i < QLD; ++i) {
         const int idx = tid + i * NW * 64;
-        qf[i] = *reinterpret_cast<const float4*>(a.q + (size_t)h0 * dr + (idx < nq4 ? idx : 0) * 4);
+        qf[i] = *reinterpret_cast<const float4*>(a.q + (size_t)h0 * (PAIR ? (uint32_t)QD : dr) + (idx < nq4 ? idx : 0) * 4);
     }
 #pragma unroll
     for (int c = 0; c < VLD; ++c) issue_v(0, c, off0);
@@ -220,7 +229,9 @@ __global__ __launch_bounds__(NW * 64) void split_mfma_kernel(SplitArgs a, uint32
             const int idx = tid + i * NW * 64;
             if (idx >= nq4) continue;
             const float4 f = qf[i];
-            const int g = PAD ? (int)((uint32_t)(idx * 4) / dr) : (idx * 4) / D, d = PAD ? idx * 4 - g * (int)dr : (idx * 4) % D;
+            const int g = PAD ? (int)((uint32_t)(idx * 4) / dr) : (idx * 4) / QD;
+            // (PAIR: the heads of the pair's second KV head use the second half of the row)
+            const int d = PAD ? idx * 4 - g * (int)dr : (idx * 4) % QD + ((PAIR && hz + (uint32_t)g >= g_all / 2u) ? 64 : 0);
             const float v4[4] = {f.x, f.y, f.z, f.w};
             _Float16 hv[4], lv[4];
 #pragma unroll
@@ -429,7 +440,8 @@ __global__ __launch_bounds__(NW * 64) void split_mfma_kernel(SplitArgs a, uint32
     // forward/runs.rs:776-821): the merge is a plain normalisation, done here, and no merge launch follows
     const bool direct = a.o_direct != nullptr;
     const float inv_l = direct ? __builtin_amdgcn_rcpf(l) : 1.0f;
-    float* const obase = (direct ? a.o_direct + (size_t)(h0 + col) * dr : a.so + pidx * dr) + ds * DV;
+    float* const obase = (direct ? a.o_direct + (size_t)(h0 + col) * (PAIR ? (uint32_t)QD : dr) : a.so + pidx * (PAIR ? (uint32_t)QD : dr)) + ds * DV;
+    const bool second_half = PAIR && (hz + (uint32_t)col) >= g_all / 2u;     // PAIR: this column's head belongs to the pair's second KV head
 #pragma unroll
     for (int t = 0; t < MT; ++t) {
         float4_t o = fw[0] * part[t][0];
@@ -439,6 +451,10 @@ __global__ __launch_bounds__(NW * 64) void split_mfma_kernel(SplitArgs a, uint32
             const float r = inv_l * (2.0f - l * inv_l);
             o *= r;
         }
+        if (PAIR) {                                    // d-tiles 0-3 are the first KV head's V columns, 4-7 the second's
+            const int dt = t * NP + wp;
+            if (writer && (dt >= 4) == second_half) *reinterpret_cast<float4_t*>(obase + (dt & 3) * 16 + kg * 4) = o;
+        } else
         if (writer && (!PAD || (uint32_t)(t * NP + wp) * 16u < dr)) *reinterpret_cast<float4_t*>(obase + (t * NP + wp) * 16 + kg * 4) = o;
     }
     if (writer && w == 0 && kg == 0 && a.o_direct == nullptr) {

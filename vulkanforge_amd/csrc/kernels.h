@@ -95,6 +95,9 @@ hipError_t launch_sigmoid_mul(float* data, uint32_t ne, const GateArgs& gate, hi
 // workgroups per KV head whatever L.tile says, so the caller may choose n_tiles freely), and when that worker would also
 // fold L.rope (which needs k_new / v_new as well).
 bool split_interleaves(const SplitLaunch& a);
+// True when launch_split will take pairs of neighbouring 64-wide FP8 KV heads as rows of 128 bytes (long spans, groups of up
+// to four heads, no folded RoPE): the launch then has half as many KV heads to give workgroups to.
+bool split_pairs_heads(const SplitLaunch& a);
 bool split_folds_rope(const SplitLaunch& a);
 // Width of the matrix-core worker that serves this head width with its tail masked off (FP8 / F16 rows of 80 / 96 / 112 ->
 // 128, 160 / 192 / 224 -> 256); 0 for every other shape.

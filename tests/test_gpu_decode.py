@@ -525,7 +525,8 @@ def test_shapes_on_the_generic_fallback_leave_a_note():
     # and vfkv_last_note says that the call was a slow one; a shape on the tiled kernels clears it
     L = vf._ffi.lib()
     r = rng(80)
-    for d, slow in ((72, True), (80, False), (128, False)):
+    valu = os.environ.get("VFKV_DECODE_WORKER", "")[:1] == "v"     # (that switch keeps the padded widths off the matrix-core worker)
+    for d, slow in ((72, True), (80, valu), (128, False)):
         heads, hkv, seq = 8, 2, 300
         q = fp16_normal(r, (heads, d))
         k, v = encode_np(fp16_normal(r, (seq, hkv, d)), vf.KvDtype.F16), encode_np(fp16_normal(r, (seq, hkv, d)), vf.KvDtype.F16)

@@ -266,6 +266,9 @@ FOLD_CASES = [
     (vf.KvDtype.F8, 96, 8, 128, 2049, 128, _ffi.ROPE_NEOX, True, False, 0, 0.0),     # 12 heads per KV head: two head slices
     (vf.KvDtype.F8, 4, 1, 512, 700, 128, _ffi.ROPE_NEOX, True, False, 0, 0.0),       # head_dim 512: the separate RoPE launch
     (vf.KvDtype.F32, 8, 2, 128, 600, 128, _ffi.ROPE_NEOX, True, False, 0, 0.0),      # F32 cache: the separate RoPE launch
+    (vf.KvDtype.F8, 64, 32, 64, 5000, 64, _ffi.ROPE_NEOX, True, False, 0, 0.0),      # FP8 heads of 64, 32 KV heads, 5 000 rows: folded, separate heads
+    (vf.KvDtype.F8, 64, 32, 64, 12500, 64, _ffi.ROPE_NEOX, True, False, 0, 0.0),     # 12 500 rows: the separate RoPE launch in front of paired KV heads
+    (vf.KvDtype.F16, 32, 32, 96, 1500, 96, _ffi.ROPE_NEOX, False, False, 0, 0.0),    # head_dim 96 (padded worker): the separate RoPE launch
 ]
 
 
@@ -318,7 +321,9 @@ def test_qk_rope_kv_write_decode_attention_equals_the_separate_calls(dtype, head
     (rk, rv, rq, rko, ro), (sk, sv, sq, sko, so_) = got
     assert (rk == sk).all() and (rv == sv).all()            # cache bytes
     assert (rq == sq).all() and (rko == sko).all()          # rotated queries and K row
-    assert np.abs(ro - so_).max() < 2e-6
+    # (the two paths may run on different workers -- the fold stays with separate KV heads where the separate calls pair FP8
+    # heads of 64 elements -- so their outputs agree to f32 rounding at the outputs' magnitude, not bit for bit)
+    assert np.abs(ro - so_).max() < 2e-6 * max(1.0, float(np.abs(so_).max()))
     # against the oracle.  The rotation: within one ulp of the f32 angle of the oracle's (the slack the reference grants its own GPU
     # at tests/correctness.rs:799-815), the stored K code a correct rounding of a value inside that band
     q_ref = oracle.rms_norm_rope(q[None], np.array([pos], np.int32), d, rotary, ts, mode=mode, weight=qw, ff=ffv, eps=1e-6)[0]

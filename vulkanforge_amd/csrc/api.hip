@@ -685,7 +685,12 @@ static int decode_attention_impl(vfkv_cache* c, uint32_t layer, uint32_t kv_laye
     L.scale = scale; L.softcap = softcap;
     // the partials stay inside the workspace, so they need not correspond to tiles
     L.interleave = true;
-    L.rope = rope;                      // (the choice of worker below depends on it)
+    // (the choice of worker below depends on whether the token's rotation will be folded into it)
+    if (rope) {
+        vfkv::SplitLaunch T = L;
+        T.k_new = k_new; T.v_new = v_new; T.append_pos = position; T.rope = rope;
+        L.rope = vfkv::split_folds_rope(T) ? rope : nullptr;
+    }
     // The interleaved worker deals the runs of the span to its workgroups whatever the tile length says: the workgroup count
     // is chosen directly (one per CU, none without a run), and the launch covers the rows from the 64-row boundary at or
     // below kv_start.

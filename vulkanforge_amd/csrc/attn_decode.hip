@@ -871,6 +871,14 @@ bool split_interleaves(const SplitLaunch& L) {
 
 bool split_folds_rope(const SplitLaunch& L) {
     if (!L.rope || !split_interleaves(L) || !split_appends(L)) return false;
+    {   // FP8 heads of 64 elements over very long spans: the rotation as a launch of its own in front of paired KV heads beats
+        // the fold into the worker for separate heads (32 / 8 / 64, us per 8-layer step, fold -> rotation launch + pairs:
+        // 16 385 keys 90.7 -> 111.9, 32 769 keys 121.8 -> 128.4, 65 537 keys 194.1 -> 171.6): no fold from three times the
+        // span at which pairs start to pay
+        SplitLaunch P = L;
+        P.rope = nullptr; P.k_new = nullptr; P.v_new = nullptr;
+        if (split_pairs_heads(P) && L.seq_len >= L.kv_start + 3u * (131072u / L.n_kv_heads)) return false;
+    }
     const RopeFold& r = *L.rope;
     const bool aligned = ((((uintptr_t)r.q_out) | ((uintptr_t)r.k_out)) & 3u) == 0u;
     return aligned && r.rotary_dim % 2u == 0u && r.rotary_dim <= L.head_dim && (r.mode == 0u || r.mode == 2u);

@@ -40,7 +40,7 @@ MFMA_F32_PEAK_TFLOPS = 157.3      # dense f32 matrix rate: what an F32 cache is 
 PROFILED_TRAFFIC = {
     "decode_fp8_32k_32layers": {
         "bytes": (65690 + 520) * 1024, "profile": "profiles/decode_fp8_32k_split_mfma_il_kernel.md",
-        "sources": ('attn_decode.hip', 'attn_decode_il.h', 'rope_device.h', 'device_utils.h'), "sha256_16": "078d12de4fc4ca9d"},
+        "sources": ('attn_decode.hip', 'attn_decode_il.h', 'rope_device.h', 'device_utils.h'), "sha256_16": "20976d6933688778"},
     "prefill_fp8_512x4608_32layers": {
         "bytes": (19411 + 10240) * 1024, "profile": "profiles/prefill_fp8_512x4608_batch_dma_kernel.md",
         "sources": ('attn_prefill.hip', 'attn_prefill_dma.h', 'device_utils.h'), "sha256_16": "01810eb838265063"},
